@@ -1,0 +1,175 @@
+"""Pins oracle/model.py against library routines, closed forms and the reference's own
+forward invariants (reference tests/model_test.py:188-199, 443-473)."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from olmo_amd.config import ModelConfig
+from oracle import model as om
+
+
+def tiny_cfg(olmo2=True, **kw):
+    base = dict(d_model=64, n_heads=4, n_layers=3, mlp_ratio=4, rope=True, alibi=False, include_bias=False,
+                weight_tying=False, vocab_size=250, embedding_size=256, max_sequence_length=64,
+                attention_dropout=0.0, residual_dropout=0.0, embedding_dropout=0.0)
+    if olmo2:
+        base.update(layer_norm_type="rms", layer_norm_with_affine=True, layer_norm_eps=1e-6,
+                    attention_layer_norm=True, norm_after=True, rope_theta=500000)
+    else:
+        base.update(layer_norm_type="default", layer_norm_with_affine=False, layer_norm_eps=1e-5,
+                    attention_layer_norm=False, norm_after=False)
+    base.update(kw)
+    return ModelConfig(**base)
+
+
+def test_layer_norm_is_textbook():
+    x = torch.randn(16, 33, 48)
+    y = om.layer_norm_np(x, 1e-5)
+    mu = x.double().mean(-1, keepdim=True)
+    var = ((x.double() - mu) ** 2).mean(-1, keepdim=True)  # biased
+    ref = ((x.double() - mu) / torch.sqrt(var + 1e-5)).float()
+    assert torch.allclose(y, ref, atol=2e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rms_norm_closed_form_and_rounding_points(dtype):
+    torch.manual_seed(0)
+    x = (torch.randn(7, 256) * 3).to(dtype)
+    w = (1 + 0.1 * torch.randn(256)).to(dtype)
+    y = om.rms_norm(x, w, 1e-6)
+    xd = x.double()
+    n = xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + 1e-6)
+    if dtype == torch.float32:
+        assert torch.allclose(y.double(), n * w.double(), rtol=1e-5, atol=1e-6)
+    else:
+        # two roundings: normalised value to bf16, then the product to bf16 (olmo/model.py:247-253).
+        # n.float() first: the reference normalises in fp32, and going fp64->bf16 directly could
+        # differ by double rounding only on exact ties, which random data does not hit
+        two = (n.float().to(dtype).double() * w.double()).float().to(dtype)
+        assert torch.equal(y, two)
+        one = (n * w.double()).float().to(dtype)
+        assert not torch.equal(y, one)  # the single-rounding variant is a different function
+    # weight == 1 reduces to x / rms(x)
+    y1 = om.rms_norm(x, torch.ones(256, dtype=dtype), 1e-6)
+    assert torch.allclose(y1.double(), n, rtol=1e-2 if dtype != torch.float32 else 1e-5, atol=1e-6)
+
+
+def test_rope_closed_form_and_invariants():
+    hd, theta, L = 32, 10000.0, 50
+    sin, cos = om.rope_tables(hd, theta, L)
+    # closed form in fp64: angle(p, j) = p * theta^(-2(j mod hd/2)/hd)
+    p = torch.arange(L, dtype=torch.float64)[:, None]
+    j = torch.arange(hd)[None, :] % (hd // 2)
+    ang = p * theta ** (-2.0 * j.double() / hd)
+    assert torch.allclose(sin.double(), ang.sin(), atol=2e-5) and torch.allclose(cos.double(), ang.cos(), atol=2e-5)
+    torch.manual_seed(1)
+    q = torch.randn(1, 2, L, hd)
+    k = torch.randn(1, 2, L, hd)
+    rq, rk = om.apply_rope(q, sin, cos), om.apply_rope(k, sin, cos)
+    assert torch.equal(rq[:, :, 0], q[:, :, 0])  # position 0 is the identity
+    # pairs (i, i+hd/2) are rotated: norms preserved
+    n0 = q[..., : hd // 2] ** 2 + q[..., hd // 2 :] ** 2
+    n1 = rq[..., : hd // 2] ** 2 + rq[..., hd // 2 :] ** 2
+    assert torch.allclose(n0, n1, rtol=1e-4, atol=1e-5)
+    # explicit complex rotation: (x1 + i x2) * exp(i ang)
+    z = torch.complex(q[..., : hd // 2].double(), q[..., hd // 2 :].double()) * torch.polar(
+        torch.ones(L, hd // 2, dtype=torch.float64), ang[:, : hd // 2])
+    assert torch.allclose(rq[..., : hd // 2].double(), z.real, atol=1e-4)
+    assert torch.allclose(rq[..., hd // 2 :].double(), z.imag, atol=1e-4)
+    # <rope(q,m), rope(k,n)> depends on m-n only
+    qq, kk = q[:, :, :1].expand(-1, -1, L, -1), k[:, :, :1].expand(-1, -1, L, -1)
+    a, b = om.apply_rope(qq, sin, cos), om.apply_rope(kk, sin, cos)
+    d1 = (a[:, :, 10] * b[:, :, 7]).sum(-1)
+    d2 = (a[:, :, 30] * b[:, :, 27]).sum(-1)
+    assert torch.allclose(d1, d2, atol=1e-4)
+
+
+def test_attention_matches_sdpa_and_bruteforce():
+    torch.manual_seed(2)
+    B, H, T, hd = 2, 3, 9, 16
+    q, k, v = torch.randn(B, H, T, hd), torch.randn(B, H, T, hd), torch.randn(B, H, T, hd)
+    ref = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+    out = om.attention(q, k, v, None, torch.float32)
+    assert torch.allclose(out, ref, atol=1e-5, rtol=1e-4)
+    # decode form: 1 query at the end of L keys == last row of the causal result
+    out1 = om.attention(q[:, :, -1:], k, v, None, torch.float32)
+    assert torch.allclose(out1, ref[:, :, -1:], atol=1e-5, rtol=1e-4)
+    # brute force one element
+    b, h, t = 1, 2, 5
+    s = [(q[b, h, t] @ k[b, h, j]).item() / math.sqrt(hd) for j in range(t + 1)]
+    m = max(s)
+    e = [math.exp(x - m) for x in s]
+    o = sum(e[j] / sum(e) * v[b, h, j] for j in range(t + 1))
+    assert torch.allclose(out[b, h, t], o, atol=1e-5)
+    # explicit additive bias path (as used with a cache) equals the causal path
+    L = T
+    bias = torch.triu(torch.ones(L, L), diagonal=1)
+    bias = bias.masked_fill(bias == 1, torch.finfo(torch.float).min).view(1, 1, L, L)
+    assert torch.allclose(om.attention(q, k, v, bias, torch.float32), ref, atol=1e-5, rtol=1e-4)
+    # GQA repeats kv heads
+    k2, v2 = k[:, :1], v[:, :1]
+    ref2 = F.scaled_dot_product_attention(q, k2.expand(-1, H, -1, -1), v2.expand(-1, H, -1, -1), is_causal=True)
+    assert torch.allclose(om.attention(q, k2, v2, None, torch.float32), ref2, atol=1e-5, rtol=1e-4)
+
+
+def test_swiglu_order():
+    x = torch.randn(4, 10)
+    assert torch.equal(om.swiglu(x), F.silu(x[:, 5:]) * x[:, :5])
+    xb = x.bfloat16()
+    # bf16 silu == fp32 silu rounded once, then a bf16 multiply
+    s = F.silu(xb[:, 5:].float()).bfloat16()
+    assert torch.equal(om.swiglu(xb), (s.float() * xb[:, :5].float()).bfloat16())
+
+
+@pytest.mark.parametrize("olmo2", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_forward_invariants(olmo2, dtype):
+    """Reference tests/model_test.py:158-199: padded batch == single sequences; cache == full."""
+    cfg = tiny_cfg(olmo2)
+    w = om.random_weights(cfg, dtype, seed=5, norm_weight_std=0.1 if olmo2 else 0.0)
+    m = om.OracleModel(cfg, w, dtype)
+    gen = torch.Generator().manual_seed(0)
+    ids1 = torch.randint(0, 250, (1, 12), generator=gen)
+    ids2 = torch.randint(0, 250, (1, 7), generator=gen)
+    tol = dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32 else dict(atol=6e-2, rtol=0)
+    l1, _ = m.forward(ids1)
+    l2, _ = m.forward(ids2)
+    # right padding + attention_mask
+    batch = torch.zeros(2, 12, dtype=torch.long)
+    batch[0] = ids1[0]
+    batch[1, :7] = ids2[0]
+    mask = torch.zeros(2, 12)
+    mask[0] = 1
+    mask[1, :7] = 1
+    lb, _ = m.forward(batch, attention_mask=mask)
+    assert torch.allclose(lb[0].float(), l1[0].float(), **tol)
+    assert torch.allclose(lb[1, :7].float(), l2[0].float(), **tol)
+    # cache: prefix then the last token
+    lp, kv = m.forward(ids1[:, :-1], use_cache=True)
+    assert len(kv) == cfg.n_layers and kv[0][0].shape == (1, cfg.n_heads, 11, cfg.d_model // cfg.n_heads)
+    ll, kv2 = m.forward(ids1[:, -1:], past_key_values=kv, use_cache=True)
+    assert kv2[0][0].shape[-2] == 12
+    assert torch.allclose(ll[:, -1].float(), l1[:, -1].float(), **tol)
+    # last_logits_only
+    lo, _ = m.forward(ids1, last_logits_only=True)
+    assert lo.shape == (1, 1, 256) and torch.allclose(lo[:, 0].float(), l1[:, -1].float(), **tol)
+
+
+def test_forward_quantised_linear_equals_dense_on_dequantised_weights():
+    cfg = tiny_cfg(True, d_model=128, n_heads=4, mlp_ratio=4)
+    wq = om.random_weights(cfg, torch.bfloat16, seed=9, quantized=True)
+    from oracle import w4
+    wd = {}
+    for k_, v_ in wq.items():
+        if k_.endswith(".qweight"):
+            p = k_[: -len(".qweight")]
+            W = w4.dequantize(wq[p + ".qweight"], wq[p + ".qzeros"], wq[p + ".scales"], 128)  # [K,N] fp16
+            wd[p + ".weight"] = W.t().contiguous()
+        elif not (k_.endswith(".qzeros") or k_.endswith(".scales")):
+            wd[k_] = v_
+    ids = torch.randint(0, 250, (2, 9), generator=torch.Generator().manual_seed(3))
+    a, _ = om.OracleModel(cfg, wq, torch.bfloat16).forward(ids)
+    b, _ = om.OracleModel(cfg, wd, torch.bfloat16).forward(ids)
+    assert torch.equal(a, b)
