@@ -1,0 +1,162 @@
+/*
+ * olmo355 -- C-ABI of the MI355X (gfx950) kernels behind the OLMo inference forward pass.
+ *
+ * Conventions, every entry point:
+ *   - plain pointers and sizes only; every pointer is a *device* pointer borrowed for the
+ *     duration of the call (nothing is allocated, freed or kept by the library);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); kernels are
+ *     launched on it asynchronously and the call returns without synchronising;
+ *   - returns 0 on success, else an O355_E* code; olmo355_status_string() names it.  No
+ *     kernel is launched when an argument check fails;
+ *   - no process-global state: safe from any host thread that has made its device current;
+ *   - `dtype` is O355_F32 or O355_BF16 (the activation dtype); fp16 appears only as the
+ *     scale / dequant-table type of the int4 format.
+ *
+ * Each declaration cites the reference interface it stands in for.  Paths are relative to
+ * the reference tree; "AGQ/" = inference/compression/dependencies/AutoGPTQ/.
+ */
+#ifndef OLMO355_H
+#define OLMO355_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define O355_OK 0
+#define O355_EINVAL 1       /* null pointer, non-positive or misaligned size */
+#define O355_EUNSUPPORTED 2 /* shape / dtype / group size outside what the kernel handles */
+#define O355_ELAUNCH 3      /* hipGetLastError() != hipSuccess after the launch */
+
+#define O355_F32 0
+#define O355_BF16 1
+
+int olmo355_version(void);
+const char* olmo355_status_string(int status);
+
+/* ---- int4 group-wise weights ------------------------------------------------------------
+ * Checkpoint layout (AGQ/auto_gptq/nn_modules/qlinear/qlinear_cuda_old.py:48-67):
+ *   qweight int32 [K/8, N]   nibble j of qweight[r][n] is q[8r+j][n]
+ *   qzeros  int32 [K/g, N/8] nibble j of qzeros[G][c] is the stored zero of column 8c+j
+ *   scales  fp16  [K/g, N]
+ *   g_idx   int32 [K]        group of row k; NULL means k / group
+ * Tiled layout ("w4t", built once by olmo355_w4_repack, K % 128 == 0, N % 16 == 0, group 128):
+ *   wt  uint32 [N/16][K/128][64 lanes][4]  lane l, word j: column 16*nt + (l&15), rows
+ *        128*g + 32*j + 8*(l>>4) + e, e = 0..7; nibble p of the word holds e = 2p (p<4) or
+ *        2(p-4)+1 (p>=4), i.e. one MFMA 16x16x32 operand fragment per word
+ *   st  fp16  [N/16][K/128][16]  scale of column 16*nt + c
+ *   zt  uint8 [N/16][K/128][8]   stored-zero nibbles of the 16 columns, low nibble first
+ */
+
+/* Dense fp16 table W[K,N] = fp16(scale * (q - (zero_stored + 1))), bit-exact with the
+ * reference's torch dequantize: AGQ qlinear_cuda_old.py:236-285 (g_idx == NULL) and
+ * qlinear_cuda.py:211-265 (g_idx given).  Also what exllama's reconstruct kernel produces
+ * (AGQ/autogptq_extension/exllama/cuda_func/q4_matrix.cu:171-225).  K % 8 == 0, N % 8 == 0,
+ * group % 8 == 0 when g_idx is NULL. */
+int olmo355_w4_dequant_fp16(const int32_t* qweight, const int32_t* qzeros, const uint16_t* scales,
+                            const int32_t* g_idx, uint16_t* out_kn, int K, int N, int group, void* stream);
+
+/* One-time re-tiling of a checkpoint-layout weight into the w4t layout; the counterpart of
+ * the reference's post_init hook that rewrites qweight for its kernels
+ * (AGQ qlinear_exllama.py:85-98, q4_matrix.cu:105-169). */
+int olmo355_w4_repack(const int32_t* qweight, const int32_t* qzeros, const uint16_t* scales, uint32_t* wt,
+                      uint16_t* st, uint8_t* zt, int K, int N, int group, void* stream);
+
+/* Same table as olmo355_w4_dequant_fp16, read from the tiled layout (checks the repack). */
+int olmo355_w4t_dequant_fp16(const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* out_kn, int K,
+                             int N, void* stream);
+
+/* y[M,N] = x[M,K] . W[K,N], bf16 in / bf16 out, fp32 accumulation, W = scale*(q-zero) exact.
+ * Small-M path (M <= 64): stands in for vecquant4matmul_faster_old
+ * (AGQ/autogptq_extension/cuda_256/autogptq_cuda_256.cpp:158-171, kernel
+ * autogptq_cuda_kernel_256.cu:1365-1435) and exllama's q4_matmul GEMV
+ * (exllama/cuda_func/q4_matmul.cu:32-143).  Deterministic (no atomics on data).
+ * `ws` is a workspace of olmo355_w4_gemv_workspace_bytes(M,N,K) bytes whose first
+ * O355_GEMV_COUNTER_BYTES bytes must be zero before the first call (the kernel leaves them
+ * zero); it may be NULL when that function returns 0. */
+#define O355_GEMV_COUNTER_BYTES 16384
+int64_t olmo355_w4_gemv_workspace_bytes(int M, int N, int K);
+int olmo355_w4_gemv(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
+                    void* ws, int M, int N, int K, void* stream);
+
+/* Large-M path: dequantise tiles into LDS as bf16 and multiply on the matrix cores.  Stands
+ * in for the reference's dequantise-then-matmul branch (AGQ qlinear_cuda_old.py:236-287) and
+ * exllama's reconstruct + cublasHgemm (exllama/cuda_func/q4_matmul.cu:222-260). */
+int olmo355_w4_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
+                    int M, int N, int K, void* stream);
+
+/* ---- dense Linear (nn.Linear without bias: olmo/model.py:452-462,695-701,1129-1139) -------
+ * bf16: weight pre-tiled by olmo355_b16_repack into [N/16][K/32][64 lanes][8 bf16]
+ * (lane l: row n = 16*nt + (l&15), columns 32*ks + 8*(l>>4) .. +7); K % 32 == 0, N % 16 == 0.
+ * fp32: weight in torch layout [N,K]. */
+int olmo355_b16_repack(const uint16_t* w_nk, uint16_t* wt, int N, int K, void* stream);
+/* small-M (<= 64) path; `ws` follows the rules of olmo355_w4_gemv (same size function) */
+int olmo355_b16_gemv(const uint16_t* x, const uint16_t* wt, uint16_t* y, void* ws, int M, int N, int K, void* stream);
+int olmo355_b16_gemm(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, void* stream);
+int olmo355_f32_linear(const float* x, const float* w_nk, float* y, int M, int N, int K, void* stream);
+
+/* ---- norms ------------------------------------------------------------------------------ */
+/* RMSLayerNorm.forward (olmo/model.py:241-255): y = w * round(x * rsqrt(mean(x^2)+eps)),
+ * both roundings to `dtype`; if `residual` != NULL, out = residual + y (the post-norm
+ * residual add of olmo/model.py:786-794,814-821).  weight may be NULL.  rows x d. */
+int olmo355_rmsnorm(const void* x, const void* weight, const void* residual, void* out, int rows, int d, float eps,
+                    int dtype, void* stream);
+/* Non-parametric LayerNorm.forward (olmo/model.py:212-225): F.layer_norm without weight/bias. */
+int olmo355_layernorm_np(const void* x, void* out, int rows, int d, float eps, int dtype, void* stream);
+
+/* ---- attention input: QK-norm + rotary + cache write --------------------------------------
+ * Per token row of the fused projection qkv [B*T, (H + 2*Hkv)*hd] (olmo/model.py:754-759):
+ *   optional RMS norm of q over all H*hd channels and of k over all Hkv*hd channels with
+ *   weights qw / kw (olmo/model.py:603-605; pass NULL for no QK-norm);
+ *   rotary embedding in fp32 at absolute position past_len + t (olmo/model.py:298-324), with
+ *   the caller's fp32 sin / cos tables [n_pos, hd] (olmo/model.py:285-296);
+ *   q -> q_out [B*T, H*hd]; k (rotated) and v -> the contiguous per-layer cache
+ *   kcache / vcache [B, Hkv, Lmax, hd] at row past_len + t.
+ * Caching the rotated key equals the reference's re-rotation of the whole cache at every
+ * step (olmo/model.py:615-625) because the rotation depends on (k, position) only.
+ * past_len_dev (device int32, may be NULL) overrides past_len when given, so that one
+ * captured launch can be replayed at successive positions. */
+int olmo355_qknorm_rope_kvwrite(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
+                                const float* cos_tab, void* q_out, void* kcache, void* vcache, int B, int T, int H,
+                                int Hkv, int hd, int Lmax, int n_pos, int past_len, const int32_t* past_len_dev,
+                                float eps, int dtype, void* stream);
+
+/* ---- attention (olmo/model.py:533-586,627-648): softmax(q k^T / sqrt(hd) + bias) v ---------
+ * q [B*T, H*hd]; caches [B, Hkv, Lmax, hd] already holding rows 0 .. past_len+T-1;
+ * out [B*T, H*hd].  Query t sits at absolute position past_len + t and sees keys 0..past_len+t.
+ * key_bias (may be NULL): fp32 [B, bias_stride] added to the scores of key j (the padding part
+ * of olmo/model.py:1337-1376); entries <= -1e30 mark the key as masked: its score is replaced
+ * by the dtype's most negative finite value (olmo/torch_util.py:81-90), never -inf. */
+int olmo355_attn_prefill(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out,
+                         int B, int T, int H, int Hkv, int hd, int Lmax, int past_len, int bias_stride, int dtype,
+                         void* stream);
+
+/* T == 1 with the keys split over workgroups.  n_keys_max bounds the number of keys for the
+ * launch grid; the true count is past_len + 1 (or *past_len_dev + 1 when given).
+ * ws: olmo355_attn_decode_workspace_bytes(B,H,hd,n_keys_max) bytes. */
+int64_t olmo355_attn_decode_workspace_bytes(int B, int H, int hd, int n_keys_max);
+int olmo355_attn_decode(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out,
+                        void* ws, int B, int H, int Hkv, int hd, int Lmax, int past_len,
+                        const int32_t* past_len_dev, int n_keys_max, int bias_stride, int dtype, void* stream);
+
+/* ---- MLP activation: SwiGLU.forward (olmo/model.py:365-368) --------------------------------
+ * x [rows, 2h]: first half "up", second half "gate"; out [rows, h] = silu(gate) * up. */
+int olmo355_swiglu(const void* x, void* out, int rows, int h, int dtype, void* stream);
+
+/* ---- small helpers on the path ---------------------------------------------------------- */
+/* wte lookup (olmo/model.py:1318): out[r,:] = table[ids[r],:]; ids int64. */
+int olmo355_embedding(const int64_t* ids, const void* table, void* out, int rows, int d, int vocab, int dtype,
+                      void* stream);
+/* out = a + b (residual add of the pre-norm block, olmo/model.py:794,821). */
+int olmo355_add(const void* a, const void* b, void* out, int64_t n, int dtype, void* stream);
+/* Greedy step (olmo/beam_search.py:102-113 with beam 1): first index of the row maximum,
+ * written as int64 to out[r], and the same value appended at ids_next when non-NULL. */
+int olmo355_argmax(const void* logits, int64_t* out, int rows, int n, int dtype, void* stream);
+/* *p += 1 for a device int32 (advances the position between captured decode steps). */
+int olmo355_incr_i32(int32_t* p, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OLMO355_H */

@@ -1,0 +1,85 @@
+"""ctypes binding of ``libolmo355.so`` (the C-ABI declared in ``include/olmo355.h``).
+
+The library is the product's only compute path: if it is missing or fails to load, every
+op raises ``Olmo355Unavailable`` -- there is no PyTorch or CPU fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+from typing import Optional
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libolmo355.so")
+
+__all__ = ["lib", "LIB_PATH", "Olmo355Unavailable", "Olmo355Error", "check", "EXPORTS"]
+
+
+class Olmo355Unavailable(RuntimeError):
+    pass
+
+
+class Olmo355Error(RuntimeError):
+    def __init__(self, fn: str, status: int, text: str):
+        super().__init__(f"{fn} failed with status {status}: {text}")
+        self.status = status
+
+
+P, I, L, F = c_void_p, c_int, c_int64, c_float
+
+# name -> (restype, argtypes); must list every symbol include/olmo355.h declares
+EXPORTS = {
+    "olmo355_version": (I, []),
+    "olmo355_status_string": (c_char_p, [I]),
+    "olmo355_w4_dequant_fp16": (I, [P, P, P, P, P, I, I, I, P]),
+    "olmo355_w4_repack": (I, [P, P, P, P, P, P, I, I, I, P]),
+    "olmo355_w4t_dequant_fp16": (I, [P, P, P, P, I, I, P]),
+    "olmo355_w4_gemv_workspace_bytes": (L, [I, I, I]),
+    "olmo355_w4_gemv": (I, [P, P, P, P, P, P, I, I, I, P]),
+    "olmo355_w4_gemm": (I, [P, P, P, P, P, I, I, I, P]),
+    "olmo355_b16_repack": (I, [P, P, I, I, P]),
+    "olmo355_b16_gemv": (I, [P, P, P, P, I, I, I, P]),
+    "olmo355_b16_gemm": (I, [P, P, P, I, I, I, P]),
+    "olmo355_f32_linear": (I, [P, P, P, I, I, I, P]),
+    "olmo355_rmsnorm": (I, [P, P, P, P, I, I, F, I, P]),
+    "olmo355_layernorm_np": (I, [P, P, I, I, F, I, P]),
+    "olmo355_qknorm_rope_kvwrite": (I, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P, F, I, P]),
+    "olmo355_attn_prefill": (I, [P, P, P, P, P, I, I, I, I, I, I, I, I, I, P]),
+    "olmo355_attn_decode_workspace_bytes": (L, [I, I, I, I]),
+    "olmo355_attn_decode": (I, [P, P, P, P, P, P, I, I, I, I, I, I, P, I, I, I, P]),
+    "olmo355_swiglu": (I, [P, P, I, I, I, P]),
+    "olmo355_embedding": (I, [P, P, P, I, I, I, I, P]),
+    "olmo355_add": (I, [P, P, P, L, I, P]),
+    "olmo355_argmax": (I, [P, P, I, I, I, P]),
+    "olmo355_incr_i32": (I, [P, P]),
+}
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def lib() -> ctypes.CDLL:
+    """Load the shared library once; fail loudly when it is not there."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise Olmo355Unavailable(
+                f"{LIB_PATH} is missing: build it with `python -m olmo_amd.build` (hipcc, gfx950). "
+                "There is no fallback path."
+            )
+        try:
+            h = ctypes.CDLL(LIB_PATH)
+        except OSError as e:  # pragma: no cover
+            raise Olmo355Unavailable(f"cannot load {LIB_PATH}: {e}") from e
+        for name, (res, args) in EXPORTS.items():
+            fn = getattr(h, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = h
+    return _lib
+
+
+def check(fn_name: str, status: int) -> None:
+    if status != 0:
+        raise Olmo355Error(fn_name, status, lib().olmo355_status_string(status).decode())

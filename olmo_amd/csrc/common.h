@@ -1,0 +1,83 @@
+// Shared device helpers for the gfx950 kernels: 16-bit conversions, wave64 reductions,
+// MFMA operand types, launch checking.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/olmo355.h"
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define O355_WAVE 64
+
+#define O355_CHECK_LAUNCH()                       \
+  do {                                            \
+    hipError_t e__ = hipGetLastError();           \
+    if (e__ != hipSuccess) return O355_ELAUNCH;   \
+    return O355_OK;                               \
+  } while (0)
+
+static inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+// ---- scalar conversions -------------------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+__device__ __forceinline__ float bf16lo_to_f32(uint32_t pair) { return __uint_as_float(pair << 16); }
+__device__ __forceinline__ float bf16hi_to_f32(uint32_t pair) { return __uint_as_float(pair & 0xffff0000u); }
+// round-to-nearest-even fp32 -> bf16 (v_cvt_pk_bf16_f32 on gfx950)
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  bf16_t b = (bf16_t)f;
+  return __builtin_bit_cast(uint16_t, b);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  bf16x2 p = {(bf16_t)lo, (bf16_t)hi};
+  return __builtin_bit_cast(uint32_t, p);
+}
+__device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+
+// Loads / stores of one activation element by dtype tag.
+template <int DT> struct Act;
+template <> struct Act<O355_F32> {
+  typedef float T;
+  static __device__ __forceinline__ float ld(const void* p, int64_t i) { return ((const float*)p)[i]; }
+  static __device__ __forceinline__ void st(void* p, int64_t i, float v) { ((float*)p)[i] = v; }
+  static __device__ __forceinline__ float rnd(float v) { return v; }
+  static __device__ __forceinline__ float lowest() { return -3.4028234663852886e38f; }
+};
+template <> struct Act<O355_BF16> {
+  typedef uint16_t T;
+  static __device__ __forceinline__ float ld(const void* p, int64_t i) {
+    return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+  }
+  static __device__ __forceinline__ void st(void* p, int64_t i, float v) { ((uint16_t*)p)[i] = f32_to_bf16_bits(v); }
+  static __device__ __forceinline__ float rnd(float v) { return round_bf16(v); }
+  static __device__ __forceinline__ float lowest() { return -3.3895313892515355e38f; }
+};
+
+// ---- wave64 reductions ------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Sum over the whole workgroup (blockDim.x a multiple of 64, at most 1024). `red` holds 16 floats.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nw; ++i) t += red[i];
+  return t;
+}

@@ -1,0 +1,370 @@
+"""Torch-tensor front end of the C-ABI: shape / dtype / contiguity checks on the host, then a
+call into ``libolmo355.so`` on the current torch stream.  PyTorch only provides device
+memory and streams here; every computation is a HIP kernel of this package.
+
+All functions require CUDA (ROCm) tensors and raise instead of falling back.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+from ._lib import check, lib
+
+F32, BF16 = 0, 1
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+GEMV_MAX_M = 64
+GEMV_COUNTER_BYTES = 16384
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported activation dtype {t.dtype}; float32 or bfloat16") from None
+
+
+def _dev(*ts: Optional[torch.Tensor]) -> None:
+    dev = None
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("olmo_amd ops run on the GPU only (tensor is on %s); there is no CPU path" % t.device)
+        if not t.is_contiguous():
+            raise ValueError("tensor must be contiguous")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise ValueError("tensors on different devices")
+
+
+def _p(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+# ---------------------------------------------------------------------------------------------
+# int4 weights
+# ---------------------------------------------------------------------------------------------
+def w4_dequant_fp16(qweight, qzeros, scales, group_size: int, g_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp16 ``[K, N]`` table, bit-exact with the reference's torch dequantize."""
+    _dev(qweight, qzeros, scales, g_idx)
+    if qweight.dtype != torch.int32 or qzeros.dtype != torch.int32 or scales.dtype != torch.float16:
+        raise TypeError("qweight/qzeros must be int32 and scales float16")
+    K, N = qweight.shape[0] * 8, qweight.shape[1]
+    if g_idx is not None:
+        if g_idx.dtype != torch.int32 or g_idx.numel() != K:
+            raise ValueError("g_idx must be int32 [K]")
+        G = scales.shape[0]
+    else:
+        G = K // group_size
+    if scales.shape != (G, N) or qzeros.shape != (G, N // 8):
+        raise ValueError(f"scales {tuple(scales.shape)} / qzeros {tuple(qzeros.shape)} do not match K={K} N={N} G={G}")
+    out = torch.empty(K, N, dtype=torch.float16, device=qweight.device)
+    check("olmo355_w4_dequant_fp16",
+          lib().olmo355_w4_dequant_fp16(_p(qweight), _p(qzeros), _p(scales), _p(g_idx), _p(out), K, N, group_size,
+                                        _stream()))
+    return out
+
+
+@dataclass
+class W4Tiled:
+    """An int4 weight in the MFMA-fragment layout (see include/olmo355.h)."""
+
+    wt: torch.Tensor  # int32 [N/16, K/128, 64, 4]
+    st: torch.Tensor  # float16 [N/16, K/128, 16]
+    zt: torch.Tensor  # uint8 [N/16, K/128, 8]
+    K: int
+    N: int
+
+    @property
+    def nbytes(self) -> int:
+        return self.wt.numel() * 4 + self.st.numel() * 2 + self.zt.numel()
+
+
+def w4_repack(qweight, qzeros, scales, group_size: int) -> W4Tiled:
+    _dev(qweight, qzeros, scales)
+    K, N = qweight.shape[0] * 8, qweight.shape[1]
+    if group_size != 128 or K % 128 or N % 16:
+        raise ValueError(f"tiled int4 layout needs group_size 128, K % 128 == 0, N % 16 == 0 (got g={group_size}, K={K}, N={N})")
+    G = K // 128
+    if scales.shape != (G, N) or qzeros.shape != (G, N // 8):
+        raise ValueError("scales / qzeros shape mismatch")
+    dev = qweight.device
+    wt = torch.empty(N // 16, G, 64, 4, dtype=torch.int32, device=dev)
+    st = torch.empty(N // 16, G, 16, dtype=torch.float16, device=dev)
+    zt = torch.empty(N // 16, G, 8, dtype=torch.uint8, device=dev)
+    check("olmo355_w4_repack",
+          lib().olmo355_w4_repack(_p(qweight), _p(qzeros), _p(scales), _p(wt), _p(st), _p(zt), K, N, group_size,
+                                  _stream()))
+    return W4Tiled(wt, st, zt, K, N)
+
+
+def w4t_dequant_fp16(w: W4Tiled) -> torch.Tensor:
+    _dev(w.wt, w.st, w.zt)
+    out = torch.empty(w.K, w.N, dtype=torch.float16, device=w.wt.device)
+    check("olmo355_w4t_dequant_fp16",
+          lib().olmo355_w4t_dequant_fp16(_p(w.wt), _p(w.st), _p(w.zt), _p(out), w.K, w.N, _stream()))
+    return out
+
+
+def gemv_workspace_bytes(M: int, N: int, K: int) -> int:
+    return int(lib().olmo355_w4_gemv_workspace_bytes(M, N, K))
+
+
+class Workspace:
+    """Device scratch shared by the small-M linear kernels on one stream: a zeroed counter
+    block followed by room for split-K partial sums.  Grows on demand (never inside a
+    captured graph: size it first with ``reserve``)."""
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self.buf = torch.zeros(GEMV_COUNTER_BYTES, dtype=torch.uint8, device=self.device)
+
+    def reserve(self, nbytes: int) -> None:
+        if nbytes > self.buf.numel():
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("workspace too small inside graph capture; call reserve() before capturing")
+            self.buf = torch.zeros(nbytes, dtype=torch.uint8, device=self.device)
+
+    def for_linear(self, M: int, N: int, K: int) -> Optional[torch.Tensor]:
+        need = gemv_workspace_bytes(M, N, K)
+        if need == 0:
+            return None
+        self.reserve(need)
+        return self.buf
+
+
+def w4_linear(x: torch.Tensor, w: W4Tiled, ws: Workspace) -> torch.Tensor:
+    """``x[..., K] @ W[K, N]`` for a tiled int4 weight; bf16 in, bf16 out."""
+    _dev(x, w.wt)
+    if x.dtype != torch.bfloat16:
+        raise TypeError("int4 linear takes bfloat16 activations")
+    if x.shape[-1] != w.K:
+        raise ValueError(f"x last dim {x.shape[-1]} != K {w.K}")
+    M = x.numel() // w.K
+    y = torch.empty(*x.shape[:-1], w.N, dtype=torch.bfloat16, device=x.device)
+    if M == 0:
+        return y
+    if M <= GEMV_MAX_M:
+        wsb = ws.for_linear(M, w.N, w.K)
+        check("olmo355_w4_gemv",
+              lib().olmo355_w4_gemv(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), _p(wsb), M, w.N, w.K, _stream()))
+    else:
+        check("olmo355_w4_gemm",
+              lib().olmo355_w4_gemm(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream()))
+    return y
+
+
+# ---------------------------------------------------------------------------------------------
+# dense weights
+# ---------------------------------------------------------------------------------------------
+@dataclass
+class B16Tiled:
+    wt: torch.Tensor  # bf16 [N/16, K/32, 64, 8]
+    K: int
+    N: int
+
+
+def b16_repack(weight_nk: torch.Tensor) -> B16Tiled:
+    _dev(weight_nk)
+    if weight_nk.dtype != torch.bfloat16 or weight_nk.dim() != 2:
+        raise TypeError("expects a bfloat16 [N, K] weight")
+    N, K = weight_nk.shape
+    if K % 64 or N % 16:
+        raise ValueError(f"dense bf16 path needs K % 64 == 0 and N % 16 == 0 (got N={N}, K={K})")
+    wt = torch.empty(N // 16, K // 32, 64, 8, dtype=torch.bfloat16, device=weight_nk.device)
+    check("olmo355_b16_repack", lib().olmo355_b16_repack(_p(weight_nk), _p(wt), N, K, _stream()))
+    return B16Tiled(wt, K, N)
+
+
+def b16_linear(x: torch.Tensor, w: B16Tiled, ws: Workspace) -> torch.Tensor:
+    _dev(x, w.wt)
+    if x.dtype != torch.bfloat16:
+        raise TypeError("dense bf16 linear takes bfloat16 activations")
+    if x.shape[-1] != w.K:
+        raise ValueError(f"x last dim {x.shape[-1]} != K {w.K}")
+    M = x.numel() // w.K
+    y = torch.empty(*x.shape[:-1], w.N, dtype=torch.bfloat16, device=x.device)
+    if M == 0:
+        return y
+    if M <= GEMV_MAX_M:
+        wsb = ws.for_linear(M, w.N, w.K) if w.K % 128 == 0 else None
+        check("olmo355_b16_gemv", lib().olmo355_b16_gemv(_p(x), _p(w.wt), _p(y), _p(wsb), M, w.N, w.K, _stream()))
+    else:
+        check("olmo355_b16_gemm", lib().olmo355_b16_gemm(_p(x), _p(w.wt), _p(y), M, w.N, w.K, _stream()))
+    return y
+
+
+def f32_linear(x: torch.Tensor, weight_nk: torch.Tensor) -> torch.Tensor:
+    _dev(x, weight_nk)
+    if x.dtype != torch.float32 or weight_nk.dtype != torch.float32:
+        raise TypeError("expects float32")
+    N, K = weight_nk.shape
+    if x.shape[-1] != K:
+        raise ValueError("shape mismatch")
+    M = x.numel() // K
+    y = torch.empty(*x.shape[:-1], N, dtype=torch.float32, device=x.device)
+    if M:
+        check("olmo355_f32_linear", lib().olmo355_f32_linear(_p(x), _p(weight_nk), _p(y), M, N, K, _stream()))
+    return y
+
+
+# ---------------------------------------------------------------------------------------------
+# norms, activation, embedding
+# ---------------------------------------------------------------------------------------------
+def rmsnorm(x, weight: Optional[torch.Tensor], eps: float, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(x, weight, residual)
+    d = x.shape[-1]
+    if weight is not None and (weight.dtype != x.dtype or weight.numel() != d):
+        raise ValueError("weight must match x's dtype and last dim")
+    if residual is not None and (residual.dtype != x.dtype or residual.shape != x.shape):
+        raise ValueError("residual must match x")
+    out = torch.empty_like(x)
+    rows = x.numel() // d
+    if rows:
+        check("olmo355_rmsnorm",
+              lib().olmo355_rmsnorm(_p(x), _p(weight), _p(residual), _p(out), rows, d, float(eps), _dt(x), _stream()))
+    return out
+
+
+def layernorm_np(x: torch.Tensor, eps: float) -> torch.Tensor:
+    _dev(x)
+    d = x.shape[-1]
+    out = torch.empty_like(x)
+    rows = x.numel() // d
+    if rows:
+        check("olmo355_layernorm_np", lib().olmo355_layernorm_np(_p(x), _p(out), rows, d, float(eps), _dt(x), _stream()))
+    return out
+
+
+def swiglu(x: torch.Tensor) -> torch.Tensor:
+    _dev(x)
+    h2 = x.shape[-1]
+    if h2 % 2:
+        raise ValueError("last dim must be even")
+    h = h2 // 2
+    out = torch.empty(*x.shape[:-1], h, dtype=x.dtype, device=x.device)
+    rows = x.numel() // h2
+    if rows:
+        check("olmo355_swiglu", lib().olmo355_swiglu(_p(x), _p(out), rows, h, _dt(x), _stream()))
+    return out
+
+
+def embedding(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    _dev(ids, table)
+    if ids.dtype != torch.int64:
+        raise TypeError("ids must be int64")
+    vocab, d = table.shape
+    out = torch.empty(*ids.shape, d, dtype=table.dtype, device=table.device)
+    if ids.numel():
+        check("olmo355_embedding",
+              lib().olmo355_embedding(_p(ids), _p(table), _p(out), ids.numel(), d, vocab, _dt(table), _stream()))
+    return out
+
+
+def add(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    _dev(a, b)
+    if a.shape != b.shape or a.dtype != b.dtype:
+        raise ValueError("shape/dtype mismatch")
+    out = torch.empty_like(a)
+    if a.numel():
+        check("olmo355_add", lib().olmo355_add(_p(a), _p(b), _p(out), a.numel(), _dt(a), _stream()))
+    return out
+
+
+def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(logits, out)
+    n = logits.shape[-1]
+    rows = logits.numel() // n
+    if out is None:
+        out = torch.empty(logits.shape[:-1], dtype=torch.int64, device=logits.device)
+    check("olmo355_argmax", lib().olmo355_argmax(_p(logits), _p(out), rows, n, _dt(logits), _stream()))
+    return out
+
+
+def incr_i32(p: torch.Tensor) -> None:
+    _dev(p)
+    if p.dtype != torch.int32:
+        raise TypeError("int32 expected")
+    check("olmo355_incr_i32", lib().olmo355_incr_i32(_p(p), _stream()))
+
+
+# ---------------------------------------------------------------------------------------------
+# attention
+# ---------------------------------------------------------------------------------------------
+def qknorm_rope_kvwrite(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, B: int, T: int, H: int, Hkv: int,
+                        hd: int, past_len: int, eps: float, past_len_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Returns q (normed + rotated) ``[B, T, H*hd]``; writes rotated k and v into the caches."""
+    _dev(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, past_len_dev)
+    if qkv.shape[-1] != (H + 2 * Hkv) * hd or qkv.numel() != B * T * (H + 2 * Hkv) * hd:
+        raise ValueError("qkv shape mismatch")
+    if kcache.shape != vcache.shape or kcache.dim() != 4 or kcache.shape[0] < B or kcache.shape[1] != Hkv or kcache.shape[3] != hd:
+        raise ValueError(f"cache shape {tuple(kcache.shape)} does not fit B={B} Hkv={Hkv} hd={hd}")
+    if kcache.dtype != qkv.dtype or sin_tab.dtype != torch.float32 or cos_tab.dtype != torch.float32:
+        raise TypeError("cache dtype must equal activation dtype; sin/cos tables float32")
+    if sin_tab.shape != cos_tab.shape or sin_tab.shape[-1] != hd:
+        raise ValueError("sin/cos tables must be [n_pos, hd]")
+    Lmax, n_pos = kcache.shape[2], sin_tab.shape[0]
+    if past_len_dev is None and past_len + T > min(Lmax, n_pos):
+        raise ValueError(f"past_len + T = {past_len + T} exceeds cache length {Lmax} or rotary table {n_pos}")
+    q = torch.empty(B, T, H * hd, dtype=qkv.dtype, device=qkv.device)
+    check("olmo355_qknorm_rope_kvwrite",
+          lib().olmo355_qknorm_rope_kvwrite(_p(qkv), _p(q_weight), _p(k_weight), _p(sin_tab), _p(cos_tab), _p(q),
+                                            _p(kcache), _p(vcache), B, T, H, Hkv, hd, Lmax, n_pos, past_len,
+                                            _p(past_len_dev), float(eps), _dt(qkv), _stream()))
+    return q
+
+
+def attn_prefill(q, kcache, vcache, B: int, T: int, H: int, Hkv: int, hd: int, past_len: int,
+                 key_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(q, kcache, vcache, key_bias)
+    Lmax = kcache.shape[2]
+    if q.numel() != B * T * H * hd or kcache.dtype != q.dtype:
+        raise ValueError("q shape / cache dtype mismatch")
+    if key_bias is not None and (key_bias.dtype != torch.float32 or key_bias.dim() != 2 or key_bias.shape[0] < B):
+        raise ValueError("key_bias must be float32 [B, n]")
+    out = torch.empty(B, T, H * hd, dtype=q.dtype, device=q.device)
+    check("olmo355_attn_prefill",
+          lib().olmo355_attn_prefill(_p(q), _p(kcache), _p(vcache), _p(key_bias), _p(out), B, T, H, Hkv, hd, Lmax,
+                                     past_len, key_bias.shape[1] if key_bias is not None else 0, _dt(q), _stream()))
+    return out
+
+
+def attn_decode_workspace(B: int, H: int, hd: int, n_keys_max: int, device) -> torch.Tensor:
+    n = int(lib().olmo355_attn_decode_workspace_bytes(B, H, hd, n_keys_max))
+    return torch.empty(n // 4, dtype=torch.float32, device=device)
+
+
+def attn_decode(q, kcache, vcache, ws, B: int, H: int, Hkv: int, hd: int, past_len: int, n_keys_max: int,
+                key_bias: Optional[torch.Tensor] = None, past_len_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(q, kcache, vcache, ws, key_bias, past_len_dev)
+    Lmax = kcache.shape[2]
+    if q.numel() != B * H * hd or kcache.dtype != q.dtype:
+        raise ValueError("q shape / cache dtype mismatch")
+    need = int(lib().olmo355_attn_decode_workspace_bytes(B, H, hd, n_keys_max))
+    if ws.numel() * ws.element_size() < need:
+        raise ValueError("attention workspace too small")
+    out = torch.empty(B, 1, H * hd, dtype=q.dtype, device=q.device)
+    check("olmo355_attn_decode",
+          lib().olmo355_attn_decode(_p(q), _p(kcache), _p(vcache), _p(key_bias), _p(out), _p(ws), B, H, Hkv, hd, Lmax,
+                                    past_len, _p(past_len_dev), n_keys_max,
+                                    key_bias.shape[1] if key_bias is not None else 0, _dt(q), _stream()))
+    return out
+
+
+def rope_tables(head_dim: int, theta: float, n_pos: int, device) -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp32 sin / cos tables ``[n_pos, hd]`` built with the reference's expression
+    (``olmo/model.py:285-296``) on the host so that device sin/cos differences cannot enter."""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float) / head_dim))
+    seq = torch.arange(n_pos, dtype=torch.float)
+    freqs = seq[:, None] * inv_freq[None, :]
+    pos = torch.cat((freqs, freqs), dim=-1)
+    return pos.sin().contiguous().to(device), pos.cos().contiguous().to(device)

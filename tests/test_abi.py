@@ -1,0 +1,54 @@
+"""CPU-side checks of the drop-in boundary: the shared library loads, exports every symbol the
+header declares, and rejects bad arguments before touching the GPU."""
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    from olmo_amd import _lib
+
+    hdr = open(os.path.join(ROOT, "include", "olmo355.h")).read()
+    declared = set(re.findall(r"\b(olmo355_\w+)\s*\(", hdr))
+    assert declared, "no declarations found"
+    assert declared == set(_lib.EXPORTS), (declared ^ set(_lib.EXPORTS))
+    h = _lib.lib()
+    for name in declared:
+        assert getattr(h, name) is not None
+    assert h.olmo355_version() >= 1
+    assert b"unsupported" in h.olmo355_status_string(2)
+
+
+def test_argument_checks_return_status_without_launching():
+    from olmo_amd import _lib
+
+    h = _lib.lib()
+    assert h.olmo355_w4_gemv(None, None, None, None, None, None, 1, 16, 128, None) == 1
+    assert h.olmo355_w4_dequant_fp16(None, None, None, None, None, 8, 8, 8, None) == 1
+    assert h.olmo355_rmsnorm(None, None, None, None, 1, 8, 1e-6, 1, None) == 1
+    # workspace sizing is pure host arithmetic
+    assert h.olmo355_w4_gemv_workspace_bytes(1, 22016, 4096) == 0
+    assert h.olmo355_w4_gemv_workspace_bytes(1, 4096, 4096) > 16384
+    assert h.olmo355_w4_gemv_workspace_bytes(65, 4096, 4096) == 0  # not a small-M shape
+    assert h.olmo355_attn_decode_workspace_bytes(1, 32, 128, 2048) == 32 * 8 * 130 * 4
+
+
+def test_ops_refuse_cpu_tensors():
+    import torch
+
+    from olmo_amd import ops
+
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ops.rmsnorm(torch.zeros(2, 8), None, 1e-6)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from olmo_amd import _lib
+
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(_lib.Olmo355Unavailable):
+        _lib.lib()

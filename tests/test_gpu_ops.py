@@ -1,0 +1,350 @@
+"""GPU parity of every HIP kernel, called through the C-ABI, against the CPU oracle on the
+same seeded inputs.  Integer / table work is bit-exact; floating point carries its tolerance
+next to the assertion."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import model as om
+from oracle import w4 as ow4
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from olmo_amd import _lib
+
+    _lib.lib()  # fail loudly if the HIP library is not built
+    return torch.device("cuda:0")
+
+
+def _ops():
+    from olmo_amd import ops
+
+    return ops
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+# ------------------------------------------------------------------------------------------------
+# int4 table: bit-exact
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("K,N,g", [(128, 16, 128), (256, 48, 128), (512, 64, 64), (4096, 256, 128), (1024, 1024, 128)])
+def test_w4_dequant_bit_exact(dev, K, N, g):
+    say("w4_dequant", K, N, g)
+    ops = _ops()
+    qw, qz, sc = ow4.random_quantized(K, N, g, seed=K * 7 + N)
+    if K == 256:  # subnormal / zero / large scales must survive
+        sc[0, :8] = torch.tensor([0.0, 6e-8, 1.2e-7, 3e-6, 5.9e-5, 6.2e-5, 1e-3, 4000.0], dtype=torch.float16)
+    ref = ow4.dequantize(qw, qz, sc, g)
+    out = ops.w4_dequant_fp16(qw.to(dev), qz.to(dev), sc.to(dev), g).cpu()
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+    if g == 128 and N % 16 == 0:
+        t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), g)
+        out2 = ops.w4t_dequant_fp16(t).cpu()
+        assert torch.equal(out2.view(torch.int16), ref.view(torch.int16))
+
+
+def test_w4_dequant_g_idx_general(dev):
+    ops = _ops()
+    K, N, g = 256, 32, 128
+    qw, qz, sc = ow4.random_quantized(K, N, g, seed=11)
+    perm = torch.randperm(K, generator=torch.Generator().manual_seed(0))
+    g_idx = (perm // g).to(torch.int32)
+    q = ow4.unpack_qweight(qw)
+    z = ow4.unpack_qzeros(qz)
+    ref = (sc.float()[g_idx.long()] * (q - z[g_idx.long()]).float()).half()
+    out = ops.w4_dequant_fp16(qw.to(dev), qz.to(dev), sc.to(dev), g, g_idx.to(dev)).cpu()
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+
+
+def test_w4_golden_vectors_through_gemv(dev, golden_dir):
+    """The reference's own kernel KATs (AGQ tests/test_q4.py) through the HIP GEMV."""
+    import json
+    import os
+
+    ops = _ops()
+    kats = json.load(open(os.path.join(golden_dir, "q4_kat.json")))
+    ws = ops.Workspace(dev)
+    for name in ("exllama_k1024_n1024", "cuda_old_half_k256_n256", "cuda_old_no_half_k256_n256"):
+        kat = kats[name]
+        k, n = kat["k"], kat["n"]
+        torch.manual_seed(42)
+        qweight = torch.randint(-100, 100, size=(k // 8, n), dtype=torch.int32)
+        scales = torch.zeros(k // 128, n, dtype=torch.float16) + 0.002
+        qzeros = torch.zeros(k // 128, n // 8, dtype=torch.int32)
+        inp = torch.rand(1, 1, k, dtype=torch.float16)
+        t = ops.w4_repack(qweight.to(dev), qzeros.to(dev), scales.to(dev), 128)
+        # inputs are fp16 values in [0,1): representable in bf16 only after rounding, so compare
+        # against the oracle on the same bf16 inputs, and against the stored vector with the
+        # input-rounding error budget (|dx| <= 2^-9, sum |w| <= k*0.2)
+        xb = inp[0].to(torch.bfloat16)
+        y = ops.w4_linear(xb.to(dev), t, ws).float().cpu()[0]
+        W = ow4.dequantize(qweight, qzeros, scales, 128)
+        ref_same_inputs = ow4.linear_fp32(xb, W)[0]
+        assert torch.allclose(y, ref_same_inputs, rtol=2 ** -8, atol=1e-3), name
+        stored = torch.tensor(kat["out"])
+        assert (y - stored).abs().max() < 0.15, name  # bf16 rounding of the inputs dominates
+
+
+# ------------------------------------------------------------------------------------------------
+# int4 linear: GEMV (M<=64) and GEMM paths
+# ------------------------------------------------------------------------------------------------
+def _w4_case(dev, M, N, K, seed):
+    ops = _ops()
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=seed)
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(seed + 1)).to(torch.bfloat16)
+    W = ow4.dequantize(qw, qz, sc, 128)
+    ref = ow4.linear_fp32(x, W)
+    t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    ws = ops.Workspace(dev)
+    y = ops.w4_linear(x.to(dev), t, ws)
+    y2 = ops.w4_linear(x.to(dev), t, ws)
+    assert torch.equal(y, y2), "not deterministic"
+    y = y.float().cpu()
+    # bf16 output rounding (2^-9 relative) + fp32 accumulation noise; GEMM path also rounds W to bf16
+    # (2^-9 relative per weight, averaging over K): budget 2^-7 relative to the row scale
+    scale = ref.abs().max().item()
+    err = (y - ref).abs().max().item()
+    return err, scale
+
+
+@pytest.mark.parametrize("M", [1, 2, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(256, 256), (4096, 4096), (1008, 1408)])
+def test_w4_gemv(dev, M, N, K):
+    say("w4_gemv", M, N, K)
+    err, scale = _w4_case(dev, M, N, K, seed=M + N + K)
+    assert err <= 2 ** -7 * scale, (err, scale)
+
+
+@pytest.mark.parametrize("M,N,K", [(65, 256, 256), (128, 512, 1024), (300, 1008, 1408), (2048, 4096, 4096),
+                                   (512, 12288, 4096)])
+def test_w4_gemm(dev, M, N, K):
+    say("w4_gemm", M, N, K)
+    err, scale = _w4_case(dev, M, N, K, seed=M + N + K)
+    assert err <= 2 ** -7 * scale, (err, scale)
+
+
+@pytest.mark.parametrize("M", [1, 8, 40, 64, 65, 300, 1024])
+@pytest.mark.parametrize("N,K", [(256, 256), (2048, 2048), (1008, 1408)])
+def test_b16_linear(dev, M, N, K):
+    say("b16_linear", M, N, K)
+    ops = _ops()
+    gen = torch.Generator().manual_seed(M + N + K)
+    w = (torch.randn(N, K, generator=gen) * 0.02).to(torch.bfloat16)
+    x = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    ref = x.float() @ w.float().t()
+    t = ops.b16_repack(w.to(dev))
+    ws = ops.Workspace(dev)
+    y = ops.b16_linear(x.to(dev), t, ws).float().cpu()
+    # exact bf16 products, fp32 accumulation, one bf16 rounding of the result
+    assert torch.allclose(y, ref, rtol=2 ** -8, atol=2 ** -8 * ref.abs().max().item())
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 50304, 256), (2048, 768, 256), (77, 130, 1024)])
+def test_f32_linear(dev, M, N, K):
+    ops = _ops()
+    gen = torch.Generator().manual_seed(M + N)
+    w = torch.randn(N, K, generator=gen) * 0.02
+    x = torch.randn(M, K, generator=gen)
+    ref = (x.double() @ w.double().t()).float()
+    y = ops.f32_linear(x.to(dev), w.to(dev)).cpu()
+    assert torch.allclose(y, ref, rtol=1e-5, atol=1e-5)
+
+
+# ------------------------------------------------------------------------------------------------
+# row kernels
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,d", [(1, 4096), (37, 2048), (5, 5120), (3, 256)])
+def test_rmsnorm(dev, dtype, rows, d):
+    ops = _ops()
+    gen = torch.Generator().manual_seed(rows + d)
+    x = (torch.randn(rows, d, generator=gen) * 3).to(dtype)
+    w = (1 + 0.1 * torch.randn(d, generator=gen)).to(dtype)
+    r = torch.randn(rows, d, generator=gen).to(dtype)
+    ref = om.rms_norm(x, w, 1e-6)
+    out = ops.rmsnorm(x.to(dev), w.to(dev), 1e-6).cpu()
+    out_r = ops.rmsnorm(x.to(dev), w.to(dev), 1e-6, residual=r.to(dev)).cpu()
+    if dtype == torch.float32:
+        assert torch.allclose(out, ref, rtol=1e-5, atol=1e-6)
+        assert torch.allclose(out_r, r + ref, rtol=1e-5, atol=1e-5)
+    else:
+        # same rounding points; the fp32 sum of squares may differ in the last bit, which can
+        # flip a bf16 rounding: allow 1 bf16 ulp on at most 0.5% of the elements
+        diff = (out.float() - ref.float()).abs()
+        ulp = 2.0 ** (torch.floor(torch.log2(ref.float().abs().clamp_min(1e-30))) - 7)
+        assert (diff <= ulp).all()
+        assert (diff > 0).float().mean().item() < 5e-3
+        assert (out_r.float() - (r + ref).float()).abs().max().item() <= 2 * ulp.max().item()
+
+
+@pytest.mark.parametrize("rows,d", [(2048, 256), (3, 1000)])
+def test_layernorm_np(dev, rows, d):
+    ops = _ops()
+    x = torch.randn(rows, d, generator=torch.Generator().manual_seed(d)) * 2 + 0.5
+    ref = om.layer_norm_np(x, 1e-5)
+    out = ops.layernorm_np(x.to(dev), 1e-5).cpu()
+    assert torch.allclose(out, ref, rtol=1e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu(dev, dtype):
+    ops = _ops()
+    x = (torch.randn(33, 2 * 1376, generator=torch.Generator().manual_seed(4)) * 2).to(dtype)
+    ref = om.swiglu(x)
+    out = ops.swiglu(x.to(dev)).cpu()
+    if dtype == torch.float32:
+        assert torch.allclose(out, ref, rtol=1e-5, atol=1e-6)
+    else:
+        diff = (out.float() - ref.float()).abs()
+        ulp = 2.0 ** (torch.floor(torch.log2(ref.float().abs().clamp_min(1e-30))) - 7)
+        assert (diff <= ulp).all() and (diff > 0).float().mean().item() < 5e-3
+
+
+def test_embedding_add_argmax(dev):
+    ops = _ops()
+    gen = torch.Generator().manual_seed(0)
+    tab = torch.randn(1000, 256, generator=gen).to(torch.bfloat16)
+    ids = torch.randint(0, 1000, (3, 7), generator=gen)
+    assert torch.equal(ops.embedding(ids.to(dev), tab.to(dev)).cpu(), tab[ids])
+    a, b = torch.randn(5, 100, generator=gen).bfloat16(), torch.randn(5, 100, generator=gen).bfloat16()
+    assert torch.equal(ops.add(a.to(dev), b.to(dev)).cpu(), a + b)
+    lg = torch.randn(4, 100352, generator=gen).bfloat16()
+    lg[1, 77] = lg[1, 5000] = 9.0  # tie: first index wins
+    assert torch.equal(ops.argmax(lg.to(dev)).cpu(), torch.argmax(lg.float(), dim=-1))
+    assert int(ops.argmax(lg.to(dev))[1]) == 77
+
+
+# ------------------------------------------------------------------------------------------------
+# attention path
+# ------------------------------------------------------------------------------------------------
+def _rope_ref(qkv, qw, kw, B, T, H, Hkv, hd, past, theta, eps, n_pos):
+    dq, dk = H * hd, Hkv * hd
+    q, k, v = qkv.view(B, T, -1).split((dq, dk, dk), dim=-1)
+    if qw is not None:
+        q, k = om.rms_norm(q, qw, eps), om.rms_norm(k, kw, eps)
+    q = q.reshape(B, T, H, hd).transpose(1, 2)
+    k = k.reshape(B, T, Hkv, hd).transpose(1, 2)
+    v = v.reshape(B, T, Hkv, hd).transpose(1, 2)
+    sin, cos = om.rope_tables(hd, theta, n_pos)
+    q = om.apply_rope(q, sin[past:past + T], cos[past:past + T])
+    k = om.apply_rope(k, sin[past:past + T], cos[past:past + T])
+    return q, k, v
+
+
+@pytest.mark.parametrize("dtype,qknorm,H,Hkv,hd", [(torch.bfloat16, True, 16, 16, 128), (torch.bfloat16, True, 8, 2, 64),
+                                                    (torch.float32, False, 8, 8, 32)])
+def test_qknorm_rope_kvwrite(dev, dtype, qknorm, H, Hkv, hd):
+    ops = _ops()
+    B, T, past, Lmax, theta, eps = 2, 5, 3, 16, 500000.0, 1e-6
+    gen = torch.Generator().manual_seed(hd)
+    qkv = torch.randn(B * T, (H + 2 * Hkv) * hd, generator=gen).to(dtype)
+    qw = (1 + 0.1 * torch.randn(H * hd, generator=gen)).to(dtype) if qknorm else None
+    kw = (1 + 0.1 * torch.randn(Hkv * hd, generator=gen)).to(dtype) if qknorm else None
+    qr, kr, vr = _rope_ref(qkv, qw, kw, B, T, H, Hkv, hd, past, theta, eps, Lmax)
+    sin, cos = ops.rope_tables(hd, theta, Lmax, dev)
+    kc = torch.zeros(B, Hkv, Lmax, hd, dtype=dtype, device=dev)
+    vc = torch.zeros_like(kc)
+    q = ops.qknorm_rope_kvwrite(qkv.to(dev), None if qw is None else qw.to(dev), None if kw is None else kw.to(dev),
+                                sin, cos, kc, vc, B, T, H, Hkv, hd, past, eps)
+    q = q.view(B, T, H, hd).transpose(1, 2).cpu()
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -7)
+    assert torch.allclose(q.float(), qr.float(), **tol)
+    assert torch.allclose(kc[:, :, past:past + T].cpu().float(), kr.float(), **tol)
+    assert torch.equal(vc[:, :, past:past + T].cpu(), vr)
+    assert (kc[:, :, :past] == 0).all() and (kc[:, :, past + T:] == 0).all()
+    if dtype == torch.bfloat16:  # same rounding points: almost every element identical
+        assert (q.float() != qr.float()).float().mean().item() < 1e-2
+
+
+@pytest.mark.parametrize("dtype,B,T,past,H,Hkv,hd", [
+    (torch.bfloat16, 1, 300, 0, 4, 4, 128),
+    (torch.bfloat16, 2, 130, 70, 4, 2, 128),
+    (torch.bfloat16, 1, 257, 0, 2, 2, 64),
+    (torch.float32, 2, 100, 0, 8, 8, 32),
+    (torch.float32, 1, 70, 30, 2, 2, 32),
+])
+def test_attn_prefill(dev, dtype, B, T, past, H, Hkv, hd):
+    say("attn_prefill", dtype, B, T, past, H, Hkv, hd)
+    ops = _ops()
+    L = past + T
+    Lmax = L + 9
+    gen = torch.Generator().manual_seed(T + hd)
+    q = torch.randn(B, H, T, hd, generator=gen).to(dtype)
+    k = torch.randn(B, Hkv, L, hd, generator=gen).to(dtype)
+    v = torch.randn(B, Hkv, L, hd, generator=gen).to(dtype)
+    ref = om.attention(q, k, v, None, dtype).transpose(1, 2).reshape(B, T, H * hd)
+    kc = torch.zeros(B, Hkv, Lmax, hd, dtype=dtype)
+    vc = torch.zeros_like(kc)
+    kc[:, :, :L], vc[:, :, :L] = k, v
+    out = ops.attn_prefill(q.transpose(1, 2).reshape(B, T, H * hd).contiguous().to(dev), kc.to(dev), vc.to(dev), B, T, H,
+                           Hkv, hd, past).cpu()
+    if dtype == torch.float32:
+        assert torch.allclose(out, ref, rtol=1e-4, atol=1e-5)
+    else:
+        # P is rounded to bf16 before the second product (2^-9 relative), output rounded to bf16
+        assert torch.allclose(out.float(), ref.float(), rtol=0, atol=2.5e-2)
+        assert (out.float() - ref.float()).abs().mean().item() < 2e-3
+    # padding: mask the first 5 keys of batch row 0 (left padding)
+    bias = torch.zeros(B, Lmax)
+    bias[0, :5] = torch.finfo(torch.float32).min
+    fb = torch.triu(torch.ones(L, L), diagonal=1).masked_fill_(torch.triu(torch.ones(L, L), diagonal=1) == 1,
+                                                               torch.finfo(torch.float32).min).view(1, 1, L, L)
+    fb = (fb + bias[:, None, None, :L])
+    fb = fb.masked_fill(fb == float("-inf"), torch.finfo(torch.float32).min)[:, :, L - T:L]
+    fb = fb.to(dtype)
+    fb = fb.masked_fill(fb == float("-inf"), torch.finfo(dtype).min)
+    ref2 = om.attention(q, k, v, fb, dtype).transpose(1, 2).reshape(B, T, H * hd)
+    out2 = ops.attn_prefill(q.transpose(1, 2).reshape(B, T, H * hd).contiguous().to(dev), kc.to(dev), vc.to(dev), B, T,
+                            H, Hkv, hd, past, key_bias=bias.to(dev)).cpu()
+    valid = slice(5, None) if past == 0 else slice(None)  # rows that see at least one real key
+    tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=0, atol=2.5e-2)
+    assert torch.allclose(out2[:, valid].float(), ref2[:, valid].float(), **tol)
+    assert torch.isfinite(out2.float()).all()
+
+
+@pytest.mark.parametrize("dtype,B,L,H,Hkv,hd", [
+    (torch.bfloat16, 1, 2048, 32, 32, 128),
+    (torch.bfloat16, 3, 700, 4, 2, 128),
+    (torch.bfloat16, 2, 1, 2, 2, 64),
+    (torch.bfloat16, 2, 257, 2, 2, 64),
+    (torch.float32, 2, 513, 8, 8, 32),
+])
+def test_attn_decode(dev, dtype, B, L, H, Hkv, hd):
+    say("attn_decode", dtype, B, L, H, Hkv, hd)
+    ops = _ops()
+    Lmax = L + 100
+    gen = torch.Generator().manual_seed(L + hd)
+    q = torch.randn(B, H, 1, hd, generator=gen).to(dtype)
+    k = torch.randn(B, Hkv, L, hd, generator=gen).to(dtype)
+    v = torch.randn(B, Hkv, L, hd, generator=gen).to(dtype)
+    ref = om.attention(q, k, v, None, dtype).transpose(1, 2).reshape(B, 1, H * hd)
+    kc = torch.zeros(B, Hkv, Lmax, hd, dtype=dtype)
+    vc = torch.zeros_like(kc)
+    kc[:, :, :L], vc[:, :, :L] = k, v
+    kc, vc = kc.to(dev), vc.to(dev)
+    qd = q.reshape(B, 1, H * hd).contiguous().to(dev)
+    ws = ops.attn_decode_workspace(B, H, hd, Lmax, dev)
+    tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -8)
+    out = ops.attn_decode(qd, kc, vc, ws, B, H, Hkv, hd, L - 1, L).cpu()
+    assert torch.allclose(out.float(), ref.float(), **tol)
+    # position read from device memory, launch grid sized for the whole cache
+    pl = torch.tensor([L - 1], dtype=torch.int32, device=dev)
+    out_d = ops.attn_decode(qd, kc, vc, ws, B, H, Hkv, hd, 0, Lmax, past_len_dev=pl).cpu()
+    assert torch.equal(out_d, out)
+    # padding mask on batch row 0
+    if L > 8:
+        bias = torch.zeros(B, Lmax)
+        bias[0, :5] = torch.finfo(torch.float32).min
+        fb = bias[:, None, None, :L].to(dtype)
+        fb = fb.masked_fill(fb == float("-inf"), torch.finfo(dtype).min)
+        ref2 = om.attention(q, k, v, fb, dtype).transpose(1, 2).reshape(B, 1, H * hd)
+        out2 = ops.attn_decode(qd, kc, vc, ws, B, H, Hkv, hd, L - 1, L, key_bias=bias.to(dev)).cpu()
+        assert torch.allclose(out2.float(), ref2.float(), **tol)
