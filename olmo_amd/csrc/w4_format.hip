@@ -5,9 +5,15 @@
 namespace {
 
 __device__ __forceinline__ uint16_t dq_one(float s, int q, int z) {
-  // exact fp32 product (11-bit x 5-bit significands), one RNE rounding to fp16, subnormals kept
-  _Float16 h = (_Float16)(s * (float)(q - z));
-  return __builtin_bit_cast(uint16_t, h);
+  // exact fp32 product (11-bit x 5-bit significands), one RNE rounding to fp16, subnormals kept.
+  // The sign is set explicitly: the compiler folds the multiply and the conversion into one
+  // mixed-precision fma with a +0 addend, which would turn a -0 product (zero scale, q < zero)
+  // into +0, and the table is compared bit for bit.
+  const int d = q - z;
+  _Float16 h = (_Float16)(s * (float)d);
+  const uint16_t mag = __builtin_bit_cast(uint16_t, h) & 0x7fffu;
+  const uint16_t sign = (uint16_t)(((__float_as_uint(s) >> 31) ^ (uint32_t)(d < 0)) << 15);
+  return mag | sign;
 }
 __device__ __forceinline__ float h2f(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
 
