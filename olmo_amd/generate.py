@@ -1,0 +1,116 @@
+"""Greedy decoding over the KV cache: prefill once, then one token per step.
+
+Stands in for the two drivers the reference reaches ``OLMo.forward`` through: the HF
+``generate`` loop behind ``hf_olmo/modeling_olmo.py:150-160`` and ``OLMo.generate`` with beam 1
+(``olmo/model.py:1603-1728``; the deterministic sampler takes ``topk(1)`` of the log-softmax,
+``olmo/beam_search.py:102-113``, i.e. the arg-max of the logits).
+
+The decode step (embedding, all blocks, final norm, head, arg-max, position increment) is
+launch-bound in Python, so it is captured once into a HIP graph and replayed: every kernel reads
+the current position from device memory, the new token is written where the next step's
+embedding lookup reads it, and no launch argument changes between steps.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import ops
+
+__all__ = ["greedy_generate", "DecodeSession"]
+
+
+class DecodeSession:
+    """State of one batched greedy decode after its prefill."""
+
+    def __init__(self, model, cache, first_ids: torch.Tensor, key_bias_full: Optional[torch.Tensor]):
+        self.model = model
+        self.cache = cache
+        self.B = first_ids.shape[0]
+        self.ids = first_ids.view(self.B, 1).contiguous()  # token to feed next; rewritten by every step
+        self.key_bias = key_bias_full
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.logits: Optional[torch.Tensor] = None
+
+    def _step_kernels(self) -> None:
+        m = self.model
+        x = m.transformer["wte"](self.ids)
+        logits, _ = m._forward_tokens(x, self.cache, self.B, 1, 0, self.key_bias, self.cache.length_dev, False)
+        self.logits = logits
+        ops.argmax(logits.view(self.B, -1), out=self.ids.view(self.B))
+        ops.incr_i32(self.cache.length_dev)
+
+    def step(self) -> None:
+        """Advance by one token: afterwards ``self.ids`` holds the new token of every sequence."""
+        if self.cache.length + 1 > self.cache.capacity:
+            raise ValueError("KV cache capacity exceeded")
+        if self.graph is not None:
+            self.graph.replay()
+        else:
+            self._step_kernels()
+        self.cache.length += 1  # host mirror of the device counter
+
+    def capture(self) -> None:
+        """Record one decode step into a HIP graph (call after at least one eager ``step`` so that
+        every workspace already has its final size)."""
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self._step_kernels()
+        self.graph = g
+
+
+def _prefill(model, input_ids, attention_mask):
+    out = model(input_ids, attention_mask=attention_mask, use_cache=True, last_logits_only=True)
+    cache = out.attn_key_values[0].cache
+    B = input_ids.shape[0]
+    first = ops.argmax(out.logits.view(B, -1))
+    key_bias_full = None
+    if attention_mask is not None:
+        am = attention_mask.to(model.device, torch.float32).view(B, -1)
+        key_bias_full = torch.zeros(B, cache.capacity, dtype=torch.float32, device=model.device)
+        key_bias_full[:, : am.shape[1]] = (1.0 - am) * torch.finfo(torch.float32).min
+    return out, cache, first, key_bias_full
+
+
+@torch.no_grad()
+def greedy_generate(model, input_ids: torch.Tensor, attention_mask: Optional[torch.Tensor], max_new_tokens: int,
+                    use_graph: bool = True, eos_token_id: Optional[int] = None, pad_token_id: Optional[int] = None,
+                    return_scores: bool = False, return_logits: bool = False):
+    """Returns ``tokens [B, max_new_tokens]`` (and, on request, the summed log-probabilities of the
+    chosen tokens and / or the per-step logits).  Always runs ``max_new_tokens`` steps; with
+    ``eos_token_id`` the tokens after a sequence's first EOS are replaced by ``pad_token_id``."""
+    if max_new_tokens < 1:
+        raise ValueError("max_new_tokens must be >= 1")
+    input_ids = input_ids.to(model.device)
+    B, T0 = input_ids.shape
+    if T0 + max_new_tokens - 1 > model.max_cache_len:
+        raise ValueError(f"prompt {T0} + {max_new_tokens} new tokens exceeds max_cache_len {model.max_cache_len}")
+    out, cache, first, key_bias_full = _prefill(model, input_ids, attention_mask)
+    sess = DecodeSession(model, cache, first, key_bias_full)
+    tokens = torch.empty(B, max_new_tokens, dtype=torch.int64, device=model.device)
+    tokens[:, 0] = sess.ids.view(B)
+    all_logits = [out.logits[:, -1].clone()] if (return_scores or return_logits) else None
+    for i in range(1, max_new_tokens):
+        if use_graph and sess.graph is None and i == 3:
+            sess.capture()
+        sess.step()
+        tokens[:, i] = sess.ids.view(B)
+        if all_logits is not None:
+            all_logits.append(sess.logits.view(B, -1).clone())
+    result = [tokens]
+    if eos_token_id is not None:
+        pad = eos_token_id if pad_token_id is None else pad_token_id
+        seen = (tokens == eos_token_id).cumsum(dim=1)
+        after = (seen - (tokens == eos_token_id).to(seen.dtype)) > 0
+        tokens = torch.where(after, torch.full_like(tokens, pad), tokens)
+        result[0] = tokens
+    if return_scores:
+        # log-probability bookkeeping of the search (olmo/model.py:1705, beam_search.py:1003-1019);
+        # not on the timed path, so plain torch on the saved logits
+        lp = torch.stack([torch.log_softmax(l.float(), dim=-1) for l in all_logits], dim=1)
+        result.append(lp.gather(-1, tokens.clamp_min(0).unsqueeze(-1)).squeeze(-1).sum(dim=1))
+    if return_logits:
+        result.append(torch.stack(all_logits, dim=1))
+    return result[0] if len(result) == 1 else tuple(result)

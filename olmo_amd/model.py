@@ -1,0 +1,436 @@
+"""``OLMo``: the reference's inference forward pass on one MI355X, computed by the HIP kernels
+of this package.
+
+Drop-in for ``olmo/model.py``'s ``OLMo.forward`` (``:1253-1465``): same arguments, same
+``OLMoOutput`` tuple, same module tree / parameter names (``transformer.wte``,
+``transformer.blocks.{i}.att_proj`` ... ``transformer.ln_f``, ``transformer.ff_out``) so that a
+reference state dict loads by name and AutoGPTQ-style ``make_quant`` can swap the block
+Linears.  PyTorch holds the parameters and device buffers; every arithmetic step is a kernel
+call through the C-ABI (``olmo_amd.ops``).
+
+KV cache.  The reference returns per layer ``(k, v)`` of shape ``[B, n_kv_heads, L, hd]`` with
+``k`` *before* rotary embedding and re-rotates the whole cache each step
+(``olmo/model.py:615-625``).  Here each layer owns one contiguous buffer of capacity
+``max_cache_len`` holding the *rotated* keys; ``attn_key_values`` are ``LayerKV`` tuples of
+views ``[:, :, :L]`` into it.  Passing them back as ``past_key_values`` continues in place with
+no copy.  Plain tensors passed as ``past_key_values`` are taken to be in the reference's
+form and are rotated into a fresh cache first.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Dict, List, NamedTuple, Optional, Sequence, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import ops
+from .config import ModelConfig, OLMoConfigurationError
+from .qlinear import QuantLinear
+
+__all__ = ["OLMo", "OLMoOutput", "OLMoGenerateOutput", "LayerKV", "KVCache", "DenseLinear"]
+
+
+class OLMoOutput(NamedTuple):
+    """``olmo/model.py:980-995``."""
+
+    logits: torch.Tensor
+    attn_key_values: Optional[List[Tuple[torch.Tensor, torch.Tensor]]]
+    hidden_states: Optional[Tuple[torch.Tensor, ...]]
+
+
+class OLMoGenerateOutput(NamedTuple):
+    """``olmo/model.py:998-1009``: ``token_ids [B, beam, steps]``, ``scores [B, beam]``."""
+
+    token_ids: torch.Tensor
+    scores: torch.Tensor
+
+
+class KVCache:
+    """Contiguous per-layer key/value buffers ``[B, n_kv_heads, capacity, hd]`` (keys rotated)."""
+
+    def __init__(self, n_layers: int, B: int, Hkv: int, capacity: int, hd: int, dtype, device):
+        self.k = [torch.empty(B, Hkv, capacity, hd, dtype=dtype, device=device) for _ in range(n_layers)]
+        self.v = [torch.empty(B, Hkv, capacity, hd, dtype=dtype, device=device) for _ in range(n_layers)]
+        self.B, self.capacity, self.length = B, capacity, 0
+        # device copy of the number of cached positions, for captured decode steps
+        self.length_dev = torch.zeros(1, dtype=torch.int32, device=device)
+
+    def views(self) -> List["LayerKV"]:
+        L = self.length
+        return [LayerKV((k[:, :, :L], v[:, :, :L]), self) for k, v in zip(self.k, self.v)]
+
+    def set_length(self, L: int) -> None:
+        self.length = L
+        self.length_dev.fill_(L)
+
+
+class LayerKV(tuple):
+    """``(k, v)`` views of one layer's cache, remembering the cache they belong to."""
+
+    def __new__(cls, kv, cache: KVCache):
+        self = super().__new__(cls, kv)
+        self.cache = cache
+        return self
+
+
+class DenseLinear(nn.Linear):
+    """``nn.Linear`` without bias whose product runs on the HIP kernels (bf16: re-tiled copy on
+    the matrix cores; fp32: FMA kernel).  Parameters are left uninitialised: weights come from a
+    state dict or from ``OLMo.reset_parameters``."""
+
+    def __init__(self, in_features: int, out_features: int, device=None, dtype=None):
+        nn.Module.__init__(self)
+        self.in_features, self.out_features = in_features, out_features
+        self.weight = nn.Parameter(torch.empty(out_features, in_features, device=device, dtype=dtype),
+                                   requires_grad=False)
+        self.register_parameter("bias", None)
+        self._tiled: Optional[ops.B16Tiled] = None
+
+    def reset_parameters(self) -> None:  # nn.Linear's default init is not wanted
+        pass
+
+    def post_init(self):
+        if self.weight.dtype == torch.bfloat16:
+            self._tiled = ops.b16_repack(self.weight.data.contiguous())
+        return self
+
+    def forward(self, x: torch.Tensor, workspace: ops.Workspace) -> torch.Tensor:
+        if self.weight.dtype == torch.float32:
+            return ops.f32_linear(x, self.weight.data)
+        if self._tiled is None:
+            self.post_init()
+        return ops.b16_linear(x, self._tiled, workspace)
+
+
+class RMSLayerNorm(nn.Module):
+    """``olmo/model.py:228-255``; parameter name ``weight`` as in the reference."""
+
+    def __init__(self, size: int, eps: float, device=None, dtype=None):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(size, device=device, dtype=dtype), requires_grad=False)
+
+    def forward(self, x, residual=None):
+        return ops.rmsnorm(x, self.weight.data, self.eps, residual=residual)
+
+
+class LayerNormNP(nn.Module):
+    """Non-parametric ``LayerNorm`` (``olmo/model.py:193-225`` with ``elementwise_affine=False``)."""
+
+    def __init__(self, size: int, eps: float):
+        super().__init__()
+        self.eps = eps
+        self.weight = None
+
+    def forward(self, x, residual=None):
+        y = ops.layernorm_np(x, self.eps)
+        return y if residual is None else ops.add(residual, y)
+
+
+def _build_norm(cfg: ModelConfig, size: int, device, dtype) -> nn.Module:
+    if cfg.layer_norm_type == "rms":
+        return RMSLayerNorm(size, cfg.layer_norm_eps, device, dtype)
+    return LayerNormNP(size, cfg.layer_norm_eps)
+
+
+class OLMoSequentialBlock(nn.Module):
+    """Module set of ``olmo/model.py:396-506,685-705``; the arithmetic is in ``OLMo._block``."""
+
+    def __init__(self, layer_id: int, cfg: ModelConfig, device, dtype, weight_device=None):
+        super().__init__()
+        self.layer_id = layer_id
+        hd = cfg.head_dim
+        dkv = cfg.effective_n_kv_heads * hd
+        wdev = weight_device if weight_device is not None else device
+        self.att_proj = DenseLinear(cfg.d_model, cfg.d_model + 2 * dkv, wdev, dtype)
+        self.attn_out = DenseLinear(cfg.d_model, cfg.d_model, wdev, dtype)
+        self.ff_proj = DenseLinear(cfg.d_model, cfg.hidden_size, wdev, dtype)
+        self.ff_out = DenseLinear(cfg.act_out_size, cfg.d_model, wdev, dtype)
+        self.attn_norm = _build_norm(cfg, cfg.d_model, device, dtype)
+        self.ff_norm = _build_norm(cfg, cfg.d_model, device, dtype)
+        if cfg.attention_layer_norm:
+            self.q_norm = RMSLayerNorm(cfg.d_model, cfg.layer_norm_eps, device, dtype)
+            self.k_norm = RMSLayerNorm(dkv, cfg.layer_norm_eps, device, dtype)
+        else:
+            self.q_norm = self.k_norm = None
+
+
+class _Embedding(nn.Module):
+    def __init__(self, n: int, d: int, device, dtype):
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty(n, d, device=device, dtype=dtype), requires_grad=False)
+
+    def forward(self, ids):
+        return ops.embedding(ids.contiguous(), self.weight.data)
+
+
+class OLMo(nn.Module):
+    def __init__(self, config: ModelConfig, device="cuda", dtype: torch.dtype = torch.bfloat16,
+                 max_cache_len: Optional[int] = None, block_weight_device=None):
+        """``block_weight_device='meta'`` leaves the four dense Linears of every block unallocated
+        (for models whose block Linears are about to be replaced by ``QuantLinear``)."""
+        super().__init__()
+        config.validate_for_inference()
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise OLMoConfigurationError("activation dtype must be bfloat16 or float32")
+        self.config = config
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self.max_cache_len = max_cache_len or config.max_sequence_length
+        V = config.logits_size
+        self.transformer = nn.ModuleDict(dict(
+            wte=_Embedding(V, config.d_model, device, dtype),
+            blocks=nn.ModuleList([OLMoSequentialBlock(i, config, device, dtype, block_weight_device)
+                                  for i in range(config.n_layers)]),
+            ln_f=_build_norm(config, config.d_model, device, dtype),
+            ff_out=DenseLinear(config.d_model, V, device, dtype),
+        ))
+        self._prepared = False
+        self._ws: Optional[ops.Workspace] = None
+        self._rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
+        self._attn_ws: Dict[Tuple[int, int], torch.Tensor] = {}
+        self._scratch_kv: Dict[Tuple[int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
+
+    # ------------------------------------------------------------------------------------------
+    # parameters
+    # ------------------------------------------------------------------------------------------
+    @torch.no_grad()
+    def reset_parameters(self, seed: int = 0) -> None:
+        """Linear and embedding weights ~ N(0, init_std), truncated at ``init_cutoff_factor`` sigmas
+        when set (``olmo/initialization.py:8-22``); norm weights 1.  (The reference's parameter
+        visiting order, hence its exact random stream, is not reproduced.)"""
+        gen = torch.Generator(device=self.device).manual_seed(seed)
+        c = self.config
+        for p in self.parameters():
+            if p.device.type == "meta":
+                continue
+            if p.dim() == 1:
+                p.fill_(1.0)
+            else:
+                t = torch.empty(p.shape, dtype=torch.float32, device=self.device).normal_(0.0, c.init_std, generator=gen)
+                if c.init_cutoff_factor:
+                    t.clamp_(-c.init_cutoff_factor * c.init_std, c.init_cutoff_factor * c.init_std)
+                p.copy_(t.to(p.dtype))
+        self._prepared = False
+
+    def post_init(self) -> "OLMo":
+        """Build the kernel-side weight layouts, rotary tables and workspaces (idempotent)."""
+        for m in self.modules():
+            if isinstance(m, (DenseLinear, QuantLinear)) and m is not self:
+                if isinstance(m, DenseLinear) and m.weight.device.type == "meta":
+                    raise RuntimeError("a block Linear is still on the meta device: swap it or load weights first")
+                m.post_init()
+        c = self.config
+        n_pos = max(self.max_cache_len, c.max_sequence_length)
+        self._rope = ops.rope_tables(c.head_dim, float(c.rope_theta), n_pos, self.device)
+        self._ws = ops.Workspace(self.device)
+        self._prepared = True
+        return self
+
+    def load_reference_state_dict(self, sd: Dict[str, torch.Tensor]) -> None:
+        """Load tensors keyed by the reference's names (``transformer....``); int4 buffers go to
+        ``QuantLinear`` modules, dense weights are cast to the model dtype."""
+        own = dict(self.named_parameters())
+        own.update(dict(self.named_buffers()))
+        missing = []
+        with torch.no_grad():
+            for name, tgt in own.items():
+                if tgt.device.type == "meta":
+                    continue
+                if name not in sd:
+                    if not name.endswith((".g_idx", ".bias")):
+                        missing.append(name)
+                    continue
+                src = sd[name]
+                if tuple(src.shape) != tuple(tgt.shape):
+                    raise ValueError(f"{name}: shape {tuple(src.shape)} != {tuple(tgt.shape)}")
+                tgt.copy_(src.to(device=tgt.device, dtype=tgt.dtype))
+        if missing:
+            raise KeyError(f"missing tensors: {missing[:5]}{'...' if len(missing) > 5 else ''}")
+        self._prepared = False
+
+    # ------------------------------------------------------------------------------------------
+    # cache handling
+    # ------------------------------------------------------------------------------------------
+    def new_cache(self, B: int, capacity: Optional[int] = None) -> KVCache:
+        c = self.config
+        return KVCache(c.n_layers, B, c.effective_n_kv_heads, capacity or self.max_cache_len, c.head_dim, self.dtype,
+                       self.device)
+
+    def _ingest_reference_cache(self, past: Sequence[Tuple[torch.Tensor, torch.Tensor]], new_tokens: int) -> KVCache:
+        """Reference-form ``past_key_values`` (keys not rotated) -> a cache of this model."""
+        c = self.config
+        B, Hkv, L, hd = past[0][0].shape
+        cache = self.new_cache(B, max(self.max_cache_len, L + new_tokens))
+        sin, cos = self._rope
+        for i, (k, v) in enumerate(past):
+            # reuse the rotary kernel: feed [q | k | v] rows with q := k (discarded), no norm
+            kt = k.to(self.device, self.dtype).transpose(1, 2).reshape(B * L, Hkv * hd)
+            vt = v.to(self.device, self.dtype).transpose(1, 2).reshape(B * L, Hkv * hd)
+            qkv = torch.cat((kt, kt, vt), dim=-1).contiguous()
+            ops.qknorm_rope_kvwrite(qkv, None, None, sin, cos, cache.k[i], cache.v[i], B, L, Hkv, Hkv, hd, 0,
+                                    c.layer_norm_eps)
+        cache.set_length(L)
+        return cache
+
+    def _scratch_cache(self, B: int, T: int):
+        key = (B, T)
+        if key not in self._scratch_kv:
+            self._scratch_kv.clear()
+            c = self.config
+            shape = (B, c.effective_n_kv_heads, T, c.head_dim)
+            self._scratch_kv[key] = (torch.empty(shape, dtype=self.dtype, device=self.device),
+                                     torch.empty(shape, dtype=self.dtype, device=self.device))
+        return self._scratch_kv[key]
+
+    def _decode_ws(self, B: int, n_keys_max: int) -> torch.Tensor:
+        key = (B, n_keys_max)
+        if key not in self._attn_ws:
+            c = self.config
+            self._attn_ws[key] = ops.attn_decode_workspace(B, c.n_heads, c.head_dim, n_keys_max, self.device)
+        return self._attn_ws[key]
+
+    # ------------------------------------------------------------------------------------------
+    # one block: olmo/model.py:728-823 (wiring), :588-654 (attention)
+    # ------------------------------------------------------------------------------------------
+    def _linear(self, m: nn.Module, x: torch.Tensor) -> torch.Tensor:
+        return m(x, self._ws)
+
+    def _block(self, blk: OLMoSequentialBlock, x, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max):
+        c = self.config
+        H, Hkv, hd = c.n_heads, c.effective_n_kv_heads, c.head_dim
+        h = x if c.norm_after else blk.attn_norm(x)
+        qkv = self._linear(blk.att_proj, h)
+        sin, cos = self._rope
+        qw = blk.q_norm.weight.data if blk.q_norm is not None else None
+        kw = blk.k_norm.weight.data if blk.k_norm is not None else None
+        q = ops.qknorm_rope_kvwrite(qkv, qw, kw, sin, cos, kc, vc, B, T, H, Hkv, hd, past_len, c.layer_norm_eps,
+                                    past_len_dev=graph_pos)
+        if T == 1 and (graph_pos is not None or past_len > 0):
+            att = ops.attn_decode(q, kc, vc, self._decode_ws(B, n_keys_max), B, H, Hkv, hd, past_len, n_keys_max,
+                                  key_bias=key_bias, past_len_dev=graph_pos)
+        else:
+            att = ops.attn_prefill(q, kc, vc, B, T, H, Hkv, hd, past_len, key_bias=key_bias)
+        att = self._linear(blk.attn_out, att)
+        x = blk.attn_norm(att, residual=x) if c.norm_after else ops.add(x, att)
+        h = x if c.norm_after else blk.ff_norm(x)
+        h = self._linear(blk.ff_proj, h)
+        h = ops.swiglu(h)
+        h = self._linear(blk.ff_out, h)
+        return blk.ff_norm(h, residual=x) if c.norm_after else ops.add(x, h)
+
+    # ------------------------------------------------------------------------------------------
+    # forward: olmo/model.py:1253-1465
+    # ------------------------------------------------------------------------------------------
+    @torch.no_grad()
+    def forward(
+        self,
+        input_ids: Optional[torch.LongTensor],
+        input_embeddings: Optional[torch.Tensor] = None,
+        attention_mask: Optional[torch.Tensor] = None,
+        attention_bias: Optional[torch.Tensor] = None,
+        past_key_values: Optional[Sequence[Tuple[torch.Tensor, torch.Tensor]]] = None,
+        use_cache: bool = False,
+        last_logits_only: bool = False,
+        output_hidden_states: Optional[bool] = None,
+        doc_lens: Optional[torch.Tensor] = None,
+        max_doc_lens: Optional[Sequence[int]] = None,
+    ) -> OLMoOutput:
+        c = self.config
+        if attention_bias is not None:
+            raise NotImplementedError("an explicit attention_bias is not implemented; causal + attention_mask only")
+        if doc_lens is not None or max_doc_lens is not None:
+            raise NotImplementedError("intra-document masking is a training feature and is not implemented")
+        if not self._prepared:
+            self.post_init()
+        if past_key_values:
+            assert len(past_key_values) == c.n_layers
+        if input_embeddings is None:
+            B, T = input_ids.shape
+            x = self.transformer["wte"](input_ids.to(self.device))
+        else:
+            B, T = input_embeddings.shape[:2]
+            x = input_embeddings.to(self.device, self.dtype).contiguous()
+
+        # ---- cache ---------------------------------------------------------------------------
+        cache: Optional[KVCache] = None
+        if past_key_values:
+            first = past_key_values[0]
+            if isinstance(first, LayerKV):
+                cache = first.cache
+                past_len = first[0].size(-2)
+                if past_len != cache.length:
+                    cache.set_length(past_len)  # caller truncated / rewound the views
+            else:
+                cache = self._ingest_reference_cache(past_key_values, T)
+                past_len = cache.length
+            if cache.B != B:
+                raise ValueError("batch size differs from the cache's")
+            if past_len + T > cache.capacity:
+                raise ValueError(f"KV cache capacity {cache.capacity} exceeded ({past_len}+{T}); "
+                                 "construct the model with a larger max_cache_len")
+        else:
+            past_len = 0
+            if use_cache:
+                cache = self.new_cache(B, max(self.max_cache_len, T))
+
+        # ---- padding mask -> additive per-key bias (olmo/model.py:1337-1340) ---------------------
+        key_bias = None
+        if attention_mask is not None:
+            am = attention_mask.to(self.device, torch.float32).view(B, -1)
+            if am.shape[1] != past_len + T:
+                raise ValueError(f"attention_mask covers {am.shape[1]} positions, expected {past_len + T}")
+            key_bias = ((1.0 - am) * torch.finfo(torch.float32).min).contiguous()
+
+        logits, hidden = self._forward_tokens(x, cache, B, T, past_len, key_bias, None, last_logits_only,
+                                              bool(output_hidden_states))
+        if cache is not None:
+            cache.set_length(past_len + T)
+        kvs = cache.views() if (use_cache and cache is not None) else None
+        return OLMoOutput(logits=logits, attn_key_values=kvs, hidden_states=hidden)
+
+    def _forward_tokens(self, x, cache: Optional[KVCache], B: int, T: int, past_len: int, key_bias, graph_pos,
+                        last_logits_only: bool, collect_hidden: bool = False):
+        """Blocks, final norm and head on embedded tokens ``x [B,T,d]``.  With ``graph_pos`` (device
+        int32 holding the number of cached positions) the launch arguments do not depend on the
+        position, so the call can be captured once and replayed; it requires ``T == 1``."""
+        n_keys_max = cache.capacity if graph_pos is not None else past_len + T
+        hidden: List[torch.Tensor] = []
+        for i, blk in enumerate(self.transformer["blocks"]):
+            if collect_hidden:
+                hidden.append(x)
+            if cache is not None:
+                kc, vc = cache.k[i], cache.v[i]
+            else:
+                kc, vc = self._scratch_cache(B, T)
+            x = self._block(blk, x, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max)
+        if last_logits_only and T > 1:
+            x = x[:, -1, :].unsqueeze(1).contiguous()
+        x = self.transformer["ln_f"](x)
+        if collect_hidden:
+            hidden.append(x)
+        logits = self._linear(self.transformer["ff_out"], x)
+        return logits, (tuple(hidden) if collect_hidden else None)
+
+    # ------------------------------------------------------------------------------------------
+    # greedy generation: olmo/model.py:1603-1728 with beam_size 1 and the deterministic sampler
+    # (olmo/beam_search.py:102-113): next = argmax(log_softmax(logits)) = argmax(logits)
+    # ------------------------------------------------------------------------------------------
+    @torch.no_grad()
+    def generate(self, input_ids: torch.LongTensor, attention_mask: Optional[torch.Tensor] = None,
+                 max_steps: int = 10, beam_size: int = 1, use_graph: bool = True,
+                 stop_at_eos: bool = False) -> OLMoGenerateOutput:
+        if beam_size != 1:
+            raise NotImplementedError("only greedy search (beam_size=1) is implemented")
+        from .generate import greedy_generate
+
+        toks, scores = greedy_generate(self, input_ids, attention_mask, max_steps, use_graph=use_graph,
+                                       eos_token_id=self.config.eos_token_id if stop_at_eos else None,
+                                       return_scores=True)
+        return OLMoGenerateOutput(token_ids=toks.unsqueeze(1), scores=scores.unsqueeze(1))
+
+    @property
+    def num_params(self) -> int:
+        return sum(p.numel() for p in self.parameters())
