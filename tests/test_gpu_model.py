@@ -83,6 +83,9 @@ def agreement(dev_tokens, oracle_logits):
     strict = (chosen == mx).float().mean().item()
     ulp = 2.0 ** (torch.floor(torch.log2(mx.abs().clamp_min(1e-30))) - 7)
     loose = (chosen >= mx - ulp).float().mean().item()
+    miss = (chosen < mx - ulp)
+    if miss.any():
+        say("  disagreements: gap to the oracle maximum in bf16 ulps:", ((mx - chosen) / ulp)[miss].tolist())
     return strict, loose
 
 
@@ -172,7 +175,10 @@ def test_forward_parity_and_invariants(dev, kind, dtype, quantized):
     # (d) last_logits_only, hidden states
     o5 = model(ids.to(dev), last_logits_only=True, output_hidden_states=True)
     assert o5.logits.shape == (2, 1, cfg.logits_size) and len(o5.hidden_states) == cfg.n_layers + 1
-    assert torch.equal(o5.logits[:, 0].cpu(), lg[:, -1])
+    # the 2-row head product takes the small-M kernel, the full one the tiled kernel: same fp32 sums in a
+    # different order, so equal up to the last bit of the rounded result
+    a5, b5 = o5.logits[:, 0].cpu().float(), lg[:, -1].float()
+    assert torch.allclose(a5, b5, rtol=2 ** -7, atol=2 ** -7 if dtype == torch.bfloat16 else 1e-5)
 
 
 @pytest.mark.parametrize("quantized", [False, True])
@@ -185,15 +191,15 @@ def test_hf_wrapper_and_greedy_generate(dev, quantized):
     cfg = small_cfg("olmo2")
     model, oracle = build_pair(cfg, torch.bfloat16, dev, quantized, seed=3)
     hf = OLMoForCausalLM(OLMoConfig.from_model_config(cfg, use_cache=True), model=model)
-    ids = torch.randint(0, cfg.vocab_size, (2, 40), generator=torch.Generator().manual_seed(5)).to(dev)
+    ids = torch.randint(0, cfg.vocab_size, (4, 40), generator=torch.Generator().manual_seed(5)).to(dev)
     o = hf(ids)
     assert torch.equal(o.logits, model(ids).logits) and o.past_key_values is not None
     with pytest.raises(ValueError):
         hf(ids, output_attentions=True)
-    steps = 48
+    steps = 128
     g = hf.generate(ids, max_new_tokens=steps, use_graph=True)
     e = hf.generate(ids, max_new_tokens=steps, use_graph=False)
-    assert g.shape == (2, 40 + steps) and torch.equal(g[:, :40], ids)
+    assert g.shape == (4, 40 + steps) and torch.equal(g[:, :40], ids)
     assert torch.equal(g, e), "graph replay differs from eager decode"
     # step-by-step through the HF forward with prepare_inputs_for_generation
     cur, past = ids, None
@@ -207,12 +213,12 @@ def test_hf_wrapper_and_greedy_generate(dev, quantized):
     full = g.cpu()
     ref, _ = oracle.forward(full[:, :-1])
     strict, loose = agreement(full[:, 40:], ref[:, 39:])
-    say(f"  greedy agreement over {steps} steps x 2: strict {strict:.4f}  ulp {loose:.4f}")
+    say(f"  greedy agreement over {steps} steps x 4: strict {strict:.4f}  ulp {loose:.4f}")
     assert loose >= 0.99
     # native generate surface
     og = model.generate(ids, max_steps=5)
-    assert og.token_ids.shape == (2, 1, 5) and torch.equal(og.token_ids[:, 0], g[:, 40:45])
-    assert og.scores.shape == (2, 1) and (og.scores <= 0).all()
+    assert og.token_ids.shape == (4, 1, 5) and torch.equal(og.token_ids[:, 0], g[:, 40:45])
+    assert og.scores.shape == (4, 1) and (og.scores <= 0).all()
 
 
 def test_quantlinear_module_surface(dev):
