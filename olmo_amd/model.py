@@ -249,6 +249,9 @@ class OLMo(nn.Module):
                 tgt.copy_(src.to(device=tgt.device, dtype=tgt.dtype))
         if missing:
             raise KeyError(f"missing tensors: {missing[:5]}{'...' if len(missing) > 5 else ''}")
+        for m in self.modules():
+            if isinstance(m, QuantLinear):
+                m._tiled = None
         self._prepared = False
 
     # ------------------------------------------------------------------------------------------

@@ -65,7 +65,9 @@ class QuantLinear(nn.Module):
 
     # -- one-time preparation ------------------------------------------------------------------
     def post_init(self, free_checkpoint_buffers: bool = False):
-        """Validate the buffers and build the tiled copy on the GPU."""
+        """Validate the buffers and build the tiled copy on the GPU (no-op when already built)."""
+        if self._tiled is not None:
+            return self
         if not self.qweight.is_cuda:
             raise RuntimeError("QuantLinear.post_init needs the buffers on the GPU; there is no CPU path")
         K = self.infeatures
@@ -81,6 +83,10 @@ class QuantLinear(nn.Module):
             self.qweight, self.qzeros = empty, empty.clone()
             self.scales = torch.empty(0, dtype=torch.float16, device=self.scales.device)
         return self
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self._tiled = None  # new buffers: the tiled copy must be rebuilt
+        return super()._load_from_state_dict(*args, **kwargs)
 
     @property
     def tiled(self) -> ops.W4Tiled:
@@ -149,10 +155,11 @@ def find_layers(module: nn.Module, layers=(nn.Linear,), name: str = ""):
 
 def make_quant(module: nn.Module, names: Iterable[str], bits: int, group_size: int, name: str = "",
                use_triton: bool = False, disable_exllama: bool = False, use_cuda_fp16: bool = True,
-               desc_act: bool = False, trainable: bool = False):
+               desc_act: bool = False, trainable: bool = False, device=None):
     """Replace every ``nn.Linear`` whose qualified name is in ``names`` by a ``QuantLinear`` with a
     zero bias buffer -- same contract as the reference's ``make_quant``
-    (``AGQ/auto_gptq/modeling/_utils.py:52-111``)."""
+    (``AGQ/auto_gptq/modeling/_utils.py:52-111``).  ``device`` (not in the reference) places the buffers of
+    layers that replace meta-device Linears."""
     if use_triton:
         raise NotImplementedError("no Triton back-end here")
     if desc_act and group_size != -1:
@@ -164,13 +171,13 @@ def make_quant(module: nn.Module, names: Iterable[str], bits: int, group_size: i
         name1 = name + "." + attr if name else attr
         if name1 in names and isinstance(child, nn.Linear):
             dev = child.weight.device
-            dev = None if dev.type == "meta" else dev
+            dev = device if dev.type == "meta" else dev  # meta: the caller says where the buffers go
             new = QuantLinear(bits, group_size, child.in_features, child.out_features, True,
                               use_cuda_fp16=use_cuda_fp16, trainable=trainable, device=dev)
             setattr(module, attr, new)
         else:
             make_quant(child, names, bits, group_size, name1, use_triton=use_triton, disable_exllama=disable_exllama,
-                       use_cuda_fp16=use_cuda_fp16, desc_act=desc_act, trainable=trainable)
+                       use_cuda_fp16=use_cuda_fp16, desc_act=desc_act, trainable=trainable, device=device)
 
 
 class OLMoGPTQForCausalLM:

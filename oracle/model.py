@@ -112,8 +112,12 @@ class OracleModel:
     ``(logits, attn_key_values)`` with the cache in the reference's form: per layer ``(k, v)``
     of shape ``[B, n_kv_heads, L, hd]``, ``k`` post-QK-norm and *pre*-RoPE (``olmo/model.py:615-625``)."""
 
-    def __init__(self, cfg, weights: Dict[str, torch.Tensor], act_dtype: torch.dtype, group_size: int = 128):
+    def __init__(self, cfg, weights: Dict[str, torch.Tensor], act_dtype: torch.dtype, group_size: int = 128,
+                 cache_weights: bool = True):
+        """``cache_weights=False`` widens / dequantises the weight on every call, as the reference's
+        ``QuantLinear.forward`` does (``AGQ:qlinear_cuda_old.py:236-287``); used when timing."""
         self.cfg = cfg
+        self.cache_weights = cache_weights
         self.w = weights
         self.act = act_dtype
         self.group_size = group_size
@@ -123,15 +127,17 @@ class OracleModel:
     # -- linear layers ---------------------------------------------------------------------
     def _weight_kn_f32(self, prefix: str) -> torch.Tensor:
         """fp32 ``[K, N]`` operand of Linear ``prefix``, dense or dequantised, cached."""
-        if prefix not in self._wf32:
-            if prefix + ".weight" in self.w:
-                self._wf32[prefix] = self.w[prefix + ".weight"].to(torch.float32).t().contiguous()
-            else:
-                w16 = w4.dequantize(
-                    self.w[prefix + ".qweight"], self.w[prefix + ".qzeros"], self.w[prefix + ".scales"], self.group_size
-                )
-                self._wf32[prefix] = w16.to(torch.float32)
-        return self._wf32[prefix]
+        if prefix in self._wf32:
+            return self._wf32[prefix]
+        if prefix + ".weight" in self.w:
+            w = self.w[prefix + ".weight"].to(torch.float32).t()
+        else:
+            w = w4.dequantize(
+                self.w[prefix + ".qweight"], self.w[prefix + ".qzeros"], self.w[prefix + ".scales"], self.group_size
+            ).to(torch.float32)
+        if self.cache_weights:
+            self._wf32[prefix] = w = w.contiguous()
+        return w
 
     def linear(self, prefix: str, x: torch.Tensor) -> torch.Tensor:
         """``nn.Linear`` without bias, or ``QuantLinear.forward``'s dequantise-then-matmul
