@@ -102,11 +102,10 @@ def main() -> int:
     shapes = linear_shapes(cfg)
     qls = [m for m in model.modules() if isinstance(m, QuantLinear)]
     xs = {k: torch.randn(1, k, device=dev).to(torch.bfloat16) for k in {s[1] for s in shapes}}
-    ws = ops.Workspace(dev)
 
     def one_step_of_linears():
         for q in qls:
-            ops.w4_linear(xs[q.infeatures], q.tiled, ws)
+            ops.w4_linear(xs[q.infeatures], q.tiled)
 
     one_step_of_linears()
     torch.cuda.synchronize()
@@ -135,12 +134,12 @@ def main() -> int:
     xp = {k: torch.randn(ctx, k, device=dev).to(torch.bfloat16) for k in {s[1] for s in shapes}}
     layer = qls[:4]
     for q in layer:
-        ops.w4_linear(xp[q.infeatures], q.tiled, ws)
+        ops.w4_linear(xp[q.infeatures], q.tiled)
     torch.cuda.synchronize()
     e0.record()
     for _ in range(3):
         for q in layer:
-            ops.w4_linear(xp[q.infeatures], q.tiled, ws)
+            ops.w4_linear(xp[q.infeatures], q.tiled)
     e1.record()
     torch.cuda.synchronize()
     flops = sum(2.0 * ctx * n * k for n, k in shapes)

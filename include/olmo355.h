@@ -71,14 +71,9 @@ int olmo355_w4t_dequant_fp16(const uint32_t* wt, const uint16_t* st, const uint8
  * Small-M path (M <= 64): stands in for vecquant4matmul_faster_old
  * (AGQ/autogptq_extension/cuda_256/autogptq_cuda_256.cpp:158-171, kernel
  * autogptq_cuda_kernel_256.cu:1365-1435) and exllama's q4_matmul GEMV
- * (exllama/cuda_func/q4_matmul.cu:32-143).  Deterministic (no atomics on data).
- * `ws` is a workspace of olmo355_w4_gemv_workspace_bytes(M,N,K) bytes whose first
- * O355_GEMV_COUNTER_BYTES bytes must be zero before the first call (the kernel leaves them
- * zero); it may be NULL when that function returns 0. */
-#define O355_GEMV_COUNTER_BYTES 16384
-int64_t olmo355_w4_gemv_workspace_bytes(int M, int N, int K);
+ * (exllama/cuda_func/q4_matmul.cu:32-143).  Deterministic: no atomics, fixed summation order. */
 int olmo355_w4_gemv(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
-                    void* ws, int M, int N, int K, void* stream);
+                    int M, int N, int K, void* stream);
 
 /* Large-M path: dequantise tiles into LDS as bf16 and multiply on the matrix cores.  Stands
  * in for the reference's dequantise-then-matmul branch (AGQ qlinear_cuda_old.py:236-287) and
@@ -91,8 +86,8 @@ int olmo355_w4_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, c
  * (lane l: row n = 16*nt + (l&15), columns 32*ks + 8*(l>>4) .. +7); K % 32 == 0, N % 16 == 0.
  * fp32: weight in torch layout [N,K]. */
 int olmo355_b16_repack(const uint16_t* w_nk, uint16_t* wt, int N, int K, void* stream);
-/* small-M (<= 64) path; `ws` follows the rules of olmo355_w4_gemv (same size function) */
-int olmo355_b16_gemv(const uint16_t* x, const uint16_t* wt, uint16_t* y, void* ws, int M, int N, int K, void* stream);
+/* small-M (<= 64) path */
+int olmo355_b16_gemv(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, void* stream);
 int olmo355_b16_gemm(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, void* stream);
 int olmo355_f32_linear(const float* x, const float* w_nk, float* y, int M, int N, int K, void* stream);
 

@@ -36,11 +36,10 @@ EXPORTS = {
     "olmo355_w4_dequant_fp16": (I, [P, P, P, P, P, I, I, I, P]),
     "olmo355_w4_repack": (I, [P, P, P, P, P, P, I, I, I, P]),
     "olmo355_w4t_dequant_fp16": (I, [P, P, P, P, I, I, P]),
-    "olmo355_w4_gemv_workspace_bytes": (L, [I, I, I]),
-    "olmo355_w4_gemv": (I, [P, P, P, P, P, P, I, I, I, P]),
+    "olmo355_w4_gemv": (I, [P, P, P, P, P, I, I, I, P]),
     "olmo355_w4_gemm": (I, [P, P, P, P, P, I, I, I, P]),
     "olmo355_b16_repack": (I, [P, P, I, I, P]),
-    "olmo355_b16_gemv": (I, [P, P, P, P, I, I, I, P]),
+    "olmo355_b16_gemv": (I, [P, P, P, I, I, I, P]),
     "olmo355_b16_gemm": (I, [P, P, P, I, I, I, P]),
     "olmo355_f32_linear": (I, [P, P, P, I, I, I, P]),
     "olmo355_rmsnorm": (I, [P, P, P, P, I, I, F, I, P]),

@@ -5,7 +5,7 @@
 //    MFMA-fragment order, S^T = K.Q^T and O^T = V^T.P^T on the matrix cores so the softmax
 //    statistics of a query stay in one lane column and P never leaves registers.
 //  * attn_decode_kernel        one query per sequence, keys split over workgroups and waves,
-//    wave-level reductions, partial (max, sum, o) merged by attn_decode_combine_kernel.
+//    DPP / wave reductions, partial (max, sum, o) merged by attn_decode_combine_kernel.
 //  * attn_generic_kernel       any dtype / head size <= 128, one query per thread (used for the
 //    fp32 model configuration).
 //
@@ -18,6 +18,29 @@
 namespace {
 
 constexpr float kMaskThreshold = -1e30f;
+
+// 8 consecutive channels as floats: one 16-byte vector of bf16 or two of fp32
+template <int DT> struct Vec8;
+template <> struct Vec8<O355_BF16> {
+  static __device__ __forceinline__ void unpack(const u32x4 (&r)[1], float (&f)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[2 * i] = bf16lo_to_f32(r[0][i]), f[2 * i + 1] = bf16hi_to_f32(r[0][i]);
+  }
+  static __device__ __forceinline__ void ld(const void* p, int64_t elem, float (&f)[8]) {
+    u32x4 r[1] = {reinterpret_cast<const u32x4*>(p)[elem >> 3]};
+    unpack(r, f);
+  }
+};
+template <> struct Vec8<O355_F32> {
+  static __device__ __forceinline__ void unpack(const u32x4 (&r)[2], float (&f)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(r[0][i]), f[4 + i] = __uint_as_float(r[1][i]);
+  }
+  static __device__ __forceinline__ void ld(const void* p, int64_t elem, float (&f)[8]) {
+    u32x4 r[2] = {reinterpret_cast<const u32x4*>(p)[elem >> 2], reinterpret_cast<const u32x4*>(p)[(elem >> 2) + 1]};
+    unpack(r, f);
+  }
+};
 
 // =====================================================================================================
 // generic: one thread per query row, K/V tiles of 32 keys in LDS as fp32
@@ -259,9 +282,29 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const uint16_t* 
 }
 
 // =====================================================================================================
-// decode: one query per (batch, head); keys split into chunks of 256 (64 per wave)
+// decode: one query per (batch, head); keys split into chunks of 128 (32 per wave)
 // =====================================================================================================
-constexpr int kDecodeChunk = 256;
+// A lane owns 8 channels of one key: LPK = HD/8 lanes cover a key row with one 16-byte load each,
+// a wave covers 64/LPK keys per load instruction.  All K and V loads of the wave's 32 keys are
+// issued before the first use (the kernel is latency-bound at batch 1); the dot product is reduced
+// over the LPK lanes with DPP adds.
+constexpr int kDecodeChunk = 128;
+constexpr int kDecodeKeysPerWave = 32;
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true);
+  return v + __builtin_bit_cast(float, t);
+}
+// sum over aligned groups of W lanes (W = 4, 8 or 16); every lane of the group gets the sum
+template <int W>
+__device__ __forceinline__ float group_sum(float v) {
+  v = dpp_add<0xB1>(v);                          // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E>(v);                          // quad_perm [2,3,0,1]
+  if constexpr (W >= 8) v = dpp_add<0x141>(v);   // row_half_mirror
+  if constexpr (W >= 16) v = dpp_add<0x140>(v);  // row_mirror
+  return v;
+}
 
 template <int DT, int HD>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const void* __restrict__ q, const void* __restrict__ kc,
@@ -270,9 +313,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const void* __restrict
                                                           int H, int Hkv, int Lmax, int past_len,
                                                           const int32_t* __restrict__ past_dev, int nchunks_max,
                                                           int bias_stride) {
-  constexpr int LPK = HD / 8;     // lanes per key (8 elements each)
-  constexpr int KPI = 64 / LPK;   // keys per wave iteration
-  constexpr int ITERS = 64 / KPI; // iterations per wave (64 keys)
+  constexpr int LPK = HD / 8;                        // lanes per key (8 channels each)
+  constexpr int KPI = 64 / LPK;                      // keys per wave iteration
+  constexpr int ITERS = kDecodeKeysPerWave / KPI;    // iterations per wave
+  constexpr int VW = DT == O355_BF16 ? 1 : 2;        // 16-byte vectors per 8 channels
   __shared__ float red_o[4][HD];
   __shared__ float red_ml[4][2];
   const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z, hk = h / (H / Hkv);
@@ -283,62 +327,60 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const void* __restrict
   const float scale = 1.f / sqrtf((float)HD);
   const float lowest = Act<DT>::lowest();
   const int64_t cbase = ((int64_t)b * Hkv + hk) * Lmax * HD;
-  float qr[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) qr[i] = Act<DT>::ld(q, ((int64_t)b * H + h) * HD + sub * 8 + i);
+  const int kbase = chunk * kDecodeChunk + wave * kDecodeKeysPerWave;
 
-  const int kbase = chunk * kDecodeChunk + wave * 64;
+  // ---- every load of this wave, issued up front -------------------------------------------------
+  u32x4 kreg[ITERS][VW], vreg[ITERS][VW];
+  float bias[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int keyc = min(kbase + it * KPI + kslot, L - 1);
+    const int64_t e = cbase + (int64_t)keyc * HD + sub * 8;
+#pragma unroll
+    for (int v = 0; v < VW; ++v) kreg[it][v] = reinterpret_cast<const u32x4*>(kc)[e * VW / 8 + v];
+  }
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int keyc = min(kbase + it * KPI + kslot, L - 1);
+    const int64_t e = cbase + (int64_t)keyc * HD + sub * 8;
+#pragma unroll
+    for (int v = 0; v < VW; ++v) vreg[it][v] = reinterpret_cast<const u32x4*>(vc)[e * VW / 8 + v];
+    bias[it] = key_bias ? key_bias[(int64_t)b * bias_stride + keyc] : 0.f;
+  }
+  float qr[8];
+  Vec8<DT>::ld(q, ((int64_t)b * H + h) * HD + sub * 8, qr);
+
   float s[ITERS];
   float wmax = -INFINITY;
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const int key = kbase + it * KPI + kslot;
-    const int keyc = min(key, L - 1);
+    float kf[8];
+    Vec8<DT>::unpack(kreg[it], kf);
     float d = 0.f;
-    if constexpr (DT == O355_BF16) {
-      const u32x4 kv = *reinterpret_cast<const u32x4*>((const uint16_t*)kc + cbase + (int64_t)keyc * HD + sub * 8);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        d = __builtin_fmaf(qr[2 * i], bf16lo_to_f32(kv[i]), d);
-        d = __builtin_fmaf(qr[2 * i + 1], bf16hi_to_f32(kv[i]), d);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) d = __builtin_fmaf(qr[i], Act<DT>::ld(kc, cbase + (int64_t)keyc * HD + sub * 8 + i), d);
-    }
-#pragma unroll
-    for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, 64);
-    const float bias = key_bias ? key_bias[(int64_t)b * bias_stride + keyc] : 0.f;
-    float v = bias <= kMaskThreshold ? lowest : d * scale + bias;
+    for (int i = 0; i < 8; ++i) d = __builtin_fmaf(qr[i], kf[i], d);
+    d = group_sum<LPK>(d);
+    float v = bias[it] <= kMaskThreshold ? lowest : d * scale + bias[it];
     v = key < L ? v : -INFINITY;
     s[it] = v;
     wmax = fmaxf(wmax, v);
   }
 #pragma unroll
   for (int o = LPK; o < 64; o <<= 1) wmax = fmaxf(wmax, __shfl_xor(wmax, o, 64));
-  // a wave whose 64 keys all lie beyond L contributes nothing
+  // a wave whose keys all lie beyond L contributes nothing
   const bool empty = (kbase >= L);
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float lsum = 0.f;
   if (!empty) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      const int key = kbase + it * KPI + kslot;
-      const int keyc = min(key, L - 1);
       const float p = __expf(s[it] - wmax);  // exp(-inf) = 0 for keys beyond L
       lsum += p;
-      if constexpr (DT == O355_BF16) {
-        const u32x4 vv = *reinterpret_cast<const u32x4*>((const uint16_t*)vc + cbase + (int64_t)keyc * HD + sub * 8);
+      float vf[8];
+      Vec8<DT>::unpack(vreg[it], vf);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          acc[2 * i] = __builtin_fmaf(p, bf16lo_to_f32(vv[i]), acc[2 * i]);
-          acc[2 * i + 1] = __builtin_fmaf(p, bf16hi_to_f32(vv[i]), acc[2 * i + 1]);
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-          acc[i] = __builtin_fmaf(p, Act<DT>::ld(vc, cbase + (int64_t)keyc * HD + sub * 8 + i), acc[i]);
-      }
+      for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, vf[i], acc[i]);
     }
     // sum over the key slots of the wave (lanes with equal `sub`)
 #pragma unroll
@@ -379,17 +421,32 @@ __global__ __launch_bounds__(HD) void attn_decode_combine_kernel(const float* __
                                                                  int H, int past_len,
                                                                  const int32_t* __restrict__ past_dev,
                                                                  int nchunks_max) {
+  constexpr int UN = 8;  // partials fetched per round, all loads before the first use
   const int h = blockIdx.x, b = blockIdx.y;
   const int L = (past_dev ? *past_dev : past_len) + 1;
   const int nch = (L + kDecodeChunk - 1) / kDecodeChunk;
   const float* src = ws + ((int64_t)b * H + h) * nchunks_max * (HD + 2);
-  float mm = -INFINITY;
-  for (int c = 0; c < nch; ++c) mm = fmaxf(mm, src[c * (HD + 2) + HD]);
-  float ov = 0.f, lv = 0.f;
-  for (int c = 0; c < nch; ++c) {
-    const float w = __expf(src[c * (HD + 2) + HD] - mm);
-    ov += src[c * (HD + 2) + threadIdx.x] * w;
-    lv += src[c * (HD + 2) + HD + 1] * w;
+  float mm = -INFINITY, ov = 0.f, lv = 0.f;
+  for (int c0 = 0; c0 < nch; c0 += UN) {
+    float m[UN], l[UN], o[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int c = min(c0 + u, nch - 1);
+      m[u] = src[c * (HD + 2) + HD], l[u] = src[c * (HD + 2) + HD + 1], o[u] = src[c * (HD + 2) + threadIdx.x];
+    }
+    float rm = mm;
+#pragma unroll
+    for (int u = 0; u < UN; ++u)
+      if (c0 + u < nch) rm = fmaxf(rm, m[u]);
+    const float a = __expf(mm - rm);  // exp(-inf) = 0 on the first round
+    ov *= a, lv *= a;
+#pragma unroll
+    for (int u = 0; u < UN; ++u)
+      if (c0 + u < nch) {
+        const float w = __expf(m[u] - rm);
+        ov += o[u] * w, lv += l[u] * w;
+      }
+    mm = rm;
   }
   Act<DT>::st(out, ((int64_t)b * H + h) * HD + threadIdx.x, ov / lv);
 }

@@ -58,6 +58,14 @@ template <> struct Act<O355_BF16> {
   static __device__ __forceinline__ float lowest() { return -3.3895313892515355e38f; }
 };
 
+// Workgroup barrier that orders LDS traffic only: global loads issued before it stay in flight
+// (a plain __syncthreads() would wait for them as well).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // ---- wave64 reductions ------------------------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -10,9 +10,9 @@
 // and the fp32 epilogue adds scale[n]*(T - (128+zero[n])*X), which equals
 // sum_k x*scale*(q-zero) with the scale and zero applied in fp32.
 //
-// K is split over the waves of a workgroup (LDS reduction in fixed order) and optionally over
-// workgroups (fp32 partials + a ticket; the last workgroup adds the partials in fixed order),
-// so the result does not depend on scheduling.
+// K is split over the waves of a workgroup only (contiguous slice per wave, LDS reduction in
+// fixed order): no atomics, no cross-workgroup pass, so the result does not depend on scheduling.
+// Each wave keeps U one-KiB weight pieces in flight and refills a slot as soon as it is consumed.
 #include "common.h"
 
 namespace {
@@ -37,12 +37,10 @@ __device__ __forceinline__ bf16x8 load_x_frag(const uint16_t* __restrict__ x, in
   return __builtin_bit_cast(bf16x8, z);
 }
 
-// Shared epilogue: reduce acc over the waves of the workgroup, then either write y or go
-// through the cross-workgroup ticket.
+// Reduce acc over the waves of the workgroup in fixed order and write y (bf16).
 template <int MT, int NT, int WAVES>
-__device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][NT], float* red, uint16_t* __restrict__ y,
-                                              float* __restrict__ partial, unsigned* __restrict__ counters, int M, int N,
-                                              int nt0, int ntiles, int ksplit) {
+__device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][NT], float* red, uint16_t* __restrict__ y, int M, int N,
+                                              int nt0, int ntiles) {
   constexpr int PER_WAVE = MT * NT * 256;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
@@ -52,8 +50,6 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][NT], float* red, 
 #pragma unroll
       for (int r = 0; r < 4; ++r) red[wave * PER_WAVE + ((mt * NT + nt) * 4 + r) * 64 + lane] = acc[mt][nt][r];
   __syncthreads();
-  const int s = blockIdx.y;
-  const int Mp = MT * 16;
   for (int i = threadIdx.x; i < PER_WAVE; i += WAVES * 64) {
     float v = 0.f;
 #pragma unroll
@@ -62,56 +58,79 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][NT], float* red, 
     const int nt = t % NT, mt = t / NT;
     const int m = mt * 16 + 4 * (l >> 4) + r;
     const int n = (nt0 + nt) * 16 + (l & 15);
-    if (nt0 + nt < ntiles) {
-      if (ksplit == 1) {
-        if (m < M) y[(int64_t)m * N + n] = f32_to_bf16_bits(v);
-      } else {
-        partial[((int64_t)s * Mp + m) * N + n] = v;
-      }
-    }
+    if (nt0 + nt < ntiles && m < M) y[(int64_t)m * N + n] = f32_to_bf16_bits(v);
   }
-  if (ksplit == 1) return;
-  __shared__ int is_last;
-  __threadfence();
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const unsigned t = atomicAdd(&counters[blockIdx.x], 1u);
-    is_last = (t == (unsigned)(ksplit - 1));
-  }
-  __syncthreads();
-  if (!is_last) return;
-  __threadfence();
-  for (int i = threadIdx.x; i < PER_WAVE; i += WAVES * 64) {
-    const int l = i & 63, r = (i >> 6) & 3, t = i >> 8;
-    const int nt = t % NT, mt = t / NT;
-    const int m = mt * 16 + 4 * (l >> 4) + r;
-    const int n = (nt0 + nt) * 16 + (l & 15);
-    if (nt0 + nt < ntiles && m < M) {
-      float v = 0.f;
-      for (int ss = 0; ss < ksplit; ++ss)
-        v += __hip_atomic_load(&partial[((int64_t)ss * Mp + m) * N + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      y[(int64_t)m * N + n] = f32_to_bf16_bits(v);
-    }
-  }
-  if (threadIdx.x == 0) __hip_atomic_store(&counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int MT, int NT, int WAVES>
+// Activation fragments.  XLDS: the workgroup first copies its M rows of x into LDS (plus one
+// zero row that the padding lanes read), and every A operand is one ds_read_b128 issued right
+// before its MFMA; otherwise the fragments come from global memory with the weight loads.
+template <bool XLDS>
+struct XSource {
+  const uint16_t* x;
+  const uint16_t* lds;  // [M+1][K] when XLDS
+  int M, K, row_off;    // row_off: element offset of this lane's row in LDS
+  __device__ __forceinline__ bf16x8 frag(int mt, int col, int k) const {
+    if constexpr (XLDS) {
+      return *reinterpret_cast<const bf16x8*>(lds + row_off + k);
+    } else {
+      return load_x_frag(x, mt * 16 + col, M, K, k);
+    }
+  }
+};
+
+// Copy of the M activation rows into LDS in two halves around the weight prologue: the global
+// loads go out first, the LDS writes (and the barrier) come after the weight loads were issued.
+constexpr int kXStageRegs = 4;
+template <int WAVES, bool XLDS>
+__device__ __forceinline__ void stage_x_begin(u32x4 (&xr)[kXStageRegs], const uint16_t* __restrict__ x, int M, int K) {
+  if constexpr (XLDS) {
+    const int total = (M * K) >> 3;  // 16-byte pieces
+#pragma unroll
+    for (int i = 0; i < kXStageRegs; ++i) {
+      const int idx = threadIdx.x + i * WAVES * 64;
+      if (idx < total) xr[i] = reinterpret_cast<const u32x4*>(x)[idx];
+    }
+  }
+}
+template <int WAVES, bool XLDS>
+__device__ __forceinline__ void stage_x_finish(u32x4 (&xr)[kXStageRegs], const uint16_t* __restrict__ x, uint16_t* xl, int M,
+                                               int K) {
+  if constexpr (XLDS) {
+    const int total = (M * K) >> 3;
+#pragma unroll
+    for (int i = 0; i < kXStageRegs; ++i) {
+      const int idx = threadIdx.x + i * WAVES * 64;
+      if (idx < total) reinterpret_cast<u32x4*>(xl)[idx] = xr[i];
+    }
+    for (int idx = threadIdx.x + kXStageRegs * WAVES * 64; idx < total; idx += WAVES * 64)
+      reinterpret_cast<u32x4*>(xl)[idx] = reinterpret_cast<const u32x4*>(x)[idx];
+    for (int i = threadIdx.x; i < (K >> 3); i += WAVES * 64)
+      reinterpret_cast<u32x4*>(xl + (int64_t)M * K)[i] = u32x4{0u, 0u, 0u, 0u};
+    lds_barrier();
+  }
+}
+
+template <int MT, int NT, int WAVES, int U, bool XLDS>
 __global__ __launch_bounds__(WAVES * 64) void w4_gemv_kernel(const uint16_t* __restrict__ x,
                                                              const u32x4* __restrict__ wt,
                                                              const uint16_t* __restrict__ st,
                                                              const uint8_t* __restrict__ zt, uint16_t* __restrict__ y,
-                                                             float* __restrict__ partial,
-                                                             unsigned* __restrict__ counters, int M, int N, int K,
-                                                             int ksplit) {
-  __shared__ float red[WAVES * MT * NT * 256];
+                                                             int M, int N, int K) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* red = reinterpret_cast<float*>(smem);                                         // [WAVES][MT*NT*256]
+  uint16_t* xl = reinterpret_cast<uint16_t*>(smem + WAVES * MT * NT * 256 * sizeof(float));  // [M+1][K]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, kq = lane >> 4;
   const int G = K >> 7, ntiles = N >> 4;
   const int nt0 = blockIdx.x * NT;
-  const int g_begin = (int)((int64_t)G * blockIdx.y / ksplit), g_end = (int)((int64_t)G * (blockIdx.y + 1) / ksplit);
+  // contiguous slice of groups per wave
+  const int g_begin = (int)((int64_t)G * wave / WAVES), g_end = (int)((int64_t)G * (wave + 1) / WAVES);
   const bf16x8 ones = ones_bf16x8();
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+
+  static_assert(!XLDS || MT == 1, "x in LDS is for M <= 16");
+  XSource<XLDS> xs_src{x, xl, M, K, (col < M ? col : M) * K};
 
   f32x4 acc[MT][NT];
 #pragma unroll
@@ -119,161 +138,216 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_kernel(const uint16_t* __r
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = zero4;
 
-  for (int g = g_begin + wave; g < g_end; g += WAVES) {
-    u32x4 w[NT];
-    float sc[NT], zc[NT];
+  u32x4 w[U][NT];
+  uint16_t s16[U][NT];
+  uint8_t z8[U][NT];
+  bf16x8 a[XLDS ? 1 : U][4][MT];
+
+  auto issue = [&](int u, int g) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const int tnt = min(nt0 + nt, ntiles - 1);  // clamp: out-of-range tiles are computed and dropped
+      const int tnt = min(nt0 + nt, ntiles - 1);  // out-of-range tiles are computed and dropped
       const int64_t tile = (int64_t)tnt * G + g;
-      w[nt] = __builtin_nontemporal_load(&wt[tile * 64 + lane]);
-      sc[nt] = (float)__builtin_bit_cast(_Float16, st[tile * 16 + col]);
-      zc[nt] = (float)(129 + (int)((zt[tile * 8 + (col >> 1)] >> (4 * (col & 1))) & 15u));  // 128 + (stored + 1)
+      w[u][nt] = __builtin_nontemporal_load(&wt[tile * 64 + lane]);
+      s16[u][nt] = st[tile * 16 + col];
+      z8[u][nt] = zt[tile * 8 + (col >> 1)];
     }
-    f32x4 t[MT][NT], xs[MT];
+    if constexpr (!XLDS) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      xs[mt] = zero4;
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) t[mt][nt] = zero4;
+        for (int mt = 0; mt < MT; ++mt) a[u][j][mt] = xs_src.frag(mt, col, 128 * g + 32 * j + 8 * kq);
     }
+  };
+
+  // x first (it comes from L2 and is needed first), then U weight pieces in flight
+  u32x4 xr[kXStageRegs];
+  stage_x_begin<WAVES, XLDS>(xr, x, M, K);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      bf16x8 a[MT];
+  for (int u = 0; u < U; ++u)
+    if (g_begin + u < g_end) issue(u, g_begin + u);
+
+  stage_x_finish<WAVES, XLDS>(xr, x, xl, M, K);
+
+  for (int base = g_begin; base < g_end; base += U) {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        a[mt] = load_x_frag(x, mt * 16 + col, M, K, 128 * g + 32 * j + 8 * kq);
-        xs[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[mt], ones, xs[mt], 0, 0, 0);
+    for (int u = 0; u < U; ++u) {
+      const int g = base + u;
+      if (g < g_end) {
+        f32x4 t[MT][NT], xsum[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          xsum[mt] = zero4;
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) t[mt][nt] = zero4;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          bf16x8 af[MT];
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            if constexpr (XLDS) af[mt] = xs_src.frag(mt, col, 128 * g + 32 * j + 8 * kq);
+            else af[mt] = a[u][j][mt];
+            xsum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], ones, xsum[mt], 0, 0, 0);
+          }
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            const bf16x8 b = unpack_w4_bias128(w[u][nt][j]);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+              t[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], b, t[mt][nt], 0, 0, 0);
+          }
+        }
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const float sc = (float)__builtin_bit_cast(_Float16, s16[u][nt]);
+          const float zc = (float)(129 + (int)((z8[u][nt] >> (4 * (col & 1))) & 15u));  // 128 + (stored + 1)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[mt][nt][r] += sc * (t[mt][nt][r] - zc * xsum[mt][r]);
+        }
+        if (g + U < g_end) issue(u, g + U);  // refill the slot just consumed
       }
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        const bf16x8 b = unpack_w4_bias128(w[nt][j]);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) t[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[mt], b, t[mt][nt], 0, 0, 0);
-      }
     }
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) acc[mt][nt][r] += sc[nt] * (t[mt][nt][r] - zc[nt] * xs[mt][r]);
   }
-  gemv_epilogue<MT, NT, WAVES>(acc, red, y, partial, counters, M, N, nt0, ntiles, ksplit);
+  gemv_epilogue<MT, NT, WAVES>(acc, red, y, M, N, nt0, ntiles);
 }
 
-template <int MT, int NT, int WAVES>
+template <int MT, int NT, int WAVES, int U, bool XLDS>
 __global__ __launch_bounds__(WAVES * 64) void b16_gemv_kernel(const uint16_t* __restrict__ x,
                                                               const bf16x8* __restrict__ wt, uint16_t* __restrict__ y,
-                                                              float* __restrict__ partial,
-                                                              unsigned* __restrict__ counters, int M, int N, int K,
-                                                              int ksplit) {
-  __shared__ float red[WAVES * MT * NT * 256];
+                                                              int M, int N, int K) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* red = reinterpret_cast<float*>(smem);
+  uint16_t* xl = reinterpret_cast<uint16_t*>(smem + WAVES * MT * NT * 256 * sizeof(float));
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, kq = lane >> 4;
   const int KS = K >> 5, ntiles = N >> 4;
   const int nt0 = blockIdx.x * NT;
-  const int s_begin = (int)((int64_t)KS * blockIdx.y / ksplit), s_end = (int)((int64_t)KS * (blockIdx.y + 1) / ksplit);
+  const int s_begin = (int)((int64_t)KS * wave / WAVES), s_end = (int)((int64_t)KS * (wave + 1) / WAVES);
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  static_assert(!XLDS || MT == 1, "x in LDS is for M <= 16");
+  XSource<XLDS> xs_src{x, xl, M, K, (col < M ? col : M) * K};
   f32x4 acc[MT][NT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = zero4;
-#pragma unroll 4
-  for (int ks = s_begin + wave; ks < s_end; ks += WAVES) {
-    bf16x8 b[NT];
+  bf16x8 b[U][NT], a[XLDS ? 1 : U][MT];
+  auto issue = [&](int u, int ks) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       const int tnt = min(nt0 + nt, ntiles - 1);
-      b[nt] = __builtin_nontemporal_load(&wt[((int64_t)tnt * KS + ks) * 64 + lane]);
+      b[u][nt] = __builtin_nontemporal_load(&wt[((int64_t)tnt * KS + ks) * 64 + lane]);
     }
+    if constexpr (!XLDS) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const bf16x8 a = load_x_frag(x, mt * 16 + col, M, K, 32 * ks + 8 * kq);
+      for (int mt = 0; mt < MT; ++mt) a[u][mt] = xs_src.frag(mt, col, 32 * ks + 8 * kq);
+    }
+  };
+  u32x4 xr[kXStageRegs];
+  stage_x_begin<WAVES, XLDS>(xr, x, M, K);
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[nt], acc[mt][nt], 0, 0, 0);
+  for (int u = 0; u < U; ++u)
+    if (s_begin + u < s_end) issue(u, s_begin + u);
+  stage_x_finish<WAVES, XLDS>(xr, x, xl, M, K);
+  for (int base = s_begin; base < s_end; base += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int ks = base + u;
+      if (ks < s_end) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          bf16x8 af;
+          if constexpr (XLDS) af = xs_src.frag(mt, col, 32 * ks + 8 * kq);
+          else af = a[u][mt];
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, b[u][nt], acc[mt][nt], 0, 0, 0);
+        }
+        if (ks + U < s_end) issue(u, ks + U);
+      }
     }
   }
-  gemv_epilogue<MT, NT, WAVES>(acc, red, y, partial, counters, M, N, nt0, ntiles, ksplit);
+  gemv_epilogue<MT, NT, WAVES>(acc, red, y, M, N, nt0, ntiles);
 }
 
-constexpr int kWaves = 4;
-constexpr int kCounterBytes = O355_GEMV_COUNTER_BYTES;
-
+// ---- launch plans -------------------------------------------------------------------------------
 struct GemvPlan {
-  int mt, nt, ksplit;
-  unsigned blocks_x;
+  int mt, nt, waves, u;
+  bool xlds;
 };
 
-// units: number of K pieces a wave can own (groups of 128 for int4, steps of 32 for bf16)
-inline GemvPlan plan_gemv(int M, int N, int units, int min_units_per_wave) {
+// Experiment hook (not part of the public interface): overrides nt / waves / u / xlds when >= 0.
+int g_dbg_nt = -1, g_dbg_waves = -1, g_dbg_u = -1, g_dbg_xlds = -1;
+
+constexpr int kXldsMaxBytes = 64 * 1024;
+
+inline GemvPlan plan_gemv(int M, int N, int K, bool w4) {
   GemvPlan p;
   p.mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
   const int ntiles = N >> 4;
-  p.nt = (p.mt == 1 && ntiles >= 2048) ? 2 : 1;
-  p.blocks_x = (unsigned)((ntiles + p.nt - 1) / p.nt);
-  const int64_t target_waves = 256 * 8;
-  int ks = (int)((target_waves + (int64_t)p.blocks_x * kWaves - 1) / ((int64_t)p.blocks_x * kWaves));
-  const int ks_max = units / (kWaves * min_units_per_wave);
-  if (ks > ks_max) ks = ks_max;
-  if (ks < 1) ks = 1;
-  if (ks > 8) ks = 8;
-  if (p.blocks_x > (unsigned)(kCounterBytes / 4)) ks = 1;
-  p.ksplit = ks;
+  const int units = w4 ? (K >> 7) : (K >> 5);   // 1 KiB pieces per column tile
+  // Measured on the 7B shapes: 2 pieces in flight per wave, 16 waves per workgroup for narrow
+  // outputs (N <= 8192, one workgroup per CU), 8 otherwise; never fewer than u pieces per wave.
+  p.nt = 1;
+  p.u = w4 ? 2 : (p.mt == 1 ? 8 : 4);
+  int waves = ntiles <= 512 ? 16 : 8;
+  while (waves > 4 && units < waves * p.u) waves /= 2;
+  p.waves = waves;
+  p.xlds = p.mt == 1 && (int64_t)(M + 1) * K * 2 <= kXldsMaxBytes;
+  if (g_dbg_nt >= 0) p.nt = g_dbg_nt;
+  if (g_dbg_waves >= 0) p.waves = g_dbg_waves;
+  if (g_dbg_u >= 0) p.u = g_dbg_u;
+  if (g_dbg_xlds >= 0) p.xlds = g_dbg_xlds && p.mt == 1 && (int64_t)(M + 1) * K * 2 <= kXldsMaxBytes;
   return p;
 }
 
-inline int64_t plan_ws_bytes(const GemvPlan& p, int N) {
-  if (p.ksplit == 1) return 0;
-  return (int64_t)kCounterBytes + (int64_t)p.ksplit * p.mt * 16 * N * 4;
+template <typename Kern, typename... Args>
+int launch_gemv(Kern kern, const GemvPlan& p, int M, int N, int K, hipStream_t stream, Args... args) {
+  const size_t lds = (size_t)p.waves * p.mt * p.nt * 256 * 4 + (p.xlds ? (size_t)(M + 1) * K * 2 : 0);
+  if (lds > 48 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return O355_ELAUNCH;
+  const unsigned blocks = (unsigned)(((N >> 4) + p.nt - 1) / p.nt);
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(p.waves * 64), lds, stream, args..., M, N, K);
+  O355_CHECK_LAUNCH();
 }
-
-#define GEMV_DISPATCH(KERNEL, MTv, NTv, ...)                                                                     \
-  hipLaunchKernelGGL((KERNEL<MTv, NTv, kWaves>), dim3(p.blocks_x, p.ksplit), dim3(kWaves * 64), 0, as_stream(stream), \
-                     __VA_ARGS__)
 
 }  // namespace
 
-extern "C" int64_t olmo355_w4_gemv_workspace_bytes(int M, int N, int K) {
-  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 127) || (N & 15)) return 0;
-  // the dense bf16 path shares the workspace: size for whichever plan needs more
-  const GemvPlan a = plan_gemv(M, N, K >> 7, 2), b = plan_gemv(M, N, K >> 5, 8);
-  const int64_t wa = plan_ws_bytes(a, N), wb = plan_ws_bytes(b, N);
-  return wa > wb ? wa : wb;
+extern "C" void olmo355_debug_set_gemv_plan(int nt, int waves, int u, int xlds) {
+  g_dbg_nt = nt, g_dbg_waves = waves, g_dbg_u = u, g_dbg_xlds = xlds;
 }
+
+#define W4_CASE(MTv, NTv, Wv, Uv, Xv)                                                                          \
+  if (p.mt == MTv && p.nt == NTv && p.waves == Wv && p.u == Uv && p.xlds == Xv)                               \
+    return launch_gemv(w4_gemv_kernel<MTv, NTv, Wv, Uv, Xv>, p, M, N, K, as_stream(stream), x, (const u32x4*)wt, st, zt, y);
+#define B16_CASE(MTv, NTv, Wv, Uv, Xv)                                                                         \
+  if (p.mt == MTv && p.nt == NTv && p.waves == Wv && p.u == Uv && p.xlds == Xv)                               \
+    return launch_gemv(b16_gemv_kernel<MTv, NTv, Wv, Uv, Xv>, p, M, N, K, as_stream(stream), x, (const bf16x8*)wt, y);
+#define FOR_WAVES(CASE, MTv, NTv, Uv, Xv) CASE(MTv, NTv, 4, Uv, Xv) CASE(MTv, NTv, 8, Uv, Xv) CASE(MTv, NTv, 16, Uv, Xv)
 
 extern "C" int olmo355_w4_gemv(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
-                               uint16_t* y, void* ws, int M, int N, int K, void* stream) {
+                               uint16_t* y, int M, int N, int K, void* stream) {
   if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
   if (M > 64 || (K & 127) || (N & 15)) return O355_EUNSUPPORTED;
-  const GemvPlan p = plan_gemv(M, N, K >> 7, 2);
-  if (p.ksplit > 1 && !ws) return O355_EINVAL;
-  unsigned* counters = (unsigned*)ws;
-  float* partial = ws ? (float*)((char*)ws + kCounterBytes) : nullptr;
-  const u32x4* w = (const u32x4*)wt;
-  if (p.mt == 1 && p.nt == 1) GEMV_DISPATCH(w4_gemv_kernel, 1, 1, x, w, st, zt, y, partial, counters, M, N, K, p.ksplit);
-  else if (p.mt == 1) GEMV_DISPATCH(w4_gemv_kernel, 1, 2, x, w, st, zt, y, partial, counters, M, N, K, p.ksplit);
-  else if (p.mt == 2) GEMV_DISPATCH(w4_gemv_kernel, 2, 1, x, w, st, zt, y, partial, counters, M, N, K, p.ksplit);
-  else GEMV_DISPATCH(w4_gemv_kernel, 4, 1, x, w, st, zt, y, partial, counters, M, N, K, p.ksplit);
-  O355_CHECK_LAUNCH();
+  const GemvPlan p = plan_gemv(M, N, K, true);
+  FOR_WAVES(W4_CASE, 1, 1, 4, true) FOR_WAVES(W4_CASE, 1, 1, 4, false)
+  FOR_WAVES(W4_CASE, 1, 1, 2, true) FOR_WAVES(W4_CASE, 1, 1, 2, false)
+  FOR_WAVES(W4_CASE, 1, 1, 8, true) FOR_WAVES(W4_CASE, 1, 2, 4, true) FOR_WAVES(W4_CASE, 1, 2, 2, true)
+  FOR_WAVES(W4_CASE, 1, 4, 2, true) FOR_WAVES(W4_CASE, 1, 2, 2, false)
+  FOR_WAVES(W4_CASE, 2, 1, 2, false) FOR_WAVES(W4_CASE, 4, 1, 2, false)
+  return O355_EUNSUPPORTED;
 }
 
-// dense bf16 small-M path; workspace rules as for olmo355_w4_gemv (same size function)
-extern "C" int olmo355_b16_gemv(const uint16_t* x, const uint16_t* wt, uint16_t* y, void* ws, int M, int N, int K,
-                                   void* stream) {
+extern "C" int olmo355_b16_gemv(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K,
+                                void* stream) {
   if (!x || !wt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
   if (M > 64 || (K & 31) || (N & 15)) return O355_EUNSUPPORTED;
-  GemvPlan p = plan_gemv(M, N, K >> 5, 8);
-  if (p.ksplit > 1 && !ws) {
-    p.ksplit = 1;
-  }
-  unsigned* counters = (unsigned*)ws;
-  float* partial = ws ? (float*)((char*)ws + kCounterBytes) : nullptr;
-  const bf16x8* w = (const bf16x8*)wt;
-  if (p.mt == 1 && p.nt == 1) GEMV_DISPATCH(b16_gemv_kernel, 1, 1, x, w, y, partial, counters, M, N, K, p.ksplit);
-  else if (p.mt == 1) GEMV_DISPATCH(b16_gemv_kernel, 1, 2, x, w, y, partial, counters, M, N, K, p.ksplit);
-  else if (p.mt == 2) GEMV_DISPATCH(b16_gemv_kernel, 2, 1, x, w, y, partial, counters, M, N, K, p.ksplit);
-  else GEMV_DISPATCH(b16_gemv_kernel, 4, 1, x, w, y, partial, counters, M, N, K, p.ksplit);
-  O355_CHECK_LAUNCH();
+  const GemvPlan p = plan_gemv(M, N, K, false);
+  FOR_WAVES(B16_CASE, 1, 1, 8, true) FOR_WAVES(B16_CASE, 1, 1, 8, false)
+  FOR_WAVES(B16_CASE, 1, 1, 4, true) FOR_WAVES(B16_CASE, 1, 2, 8, true) FOR_WAVES(B16_CASE, 1, 2, 4, true)
+  FOR_WAVES(B16_CASE, 2, 1, 4, false) FOR_WAVES(B16_CASE, 4, 1, 4, false)
+  return O355_EUNSUPPORTED;
 }

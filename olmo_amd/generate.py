@@ -54,7 +54,7 @@ class DecodeSession:
 
     def capture(self) -> None:
         """Record one decode step into a HIP graph (call after at least one eager ``step`` so that
-        every workspace already has its final size)."""
+        the attention workspace already exists)."""
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             self._step_kernels()

@@ -96,12 +96,12 @@ class DenseLinear(nn.Linear):
             self._tiled = ops.b16_repack(self.weight.data.contiguous())
         return self
 
-    def forward(self, x: torch.Tensor, workspace: ops.Workspace) -> torch.Tensor:
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.weight.dtype == torch.float32:
             return ops.f32_linear(x, self.weight.data)
         if self._tiled is None:
             self.post_init()
-        return ops.b16_linear(x, self._tiled, workspace)
+        return ops.b16_linear(x, self._tiled)
 
 
 class RMSLayerNorm(nn.Module):
@@ -188,7 +188,6 @@ class OLMo(nn.Module):
             ff_out=DenseLinear(config.d_model, V, device, dtype),
         ))
         self._prepared = False
-        self._ws: Optional[ops.Workspace] = None
         self._rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
         self._attn_ws: Dict[Tuple[int, int], torch.Tensor] = {}
         self._scratch_kv: Dict[Tuple[int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
@@ -216,7 +215,7 @@ class OLMo(nn.Module):
         self._prepared = False
 
     def post_init(self) -> "OLMo":
-        """Build the kernel-side weight layouts, rotary tables and workspaces (idempotent)."""
+        """Build the kernel-side weight layouts, rotary tables (idempotent)."""
         for m in self.modules():
             if isinstance(m, (DenseLinear, QuantLinear)) and m is not self:
                 if isinstance(m, DenseLinear) and m.weight.device.type == "meta":
@@ -225,7 +224,6 @@ class OLMo(nn.Module):
         c = self.config
         n_pos = max(self.max_cache_len, c.max_sequence_length)
         self._rope = ops.rope_tables(c.head_dim, float(c.rope_theta), n_pos, self.device)
-        self._ws = ops.Workspace(self.device)
         self._prepared = True
         return self
 
@@ -299,7 +297,7 @@ class OLMo(nn.Module):
     # one block: olmo/model.py:728-823 (wiring), :588-654 (attention)
     # ------------------------------------------------------------------------------------------
     def _linear(self, m: nn.Module, x: torch.Tensor) -> torch.Tensor:
-        return m(x, self._ws)
+        return m(x)
 
     def _block(self, blk: OLMoSequentialBlock, x, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max):
         c = self.config

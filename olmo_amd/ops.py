@@ -17,7 +17,6 @@ from ._lib import check, lib
 F32, BF16 = 0, 1
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
 GEMV_MAX_M = 64
-GEMV_COUNTER_BYTES = 16384
 
 
 def _dt(t: torch.Tensor) -> int:
@@ -115,34 +114,7 @@ def w4t_dequant_fp16(w: W4Tiled) -> torch.Tensor:
     return out
 
 
-def gemv_workspace_bytes(M: int, N: int, K: int) -> int:
-    return int(lib().olmo355_w4_gemv_workspace_bytes(M, N, K))
-
-
-class Workspace:
-    """Device scratch shared by the small-M linear kernels on one stream: a zeroed counter
-    block followed by room for split-K partial sums.  Grows on demand (never inside a
-    captured graph: size it first with ``reserve``)."""
-
-    def __init__(self, device):
-        self.device = torch.device(device)
-        self.buf = torch.zeros(GEMV_COUNTER_BYTES, dtype=torch.uint8, device=self.device)
-
-    def reserve(self, nbytes: int) -> None:
-        if nbytes > self.buf.numel():
-            if torch.cuda.is_current_stream_capturing():
-                raise RuntimeError("workspace too small inside graph capture; call reserve() before capturing")
-            self.buf = torch.zeros(nbytes, dtype=torch.uint8, device=self.device)
-
-    def for_linear(self, M: int, N: int, K: int) -> Optional[torch.Tensor]:
-        need = gemv_workspace_bytes(M, N, K)
-        if need == 0:
-            return None
-        self.reserve(need)
-        return self.buf
-
-
-def w4_linear(x: torch.Tensor, w: W4Tiled, ws: Workspace) -> torch.Tensor:
+def w4_linear(x: torch.Tensor, w: W4Tiled) -> torch.Tensor:
     """``x[..., K] @ W[K, N]`` for a tiled int4 weight; bf16 in, bf16 out."""
     _dev(x, w.wt)
     if x.dtype != torch.bfloat16:
@@ -154,9 +126,8 @@ def w4_linear(x: torch.Tensor, w: W4Tiled, ws: Workspace) -> torch.Tensor:
     if M == 0:
         return y
     if M <= GEMV_MAX_M:
-        wsb = ws.for_linear(M, w.N, w.K)
         check("olmo355_w4_gemv",
-              lib().olmo355_w4_gemv(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), _p(wsb), M, w.N, w.K, _stream()))
+              lib().olmo355_w4_gemv(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream()))
     else:
         check("olmo355_w4_gemm",
               lib().olmo355_w4_gemm(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream()))
@@ -185,7 +156,7 @@ def b16_repack(weight_nk: torch.Tensor) -> B16Tiled:
     return B16Tiled(wt, K, N)
 
 
-def b16_linear(x: torch.Tensor, w: B16Tiled, ws: Workspace) -> torch.Tensor:
+def b16_linear(x: torch.Tensor, w: B16Tiled) -> torch.Tensor:
     _dev(x, w.wt)
     if x.dtype != torch.bfloat16:
         raise TypeError("dense bf16 linear takes bfloat16 activations")
@@ -196,8 +167,7 @@ def b16_linear(x: torch.Tensor, w: B16Tiled, ws: Workspace) -> torch.Tensor:
     if M == 0:
         return y
     if M <= GEMV_MAX_M:
-        wsb = ws.for_linear(M, w.N, w.K) if w.K % 128 == 0 else None
-        check("olmo355_b16_gemv", lib().olmo355_b16_gemv(_p(x), _p(w.wt), _p(y), _p(wsb), M, w.N, w.K, _stream()))
+        check("olmo355_b16_gemv", lib().olmo355_b16_gemv(_p(x), _p(w.wt), _p(y), M, w.N, w.K, _stream()))
     else:
         check("olmo355_b16_gemm", lib().olmo355_b16_gemm(_p(x), _p(w.wt), _p(y), M, w.N, w.K, _stream()))
     return y

@@ -61,7 +61,6 @@ class QuantLinear(nn.Module):
         self.kernel_switch_threshold = kernel_switch_threshold
         self.trainable = trainable
         self._tiled: Optional[ops.W4Tiled] = None
-        self._ws: Optional[ops.Workspace] = None
 
     # -- one-time preparation ------------------------------------------------------------------
     def post_init(self, free_checkpoint_buffers: bool = False):
@@ -127,16 +126,11 @@ class QuantLinear(nn.Module):
         self._tiled = None
 
     # -- forward ---------------------------------------------------------------------------------
-    def forward(self, x: torch.Tensor, workspace: Optional[ops.Workspace] = None) -> torch.Tensor:
-        ws = workspace
-        if ws is None:
-            if self._ws is None:
-                self._ws = ops.Workspace(x.device)
-            ws = self._ws
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
         in_dtype = x.dtype
         if in_dtype != torch.bfloat16:
             x = x.to(torch.bfloat16)  # the reference casts to float16 here (qlinear_cuda_old.py:287)
-        y = ops.w4_linear(x.contiguous(), self.tiled, ws)
+        y = ops.w4_linear(x.contiguous(), self.tiled)
         return y if in_dtype == torch.bfloat16 else y.to(in_dtype)
 
     def extra_repr(self):

@@ -71,7 +71,6 @@ def test_w4_golden_vectors_through_gemv(dev, golden_dir):
 
     ops = _ops()
     kats = json.load(open(os.path.join(golden_dir, "q4_kat.json")))
-    ws = ops.Workspace(dev)
     for name in ("exllama_k1024_n1024", "cuda_old_half_k256_n256", "cuda_old_no_half_k256_n256"):
         kat = kats[name]
         k, n = kat["k"], kat["n"]
@@ -85,7 +84,7 @@ def test_w4_golden_vectors_through_gemv(dev, golden_dir):
         # against the oracle on the same bf16 inputs, and against the stored vector with the
         # input-rounding error budget (|dx| <= 2^-9, sum |w| <= k*0.2)
         xb = inp[0].to(torch.bfloat16)
-        y = ops.w4_linear(xb.to(dev), t, ws).float().cpu()[0]
+        y = ops.w4_linear(xb.to(dev), t).float().cpu()[0]
         W = ow4.dequantize(qweight, qzeros, scales, 128)
         ref_same_inputs = ow4.linear_fp32(xb, W)[0]
         assert torch.allclose(y, ref_same_inputs, rtol=2 ** -8, atol=1e-3), name
@@ -103,9 +102,8 @@ def _w4_case(dev, M, N, K, seed):
     W = ow4.dequantize(qw, qz, sc, 128)
     ref = ow4.linear_fp32(x, W)
     t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
-    ws = ops.Workspace(dev)
-    y = ops.w4_linear(x.to(dev), t, ws)
-    y2 = ops.w4_linear(x.to(dev), t, ws)
+    y = ops.w4_linear(x.to(dev), t)
+    y2 = ops.w4_linear(x.to(dev), t)
     assert torch.equal(y, y2), "not deterministic"
     y = y.float().cpu()
     # bf16 output rounding (2^-9 relative) + fp32 accumulation noise; GEMM path also rounds W to bf16
@@ -141,8 +139,7 @@ def test_b16_linear(dev, M, N, K):
     x = torch.randn(M, K, generator=gen).to(torch.bfloat16)
     ref = x.float() @ w.float().t()
     t = ops.b16_repack(w.to(dev))
-    ws = ops.Workspace(dev)
-    y = ops.b16_linear(x.to(dev), t, ws).float().cpu()
+    y = ops.b16_linear(x.to(dev), t).float().cpu()
     # exact bf16 products, fp32 accumulation, one bf16 rounding of the result
     assert torch.allclose(y, ref, rtol=2 ** -8, atol=2 ** -8 * ref.abs().max().item())
 
