@@ -75,6 +75,17 @@ int olmo355_w4t_dequant_fp16(const uint32_t* wt, const uint16_t* st, const uint8
 int olmo355_w4_gemv(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
                     int M, int N, int K, void* stream);
 
+/* The same product with up to two neighbouring steps of a decode block folded in (M <= 16):
+ *   resid != NULL: the activations are first formed as x' = resid + rmsnorm(x; norm_w, eps) -- the
+ *     post-norm residual update that precedes att_proj / ff_proj (olmo/model.py:786-794,814-821),
+ *     with RMSLayerNorm's rounding points (olmo/model.py:241-255) -- and also written to x_out [M,K];
+ *   swiglu != 0: y [M, N/2] = silu(gate) * up of the two halves of the product (olmo/model.py:365-368).
+ * Returns O355_EUNSUPPORTED for shapes the fused kernels do not cover (the caller then issues the
+ * separate kernels). */
+int olmo355_w4_gemv_fused(const uint16_t* x, const uint16_t* resid, const uint16_t* norm_w, float eps,
+                          uint16_t* x_out, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
+                          int M, int N, int K, int swiglu, void* stream);
+
 /* Large-M path: dequantise tiles into LDS as bf16 and multiply on the matrix cores.  Stands
  * in for the reference's dequantise-then-matmul branch (AGQ qlinear_cuda_old.py:236-287) and
  * exllama's reconstruct + cublasHgemm (exllama/cuda_func/q4_matmul.cu:222-260). */
@@ -88,6 +99,9 @@ int olmo355_w4_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, c
 int olmo355_b16_repack(const uint16_t* w_nk, uint16_t* wt, int N, int K, void* stream);
 /* small-M (<= 64) path */
 int olmo355_b16_gemv(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, void* stream);
+int olmo355_b16_gemv_fused(const uint16_t* x, const uint16_t* resid, const uint16_t* norm_w, float eps,
+                           uint16_t* x_out, const uint16_t* wt, uint16_t* y, int M, int N, int K, int swiglu,
+                           void* stream);
 int olmo355_b16_gemm(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, void* stream);
 int olmo355_f32_linear(const float* x, const float* w_nk, float* y, int M, int N, int K, void* stream);
 

@@ -37,6 +37,8 @@ EXPORTS = {
     "olmo355_w4_repack": (I, [P, P, P, P, P, P, I, I, I, P]),
     "olmo355_w4t_dequant_fp16": (I, [P, P, P, P, I, I, P]),
     "olmo355_w4_gemv": (I, [P, P, P, P, P, I, I, I, P]),
+    "olmo355_w4_gemv_fused": (I, [P, P, P, F, P, P, P, P, P, I, I, I, I, P]),
+    "olmo355_b16_gemv_fused": (I, [P, P, P, F, P, P, P, I, I, I, I, P]),
     "olmo355_w4_gemm": (I, [P, P, P, P, P, I, I, I, P]),
     "olmo355_b16_repack": (I, [P, P, I, I, P]),
     "olmo355_b16_gemv": (I, [P, P, P, I, I, I, P]),

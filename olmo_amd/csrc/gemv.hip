@@ -13,9 +13,27 @@
 // K is split over the waves of a workgroup only (contiguous slice per wave, LDS reduction in
 // fixed order): no atomics, no cross-workgroup pass, so the result does not depend on scheduling.
 // Each wave keeps U one-KiB weight pieces in flight and refills a slot as soon as it is consumed.
+//
+// Two optional fusions remove whole launches from a decode step (each launch costs several
+// microseconds against kernels that themselves run for 5-10):
+//   prologue  x := resid + rmsnorm(a; w, eps)   the post-norm residual update of the previous
+//             sub-block (olmo/model.py:786-794,814-821), recomputed by every workgroup while
+//             its first weight pieces are in flight; workgroup 0 also writes x to memory;
+//   epilogue  y := silu(gate) * up              SwiGLU (olmo/model.py:365-368) on the two column
+//             tiles a workgroup owns (tile p of the first half and tile p of the second half).
 #include "common.h"
 
 namespace {
+
+struct GemvArgs {
+  const uint16_t* x;       // [M,K] activations; with a prologue: the tensor to be normalised
+  const uint16_t* resid;   // [M,K] residual stream (prologue) or null
+  const uint16_t* norm_w;  // [K] RMSNorm weight (prologue) or null
+  uint16_t* x_out;         // [M,K] resid + norm(x), written by workgroup 0 (prologue)
+  uint16_t* y;             // [M,N], or [M,N/2] with the SwiGLU epilogue
+  float eps;
+  int M, N, K;
+};
 
 __device__ __forceinline__ bf16x8 unpack_w4_bias128(uint32_t w) {
   u32x4 r;
@@ -37,10 +55,115 @@ __device__ __forceinline__ bf16x8 load_x_frag(const uint16_t* __restrict__ x, in
   return __builtin_bit_cast(bf16x8, z);
 }
 
-// Reduce acc over the waves of the workgroup in fixed order and write y (bf16).
-template <int MT, int NT, int WAVES>
-__device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][NT], float* red, uint16_t* __restrict__ y, int M, int N,
-                                              int nt0, int ntiles) {
+__device__ __forceinline__ void unpack8(const u32x4& v, float (&f)[8]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f[2 * i] = bf16lo_to_f32(v[i]), f[2 * i + 1] = bf16hi_to_f32(v[i]);
+}
+
+// ---- activation staging --------------------------------------------------------------------------
+// XLDS: the M rows of x live in LDS as [M+1][K] (the extra row is zero and is what the padding
+// lanes of the A operand read); every A fragment is one ds_read_b128 right before its MFMA.
+// The global loads are issued in begin() -- before the weight prologue -- and consumed in
+// finish(), after the weight loads have been issued; the barrier orders LDS only.
+constexpr int kXStageRegs = 4;  // plain copy: 16-byte pieces per thread held across the weight prologue
+constexpr int kNormVPL = 10;    // prologue: 16-byte pieces of a row per lane (K <= 5120)
+
+template <int WAVES, bool XLDS, int PRO>
+struct XStage {
+  __device__ __forceinline__ void begin(const GemvArgs&) {}
+  __device__ __forceinline__ void finish(const GemvArgs&, uint16_t*) {}
+};
+
+template <int WAVES>
+struct XStage<WAVES, true, 0> {
+  u32x4 xr[kXStageRegs];
+  __device__ __forceinline__ void begin(const GemvArgs& a) {
+    const int total = (a.M * a.K) >> 3;
+#pragma unroll
+    for (int i = 0; i < kXStageRegs; ++i) {
+      const int idx = threadIdx.x + i * WAVES * 64;
+      if (idx < total) xr[i] = reinterpret_cast<const u32x4*>(a.x)[idx];
+    }
+  }
+  __device__ __forceinline__ void finish(const GemvArgs& a, uint16_t* xl) {
+    const int total = (a.M * a.K) >> 3;
+#pragma unroll
+    for (int i = 0; i < kXStageRegs; ++i) {
+      const int idx = threadIdx.x + i * WAVES * 64;
+      if (idx < total) reinterpret_cast<u32x4*>(xl)[idx] = xr[i];
+    }
+    for (int idx = threadIdx.x + kXStageRegs * WAVES * 64; idx < total; idx += WAVES * 64)
+      reinterpret_cast<u32x4*>(xl)[idx] = reinterpret_cast<const u32x4*>(a.x)[idx];
+    for (int i = threadIdx.x; i < (a.K >> 3); i += WAVES * 64)
+      reinterpret_cast<u32x4*>(xl + (int64_t)a.M * a.K)[i] = u32x4{0u, 0u, 0u, 0u};
+    lds_barrier();
+  }
+};
+
+// x := resid + w * round(a * rsqrt(mean(a^2) + eps)), rounding points of olmo/model.py:241-255 and
+// of the bf16 residual add.  Wave m normalises row m (M <= WAVES), so only wave reductions are needed.
+template <int WAVES>
+struct XStage<WAVES, true, 1> {
+  u32x4 av[kNormVPL], rv[kNormVPL], wv[kNormVPL];
+  __device__ __forceinline__ void begin(const GemvArgs& a) {
+    const int lane = threadIdx.x & 63, m = threadIdx.x >> 6, nvec = a.K >> 3;
+    if (m < a.M) {
+#pragma unroll
+      for (int i = 0; i < kNormVPL; ++i) {
+        const int idx = lane + 64 * i;
+        if (idx < nvec) {
+          av[i] = reinterpret_cast<const u32x4*>(a.x)[(int64_t)m * nvec + idx];
+          rv[i] = reinterpret_cast<const u32x4*>(a.resid)[(int64_t)m * nvec + idx];
+          wv[i] = reinterpret_cast<const u32x4*>(a.norm_w)[idx];
+        }
+      }
+    }
+  }
+  __device__ __forceinline__ void finish(const GemvArgs& a, uint16_t* xl) {
+    const int lane = threadIdx.x & 63, m = threadIdx.x >> 6, nvec = a.K >> 3;
+    if (m < a.M) {
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < kNormVPL; ++i) {
+        if (lane + 64 * i < nvec) {
+          float f[8];
+          unpack8(av[i], f);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+        }
+      }
+      ss = wave_sum(ss);
+      const float rstd = 1.f / sqrtf(ss / (float)a.K + a.eps);
+#pragma unroll
+      for (int i = 0; i < kNormVPL; ++i) {
+        const int idx = lane + 64 * i;
+        if (idx < nvec) {
+          float f[8], r[8], w[8];
+          unpack8(av[i], f);
+          unpack8(rv[i], r);
+          unpack8(wv[i], w);
+          u32x4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float y0 = round_bf16(w[2 * e] * round_bf16(f[2 * e] * rstd));
+            const float y1 = round_bf16(w[2 * e + 1] * round_bf16(f[2 * e + 1] * rstd));
+            o[e] = pack_bf16x2(r[2 * e] + y0, r[2 * e + 1] + y1);
+          }
+          reinterpret_cast<u32x4*>(xl)[(int64_t)m * nvec + idx] = o;
+          if (blockIdx.x == 0) reinterpret_cast<u32x4*>(a.x_out)[(int64_t)m * nvec + idx] = o;
+        }
+      }
+    }
+    for (int i = threadIdx.x; i < nvec; i += WAVES * 64)
+      reinterpret_cast<u32x4*>(xl + (int64_t)a.M * a.K)[i] = u32x4{0u, 0u, 0u, 0u};
+    lds_barrier();
+  }
+};
+
+// ---- epilogue: reduce over the waves in fixed order, write y (bf16) -----------------------------------
+template <int MT, int NT, int WAVES, int EPI>
+__device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][NT], float* red, const GemvArgs& a,
+                                              const int (&tile)[NT], int ntiles) {
   constexpr int PER_WAVE = MT * NT * 256;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
@@ -50,87 +173,65 @@ __device__ __forceinline__ void gemv_epilogue(f32x4 (&acc)[MT][NT], float* red, 
 #pragma unroll
       for (int r = 0; r < 4; ++r) red[wave * PER_WAVE + ((mt * NT + nt) * 4 + r) * 64 + lane] = acc[mt][nt][r];
   __syncthreads();
-  for (int i = threadIdx.x; i < PER_WAVE; i += WAVES * 64) {
-    float v = 0.f;
+  if constexpr (EPI == 0) {
+    for (int i = threadIdx.x; i < PER_WAVE; i += WAVES * 64) {
+      float v = 0.f;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) v += red[w * PER_WAVE + i];
-    const int l = i & 63, r = (i >> 6) & 3, t = i >> 8;
-    const int nt = t % NT, mt = t / NT;
-    const int m = mt * 16 + 4 * (l >> 4) + r;
-    const int n = (nt0 + nt) * 16 + (l & 15);
-    if (nt0 + nt < ntiles && m < M) y[(int64_t)m * N + n] = f32_to_bf16_bits(v);
-  }
-}
-
-// Activation fragments.  XLDS: the workgroup first copies its M rows of x into LDS (plus one
-// zero row that the padding lanes read), and every A operand is one ds_read_b128 issued right
-// before its MFMA; otherwise the fragments come from global memory with the weight loads.
-template <bool XLDS>
-struct XSource {
-  const uint16_t* x;
-  const uint16_t* lds;  // [M+1][K] when XLDS
-  int M, K, row_off;    // row_off: element offset of this lane's row in LDS
-  __device__ __forceinline__ bf16x8 frag(int mt, int col, int k) const {
-    if constexpr (XLDS) {
-      return *reinterpret_cast<const bf16x8*>(lds + row_off + k);
-    } else {
-      return load_x_frag(x, mt * 16 + col, M, K, k);
+      for (int w = 0; w < WAVES; ++w) v += red[w * PER_WAVE + i];
+      const int l = i & 63, r = (i >> 6) & 3, t = i >> 8;
+      const int nt = t % NT, mt = t / NT;
+      const int m = mt * 16 + 4 * (l >> 4) + r;
+      if (tile[nt] < ntiles && m < a.M) a.y[(int64_t)m * a.N + tile[nt] * 16 + (l & 15)] = f32_to_bf16_bits(v);
     }
-  }
-};
-
-// Copy of the M activation rows into LDS in two halves around the weight prologue: the global
-// loads go out first, the LDS writes (and the barrier) come after the weight loads were issued.
-constexpr int kXStageRegs = 4;
-template <int WAVES, bool XLDS>
-__device__ __forceinline__ void stage_x_begin(u32x4 (&xr)[kXStageRegs], const uint16_t* __restrict__ x, int M, int K) {
-  if constexpr (XLDS) {
-    const int total = (M * K) >> 3;  // 16-byte pieces
+  } else {
+    static_assert(EPI == 0 || NT == 2, "the SwiGLU epilogue owns one up tile and one gate tile");
+    const int half_n = a.N >> 1;
+    for (int i = threadIdx.x; i < MT * 256; i += WAVES * 64) {
+      const int l = i & 63, r = (i >> 6) & 3, mt = i >> 8;
+      const int iu = ((mt * 2 + 0) * 4 + r) * 64 + l, ig = ((mt * 2 + 1) * 4 + r) * 64 + l;
+      float up = 0.f, gate = 0.f;
 #pragma unroll
-    for (int i = 0; i < kXStageRegs; ++i) {
-      const int idx = threadIdx.x + i * WAVES * 64;
-      if (idx < total) xr[i] = reinterpret_cast<const u32x4*>(x)[idx];
+      for (int w = 0; w < WAVES; ++w) up += red[w * PER_WAVE + iu], gate += red[w * PER_WAVE + ig];
+      up = round_bf16(up), gate = round_bf16(gate);  // the Linear's bf16 output
+      const float s = round_bf16(gate / (1.f + expf(-gate)));
+      const int m = mt * 16 + 4 * (l >> 4) + r;
+      if (m < a.M) a.y[(int64_t)m * half_n + tile[0] * 16 + (l & 15)] = f32_to_bf16_bits(s * up);
     }
   }
 }
-template <int WAVES, bool XLDS>
-__device__ __forceinline__ void stage_x_finish(u32x4 (&xr)[kXStageRegs], const uint16_t* __restrict__ x, uint16_t* xl, int M,
-                                               int K) {
-  if constexpr (XLDS) {
-    const int total = (M * K) >> 3;
+
+template <int NT, int EPI>
+__device__ __forceinline__ void owned_tiles(int (&tile)[NT], int ntiles) {
+  if constexpr (EPI == 1) {
+    tile[0] = blockIdx.x;
+    tile[1] = blockIdx.x + (ntiles >> 1);
+  } else {
 #pragma unroll
-    for (int i = 0; i < kXStageRegs; ++i) {
-      const int idx = threadIdx.x + i * WAVES * 64;
-      if (idx < total) reinterpret_cast<u32x4*>(xl)[idx] = xr[i];
-    }
-    for (int idx = threadIdx.x + kXStageRegs * WAVES * 64; idx < total; idx += WAVES * 64)
-      reinterpret_cast<u32x4*>(xl)[idx] = reinterpret_cast<const u32x4*>(x)[idx];
-    for (int i = threadIdx.x; i < (K >> 3); i += WAVES * 64)
-      reinterpret_cast<u32x4*>(xl + (int64_t)M * K)[i] = u32x4{0u, 0u, 0u, 0u};
-    lds_barrier();
+    for (int nt = 0; nt < NT; ++nt) tile[nt] = blockIdx.x * NT + nt;
   }
 }
 
-template <int MT, int NT, int WAVES, int U, bool XLDS>
-__global__ __launch_bounds__(WAVES * 64) void w4_gemv_kernel(const uint16_t* __restrict__ x,
-                                                             const u32x4* __restrict__ wt,
+// ---- int4 -----------------------------------------------------------------------------------------------
+template <int MT, int NT, int WAVES, int U, bool XLDS, int PRO, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void w4_gemv_kernel(GemvArgs args, const u32x4* __restrict__ wt,
                                                              const uint16_t* __restrict__ st,
-                                                             const uint8_t* __restrict__ zt, uint16_t* __restrict__ y,
-                                                             int M, int N, int K) {
+                                                             const uint8_t* __restrict__ zt) {
+  static_assert(!XLDS || MT == 1, "x in LDS is for M <= 16");
+  static_assert(PRO == 0 || XLDS, "the norm prologue writes x into LDS");
   extern __shared__ __align__(16) unsigned char smem[];
-  float* red = reinterpret_cast<float*>(smem);                                         // [WAVES][MT*NT*256]
-  uint16_t* xl = reinterpret_cast<uint16_t*>(smem + WAVES * MT * NT * 256 * sizeof(float));  // [M+1][K]
+  float* red = reinterpret_cast<float*>(smem);                                                // [WAVES][MT*NT*256]
+  uint16_t* xl = reinterpret_cast<uint16_t*>(smem + WAVES * MT * NT * 256 * sizeof(float));   // [M+1][K]
+  const int M = args.M, K = args.K;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, kq = lane >> 4;
-  const int G = K >> 7, ntiles = N >> 4;
-  const int nt0 = blockIdx.x * NT;
+  const int G = K >> 7, ntiles = args.N >> 4;
+  int tile[NT];
+  owned_tiles<NT, EPI>(tile, ntiles);
   // contiguous slice of groups per wave
   const int g_begin = (int)((int64_t)G * wave / WAVES), g_end = (int)((int64_t)G * (wave + 1) / WAVES);
   const bf16x8 ones = ones_bf16x8();
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
-
-  static_assert(!XLDS || MT == 1, "x in LDS is for M <= 16");
-  XSource<XLDS> xs_src{x, xl, M, K, (col < M ? col : M) * K};
+  const uint16_t* xrow = xl + (col < M ? col : M) * K;  // this lane's row in LDS (XLDS)
 
   f32x4 acc[MT][NT];
 #pragma unroll
@@ -146,28 +247,27 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_kernel(const uint16_t* __r
   auto issue = [&](int u, int g) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const int tnt = min(nt0 + nt, ntiles - 1);  // out-of-range tiles are computed and dropped
-      const int64_t tile = (int64_t)tnt * G + g;
-      w[u][nt] = __builtin_nontemporal_load(&wt[tile * 64 + lane]);
-      s16[u][nt] = st[tile * 16 + col];
-      z8[u][nt] = zt[tile * 8 + (col >> 1)];
+      const int tnt = min(tile[nt], ntiles - 1);  // out-of-range tiles are computed and dropped
+      const int64_t t = (int64_t)tnt * G + g;
+      w[u][nt] = __builtin_nontemporal_load(&wt[t * 64 + lane]);
+      s16[u][nt] = st[t * 16 + col];
+      z8[u][nt] = zt[t * 8 + (col >> 1)];
     }
     if constexpr (!XLDS) {
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) a[u][j][mt] = xs_src.frag(mt, col, 128 * g + 32 * j + 8 * kq);
+        for (int mt = 0; mt < MT; ++mt) a[u][j][mt] = load_x_frag(args.x, mt * 16 + col, M, K, 128 * g + 32 * j + 8 * kq);
     }
   };
 
   // x first (it comes from L2 and is needed first), then U weight pieces in flight
-  u32x4 xr[kXStageRegs];
-  stage_x_begin<WAVES, XLDS>(xr, x, M, K);
+  XStage<WAVES, XLDS, PRO> stage;
+  stage.begin(args);
 #pragma unroll
   for (int u = 0; u < U; ++u)
     if (g_begin + u < g_end) issue(u, g_begin + u);
-
-  stage_x_finish<WAVES, XLDS>(xr, x, xl, M, K);
+  stage.finish(args, xl);
 
   for (int base = g_begin; base < g_end; base += U) {
 #pragma unroll
@@ -186,7 +286,7 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_kernel(const uint16_t* __r
           bf16x8 af[MT];
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
-            if constexpr (XLDS) af[mt] = xs_src.frag(mt, col, 128 * g + 32 * j + 8 * kq);
+            if constexpr (XLDS) af[mt] = *reinterpret_cast<const bf16x8*>(xrow + 128 * g + 32 * j + 8 * kq);
             else af[mt] = a[u][j][mt];
             xsum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], ones, xsum[mt], 0, 0, 0);
           }
@@ -211,24 +311,26 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_kernel(const uint16_t* __r
       }
     }
   }
-  gemv_epilogue<MT, NT, WAVES>(acc, red, y, M, N, nt0, ntiles);
+  gemv_epilogue<MT, NT, WAVES, EPI>(acc, red, args, tile, ntiles);
 }
 
-template <int MT, int NT, int WAVES, int U, bool XLDS>
-__global__ __launch_bounds__(WAVES * 64) void b16_gemv_kernel(const uint16_t* __restrict__ x,
-                                                              const bf16x8* __restrict__ wt, uint16_t* __restrict__ y,
-                                                              int M, int N, int K) {
+// ---- dense bf16 --------------------------------------------------------------------------------------------
+template <int MT, int NT, int WAVES, int U, bool XLDS, int PRO, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void b16_gemv_kernel(GemvArgs args, const bf16x8* __restrict__ wt) {
+  static_assert(!XLDS || MT == 1, "x in LDS is for M <= 16");
+  static_assert(PRO == 0 || XLDS, "the norm prologue writes x into LDS");
   extern __shared__ __align__(16) unsigned char smem[];
   float* red = reinterpret_cast<float*>(smem);
   uint16_t* xl = reinterpret_cast<uint16_t*>(smem + WAVES * MT * NT * 256 * sizeof(float));
+  const int M = args.M, K = args.K;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, kq = lane >> 4;
-  const int KS = K >> 5, ntiles = N >> 4;
-  const int nt0 = blockIdx.x * NT;
+  const int KS = K >> 5, ntiles = args.N >> 4;
+  int tile[NT];
+  owned_tiles<NT, EPI>(tile, ntiles);
   const int s_begin = (int)((int64_t)KS * wave / WAVES), s_end = (int)((int64_t)KS * (wave + 1) / WAVES);
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
-  static_assert(!XLDS || MT == 1, "x in LDS is for M <= 16");
-  XSource<XLDS> xs_src{x, xl, M, K, (col < M ? col : M) * K};
+  const uint16_t* xrow = xl + (col < M ? col : M) * K;
   f32x4 acc[MT][NT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
@@ -238,20 +340,20 @@ __global__ __launch_bounds__(WAVES * 64) void b16_gemv_kernel(const uint16_t* __
   auto issue = [&](int u, int ks) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      const int tnt = min(nt0 + nt, ntiles - 1);
+      const int tnt = min(tile[nt], ntiles - 1);
       b[u][nt] = __builtin_nontemporal_load(&wt[((int64_t)tnt * KS + ks) * 64 + lane]);
     }
     if constexpr (!XLDS) {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) a[u][mt] = xs_src.frag(mt, col, 32 * ks + 8 * kq);
+      for (int mt = 0; mt < MT; ++mt) a[u][mt] = load_x_frag(args.x, mt * 16 + col, M, K, 32 * ks + 8 * kq);
     }
   };
-  u32x4 xr[kXStageRegs];
-  stage_x_begin<WAVES, XLDS>(xr, x, M, K);
+  XStage<WAVES, XLDS, PRO> stage;
+  stage.begin(args);
 #pragma unroll
   for (int u = 0; u < U; ++u)
     if (s_begin + u < s_end) issue(u, s_begin + u);
-  stage_x_finish<WAVES, XLDS>(xr, x, xl, M, K);
+  stage.finish(args, xl);
   for (int base = s_begin; base < s_end; base += U) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -260,7 +362,7 @@ __global__ __launch_bounds__(WAVES * 64) void b16_gemv_kernel(const uint16_t* __
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           bf16x8 af;
-          if constexpr (XLDS) af = xs_src.frag(mt, col, 32 * ks + 8 * kq);
+          if constexpr (XLDS) af = *reinterpret_cast<const bf16x8*>(xrow + 32 * ks + 8 * kq);
           else af = a[u][mt];
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, b[u][nt], acc[mt][nt], 0, 0, 0);
@@ -269,85 +371,136 @@ __global__ __launch_bounds__(WAVES * 64) void b16_gemv_kernel(const uint16_t* __
       }
     }
   }
-  gemv_epilogue<MT, NT, WAVES>(acc, red, y, M, N, nt0, ntiles);
+  gemv_epilogue<MT, NT, WAVES, EPI>(acc, red, args, tile, ntiles);
 }
 
 // ---- launch plans -------------------------------------------------------------------------------
 struct GemvPlan {
-  int mt, nt, waves, u;
+  int mt, nt, waves;
   bool xlds;
+  int pro, epi;
 };
 
-// Experiment hook (not part of the public interface): overrides nt / waves / u / xlds when >= 0.
-int g_dbg_nt = -1, g_dbg_waves = -1, g_dbg_u = -1, g_dbg_xlds = -1;
+// Experiment hook (not part of the public interface): overrides waves / xlds when >= 0.
+int g_dbg_waves = -1, g_dbg_xlds = -1;
 
 constexpr int kXldsMaxBytes = 64 * 1024;
 
-inline GemvPlan plan_gemv(int M, int N, int K, bool w4) {
+// u (pieces in flight per wave) is fixed per format: 2 KiB-groups for int4, 8 (4 for M > 16) 32-row steps for bf16
+inline GemvPlan plan_gemv(int M, int N, int K, bool w4, bool pro, bool epi) {
   GemvPlan p;
   p.mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  p.nt = epi ? 2 : 1;
+  p.pro = pro, p.epi = epi;
   const int ntiles = N >> 4;
-  const int units = w4 ? (K >> 7) : (K >> 5);   // 1 KiB pieces per column tile
-  // Measured on the 7B shapes: 2 pieces in flight per wave, 16 waves per workgroup for narrow
-  // outputs (N <= 8192, one workgroup per CU), 8 otherwise; never fewer than u pieces per wave.
-  p.nt = 1;
-  p.u = w4 ? 2 : (p.mt == 1 ? 8 : 4);
+  const int units = w4 ? (K >> 7) : (K >> 5);  // 1 KiB pieces per column tile
+  const int u = w4 ? 2 : (p.mt == 1 ? 8 : 4);
+  // Measured on the 7B shapes: 16 waves per workgroup for narrow outputs (N <= 8192, one workgroup
+  // per CU), 8 otherwise; never fewer than u pieces per wave.
   int waves = ntiles <= 512 ? 16 : 8;
-  while (waves > 4 && units < waves * p.u) waves /= 2;
+  while (waves > 4 && units < waves * u) waves /= 2;
+  if (pro && waves < M) waves = 0;  // the prologue needs one wave per row: no kernel, caller falls back
   p.waves = waves;
   p.xlds = p.mt == 1 && (int64_t)(M + 1) * K * 2 <= kXldsMaxBytes;
-  if (g_dbg_nt >= 0) p.nt = g_dbg_nt;
-  if (g_dbg_waves >= 0) p.waves = g_dbg_waves;
-  if (g_dbg_u >= 0) p.u = g_dbg_u;
-  if (g_dbg_xlds >= 0) p.xlds = g_dbg_xlds && p.mt == 1 && (int64_t)(M + 1) * K * 2 <= kXldsMaxBytes;
+  if (g_dbg_waves >= 0 && !pro && !epi) p.waves = g_dbg_waves;
+  if (g_dbg_xlds >= 0 && !pro && !epi) p.xlds = g_dbg_xlds && p.xlds;
   return p;
 }
 
 template <typename Kern, typename... Args>
-int launch_gemv(Kern kern, const GemvPlan& p, int M, int N, int K, hipStream_t stream, Args... args) {
-  const size_t lds = (size_t)p.waves * p.mt * p.nt * 256 * 4 + (p.xlds ? (size_t)(M + 1) * K * 2 : 0);
+int launch_gemv(Kern kern, const GemvPlan& p, const GemvArgs& a, hipStream_t stream, Args... args) {
+  const size_t lds = (size_t)p.waves * p.mt * p.nt * 256 * 4 + (p.xlds ? (size_t)(a.M + 1) * a.K * 2 : 0);
   if (lds > 48 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
     return O355_ELAUNCH;
-  const unsigned blocks = (unsigned)(((N >> 4) + p.nt - 1) / p.nt);
-  hipLaunchKernelGGL(kern, dim3(blocks), dim3(p.waves * 64), lds, stream, args..., M, N, K);
+  const int ntiles = a.N >> 4;
+  const unsigned blocks = p.epi ? (unsigned)(ntiles >> 1) : (unsigned)((ntiles + p.nt - 1) / p.nt);
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(p.waves * 64), lds, stream, a, args...);
   O355_CHECK_LAUNCH();
+}
+
+int check_fused(const GemvArgs& a, bool pro, bool epi) {
+  if (pro && (!a.resid || !a.norm_w || !a.x_out || a.M > 16 || (a.K >> 3) > 64 * kNormVPL)) return O355_EUNSUPPORTED;
+  if ((pro || epi) && (int64_t)(a.M + 1) * a.K * 2 > kXldsMaxBytes) return O355_EUNSUPPORTED;
+  if (epi && ((a.N & 31) || a.M > 16)) return O355_EUNSUPPORTED;
+  return O355_OK;
+}
+
+#define GEMV_CASE(KERNEL, MTv, NTv, Wv, Uv, Xv, Pv, Ev, ...)                                                  \
+  if (p.mt == MTv && p.nt == NTv && p.waves == Wv && p.xlds == Xv && p.pro == Pv && p.epi == Ev)             \
+    return launch_gemv(KERNEL<MTv, NTv, Wv, Uv, Xv, Pv, Ev>, p, a, as_stream(stream), __VA_ARGS__);
+#define GEMV_WAVES(KERNEL, MTv, NTv, Uv, Xv, Pv, Ev, ...)        \
+  GEMV_CASE(KERNEL, MTv, NTv, 4, Uv, Xv, Pv, Ev, __VA_ARGS__)    \
+  GEMV_CASE(KERNEL, MTv, NTv, 8, Uv, Xv, Pv, Ev, __VA_ARGS__)    \
+  GEMV_CASE(KERNEL, MTv, NTv, 16, Uv, Xv, Pv, Ev, __VA_ARGS__)
+
+int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, bool pro, bool epi,
+                     void* stream) {
+  const GemvPlan p = plan_gemv(a.M, a.N, a.K, true, pro, epi);
+  const u32x4* w = (const u32x4*)wt;
+  GEMV_WAVES(w4_gemv_kernel, 1, 1, 2, true, 0, 0, w, st, zt)
+  GEMV_WAVES(w4_gemv_kernel, 1, 1, 2, false, 0, 0, w, st, zt)
+  GEMV_WAVES(w4_gemv_kernel, 2, 1, 2, false, 0, 0, w, st, zt)
+  GEMV_WAVES(w4_gemv_kernel, 4, 1, 2, false, 0, 0, w, st, zt)
+  GEMV_WAVES(w4_gemv_kernel, 1, 1, 2, true, 1, 0, w, st, zt)
+  GEMV_WAVES(w4_gemv_kernel, 1, 2, 2, true, 0, 1, w, st, zt)
+  GEMV_WAVES(w4_gemv_kernel, 1, 2, 2, true, 1, 1, w, st, zt)
+  return O355_EUNSUPPORTED;
+}
+
+int b16_gemv_dispatch(const GemvArgs& a, const uint16_t* wt, bool pro, bool epi, void* stream) {
+  const GemvPlan p = plan_gemv(a.M, a.N, a.K, false, pro, epi);
+  const bf16x8* w = (const bf16x8*)wt;
+  GEMV_WAVES(b16_gemv_kernel, 1, 1, 8, true, 0, 0, w)
+  GEMV_WAVES(b16_gemv_kernel, 1, 1, 8, false, 0, 0, w)
+  GEMV_WAVES(b16_gemv_kernel, 2, 1, 4, false, 0, 0, w)
+  GEMV_WAVES(b16_gemv_kernel, 4, 1, 4, false, 0, 0, w)
+  GEMV_WAVES(b16_gemv_kernel, 1, 1, 8, true, 1, 0, w)
+  GEMV_WAVES(b16_gemv_kernel, 1, 2, 8, true, 0, 1, w)
+  GEMV_WAVES(b16_gemv_kernel, 1, 2, 8, true, 1, 1, w)
+  return O355_EUNSUPPORTED;
 }
 
 }  // namespace
 
-extern "C" void olmo355_debug_set_gemv_plan(int nt, int waves, int u, int xlds) {
-  g_dbg_nt = nt, g_dbg_waves = waves, g_dbg_u = u, g_dbg_xlds = xlds;
-}
-
-#define W4_CASE(MTv, NTv, Wv, Uv, Xv)                                                                          \
-  if (p.mt == MTv && p.nt == NTv && p.waves == Wv && p.u == Uv && p.xlds == Xv)                               \
-    return launch_gemv(w4_gemv_kernel<MTv, NTv, Wv, Uv, Xv>, p, M, N, K, as_stream(stream), x, (const u32x4*)wt, st, zt, y);
-#define B16_CASE(MTv, NTv, Wv, Uv, Xv)                                                                         \
-  if (p.mt == MTv && p.nt == NTv && p.waves == Wv && p.u == Uv && p.xlds == Xv)                               \
-    return launch_gemv(b16_gemv_kernel<MTv, NTv, Wv, Uv, Xv>, p, M, N, K, as_stream(stream), x, (const bf16x8*)wt, y);
-#define FOR_WAVES(CASE, MTv, NTv, Uv, Xv) CASE(MTv, NTv, 4, Uv, Xv) CASE(MTv, NTv, 8, Uv, Xv) CASE(MTv, NTv, 16, Uv, Xv)
+extern "C" void olmo355_debug_set_gemv_plan(int waves, int xlds) { g_dbg_waves = waves, g_dbg_xlds = xlds; }
 
 extern "C" int olmo355_w4_gemv(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
                                uint16_t* y, int M, int N, int K, void* stream) {
   if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
   if (M > 64 || (K & 127) || (N & 15)) return O355_EUNSUPPORTED;
-  const GemvPlan p = plan_gemv(M, N, K, true);
-  FOR_WAVES(W4_CASE, 1, 1, 4, true) FOR_WAVES(W4_CASE, 1, 1, 4, false)
-  FOR_WAVES(W4_CASE, 1, 1, 2, true) FOR_WAVES(W4_CASE, 1, 1, 2, false)
-  FOR_WAVES(W4_CASE, 1, 1, 8, true) FOR_WAVES(W4_CASE, 1, 2, 4, true) FOR_WAVES(W4_CASE, 1, 2, 2, true)
-  FOR_WAVES(W4_CASE, 1, 4, 2, true) FOR_WAVES(W4_CASE, 1, 2, 2, false)
-  FOR_WAVES(W4_CASE, 2, 1, 2, false) FOR_WAVES(W4_CASE, 4, 1, 2, false)
-  return O355_EUNSUPPORTED;
+  const GemvArgs a{x, nullptr, nullptr, nullptr, y, 0.f, M, N, K};
+  return w4_gemv_dispatch(a, wt, st, zt, false, false, stream);
 }
 
 extern "C" int olmo355_b16_gemv(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K,
                                 void* stream) {
   if (!x || !wt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
   if (M > 64 || (K & 31) || (N & 15)) return O355_EUNSUPPORTED;
-  const GemvPlan p = plan_gemv(M, N, K, false);
-  FOR_WAVES(B16_CASE, 1, 1, 8, true) FOR_WAVES(B16_CASE, 1, 1, 8, false)
-  FOR_WAVES(B16_CASE, 1, 1, 4, true) FOR_WAVES(B16_CASE, 1, 2, 8, true) FOR_WAVES(B16_CASE, 1, 2, 4, true)
-  FOR_WAVES(B16_CASE, 2, 1, 4, false) FOR_WAVES(B16_CASE, 4, 1, 4, false)
-  return O355_EUNSUPPORTED;
+  const GemvArgs a{x, nullptr, nullptr, nullptr, y, 0.f, M, N, K};
+  return b16_gemv_dispatch(a, wt, false, false, stream);
+}
+
+extern "C" int olmo355_w4_gemv_fused(const uint16_t* x, const uint16_t* resid, const uint16_t* norm_w, float eps,
+                                     uint16_t* x_out, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
+                                     uint16_t* y, int M, int N, int K, int swiglu, void* stream) {
+  if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
+  if (M > 64 || (K & 127) || (N & 15)) return O355_EUNSUPPORTED;
+  const GemvArgs a{x, resid, norm_w, x_out, y, eps, M, N, K};
+  const bool pro = resid != nullptr, epi = swiglu != 0;
+  const int chk = check_fused(a, pro, epi);
+  if (chk != O355_OK) return chk;
+  return w4_gemv_dispatch(a, wt, st, zt, pro, epi, stream);
+}
+
+extern "C" int olmo355_b16_gemv_fused(const uint16_t* x, const uint16_t* resid, const uint16_t* norm_w, float eps,
+                                      uint16_t* x_out, const uint16_t* wt, uint16_t* y, int M, int N, int K, int swiglu,
+                                      void* stream) {
+  if (!x || !wt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
+  if (M > 64 || (K & 31) || (N & 15)) return O355_EUNSUPPORTED;
+  const GemvArgs a{x, resid, norm_w, x_out, y, eps, M, N, K};
+  const bool pro = resid != nullptr, epi = swiglu != 0;
+  const int chk = check_fused(a, pro, epi);
+  if (chk != O355_OK) return chk;
+  return b16_gemv_dispatch(a, wt, pro, epi, stream);
 }

@@ -96,12 +96,15 @@ class DenseLinear(nn.Linear):
             self._tiled = ops.b16_repack(self.weight.data.contiguous())
         return self
 
+    def tiled_weight(self) -> ops.B16Tiled:
+        if self._tiled is None:
+            self.post_init()
+        return self._tiled
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.weight.dtype == torch.float32:
             return ops.f32_linear(x, self.weight.data)
-        if self._tiled is None:
-            self.post_init()
-        return ops.b16_linear(x, self._tiled)
+        return ops.b16_linear(x, self.tiled_weight())
 
 
 class RMSLayerNorm(nn.Module):
@@ -299,21 +302,24 @@ class OLMo(nn.Module):
     def _linear(self, m: nn.Module, x: torch.Tensor) -> torch.Tensor:
         return m(x)
 
-    def _block(self, blk: OLMoSequentialBlock, x, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max):
+    def _attention(self, blk, qkv, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max):
         c = self.config
         H, Hkv, hd = c.n_heads, c.effective_n_kv_heads, c.head_dim
-        h = x if c.norm_after else blk.attn_norm(x)
-        qkv = self._linear(blk.att_proj, h)
         sin, cos = self._rope
         qw = blk.q_norm.weight.data if blk.q_norm is not None else None
         kw = blk.k_norm.weight.data if blk.k_norm is not None else None
         q = ops.qknorm_rope_kvwrite(qkv, qw, kw, sin, cos, kc, vc, B, T, H, Hkv, hd, past_len, c.layer_norm_eps,
                                     past_len_dev=graph_pos)
         if T == 1 and (graph_pos is not None or past_len > 0):
-            att = ops.attn_decode(q, kc, vc, self._decode_ws(B, n_keys_max), B, H, Hkv, hd, past_len, n_keys_max,
-                                  key_bias=key_bias, past_len_dev=graph_pos)
-        else:
-            att = ops.attn_prefill(q, kc, vc, B, T, H, Hkv, hd, past_len, key_bias=key_bias)
+            return ops.attn_decode(q, kc, vc, self._decode_ws(B, n_keys_max), B, H, Hkv, hd, past_len, n_keys_max,
+                                   key_bias=key_bias, past_len_dev=graph_pos)
+        return ops.attn_prefill(q, kc, vc, B, T, H, Hkv, hd, past_len, key_bias=key_bias)
+
+    def _block(self, blk: OLMoSequentialBlock, x, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max):
+        c = self.config
+        h = x if c.norm_after else blk.attn_norm(x)
+        qkv = self._linear(blk.att_proj, h)
+        att = self._attention(blk, qkv, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max)
         att = self._linear(blk.attn_out, att)
         x = blk.attn_norm(att, residual=x) if c.norm_after else ops.add(x, att)
         h = x if c.norm_after else blk.ff_norm(x)
@@ -321,6 +327,33 @@ class OLMo(nn.Module):
         h = ops.swiglu(h)
         h = self._linear(blk.ff_out, h)
         return blk.ff_norm(h, residual=x) if c.norm_after else ops.add(x, h)
+
+    # Decode form of the OLMo-2 (post-norm, RMS) block with the residual/norm updates folded into the
+    # linear that consumes them and SwiGLU into ff_proj: 6 launches per layer instead of 10.
+    #   x      residual stream entering the block, *before* the previous block's pending update
+    #   pend   (f_prev, ff_norm weight of the previous block) or None: x := x + norm(f_prev) is applied
+    #          inside this block's att_proj launch
+    def _fused_decode_ok(self, M: int, collect_hidden: bool) -> bool:
+        c = self.config
+        return (M <= 16 and self.dtype == torch.bfloat16 and c.norm_after and c.layer_norm_type == "rms"
+                and not collect_hidden and c.d_model * 2 * (M + 1) <= 64 * 1024 and c.d_model <= 5120)
+
+    @staticmethod
+    def _tiled(m: nn.Module):
+        return m.tiled if isinstance(m, QuantLinear) else m.tiled_weight()
+
+    def _block_decode_fused(self, blk, x, pend, kc, vc, B, past_len, key_bias, graph_pos, n_keys_max):
+        eps = self.config.layer_norm_eps
+        if pend is None:
+            qkv = self._linear(blk.att_proj, x)
+        else:
+            qkv, x = ops.linear_fused(pend[0], self._tiled(blk.att_proj), resid=x, norm_w=pend[1], eps=eps)
+        att = self._attention(blk, qkv, kc, vc, B, 1, past_len, key_bias, graph_pos, n_keys_max)
+        a = self._linear(blk.attn_out, att)
+        u, x = ops.linear_fused(a, self._tiled(blk.ff_proj), resid=x, norm_w=blk.attn_norm.weight.data, eps=eps,
+                                swiglu_out=True)
+        f = self._linear(blk.ff_out, u)
+        return x, (f, blk.ff_norm.weight.data)
 
     # ------------------------------------------------------------------------------------------
     # forward: olmo/model.py:1253-1465
@@ -399,6 +432,8 @@ class OLMo(nn.Module):
         position, so the call can be captured once and replayed; it requires ``T == 1``."""
         n_keys_max = cache.capacity if graph_pos is not None else past_len + T
         hidden: List[torch.Tensor] = []
+        fused = T == 1 and cache is not None and self._fused_decode_ok(B, collect_hidden)
+        pend = None
         for i, blk in enumerate(self.transformer["blocks"]):
             if collect_hidden:
                 hidden.append(x)
@@ -406,7 +441,12 @@ class OLMo(nn.Module):
                 kc, vc = cache.k[i], cache.v[i]
             else:
                 kc, vc = self._scratch_cache(B, T)
-            x = self._block(blk, x, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max)
+            if fused:
+                x, pend = self._block_decode_fused(blk, x, pend, kc, vc, B, past_len, key_bias, graph_pos, n_keys_max)
+            else:
+                x = self._block(blk, x, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max)
+        if pend is not None:  # the last block's update has no following linear to ride on
+            x = ops.rmsnorm(pend[0], pend[1], self.config.layer_norm_eps, residual=x)
         if last_logits_only and T > 1:
             x = x[:, -1, :].unsqueeze(1).contiguous()
         x = self.transformer["ln_f"](x)

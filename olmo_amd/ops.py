@@ -173,6 +173,38 @@ def b16_linear(x: torch.Tensor, w: B16Tiled) -> torch.Tensor:
     return y
 
 
+def linear_fused(x: torch.Tensor, w, resid: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None,
+                 eps: float = 0.0, swiglu_out: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Decode-step linear with its neighbours folded into the same launch: returns ``(y, x_new)`` with
+    ``x_new = resid + rmsnorm(x; norm_w, eps)`` (``x`` itself without ``resid``) and
+    ``y = x_new @ W`` (``swiglu(x_new @ W)`` with ``swiglu_out``).  Falls back to the separate kernels
+    for shapes the fused kernels do not cover.  ``w``: ``W4Tiled`` or ``B16Tiled``."""
+    _dev(x, resid, norm_w)
+    if x.dtype != torch.bfloat16:
+        raise TypeError("bfloat16 activations expected")
+    M = x.numel() // w.K
+    n_out = w.N // 2 if swiglu_out else w.N
+    if M and M <= 16 and (resid is not None or swiglu_out):
+        y = torch.empty(*x.shape[:-1], n_out, dtype=torch.bfloat16, device=x.device)
+        x_new = torch.empty_like(x) if resid is not None else x
+        xo = _p(x_new) if resid is not None else None
+        if isinstance(w, W4Tiled):
+            st = lib().olmo355_w4_gemv_fused(_p(x), _p(resid), _p(norm_w), float(eps), xo, _p(w.wt), _p(w.st), _p(w.zt),
+                                             _p(y), M, w.N, w.K, int(swiglu_out), _stream())
+            name = "olmo355_w4_gemv_fused"
+        else:
+            st = lib().olmo355_b16_gemv_fused(_p(x), _p(resid), _p(norm_w), float(eps), xo, _p(w.wt), _p(y), M, w.N, w.K,
+                                              int(swiglu_out), _stream())
+            name = "olmo355_b16_gemv_fused"
+        if st == 0:
+            return y, x_new
+        if st != 2:
+            check(name, st)
+    x_new = rmsnorm(x, norm_w, eps, residual=resid) if resid is not None else x
+    y = w4_linear(x_new, w) if isinstance(w, W4Tiled) else b16_linear(x_new, w)
+    return (swiglu(y) if swiglu_out else y), x_new
+
+
 def f32_linear(x: torch.Tensor, weight_nk: torch.Tensor) -> torch.Tensor:
     _dev(x, weight_nk)
     if x.dtype != torch.float32 or weight_nk.dtype != torch.float32:
