@@ -66,12 +66,11 @@ __device__ __forceinline__ void unpack8(const u32x4& v, float (&f)[8]) {
 // The global loads are issued in begin() -- before the weight prologue -- and consumed in
 // finish(), after the weight loads have been issued; the barrier orders LDS only.
 constexpr int kXStageRegs = 4;  // plain copy: 16-byte pieces per thread held across the weight prologue
-constexpr int kNormVPL = 10;    // prologue: 16-byte pieces of a row per lane (K <= 5120)
 
 template <int WAVES, bool XLDS, int PRO>
 struct XStage {
   __device__ __forceinline__ void begin(const GemvArgs&) {}
-  __device__ __forceinline__ void finish(const GemvArgs&, uint16_t*) {}
+  __device__ __forceinline__ void finish(const GemvArgs&, uint16_t*, float*) {}
 };
 
 template <int WAVES>
@@ -85,7 +84,7 @@ struct XStage<WAVES, true, 0> {
       if (idx < total) xr[i] = reinterpret_cast<const u32x4*>(a.x)[idx];
     }
   }
-  __device__ __forceinline__ void finish(const GemvArgs& a, uint16_t* xl) {
+  __device__ __forceinline__ void finish(const GemvArgs& a, uint16_t* xl, float*) {
     const int total = (a.M * a.K) >> 3;
 #pragma unroll
     for (int i = 0; i < kXStageRegs; ++i) {
@@ -101,57 +100,64 @@ struct XStage<WAVES, true, 0> {
 };
 
 // x := resid + w * round(a * rsqrt(mean(a^2) + eps)), rounding points of olmo/model.py:241-255 and
-// of the bf16 residual add.  Wave m normalises row m (M <= WAVES), so only wave reductions are needed.
-template <int WAVES>
-struct XStage<WAVES, true, 1> {
-  u32x4 av[kNormVPL], rv[kNormVPL], wv[kNormVPL];
+// of the bf16 residual add.  The whole workgroup shares the rows: thread t owns the 16-byte pieces
+// t, t + threads, ... (VPT of them), a wave's 64 pieces lie in one row (K % 512 == 0), the per-wave
+// sums of squares meet in LDS and are added in a fixed order.
+template <int WAVES, int VPT>
+struct NormStage {
+  u32x4 av[VPT], rv[VPT], wv[VPT];
   __device__ __forceinline__ void begin(const GemvArgs& a) {
-    const int lane = threadIdx.x & 63, m = threadIdx.x >> 6, nvec = a.K >> 3;
-    if (m < a.M) {
+    const int nvec = a.K >> 3, total = a.M * nvec;
 #pragma unroll
-      for (int i = 0; i < kNormVPL; ++i) {
-        const int idx = lane + 64 * i;
-        if (idx < nvec) {
-          av[i] = reinterpret_cast<const u32x4*>(a.x)[(int64_t)m * nvec + idx];
-          rv[i] = reinterpret_cast<const u32x4*>(a.resid)[(int64_t)m * nvec + idx];
-          wv[i] = reinterpret_cast<const u32x4*>(a.norm_w)[idx];
-        }
+    for (int i = 0; i < VPT; ++i) {
+      const int idx = threadIdx.x + i * WAVES * 64;
+      if (idx < total) {
+        av[i] = reinterpret_cast<const u32x4*>(a.x)[idx];
+        rv[i] = reinterpret_cast<const u32x4*>(a.resid)[idx];
+        wv[i] = reinterpret_cast<const u32x4*>(a.norm_w)[idx % nvec];
       }
     }
   }
-  __device__ __forceinline__ void finish(const GemvArgs& a, uint16_t* xl) {
-    const int lane = threadIdx.x & 63, m = threadIdx.x >> 6, nvec = a.K >> 3;
-    if (m < a.M) {
+  __device__ __forceinline__ void finish(const GemvArgs& a, uint16_t* xl, float* part /* [VPT*WAVES] */) {
+    const int nvec = a.K >> 3, total = a.M * nvec;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
       float ss = 0.f;
+      if (threadIdx.x + i * WAVES * 64 < total) {
+        float f[8];
+        unpack8(av[i], f);
 #pragma unroll
-      for (int i = 0; i < kNormVPL; ++i) {
-        if (lane + 64 * i < nvec) {
-          float f[8];
-          unpack8(av[i], f);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
-        }
+        for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
       }
       ss = wave_sum(ss);
-      const float rstd = 1.f / sqrtf(ss / (float)a.K + a.eps);
+      if (lane == 0) part[i * WAVES + wave] = ss;
+    }
+    lds_barrier();
 #pragma unroll
-      for (int i = 0; i < kNormVPL; ++i) {
-        const int idx = lane + 64 * i;
-        if (idx < nvec) {
-          float f[8], r[8], w[8];
-          unpack8(av[i], f);
-          unpack8(rv[i], r);
-          unpack8(wv[i], w);
-          u32x4 o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float y0 = round_bf16(w[2 * e] * round_bf16(f[2 * e] * rstd));
-            const float y1 = round_bf16(w[2 * e + 1] * round_bf16(f[2 * e + 1] * rstd));
-            o[e] = pack_bf16x2(r[2 * e] + y0, r[2 * e + 1] + y1);
-          }
-          reinterpret_cast<u32x4*>(xl)[(int64_t)m * nvec + idx] = o;
-          if (blockIdx.x == 0) reinterpret_cast<u32x4*>(a.x_out)[(int64_t)m * nvec + idx] = o;
+    for (int i = 0; i < VPT; ++i) {
+      const int idx = threadIdx.x + i * WAVES * 64;
+      if (idx < total) {
+        const int m = idx / nvec;
+        float ss = 0.f;  // partials of row m, in (i, wave) order
+        for (int j = 0; j < VPT * WAVES; ++j) {
+          const int first = (j % WAVES) * 64 + (j / WAVES) * WAVES * 64;  // first piece of that partial
+          if (first < total && first / nvec == m) ss += part[j];
         }
+        const float rstd = 1.f / sqrtf(ss / (float)a.K + a.eps);
+        float f[8], r[8], w[8];
+        unpack8(av[i], f);
+        unpack8(rv[i], r);
+        unpack8(wv[i], w);
+        u32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float y0 = round_bf16(w[2 * e] * round_bf16(f[2 * e] * rstd));
+          const float y1 = round_bf16(w[2 * e + 1] * round_bf16(f[2 * e + 1] * rstd));
+          o[e] = pack_bf16x2(r[2 * e] + y0, r[2 * e + 1] + y1);
+        }
+        reinterpret_cast<u32x4*>(xl)[idx] = o;
+        if (blockIdx.x == 0) reinterpret_cast<u32x4*>(a.x_out)[idx] = o;
       }
     }
     for (int i = threadIdx.x; i < nvec; i += WAVES * 64)
@@ -159,6 +165,10 @@ struct XStage<WAVES, true, 1> {
     lds_barrier();
   }
 };
+template <int WAVES>
+struct XStage<WAVES, true, 1> : NormStage<WAVES, 1> {};
+template <int WAVES>
+struct XStage<WAVES, true, 4> : NormStage<WAVES, 4> {};
 
 // ---- epilogue: reduce over the waves in fixed order, write y (bf16) -----------------------------------
 template <int MT, int NT, int WAVES, int EPI>
@@ -267,7 +277,7 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_kernel(GemvArgs args, cons
 #pragma unroll
   for (int u = 0; u < U; ++u)
     if (g_begin + u < g_end) issue(u, g_begin + u);
-  stage.finish(args, xl);
+  stage.finish(args, xl, red);
 
   for (int base = g_begin; base < g_end; base += U) {
 #pragma unroll
@@ -353,7 +363,7 @@ __global__ __launch_bounds__(WAVES * 64) void b16_gemv_kernel(GemvArgs args, con
 #pragma unroll
   for (int u = 0; u < U; ++u)
     if (s_begin + u < s_end) issue(u, s_begin + u);
-  stage.finish(args, xl);
+  stage.finish(args, xl, red);
   for (int base = s_begin; base < s_end; base += U) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -399,7 +409,12 @@ inline GemvPlan plan_gemv(int M, int N, int K, bool w4, bool pro, bool epi) {
   // per CU), 8 otherwise; never fewer than u pieces per wave.
   int waves = ntiles <= 512 ? 16 : 8;
   while (waves > 4 && units < waves * u) waves /= 2;
-  if (pro && waves < M) waves = 0;  // the prologue needs one wave per row: no kernel, caller falls back
+  if (p.mt > 1 && waves > 8) waves = 8;  // register budget of the wider accumulators
+  if (pro) {  // rows shared by the whole workgroup: 1 or 4 pieces per thread
+    const int pieces = M * (K >> 3);
+    if (pieces > waves * 64 && waves < 16 && units >= 16 * u) waves = 16;
+    p.pro = pieces <= waves * 64 ? 1 : (pieces <= 4 * waves * 64 ? 4 : -1);
+  }
   p.waves = waves;
   p.xlds = p.mt == 1 && (int64_t)(M + 1) * K * 2 <= kXldsMaxBytes;
   if (g_dbg_waves >= 0 && !pro && !epi) p.waves = g_dbg_waves;
@@ -420,7 +435,7 @@ int launch_gemv(Kern kern, const GemvPlan& p, const GemvArgs& a, hipStream_t str
 }
 
 int check_fused(const GemvArgs& a, bool pro, bool epi) {
-  if (pro && (!a.resid || !a.norm_w || !a.x_out || a.M > 16 || (a.K >> 3) > 64 * kNormVPL)) return O355_EUNSUPPORTED;
+  if (pro && (!a.resid || !a.norm_w || !a.x_out || a.M > 16 || (a.K & 511))) return O355_EUNSUPPORTED;
   if ((pro || epi) && (int64_t)(a.M + 1) * a.K * 2 > kXldsMaxBytes) return O355_EUNSUPPORTED;
   if (epi && ((a.N & 31) || a.M > 16)) return O355_EUNSUPPORTED;
   return O355_OK;
@@ -443,8 +458,10 @@ int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, 
   GEMV_WAVES(w4_gemv_kernel, 2, 1, 2, false, 0, 0, w, st, zt)
   GEMV_WAVES(w4_gemv_kernel, 4, 1, 2, false, 0, 0, w, st, zt)
   GEMV_WAVES(w4_gemv_kernel, 1, 1, 2, true, 1, 0, w, st, zt)
+  GEMV_WAVES(w4_gemv_kernel, 1, 1, 2, true, 4, 0, w, st, zt)
   GEMV_WAVES(w4_gemv_kernel, 1, 2, 2, true, 0, 1, w, st, zt)
   GEMV_WAVES(w4_gemv_kernel, 1, 2, 2, true, 1, 1, w, st, zt)
+  GEMV_WAVES(w4_gemv_kernel, 1, 2, 2, true, 4, 1, w, st, zt)
   return O355_EUNSUPPORTED;
 }
 
@@ -456,8 +473,10 @@ int b16_gemv_dispatch(const GemvArgs& a, const uint16_t* wt, bool pro, bool epi,
   GEMV_WAVES(b16_gemv_kernel, 2, 1, 4, false, 0, 0, w)
   GEMV_WAVES(b16_gemv_kernel, 4, 1, 4, false, 0, 0, w)
   GEMV_WAVES(b16_gemv_kernel, 1, 1, 8, true, 1, 0, w)
+  GEMV_WAVES(b16_gemv_kernel, 1, 1, 8, true, 4, 0, w)
   GEMV_WAVES(b16_gemv_kernel, 1, 2, 8, true, 0, 1, w)
   GEMV_WAVES(b16_gemv_kernel, 1, 2, 8, true, 1, 1, w)
+  GEMV_WAVES(b16_gemv_kernel, 1, 2, 8, true, 4, 1, w)
   return O355_EUNSUPPORTED;
 }
 

@@ -33,14 +33,14 @@ def dev():
 
 def small_cfg(kind: str) -> ModelConfig:
     if kind == "olmo2":  # OLMo-2 wiring: post-norm, RMS, QK-norm, rope theta 5e5, head_dim 128
-        return ModelConfig(d_model=256, n_heads=2, n_layers=4, mlp_hidden_size=1024, rope=True, alibi=False,
+        return ModelConfig(d_model=512, n_heads=4, n_layers=4, mlp_hidden_size=2048, rope=True, alibi=False,
                            include_bias=False, weight_tying=False, vocab_size=1000, embedding_size=1024,
                            max_sequence_length=512, layer_norm_type="rms", layer_norm_with_affine=True,
                            layer_norm_eps=1e-6, attention_layer_norm=True, norm_after=True, rope_theta=500000,
                            attention_dropout=0.0, residual_dropout=0.0, embedding_dropout=0.0)
     if kind == "olmo2-gqa":
         c = small_cfg("olmo2")
-        c.n_heads, c.n_kv_heads, c.d_model, c.mlp_hidden_size = 4, 2, 256, 768
+        c.n_heads, c.n_kv_heads, c.d_model, c.mlp_hidden_size = 8, 2, 512, 1536
         return c
     if kind == "ln":  # pre-norm, non-parametric LayerNorm, head_dim 32 (the fp32 configuration's wiring)
         return ModelConfig(d_model=128, n_heads=4, n_layers=3, mlp_ratio=8, rope=True, alibi=False, include_bias=False,

@@ -345,3 +345,45 @@ def test_attn_decode(dev, dtype, B, L, H, Hkv, hd):
         ref2 = om.attention(q, k, v, fb, dtype).transpose(1, 2).reshape(B, 1, H * hd)
         out2 = ops.attn_decode(qd, kc, vc, ws, B, H, Hkv, hd, L - 1, L, key_bias=bias.to(dev)).cpu()
         assert torch.allclose(out2.float(), ref2.float(), **tol)
+
+
+# ------------------------------------------------------------------------------------------------
+# decode-step fusions: x' = resid + rmsnorm(a) in the prologue, SwiGLU in the epilogue
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("quant", [True, False])
+@pytest.mark.parametrize("M", [1, 3, 8, 16])
+@pytest.mark.parametrize("N,K,pro,epi", [(768, 256, True, False), (1024, 256, True, True), (12288, 4096, True, False),
+                                         (22016, 4096, True, True), (22016, 4096, False, True), (16384, 2048, True, True)])
+def test_linear_fused(dev, quant, M, N, K, pro, epi):
+    say("linear_fused", quant, M, N, K, pro, epi)
+    ops = _ops()
+    gen = torch.Generator().manual_seed(M + N + K)
+    a = (torch.randn(M, K, generator=gen) * 2).to(torch.bfloat16)
+    resid = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    nw = (1 + 0.1 * torch.randn(K, generator=gen)).to(torch.bfloat16)
+    if quant:
+        qw, qz, sc = ow4.random_quantized(K, N, 128, seed=N + K)
+        Wf = ow4.dequantize(qw, qz, sc, 128).float()  # [K,N]
+        w = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    else:
+        wd = (torch.randn(N, K, generator=gen) * 0.02).to(torch.bfloat16)
+        Wf = wd.float().t()
+        w = ops.b16_repack(wd.to(dev))
+    x_ref = (resid + om.rms_norm(a, nw, 1e-6)) if pro else a
+    y_ref = (x_ref.float() @ Wf).to(torch.bfloat16)
+    if epi:
+        y_ref = om.swiglu(y_ref)
+    y, x_new = ops.linear_fused(a.to(dev), w, resid=resid.to(dev) if pro else None, norm_w=nw.to(dev) if pro else None,
+                                eps=1e-6, swiglu_out=epi)
+    y, x_new = y.cpu(), x_new.cpu()
+    assert y.shape == y_ref.shape
+    # x': same rounding points as the separate kernel (1 bf16 ulp where the fp32 sum of squares differs)
+    dx = (x_new.float() - x_ref.float()).abs()
+    assert (dx <= 2.0 ** (torch.floor(torch.log2(x_ref.float().abs().clamp_min(1e-30))) - 7)).all()
+    scale = y_ref.float().abs().max().item()
+    assert (y.float() - y_ref.float()).abs().max().item() <= 2 ** -6 * scale
+    # and equal to the unfused sequence of kernels up to the last bit of each rounding
+    x2 = ops.rmsnorm(a.to(dev), nw.to(dev), 1e-6, residual=resid.to(dev)) if pro else a.to(dev)
+    y2 = ops.w4_linear(x2, w) if quant else ops.b16_linear(x2, w)
+    y2 = (ops.swiglu(y2) if epi else y2).cpu()
+    assert (y.float() - y2.float()).abs().max().item() <= 2 ** -6 * scale
