@@ -149,6 +149,15 @@ int olmo355_attn_decode(const void* q, const void* kcache, const void* vcache, c
                         void* ws, int B, int H, int Hkv, int hd, int Lmax, int past_len,
                         const int32_t* past_len_dev, int n_keys_max, int bias_stride, int dtype, void* stream);
 
+/* olmo355_qknorm_rope_kvwrite (T == 1) and olmo355_attn_decode in one pass over the new token's
+ * fused projection qkv [B, (H+2*Hkv)*hd]: bf16, hd 64 or 128; O355_EUNSUPPORTED otherwise (the caller
+ * then issues the two separate calls).  Same workspace as olmo355_attn_decode. */
+int olmo355_attn_decode_fused(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
+                              const float* cos_tab, void* kcache, void* vcache, const float* key_bias, void* out,
+                              void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos, int past_len,
+                              const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps, int dtype,
+                              void* stream);
+
 /* ---- MLP activation: SwiGLU.forward (olmo/model.py:365-368) --------------------------------
  * x [rows, 2h]: first half "up", second half "gate"; out [rows, h] = silu(gate) * up. */
 int olmo355_swiglu(const void* x, void* out, int rows, int h, int dtype, void* stream);

@@ -145,7 +145,7 @@ __global__ __launch_bounds__(256) void qknorm_rope_vec_kernel(const uint16_t* __
                                                               const float* __restrict__ sin_t,
                                                               const float* __restrict__ cos_t, uint16_t* __restrict__ q_out,
                                                               uint16_t* __restrict__ kc, uint16_t* __restrict__ vc, int T,
-                                                              int H, int Hkv, int hd, int Lmax, int past_len,
+                                                              int H, int Hkv, int hd, int Lmax, int n_pos, int past_len,
                                                               const int32_t* __restrict__ past_dev, float eps) {
   constexpr int DT = O355_BF16;
   __shared__ float red[16];
@@ -153,6 +153,7 @@ __global__ __launch_bounds__(256) void qknorm_rope_vec_kernel(const uint16_t* __
   const int dq = H * hd, dk = Hkv * hd, half = hd >> 1, cph = hd >> 4;  // chunks per head
   const int64_t in_base = (int64_t)row * (dq + 2 * dk);
   const int pos = (past_dev ? *past_dev : past_len) + t;
+  if (pos >= Lmax || pos >= n_pos) return;  // a device-side position beyond the cache: write nothing
   const bool norm = (qw != nullptr);
   const int nq = H * cph, nk = Hkv * cph;
 
@@ -248,7 +249,7 @@ __global__ __launch_bounds__(256) void qknorm_rope_kernel(const void* __restrict
                                                           const void* __restrict__ kw, const float* __restrict__ sin_t,
                                                           const float* __restrict__ cos_t, void* __restrict__ q_out,
                                                           void* __restrict__ kc, void* __restrict__ vc, int T, int H,
-                                                          int Hkv, int hd, int Lmax, int past_len,
+                                                          int Hkv, int hd, int Lmax, int n_pos, int past_len,
                                                           const int32_t* __restrict__ past_dev, float eps) {
   __shared__ float red[16];
   const int row = blockIdx.x;  // b*T + t
@@ -257,6 +258,7 @@ __global__ __launch_bounds__(256) void qknorm_rope_kernel(const void* __restrict
   const int64_t in_base = (int64_t)row * (dq + 2 * dk);
   const int past = past_dev ? *past_dev : past_len;
   const int pos = past + t;
+  if (pos >= Lmax || pos >= n_pos) return;  // a device-side position beyond the cache: write nothing
   const bool norm = (qw != nullptr);
 
   float rq = 1.f, rk = 1.f;
@@ -475,7 +477,7 @@ extern "C" int olmo355_qknorm_rope_kvwrite(const void* qkv, const void* qw, cons
 #define QK_VEC(CPT)                                                                                                 \
   hipLaunchKernelGGL(qknorm_rope_vec_kernel<CPT>, dim3(B * T), dim3(256), 0, s, (const uint16_t*)qkv,              \
                      (const uint16_t*)qw, (const uint16_t*)kw, sin_tab, cos_tab, (uint16_t*)q_out, (uint16_t*)kcache, \
-                     (uint16_t*)vcache, T, H, Hkv, hd, Lmax, past_len, past_len_dev, eps)
+                     (uint16_t*)vcache, T, H, Hkv, hd, Lmax, n_pos, past_len, past_len_dev, eps)
     if (chunks <= 256) QK_VEC(1);
     else if (chunks <= 512) QK_VEC(2);
     else QK_VEC(4);
@@ -483,7 +485,7 @@ extern "C" int olmo355_qknorm_rope_kvwrite(const void* qkv, const void* qw, cons
     O355_CHECK_LAUNCH();
   }
   DT_SWITCH(dtype, hipLaunchKernelGGL(qknorm_rope_kernel<DT>, dim3(B * T), dim3(256), 0, s, qkv, qw, kw, sin_tab,
-                                      cos_tab, q_out, kcache, vcache, T, H, Hkv, hd, Lmax, past_len, past_len_dev,
+                                      cos_tab, q_out, kcache, vcache, T, H, Hkv, hd, Lmax, n_pos, past_len, past_len_dev,
                                       eps));
   O355_CHECK_LAUNCH();
 }

@@ -308,9 +308,16 @@ class OLMo(nn.Module):
         sin, cos = self._rope
         qw = blk.q_norm.weight.data if blk.q_norm is not None else None
         kw = blk.k_norm.weight.data if blk.k_norm is not None else None
+        decode = T == 1 and (graph_pos is not None or past_len > 0)
+        if decode:
+            att = ops.attn_decode_fused(qkv, qw, kw, sin, cos, kc, vc, self._decode_ws(B, n_keys_max), B, H, Hkv, hd,
+                                        past_len, n_keys_max, c.layer_norm_eps, key_bias=key_bias,
+                                        past_len_dev=graph_pos)
+            if att is not None:
+                return att
         q = ops.qknorm_rope_kvwrite(qkv, qw, kw, sin, cos, kc, vc, B, T, H, Hkv, hd, past_len, c.layer_norm_eps,
                                     past_len_dev=graph_pos)
-        if T == 1 and (graph_pos is not None or past_len > 0):
+        if decode:
             return ops.attn_decode(q, kc, vc, self._decode_ws(B, n_keys_max), B, H, Hkv, hd, past_len, n_keys_max,
                                    key_bias=key_bias, past_len_dev=graph_pos)
         return ops.attn_prefill(q, kc, vc, B, T, H, Hkv, hd, past_len, key_bias=key_bias)

@@ -362,6 +362,31 @@ def attn_decode(q, kcache, vcache, ws, B: int, H: int, Hkv: int, hd: int, past_l
     return out
 
 
+def attn_decode_fused(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, ws, B: int, H: int, Hkv: int, hd: int,
+                      past_len: int, n_keys_max: int, eps: float, key_bias: Optional[torch.Tensor] = None,
+                      past_len_dev: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """One new token per sequence: QK-norm, rotary, cache append and attention in one pass.  Returns
+    ``None`` when the fused kernel does not cover the shape (use the separate calls then)."""
+    _dev(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, ws, key_bias, past_len_dev)
+    if qkv.dtype != torch.bfloat16 or hd not in (64, 128):
+        return None
+    if qkv.numel() != B * (H + 2 * Hkv) * hd or kcache.shape != vcache.shape or kcache.shape[1] != Hkv or kcache.shape[3] != hd:
+        raise ValueError("qkv / cache shape mismatch")
+    Lmax, n_pos = kcache.shape[2], sin_tab.shape[0]
+    need = int(lib().olmo355_attn_decode_workspace_bytes(B, H, hd, n_keys_max))
+    if ws.numel() * ws.element_size() < need:
+        raise ValueError("attention workspace too small")
+    out = torch.empty(B, 1, H * hd, dtype=qkv.dtype, device=qkv.device)
+    st = lib().olmo355_attn_decode_fused(_p(qkv), _p(q_weight), _p(k_weight), _p(sin_tab), _p(cos_tab), _p(kcache),
+                                         _p(vcache), _p(key_bias), _p(out), _p(ws), B, H, Hkv, hd, Lmax, n_pos, past_len,
+                                         _p(past_len_dev), n_keys_max, key_bias.shape[1] if key_bias is not None else 0,
+                                         float(eps), _dt(qkv), _stream())
+    if st == 2:
+        return None
+    check("olmo355_attn_decode_fused", st)
+    return out
+
+
 def rope_tables(head_dim: int, theta: float, n_pos: int, device) -> Tuple[torch.Tensor, torch.Tensor]:
     """fp32 sin / cos tables ``[n_pos, hd]`` built with the reference's expression
     (``olmo/model.py:285-296``) on the host so that device sin/cos differences cannot enter."""

@@ -387,3 +387,62 @@ def test_linear_fused(dev, quant, M, N, K, pro, epi):
     y2 = ops.w4_linear(x2, w) if quant else ops.b16_linear(x2, w)
     y2 = (ops.swiglu(y2) if epi else y2).cpu()
     assert (y.float() - y2.float()).abs().max().item() <= 2 ** -6 * scale
+
+
+@pytest.mark.parametrize("qknorm,B,past,H,Hkv,hd", [(True, 1, 2048, 32, 32, 128), (True, 3, 700, 4, 2, 128),
+                                                     (False, 2, 0, 2, 2, 64), (True, 2, 127, 8, 8, 64),
+                                                     (True, 2, 128, 4, 4, 128)])
+def test_attn_decode_fused(dev, qknorm, B, past, H, Hkv, hd):
+    """QK-norm + rotary + cache append + attention in one pass == the two separate kernels == the oracle."""
+    say("attn_decode_fused", qknorm, B, past, H, Hkv, hd)
+    ops = _ops()
+    dtype, theta, eps = torch.bfloat16, 500000.0, 1e-6
+    Lmax = past + 200
+    gen = torch.Generator().manual_seed(past + hd + H)
+    qkv = torch.randn(B, (H + 2 * Hkv) * hd, generator=gen).to(dtype)
+    qw = (1 + 0.1 * torch.randn(H * hd, generator=gen)).to(dtype) if qknorm else None
+    kw = (1 + 0.1 * torch.randn(Hkv * hd, generator=gen)).to(dtype) if qknorm else None
+    k_old = torch.randn(B, Hkv, past, hd, generator=gen).to(dtype)
+    v_old = torch.randn(B, Hkv, past, hd, generator=gen).to(dtype)
+    qr, kr, vr = _rope_ref(qkv, qw, kw, B, 1, H, Hkv, hd, past, theta, eps, Lmax)
+    ref = om.attention(qr, torch.cat((k_old, kr), 2), torch.cat((v_old, vr), 2), None, dtype)
+    ref = ref.transpose(1, 2).reshape(B, 1, H * hd)
+    sin, cos = ops.rope_tables(hd, theta, Lmax, dev)
+
+    def fresh():
+        kc = torch.full((B, Hkv, Lmax, hd), float("nan"), dtype=dtype)  # unwritten rows must never matter
+        vc = torch.full((B, Hkv, Lmax, hd), float("nan"), dtype=dtype)
+        kc[:, :, :past], vc[:, :, :past] = k_old, v_old
+        return kc.to(dev), vc.to(dev)
+
+    d = lambda t: None if t is None else t.to(dev)
+    ws = ops.attn_decode_workspace(B, H, hd, Lmax, dev)
+    kc, vc = fresh()
+    out = ops.attn_decode_fused(qkv.to(dev), d(qw), d(kw), sin, cos, kc, vc, ws, B, H, Hkv, hd, past, past + 1, eps)
+    assert out is not None
+    assert torch.allclose(out.cpu().float(), ref.float(), rtol=2 ** -7, atol=2 ** -7)
+    assert torch.allclose(kc[:, :, past].cpu().float(), kr[:, :, 0].float(), rtol=2 ** -7, atol=2 ** -7)
+    assert torch.equal(vc[:, :, past].cpu(), vr[:, :, 0])
+    assert torch.isnan(kc[:, :, past + 1:].float()).all()  # nothing else written
+    # same rounding points as the separate kernels; only the fp32 summation order of the softmax differs
+    kc2, vc2 = fresh()
+    q2 = ops.qknorm_rope_kvwrite(qkv.to(dev), d(qw), d(kw), sin, cos, kc2, vc2, B, 1, H, Hkv, hd, past, eps)
+    out2 = ops.attn_decode(q2, kc2, vc2, ws, B, H, Hkv, hd, past, past + 1)
+    assert torch.equal(kc2[:, :, past], kc[:, :, past])
+    assert torch.allclose(out2.float(), out.float(), rtol=2 ** -8, atol=2 ** -10)
+    # position from device memory, grid sized for the whole cache, padding bias
+    kc3, vc3 = fresh()
+    bias = torch.zeros(B, Lmax)
+    if past > 8:
+        bias[0, :5] = torch.finfo(torch.float32).min
+    pl = torch.tensor([past], dtype=torch.int32, device=dev)
+    out3 = ops.attn_decode_fused(qkv.to(dev), d(qw), d(kw), sin, cos, kc3, vc3, ws, B, H, Hkv, hd, 0, Lmax, eps,
+                                 key_bias=bias.to(dev), past_len_dev=pl)
+    if past > 8:
+        fb = bias[:, None, None, :past + 1].to(dtype)
+        fb = fb.masked_fill(fb == float("-inf"), torch.finfo(dtype).min)
+        ref3 = om.attention(qr, torch.cat((k_old, kr), 2), torch.cat((v_old, vr), 2), fb, dtype)
+        ref3 = ref3.transpose(1, 2).reshape(B, 1, H * hd)
+        assert torch.allclose(out3.cpu().float(), ref3.float(), rtol=2 ** -7, atol=2 ** -7)
+    else:
+        assert torch.allclose(out3.float(), out.float(), rtol=2 ** -8, atol=2 ** -10)
