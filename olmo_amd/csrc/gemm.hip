@@ -52,78 +52,112 @@ __device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& 
   }
 }
 
-template <int WMT, int WNT, bool W4>  // 32x32 MFMA tiles per wave along M and N
-__global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wt,
-                                                   const uint16_t* __restrict__ st, const uint8_t* __restrict__ zt,
-                                                   uint16_t* __restrict__ y, int M, int N, int K, int tiles_m,
-                                                   int tiles_n) {
-  constexpr int BM = 64 * WMT, BN = 64 * WNT;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// buffer resource over [base, base + bytes): loads past the end return zero, which is what pads
+// ragged M and N edges
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int64_t bytes) {
+  const int64_t cap = 0xffffffffll;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)(uint32_t)(bytes < cap ? (bytes < 0 ? 0 : bytes) : cap),
+                                           0x00020000);
+}
+
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4>  // wave grid, 32x32 MFMA tiles per wave
+__device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wt,
+                                          const uint16_t* __restrict__ st, const uint8_t* __restrict__ zt,
+                                          uint16_t* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n) {
+  constexpr int NW = WAVES_M * WAVES_N, NT = 64 * NW;
+  constexpr int BM = 32 * WMT * WAVES_M, BN = 32 * WNT * WAVES_N;
   constexpr int A_FRAGS = (BM / 32) * KSTEPS, B_FRAGS = (BN / 32) * KSTEPS;  // 1 KiB fragments per stage
-  constexpr int A_LD = (BM * 8) / 256;           // 16-byte activation pieces per thread per stage
-  constexpr int B_ITEMS = (BN / 16) * 64 / 256;  // (16-column weight tile, lane) items per thread per stage
+  constexpr int A_PW = A_FRAGS / NW;                 // activation fragments each wave brings in per stage
+  constexpr int B_PW = B_FRAGS / NW;                 // dense weights: same
+  constexpr int B_ITEMS = (BN / 16) * 64 / NT;       // int4: (16-column tile, lane) items per thread per stage
+  static_assert(A_FRAGS % NW == 0 && B_FRAGS % NW == 0 && ((BN / 16) * 64) % NT == 0, "tile / wave split");
   extern __shared__ __align__(16) unsigned char smem[];
   u32x4* lds_a = reinterpret_cast<u32x4*>(smem);  // [2][A_FRAGS][64]
   u32x4* lds_b = lds_a + 2 * A_FRAGS * 64;        // [2][B_FRAGS][64]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   int tile_m, tile_n;
   tile_of(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
   const int m0 = tile_m * BM, nt0 = tile_n * (BN / 16);
   const int ntiles = N >> 4;
   const int G = K >> 7, KS = K >> 5;
   const int stages = K / BK;
+  const int row32 = lane & 31, kh = lane >> 5;
 
-  // ---- global -> register staging -----------------------------------------------------------
-  u32x4 ra[A_LD];
-  u32x2 rbw[B_ITEMS];  // int4: two tiled words (32-row steps 2h, 2h+1 of the group)
-  u32x4 rbd[W4 ? 1 : B_ITEMS][2];
-  float rs[B_ITEMS], rc[B_ITEMS];
-
-  // rows past M are clamped to the last row (their products are computed and never stored): the
-  // loop body stays free of branches, which is what lets the compiler interleave it
-  auto fetch_a = [&](int s, int i) {
-    const int row = (tid >> 3) + 32 * i, c = tid & 7;
-    const int gm = min(m0 + row, M - 1);
-    ra[i] = *reinterpret_cast<const u32x4*>(x + (int64_t)gm * K + s * BK + 8 * c);
+  // ---- activations: memory -> LDS directly, one 1 KiB fragment per instruction -----------------
+  // fragment (row tile rt, k-step ks): lane (row32, kh) holds x[m0 + 32 rt + row32][k0 + 16 ks + 8 kh ..+8]
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(x + (int64_t)m0 * K, (int64_t)(M - m0) * K * 2);
+  int a_voff[A_PW];
+#pragma unroll
+  for (int i = 0; i < A_PW; ++i) {
+    const int f = wave * A_PW + i, rt = f / KSTEPS, ks = f % KSTEPS;
+    a_voff[i] = ((rt * 32 + row32) * K + ks * 16 + kh * 8) * 2;
+  }
+  auto load_a = [&](int s, int buf) {
+#pragma unroll
+    for (int i = 0; i < A_PW; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(smem + ((buf * A_FRAGS + wave * A_PW + i) << 10)), 16, a_voff[i],
+                                               s * (BK * 2), 0, 0);
   };
-  auto fetch_b = [&](int s, int i) {
-    const int k0 = s * BK;
-    const int nt = min(nt0 + (tid >> 6) + 4 * i, ntiles - 1);
-    if constexpr (W4) {
-      const int g = k0 >> 7, h = (k0 >> 6) & 1;
-      const int64_t tile = (int64_t)nt * G + g;
-      rbw[i] = *reinterpret_cast<const u32x2*>(wt + (tile * 64 + lane) * 4 + 2 * h);
-      const int col = lane & 15;
-      const float sc = (float)__builtin_bit_cast(_Float16, st[tile * 16 + col]);
-      const int z = 129 + (int)((zt[tile * 8 + (col >> 1)] >> (4 * (col & 1))) & 15u);
-      rs[i] = sc;
-      rc[i] = -(float)z * sc;
-    } else {
-      const u32x4* src = reinterpret_cast<const u32x4*>(wt) + ((int64_t)nt * KS + (k0 >> 5)) * 64 + lane;
-      rbd[i][0] = src[0];
-      rbd[i][1] = src[64];
+
+  // ---- weights ---------------------------------------------------------------------------------
+  // int4: registers, dequantised on the way into LDS.  dense: memory -> LDS directly.
+  const __amdgpu_buffer_rsrc_t rw =
+      W4 ? make_rsrc(wt + (int64_t)nt0 * G * 256, (int64_t)(ntiles - nt0) * G * 1024)
+         : make_rsrc(wt + (int64_t)nt0 * KS * 256, (int64_t)(ntiles - nt0) * KS * 1024);
+  const __amdgpu_buffer_rsrc_t rs_ = make_rsrc(W4 ? st + (int64_t)nt0 * G * 16 : x, W4 ? (int64_t)(ntiles - nt0) * G * 32 : 0);
+  const __amdgpu_buffer_rsrc_t rz_ = make_rsrc(W4 ? zt + (int64_t)nt0 * G * 8 : (const uint8_t*)x, W4 ? (int64_t)(ntiles - nt0) * G * 8 : 0);
+  constexpr int NBI = W4 ? B_ITEMS : 1;
+  u32x2 rbw[2][NBI];
+  uint32_t rsc[2][NBI], rzb[2][NBI];
+  int bw_voff[NBI], bs_voff[NBI], bz_voff[NBI];
+  int bd_voff[W4 ? 1 : B_PW];
+  if constexpr (W4) {
+#pragma unroll
+    for (int i = 0; i < B_ITEMS; ++i) {
+      const int ntl = (tid >> 6) + NW * i, col = lane & 15;
+      bw_voff[i] = (ntl * G * 64 + lane) * 16;
+      bs_voff[i] = (ntl * G * 16 + col) * 2;
+      bz_voff[i] = ntl * G * 8 + (col >> 1);
+    }
+  } else {
+    // fragment (column tile ct of 32, k-step ks): lane (n32, kh) <- tiled piece
+    // [2 ct + n32/16][k32 = ks/2][(n32 & 15) + 16 (2 (ks & 1) + kh)]
+#pragma unroll
+    for (int i = 0; i < B_PW; ++i) {
+      const int f = wave * B_PW + i, ct = f / KSTEPS, ks = f % KSTEPS;
+      bd_voff[i] = (((2 * ct + (row32 >> 4)) * KS + (ks >> 1)) * 64 + (row32 & 15) + 16 * (2 * (ks & 1) + kh)) * 16;
+    }
+  }
+  auto fetch_b = [&](int s, int set) {  // int4 only
+    const int g = s >> 1, h = s & 1;
+#pragma unroll
+    for (int i = 0; i < NBI; ++i) {
+      rbw[set][i] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rw, bw_voff[i], g * 1024 + 8 * h, 0));
+      rsc[set][i] = __builtin_amdgcn_raw_buffer_load_b16(rs_, bs_voff[i], g * 32, 0);
+      rzb[set][i] = __builtin_amdgcn_raw_buffer_load_b8(rz_, bz_voff[i], g * 8, 0);
     }
   };
-  // piece (row, chunk c of 8 columns) -> fragment (row/32, c/2), slot (c&1)*32 + (row%32 ^ 2c mod 16)
-  auto stash_a = [&](u32x4* a, int i) {
-    const int row = (tid >> 3) + 32 * i, c = tid & 7;
-    a[((row >> 5) * KSTEPS + (c >> 1)) * 64 + (c & 1) * 32 + ((row & 31) ^ ((2 * c) & 15))] = ra[i];
+  auto load_b_dense = [&](int s, int buf) {
+#pragma unroll
+    for (int i = 0; i < (W4 ? 0 : B_PW); ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(smem + ((2 * A_FRAGS + buf * B_FRAGS + wave * B_PW + i) << 10)), 16,
+                                               bd_voff[i], s * 2048, 0, 0);
   };
-  // weight piece of lane l (column l&15 of its 16-column tile, rows 8*(l>>4).. of 32-row step j):
+  // int4 piece of lane l (column l&15 of its 16-column tile, rows 8*(l>>4).. of 32-row step j):
   // fragment (tile/2, 2j + (l>>5)), slot ((l>>4)&1)*32 + (tile&1)*16 + (l&15)
-  auto stash_b = [&](u32x4* b, int i) {
-    const int ntl = (tid >> 6) + 4 * i;
+  auto stash_b_word = [&](u32x4* b, int set, int i, int wsel) {
+    const int ntl = (tid >> 6) + NW * i;
     const int kq = lane >> 4;
     const int slot = (kq & 1) * 32 + (ntl & 1) * 16 + (lane & 15);
-    const int f0 = (ntl >> 1) * KSTEPS + (kq >> 1);
-    if constexpr (W4) {
-      b[(f0 + 0) * 64 + slot] = dequant_word_bf16(rbw[i].x, rs[i], rc[i]);
-      b[(f0 + 2) * 64 + slot] = dequant_word_bf16(rbw[i].y, rs[i], rc[i]);
-    } else {
-      b[(f0 + 0) * 64 + slot] = rbd[i][0];
-      b[(f0 + 2) * 64 + slot] = rbd[i][1];
-    }
+    const int f0 = (ntl >> 1) * KSTEPS + (kq >> 1) + 2 * wsel;
+    const float sc = (float)__builtin_bit_cast(_Float16, (uint16_t)rsc[set][i]);
+    const int z = 129 + (int)((rzb[set][i] >> (4 * (lane & 1))) & 15u);
+    b[f0 * 64 + slot] = dequant_word_bf16(wsel ? rbw[set][i].y : rbw[set][i].x, sc, -(float)z * sc);
   };
 
   f32x16 acc[WMT][WNT];
@@ -134,53 +168,68 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+  bf16x8 fa[2][WMT], fb[2][WNT];
+  auto load_frags = [&](int set, const u32x4* a, const u32x4* b, int ks) {
 #pragma unroll
-  for (int i = 0; i < A_LD; ++i) fetch_a(0, i);
+    for (int i = 0; i < WMT; ++i) fa[set][i] = __builtin_bit_cast(bf16x8, a[((wm * WMT + i) * KSTEPS + ks) * 64 + lane]);
 #pragma unroll
-  for (int i = 0; i < B_ITEMS; ++i) fetch_b(0, i);
+    for (int j = 0; j < WNT; ++j) fb[set][j] = __builtin_bit_cast(bf16x8, b[((wn * WNT + j) * KSTEPS + ks) * 64 + lane]);
+  };
+  auto mfmas = [&](int set) {
 #pragma unroll
-  for (int i = 0; i < A_LD; ++i) stash_a(lds_a, i);
+    for (int i = 0; i < WMT; ++i)
 #pragma unroll
-  for (int i = 0; i < B_ITEMS; ++i) stash_b(lds_b, i);
-#pragma unroll
-  for (int i = 0; i < A_LD; ++i) fetch_a(min(1, stages - 1), i);
-#pragma unroll
-  for (int i = 0; i < B_ITEMS; ++i) fetch_b(min(1, stages - 1), i);
-  lds_barrier();
+      for (int j = 0; j < WNT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
+  };
+  // everything this wave sent towards LDS (through registers or directly) has landed, then meet
+  auto stage_barrier = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+  };
 
-  const int row32 = lane & 31, kh = lane >> 5;
+  // ---- prologue: stage 0 into buffer 0, stage 1's int4 words into registers --------------------
+  load_a(0, 0);
+  if constexpr (W4) {
+    fetch_b(0, 0);
+#pragma unroll
+    for (int i = 0; i < 2 * B_ITEMS; ++i) stash_b_word(lds_b, 0, i >> 1, i & 1);
+    fetch_b(min(1, stages - 1), 1);
+  } else {
+    load_b_dense(0, 0);
+  }
+  stage_barrier();
+  load_frags(0, lds_a, lds_b, 0);
+
   for (int s = 0; s < stages; ++s) {
     const int buf = s & 1;
     const u32x4* a = lds_a + buf * A_FRAGS * 64;
     const u32x4* b = lds_b + buf * B_FRAGS * 64;
     u32x4* an = lds_a + (buf ^ 1) * A_FRAGS * 64;
     u32x4* bn = lds_b + (buf ^ 1) * B_FRAGS * 64;
-    // the last stage stashes into a buffer nobody reads again and the last two re-fetch the final
-    // stage: redundant, but unconditional
-    const int sf = min(s + 2, stages - 1);
+    // the last iterations re-fetch the final stage into buffers nobody reads again: redundant, but
+    // it keeps the loop body free of branches
+    const int s1 = min(s + 1, stages - 1), s2 = min(s + 2, stages - 1);
+    load_a(s1, buf ^ 1);
+    if constexpr (!W4) load_b_dense(s1, buf ^ 1);
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      bf16x8 af[WMT], bfr[WNT];
-      const int aslot = kh * 32 + (row32 ^ ((2 * (2 * ks + kh)) & 15));
+    for (int ks = 0; ks < 3; ++ks) {
+      load_frags((ks + 1) & 1, a, b, ks + 1);
+      mfmas(ks & 1);
+      if constexpr (W4) {
 #pragma unroll
-      for (int i = 0; i < WMT; ++i) af[i] = __builtin_bit_cast(bf16x8, a[((wm * WMT + i) * KSTEPS + ks) * 64 + aslot]);
-#pragma unroll
-      for (int j = 0; j < WNT; ++j) bfr[j] = __builtin_bit_cast(bf16x8, b[((wn * WNT + j) * KSTEPS + ks) * 64 + lane]);
-#pragma unroll
-      for (int i = 0; i < WMT; ++i)
-#pragma unroll
-        for (int j = 0; j < WNT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
-      // a quarter of the staging work per k-step, issued behind this step's MFMAs
-#pragma unroll
-      for (int i = ks; i < A_LD; i += KSTEPS) stash_a(an, i);
-#pragma unroll
-      for (int i = ks; i < B_ITEMS; i += KSTEPS) stash_b(bn, i);
-#pragma unroll
-      for (int i = ks; i < A_LD; i += KSTEPS) fetch_a(sf, i);
-#pragma unroll
-      for (int i = ks; i < B_ITEMS; i += KSTEPS) fetch_b(sf, i);
+        for (int i = 0; i < 2 * B_ITEMS; ++i)
+          if (i * 3 / (2 * B_ITEMS) == ks) stash_b_word(bn, 1, i >> 1, i & 1);
+      }
     }
-    lds_barrier();  // orders LDS only: the global loads of stage s+2 stay in flight across it
+    if constexpr (W4) {
+      // register set 1 (stage s+1) is in LDS now; set 0 <- stage s+2, and rotate
+#pragma unroll
+      for (int i = 0; i < NBI; ++i) rbw[0][i] = rbw[1][i], rsc[0][i] = rsc[1][i], rzb[0][i] = rzb[1][i];
+    }
+    stage_barrier();
+    if constexpr (W4) fetch_b(s2, 1);
+    load_frags(0, an, bn, 0);
+    mfmas(1);
   }
 
   // ---- epilogue: D[m = 8*(r/4) + 4*(lane>>5) + r%4][n = lane&31] of each 32x32 tile ---------------------
@@ -198,32 +247,37 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint16_t* __restrict__ 
     }
 }
 
-template <int WMT, int WNT, bool W4>
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const uint16_t* __restrict__ x,
+                                                                     const uint32_t* __restrict__ wt,
+                                                                     const uint16_t* __restrict__ st,
+                                                                     const uint8_t* __restrict__ zt,
+                                                                     uint16_t* __restrict__ y, int M, int N, int K,
+                                                                     int tiles_m, int tiles_n) {
+  gemm_body<WAVES_M, WAVES_N, WMT, WNT, W4>(x, wt, st, zt, y, M, N, K, tiles_m, tiles_n);
+}
+
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4>
 int launch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M, int N,
                 int K, hipStream_t stream) {
-  constexpr int BM = 64 * WMT, BN = 64 * WNT;
+  constexpr int BM = 32 * WMT * WAVES_M, BN = 32 * WNT * WAVES_N;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const size_t lds = (size_t)2 * ((BM / 32) + (BN / 32)) * KSTEPS * 64 * 16;
-  auto kern = gemm_kernel<WMT, WNT, W4>;
+  auto kern = gemm_kernel<WAVES_M, WAVES_N, WMT, WNT, W4>;
   if (lds > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
         hipSuccess)
       return O355_ELAUNCH;
   }
-  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), lds, stream, x, wt, st, zt, y, M, N, K,
-                     tiles_m, tiles_n);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(64 * WAVES_M * WAVES_N), lds, stream, x, wt, st, zt,
+                     y, M, N, K, tiles_m, tiles_n);
   O355_CHECK_LAUNCH();
 }
 
 template <bool W4>
 int dispatch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M,
                   int N, int K, hipStream_t stream) {
-  // Big tiles when they still give at least one workgroup per CU; otherwise smaller ones.
-  const int64_t big = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-  if (big >= 256) return launch_gemm<4, 4, W4>(x, wt, st, zt, y, M, N, K, stream);
-  const int64_t mid = (int64_t)((M + 255) / 256) * ((N + 127) / 128);
-  if (mid >= 256) return launch_gemm<4, 2, W4>(x, wt, st, zt, y, M, N, K, stream);
-  return launch_gemm<2, 2, W4>(x, wt, st, zt, y, M, N, K, stream);
+  return launch_gemm<2, 4, 4, 2, W4>(x, wt, st, zt, y, M, N, K, stream);
 }
 
 }  // namespace
