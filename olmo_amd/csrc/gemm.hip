@@ -16,6 +16,7 @@
 //
 // The int4 operand is W = bf16(scale * (q - zero)) (fp32 product, one rounding).
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
@@ -68,14 +69,14 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
                                           uint16_t* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n) {
   constexpr int NW = WAVES_M * WAVES_N, NT = 64 * NW;
   constexpr int BM = 32 * WMT * WAVES_M, BN = 32 * WNT * WAVES_N;
-  constexpr int A_FRAGS = (BM / 32) * KSTEPS, B_FRAGS = (BN / 32) * KSTEPS;  // 1 KiB fragments per stage
-  constexpr int A_PW = A_FRAGS / NW;                 // activation fragments each wave brings in per stage
-  constexpr int B_PW = B_FRAGS / NW;                 // dense weights: same
-  constexpr int B_ITEMS = (BN / 16) * 64 / NT;       // int4: (16-column tile, lane) items per thread per stage
-  static_assert(A_FRAGS % NW == 0 && B_FRAGS % NW == 0 && ((BN / 16) * 64) % NT == 0, "tile / wave split");
+  constexpr int A_BLK = BM / 8;        // 1 KiB blocks per stage: activations, 8 rows x 128 bytes each
+  constexpr int B_BLK = BN / 8;        // weights: 32x16 bf16 pieces (either layout)
+  constexpr int A_PW = A_BLK / NW, B_PW = B_BLK / NW;
+  constexpr int B_ITEMS = (BN / 16) * 64 / NT;  // int4: (16-column tile, lane) items per thread per group of 128 rows
+  static_assert(A_BLK % NW == 0 && B_BLK % NW == 0 && ((BN / 16) * 64) % NT == 0, "tile / wave split");
   extern __shared__ __align__(16) unsigned char smem[];
-  u32x4* lds_a = reinterpret_cast<u32x4*>(smem);  // [2][A_FRAGS][64]
-  u32x4* lds_b = lds_a + 2 * A_FRAGS * 64;        // [2][B_FRAGS][64]
+  u32x4* lds_a = reinterpret_cast<u32x4*>(smem);  // [2][A_BLK][64]
+  u32x4* lds_b = lds_a + 2 * A_BLK * 64;          // [2][B_BLK][64]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -88,77 +89,92 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   const int stages = K / BK;
   const int row32 = lane & 31, kh = lane >> 5;
 
-  // ---- activations: memory -> LDS directly, one 1 KiB fragment per instruction -----------------
-  // fragment (row tile rt, k-step ks): lane (row32, kh) holds x[m0 + 32 rt + row32][k0 + 16 ks + 8 kh ..+8]
+  // ---- activations: memory -> LDS directly ------------------------------------------------------
+  // One instruction moves 8 rows x 128 bytes (the 64 k of a stage): 8 consecutive lanes cover one
+  // row's cache line.  LDS keeps the rows 128 bytes apart with the 16-byte chunks of row r stored at
+  // position chunk ^ ((r >> 1) & 7), which makes the MFMA operand reads (32 rows, one chunk) hit
+  // every bank once; the swizzle is applied on the memory side because the LDS side of these loads
+  // is lane-linear.
   const __amdgpu_buffer_rsrc_t rx = make_rsrc(x + (int64_t)m0 * K, (int64_t)(M - m0) * K * 2);
   int a_voff[A_PW];
 #pragma unroll
   for (int i = 0; i < A_PW; ++i) {
-    const int f = wave * A_PW + i, rt = f / KSTEPS, ks = f % KSTEPS;
-    a_voff[i] = ((rt * 32 + row32) * K + ks * 16 + kh * 8) * 2;
+    const int row = 8 * (wave * A_PW + i) + (lane >> 3);
+    const int c = (lane & 7) ^ ((row >> 1) & 7);
+    a_voff[i] = (row * K + 8 * c) * 2;
   }
   auto load_a = [&](int s, int buf) {
 #pragma unroll
     for (int i = 0; i < A_PW; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(smem + ((buf * A_FRAGS + wave * A_PW + i) << 10)), 16, a_voff[i],
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(smem + ((buf * A_BLK + wave * A_PW + i) << 10)), 16, a_voff[i],
                                                s * (BK * 2), 0, 0);
   };
+  // operand read: lane (row32, kh), row tile rt, k-step ks -> 16-byte slot
+  const int a_swz = (row32 >> 1) & 7;
+  int a_rd[KSTEPS];
+#pragma unroll
+  for (int ks = 0; ks < KSTEPS; ++ks) a_rd[ks] = row32 * 8 + ((2 * ks + kh) ^ a_swz);
 
   // ---- weights ---------------------------------------------------------------------------------
-  // int4: registers, dequantised on the way into LDS.  dense: memory -> LDS directly.
   const __amdgpu_buffer_rsrc_t rw =
       W4 ? make_rsrc(wt + (int64_t)nt0 * G * 256, (int64_t)(ntiles - nt0) * G * 1024)
          : make_rsrc(wt + (int64_t)nt0 * KS * 256, (int64_t)(ntiles - nt0) * KS * 1024);
   const __amdgpu_buffer_rsrc_t rs_ = make_rsrc(W4 ? st + (int64_t)nt0 * G * 16 : x, W4 ? (int64_t)(ntiles - nt0) * G * 32 : 0);
   const __amdgpu_buffer_rsrc_t rz_ = make_rsrc(W4 ? zt + (int64_t)nt0 * G * 8 : (const uint8_t*)x, W4 ? (int64_t)(ntiles - nt0) * G * 8 : 0);
+  // int4: one 16-byte piece (4 tiled words = the lane's share of a 128-row group), scale and zero per
+  // item, fetched a group ahead into registers and dequantised on the way into LDS, fragment-major:
+  // piece of lane l (column l&15 of its 16-column tile, rows 8*(l>>4).. of 32-row step j) goes to
+  // fragment (tile/2, k-step 2j + (l>>5)), slot ((l>>4)&1)*32 + (tile&1)*16 + (l&15).
   constexpr int NBI = W4 ? B_ITEMS : 1;
-  u32x2 rbw[2][NBI];
-  uint32_t rsc[2][NBI], rzb[2][NBI];
+  u32x4 rbw[2][NBI];
+  float rsc[2][NBI], rcc[2][NBI];
   int bw_voff[NBI], bs_voff[NBI], bz_voff[NBI];
-  int bd_voff[W4 ? 1 : B_PW];
   if constexpr (W4) {
 #pragma unroll
     for (int i = 0; i < B_ITEMS; ++i) {
-      const int ntl = (tid >> 6) + NW * i, col = lane & 15;
+      const int ntl = wave + NW * i, col = lane & 15;
       bw_voff[i] = (ntl * G * 64 + lane) * 16;
       bs_voff[i] = (ntl * G * 16 + col) * 2;
       bz_voff[i] = ntl * G * 8 + (col >> 1);
     }
-  } else {
-    // fragment (column tile ct of 32, k-step ks): lane (n32, kh) <- tiled piece
-    // [2 ct + n32/16][k32 = ks/2][(n32 & 15) + 16 (2 (ks & 1) + kh)]
-#pragma unroll
-    for (int i = 0; i < B_PW; ++i) {
-      const int f = wave * B_PW + i, ct = f / KSTEPS, ks = f % KSTEPS;
-      bd_voff[i] = (((2 * ct + (row32 >> 4)) * KS + (ks >> 1)) * 64 + (row32 & 15) + 16 * (2 * (ks & 1) + kh)) * 16;
-    }
   }
-  auto fetch_b = [&](int s, int set) {  // int4 only
-    const int g = s >> 1, h = s & 1;
+  auto fetch_b = [&](int g, int set) {
 #pragma unroll
     for (int i = 0; i < NBI; ++i) {
-      rbw[set][i] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rw, bw_voff[i], g * 1024 + 8 * h, 0));
-      rsc[set][i] = __builtin_amdgcn_raw_buffer_load_b16(rs_, bs_voff[i], g * 32, 0);
-      rzb[set][i] = __builtin_amdgcn_raw_buffer_load_b8(rz_, bz_voff[i], g * 8, 0);
+      rbw[set][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, bw_voff[i], g * 1024, 0));
+      const uint32_t sb = __builtin_amdgcn_raw_buffer_load_b16(rs_, bs_voff[i], g * 32, 0);
+      const uint32_t zb = __builtin_amdgcn_raw_buffer_load_b8(rz_, bz_voff[i], g * 8, 0);
+      const float sc = (float)__builtin_bit_cast(_Float16, (uint16_t)sb);
+      rsc[set][i] = sc;
+      rcc[set][i] = -(float)(129 + (int)((zb >> (4 * (lane & 1))) & 15u)) * sc;
     }
   };
+  auto stash_b_word = [&](int buf, int set, int i, int j) {  // word j (32-row step j of the group) of item i
+    const int ntl = wave + NW * i;
+    const int kq = lane >> 4;
+    const int slot = (kq & 1) * 32 + (ntl & 1) * 16 + (lane & 15);
+    const int f = (ntl >> 1) * KSTEPS + 2 * (j & 1) + (kq >> 1);
+    lds_b[(buf * B_BLK + f) * 64 + slot] = dequant_word_bf16(rbw[set][i][j], rsc[set][i], rcc[set][i]);
+  };
+  // dense: the tiled pieces [16-column tile][32-row step][64][16 B] are copied as they are
+  int bd_voff[W4 ? 1 : B_PW];
+  if constexpr (!W4) {
+#pragma unroll
+    for (int i = 0; i < B_PW; ++i) {
+      const int q = wave * B_PW + i;
+      bd_voff[i] = (((q >> 1) * KS + (q & 1)) * 64 + lane) * 16;
+    }
+  }
   auto load_b_dense = [&](int s, int buf) {
 #pragma unroll
     for (int i = 0; i < (W4 ? 0 : B_PW); ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(smem + ((2 * A_FRAGS + buf * B_FRAGS + wave * B_PW + i) << 10)), 16,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(smem + ((2 * A_BLK + buf * B_BLK + wave * B_PW + i) << 10)), 16,
                                                bd_voff[i], s * 2048, 0, 0);
   };
-  // int4 piece of lane l (column l&15 of its 16-column tile, rows 8*(l>>4).. of 32-row step j):
-  // fragment (tile/2, 2j + (l>>5)), slot ((l>>4)&1)*32 + (tile&1)*16 + (l&15)
-  auto stash_b_word = [&](u32x4* b, int set, int i, int wsel) {
-    const int ntl = (tid >> 6) + NW * i;
-    const int kq = lane >> 4;
-    const int slot = (kq & 1) * 32 + (ntl & 1) * 16 + (lane & 15);
-    const int f0 = (ntl >> 1) * KSTEPS + (kq >> 1) + 2 * wsel;
-    const float sc = (float)__builtin_bit_cast(_Float16, (uint16_t)rsc[set][i]);
-    const int z = 129 + (int)((rzb[set][i] >> (4 * (lane & 1))) & 15u);
-    b[f0 * 64 + slot] = dequant_word_bf16(wsel ? rbw[set][i].y : rbw[set][i].x, sc, -(float)z * sc);
-  };
+  // operand read of column tile ct, k-step ks: int4 fragment-major; dense: piece (2 ct + n32/16, ks/2),
+  // lane (n32 & 15) + 16 (2 (ks & 1) + kh)
+  const int b_rd = W4 ? lane : (row32 >> 4) * 128 + (row32 & 15) + 16 * kh;
+  auto b_slot = [&](int ct, int ks) { return W4 ? (ct * KSTEPS + ks) * 64 : ct * 256 + (ks >> 1) * 64 + (ks & 1) * 32; };
 
   f32x16 acc[WMT][WNT];
 #pragma unroll
@@ -169,11 +185,13 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   bf16x8 fa[2][WMT], fb[2][WNT];
-  auto load_frags = [&](int set, const u32x4* a, const u32x4* b, int ks) {
+  auto load_frags = [&](int set, int buf, int ks) {
+    const u32x4* a = lds_a + buf * A_BLK * 64;
+    const u32x4* b = lds_b + buf * B_BLK * 64;
 #pragma unroll
-    for (int i = 0; i < WMT; ++i) fa[set][i] = __builtin_bit_cast(bf16x8, a[((wm * WMT + i) * KSTEPS + ks) * 64 + lane]);
+    for (int i = 0; i < WMT; ++i) fa[set][i] = __builtin_bit_cast(bf16x8, a[(wm * WMT + i) * 256 + a_rd[ks]]);
 #pragma unroll
-    for (int j = 0; j < WNT; ++j) fb[set][j] = __builtin_bit_cast(bf16x8, b[((wn * WNT + j) * KSTEPS + ks) * 64 + lane]);
+    for (int j = 0; j < WNT; ++j) fb[set][j] = __builtin_bit_cast(bf16x8, b[b_slot(wn * WNT + j, ks) + b_rd]);
   };
   auto mfmas = [&](int set) {
 #pragma unroll
@@ -187,50 +205,56 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     __builtin_amdgcn_s_barrier();
   };
 
-  // ---- prologue: stage 0 into buffer 0, stage 1's int4 words into registers --------------------
+  // One stage: MFMAs on LDS buffer h while the next stage is brought in.  h is the stage's parity,
+  // which for int4 is also its half of the 128-row group: register set 0 holds the current group,
+  // set 1 the next one.
+  auto do_stage = [&](int s, auto hc) {
+    constexpr int h = decltype(hc)::value;
+    const int s1 = min(s + 1, stages - 1);  // past the end: re-fetch the last stage into a buffer nobody reads
+    load_a(s1, h ^ 1);
+    if constexpr (W4) {
+      if constexpr (h == 0) fetch_b(min((s >> 1) + 1, G - 1), 1);
+    } else {
+      load_b_dense(s1, h ^ 1);
+    }
+#pragma unroll
+    for (int ks = 0; ks < 3; ++ks) {
+      load_frags((ks + 1) & 1, h, ks + 1);
+      mfmas(ks & 1);
+      if constexpr (W4) {
+        // next stage's words: second half of this group (h == 0) or first half of the next (h == 1)
+#pragma unroll
+        for (int i = 0; i < 2 * B_ITEMS; ++i)
+          if (i * 3 / (2 * B_ITEMS) == ks) stash_b_word(h ^ 1, h, i >> 1, 2 * (h ^ 1) + (i & 1));
+      }
+    }
+    stage_barrier();
+    if constexpr (W4 && h == 1) {
+#pragma unroll
+      for (int i = 0; i < NBI; ++i) rbw[0][i] = rbw[1][i], rsc[0][i] = rsc[1][i], rcc[0][i] = rcc[1][i];
+    }
+    load_frags(0, h ^ 1, 0);
+    mfmas(1);
+  };
+
+  // ---- prologue: stage 0 into buffer 0 -----------------------------------------------------------
   load_a(0, 0);
   if constexpr (W4) {
     fetch_b(0, 0);
 #pragma unroll
-    for (int i = 0; i < 2 * B_ITEMS; ++i) stash_b_word(lds_b, 0, i >> 1, i & 1);
-    fetch_b(min(1, stages - 1), 1);
+    for (int i = 0; i < 2 * B_ITEMS; ++i) stash_b_word(0, 0, i >> 1, i & 1);
   } else {
     load_b_dense(0, 0);
   }
   stage_barrier();
-  load_frags(0, lds_a, lds_b, 0);
+  load_frags(0, 0, 0);
 
-  for (int s = 0; s < stages; ++s) {
-    const int buf = s & 1;
-    const u32x4* a = lds_a + buf * A_FRAGS * 64;
-    const u32x4* b = lds_b + buf * B_FRAGS * 64;
-    u32x4* an = lds_a + (buf ^ 1) * A_FRAGS * 64;
-    u32x4* bn = lds_b + (buf ^ 1) * B_FRAGS * 64;
-    // the last iterations re-fetch the final stage into buffers nobody reads again: redundant, but
-    // it keeps the loop body free of branches
-    const int s1 = min(s + 1, stages - 1), s2 = min(s + 2, stages - 1);
-    load_a(s1, buf ^ 1);
-    if constexpr (!W4) load_b_dense(s1, buf ^ 1);
-#pragma unroll
-    for (int ks = 0; ks < 3; ++ks) {
-      load_frags((ks + 1) & 1, a, b, ks + 1);
-      mfmas(ks & 1);
-      if constexpr (W4) {
-#pragma unroll
-        for (int i = 0; i < 2 * B_ITEMS; ++i)
-          if (i * 3 / (2 * B_ITEMS) == ks) stash_b_word(bn, 1, i >> 1, i & 1);
-      }
-    }
-    if constexpr (W4) {
-      // register set 1 (stage s+1) is in LDS now; set 0 <- stage s+2, and rotate
-#pragma unroll
-      for (int i = 0; i < NBI; ++i) rbw[0][i] = rbw[1][i], rsc[0][i] = rsc[1][i], rzb[0][i] = rzb[1][i];
-    }
-    stage_barrier();
-    if constexpr (W4) fetch_b(s2, 1);
-    load_frags(0, an, bn, 0);
-    mfmas(1);
+  int s = 0;
+  for (; s + 1 < stages; s += 2) {
+    do_stage(s, std::integral_constant<int, 0>{});
+    do_stage(s + 1, std::integral_constant<int, 1>{});
   }
+  if (s < stages) do_stage(s, std::integral_constant<int, 0>{});
 
   // ---- epilogue: D[m = 8*(r/4) + 4*(lane>>5) + r%4][n = lane&31] of each 32x32 tile ---------------------
 #pragma unroll
@@ -262,7 +286,7 @@ int launch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const
                 int K, hipStream_t stream) {
   constexpr int BM = 32 * WMT * WAVES_M, BN = 32 * WNT * WAVES_N;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  const size_t lds = (size_t)2 * ((BM / 32) + (BN / 32)) * KSTEPS * 64 * 16;
+  const size_t lds = (size_t)2 * (BM / 8 + BN / 8) * 1024;
   auto kern = gemm_kernel<WAVES_M, WAVES_N, WMT, WNT, W4>;
   if (lds > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
