@@ -72,8 +72,11 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   constexpr int A_BLK = BM / 8;        // 1 KiB blocks per stage: activations, 8 rows x 128 bytes each
   constexpr int B_BLK = BN / 8;        // weights: 32x16 bf16 pieces (either layout)
   constexpr int A_PW = A_BLK / NW, B_PW = B_BLK / NW;
-  constexpr int B_ITEMS = (BN / 16) * 64 / NT;  // int4: (16-column tile, lane) items per thread per group of 128 rows
-  static_assert(A_BLK % NW == 0 && B_BLK % NW == 0 && ((BN / 16) * 64) % NT == 0, "tile / wave split");
+  // int4: (16-column tile, lane) items per thread per group of 128 rows; when the tiles do not divide
+  // evenly among the waves the last item exists on the first waves only
+  constexpr int B_ITEMS = (BN / 16 + NW - 1) / NW;
+  constexpr bool B_RAGGED = (BN / 16) % NW != 0;
+  static_assert(A_BLK % NW == 0 && B_BLK % NW == 0, "tile / wave split");
   extern __shared__ __align__(16) unsigned char smem[];
   u32x4* lds_a = reinterpret_cast<u32x4*>(smem);  // [2][A_BLK][64]
   u32x4* lds_b = lds_a + 2 * A_BLK * 64;          // [2][B_BLK][64]
@@ -151,6 +154,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   };
   auto stash_b_word = [&](int buf, int set, int i, int j) {  // word j (32-row step j of the group) of item i
     const int ntl = wave + NW * i;
+    if (B_RAGGED && ntl >= BN / 16) return;  // wave-uniform
     const int kq = lane >> 4;
     const int slot = (kq & 1) * 32 + (ntl & 1) * 16 + (lane & 15);
     const int f = (ntl >> 1) * KSTEPS + 2 * (j & 1) + (kq >> 1);
@@ -298,13 +302,33 @@ int launch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const
   O355_CHECK_LAUNCH();
 }
 
+int g_force_tile = 0;  // debug: 0 = choose, else 256 / 192 / 128 = the tile's width
+
+// Tiles are 256 rows by 256, 192 or 128 columns.  A launch runs in rounds of one tile per CU, so the
+// width is picked to minimise rounds x width (narrow tiles cost a little more per column: more
+// operand traffic per MFMA).
 template <bool W4>
 int dispatch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M,
                   int N, int K, hipStream_t stream) {
-  return launch_gemm<2, 4, 4, 2, W4>(x, wt, st, zt, y, M, N, K, stream);
+  int cus = 256;
+  const int64_t tm = (M + 255) / 256;
+  auto cost = [&](int bn, double penalty) {
+    const int64_t tiles = tm * ((N + bn - 1) / bn);
+    return (double)((tiles + cus - 1) / cus) * bn * penalty;
+  };
+  int best = 256;
+  double c = cost(256, 1.0);
+  if (cost(192, 1.04) < c) best = 192, c = cost(192, 1.04);
+  if (cost(128, 1.10) < c) best = 128, c = cost(128, 1.10);
+  if (g_force_tile) best = g_force_tile;
+  if (best == 256) return launch_gemm<2, 4, 4, 2, W4>(x, wt, st, zt, y, M, N, K, stream);
+  if (best == 192) return launch_gemm<4, 2, 2, 3, W4>(x, wt, st, zt, y, M, N, K, stream);
+  return launch_gemm<4, 2, 2, 2, W4>(x, wt, st, zt, y, M, N, K, stream);
 }
 
 }  // namespace
+
+extern "C" void olmo355_debug_set_gemm_tile(int width) { g_force_tile = width; }
 
 extern "C" int olmo355_w4_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
                                uint16_t* y, int M, int N, int K, void* stream) {
