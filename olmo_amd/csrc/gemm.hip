@@ -78,8 +78,8 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   constexpr bool B_RAGGED = (BN / 16) % NW != 0;
   static_assert(A_BLK % NW == 0 && B_BLK % NW == 0, "tile / wave split");
   extern __shared__ __align__(16) unsigned char smem[];
-  u32x4* lds_a = reinterpret_cast<u32x4*>(smem);  // [2][A_BLK][64]
-  u32x4* lds_b = lds_a + 2 * A_BLK * 64;          // [2][B_BLK][64]
+  u32x4* lds_a = reinterpret_cast<u32x4*>(smem);  // [3][A_BLK][64]: ring of three stages
+  u32x4* lds_b = lds_a + 3 * A_BLK * 64;          // [2][B_BLK][64]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -106,10 +106,11 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     const int c = (lane & 7) ^ ((row >> 1) & 7);
     a_voff[i] = (row * K + 8 * c) * 2;
   }
-  auto load_a = [&](int s, int buf) {
+  auto load_a = [&](int s, int buf, int part = -1) {  // part: only the requests of that k-step's share
 #pragma unroll
     for (int i = 0; i < A_PW; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(smem + ((buf * A_BLK + wave * A_PW + i) << 10)), 16, a_voff[i],
+      if (part < 0 || i * KSTEPS / A_PW == part)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(smem + ((buf * A_BLK + wave * A_PW + i) << 10)), 16, a_voff[i],
                                                s * (BK * 2), 0, 0);
   };
   // operand read: lane (row32, kh), row tile rt, k-step ks -> 16-byte slot
@@ -130,7 +131,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   // fragment (tile/2, k-step 2j + (l>>5)), slot ((l>>4)&1)*32 + (tile&1)*16 + (l&15).
   constexpr int NBI = W4 ? B_ITEMS : 1;
   u32x4 rbw[2][NBI];
-  float rsc[2][NBI], rcc[2][NBI];
+  uint32_t rsb[2][NBI], rzb[2][NBI];
   int bw_voff[NBI], bs_voff[NBI], bz_voff[NBI];
   if constexpr (W4) {
 #pragma unroll
@@ -141,15 +142,14 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
       bz_voff[i] = ntl * G * 8 + (col >> 1);
     }
   }
-  auto fetch_b = [&](int g, int set) {
+  auto fetch_b = [&](int g, int set, int part = -1) {  // part: as for the activations
 #pragma unroll
     for (int i = 0; i < NBI; ++i) {
+      if (part >= 0 && (2 * i + 1) * KSTEPS / (2 * NBI) != part) continue;
       rbw[set][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, bw_voff[i], g * 1024, 0));
-      const uint32_t sb = __builtin_amdgcn_raw_buffer_load_b16(rs_, bs_voff[i], g * 32, 0);
-      const uint32_t zb = __builtin_amdgcn_raw_buffer_load_b8(rz_, bz_voff[i], g * 8, 0);
-      const float sc = (float)__builtin_bit_cast(_Float16, (uint16_t)sb);
-      rsc[set][i] = sc;
-      rcc[set][i] = -(float)(129 + (int)((zb >> (4 * (lane & 1))) & 15u)) * sc;
+      // kept raw: converting here would make the wave wait for the loads it has just issued
+      rsb[set][i] = __builtin_amdgcn_raw_buffer_load_b16(rs_, bs_voff[i], g * 32, 0);
+      rzb[set][i] = __builtin_amdgcn_raw_buffer_load_b8(rz_, bz_voff[i], g * 8, 0);
     }
   };
   auto stash_b_word = [&](int buf, int set, int i, int j) {  // word j (32-row step j of the group) of item i
@@ -158,7 +158,9 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     const int kq = lane >> 4;
     const int slot = (kq & 1) * 32 + (ntl & 1) * 16 + (lane & 15);
     const int f = (ntl >> 1) * KSTEPS + 2 * (j & 1) + (kq >> 1);
-    lds_b[(buf * B_BLK + f) * 64 + slot] = dequant_word_bf16(rbw[set][i][j], rsc[set][i], rcc[set][i]);
+    const float sc = (float)__builtin_bit_cast(_Float16, (uint16_t)rsb[set][i]);
+    const float cc = -(float)(129 + (int)((rzb[set][i] >> (4 * (lane & 1))) & 15u)) * sc;
+    lds_b[(buf * B_BLK + f) * 64 + slot] = dequant_word_bf16(rbw[set][i][j], sc, cc);
   };
   // dense: the tiled pieces [16-column tile][32-row step][64][16 B] are copied as they are
   int bd_voff[W4 ? 1 : B_PW];
@@ -172,7 +174,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   auto load_b_dense = [&](int s, int buf) {
 #pragma unroll
     for (int i = 0; i < (W4 ? 0 : B_PW); ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(smem + ((2 * A_BLK + buf * B_BLK + wave * B_PW + i) << 10)), 16,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(smem + ((3 * A_BLK + buf * B_BLK + wave * B_PW + i) << 10)), 16,
                                                bd_voff[i], s * 2048, 0, 0);
   };
   // operand read of column tile ct, k-step ks: int4 fragment-major; dense: piece (2 ct + n32/16, ks/2),
@@ -188,77 +190,95 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  bf16x8 fa[2][WMT], fb[2][WNT];
-  auto load_frags = [&](int set, int buf, int ks) {
-    const u32x4* a = lds_a + buf * A_BLK * 64;
-    const u32x4* b = lds_b + buf * B_BLK * 64;
+  bf16x8 fa[WMT], fb[WNT];
+  auto load_frags = [&](int abuf, int bbuf, int ks) {
+    const u32x4* a = lds_a + abuf * A_BLK * 64;
+    const u32x4* b = lds_b + bbuf * B_BLK * 64;
 #pragma unroll
-    for (int i = 0; i < WMT; ++i) fa[set][i] = __builtin_bit_cast(bf16x8, a[(wm * WMT + i) * 256 + a_rd[ks]]);
+    for (int i = 0; i < WMT; ++i) fa[i] = __builtin_bit_cast(bf16x8, a[(wm * WMT + i) * 256 + a_rd[ks]]);
 #pragma unroll
-    for (int j = 0; j < WNT; ++j) fb[set][j] = __builtin_bit_cast(bf16x8, b[b_slot(wn * WNT + j, ks) + b_rd]);
+    for (int j = 0; j < WNT; ++j) fb[j] = __builtin_bit_cast(bf16x8, b[b_slot(wn * WNT + j, ks) + b_rd]);
   };
-  auto mfmas = [&](int set) {
+  auto mfmas = [&]() {
 #pragma unroll
     for (int i = 0; i < WMT; ++i)
 #pragma unroll
-      for (int j = 0; j < WNT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < WNT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
   };
-  // everything this wave sent towards LDS (through registers or directly) has landed, then meet
-  auto stage_barrier = [&]() {
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-    __builtin_amdgcn_s_barrier();
-  };
+  auto ring_next = [](int ab) { return ab == 2 ? 0 : ab + 1; };
 
-  // One stage: MFMAs on LDS buffer h while the next stage is brought in.  h is the stage's parity,
-  // which for int4 is also its half of the 128-row group: register set 0 holds the current group,
-  // set 1 the next one.
-  auto do_stage = [&](int s, auto hc) {
-    constexpr int h = decltype(hc)::value;
-    const int s1 = min(s + 1, stages - 1);  // past the end: re-fetch the last stage into a buffer nobody reads
-    load_a(s1, h ^ 1);
-    if constexpr (W4) {
-      if constexpr (h == 0) fetch_b(min((s >> 1) + 1, G - 1), 1);
-    } else {
-      load_b_dense(s1, h ^ 1);
+  // One stage.  Activations sit in a ring of three LDS buffers and are requested two stages ahead;
+  // the weights are double-buffered in LDS (int4: requested two stages ahead into registers, set
+  // = parity of the 128-row group, and dequantised into LDS one stage ahead; dense: copied one stage
+  // ahead).  Memory operations complete in order, so waiting until only this stage's own requests
+  // (KEEP of them) are outstanding means everything the next stage reads has landed.
+  //   h = parity of the stage = weight LDS buffer (and, int4, the half of the group)
+  //   p = parity of the group (int4 register set)
+  auto do_stage = [&](int s, int ab, auto hc, auto pc) {
+    constexpr int h = decltype(hc)::value, p = decltype(pc)::value;
+    const int s2 = min(s + 2, stages - 1);  // past the end: re-fetch the last stage into a buffer nobody reads
+    const int ab2 = ring_next(ring_next(ab));
+    if constexpr (!W4) {
+      load_b_dense(min(s + 1, stages - 1), h ^ 1);
+      __builtin_amdgcn_sched_barrier(0);  // keep the order: the weights' requests are the older ones
     }
 #pragma unroll
-    for (int ks = 0; ks < 3; ++ks) {
-      load_frags((ks + 1) & 1, h, ks + 1);
-      mfmas(ks & 1);
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      load_frags(ab, h, ks);
+      // requests are spread over the stage: a burst of them stalls the wave at issue
+      load_a(s2, ab2, ks);
+      if constexpr (W4 && h == 1) fetch_b(min((s >> 1) + 2, G - 1), p, ks);
+      __builtin_amdgcn_sched_barrier(0);
+      mfmas();
       if constexpr (W4) {
         // next stage's words: second half of this group (h == 0) or first half of the next (h == 1)
 #pragma unroll
         for (int i = 0; i < 2 * B_ITEMS; ++i)
-          if (i * 3 / (2 * B_ITEMS) == ks) stash_b_word(h ^ 1, h, i >> 1, 2 * (h ^ 1) + (i & 1));
+          if (i * KSTEPS / (2 * B_ITEMS) == ks) stash_b_word(h ^ 1, p ^ h, i >> 1, 2 * (h ^ 1) + (i & 1));
       }
     }
-    stage_barrier();
-    if constexpr (W4 && h == 1) {
-#pragma unroll
-      for (int i = 0; i < NBI; ++i) rbw[0][i] = rbw[1][i], rsc[0][i] = rsc[1][i], rcc[0][i] = rcc[1][i];
-    }
-    load_frags(0, h ^ 1, 0);
-    mfmas(1);
+    constexpr int KEEP = A_PW + ((W4 && h == 1) ? 3 * NBI : 0);
+    static_assert(KEEP < 64, "vmcnt range");
+    __builtin_amdgcn_s_waitcnt((KEEP & 15) | ((KEEP >> 4) << 14) | 0x0070);  // vmcnt(KEEP) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
   };
 
-  // ---- prologue: stage 0 into buffer 0 -----------------------------------------------------------
+  // ---- prologue: stages 0 and 1 of the activations, stage 0 of the weights -----------------------
   load_a(0, 0);
+  load_a(min(1, stages - 1), 1);
   if constexpr (W4) {
     fetch_b(0, 0);
 #pragma unroll
     for (int i = 0; i < 2 * B_ITEMS; ++i) stash_b_word(0, 0, i >> 1, i & 1);
+    fetch_b(min(1, G - 1), 1);
   } else {
     load_b_dense(0, 0);
   }
-  stage_barrier();
-  load_frags(0, 0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
 
-  int s = 0;
-  for (; s + 1 < stages; s += 2) {
-    do_stage(s, std::integral_constant<int, 0>{});
-    do_stage(s + 1, std::integral_constant<int, 1>{});
+  using H0 = std::integral_constant<int, 0>;
+  using H1 = std::integral_constant<int, 1>;
+  int s = 0, ab = 0;
+  for (; s + 3 < stages; s += 4) {
+    do_stage(s, ab, H0{}, H0{});
+    ab = ring_next(ab);
+    do_stage(s + 1, ab, H1{}, H0{});
+    ab = ring_next(ab);
+    do_stage(s + 2, ab, H0{}, H1{});
+    ab = ring_next(ab);
+    do_stage(s + 3, ab, H1{}, H1{});
+    ab = ring_next(ab);
   }
-  if (s < stages) do_stage(s, std::integral_constant<int, 0>{});
+  if (s < stages) {  // up to three stages left; s is a multiple of four, so the parities are known
+    do_stage(s, ab, H0{}, H0{});
+    ab = ring_next(ab);
+    if (s + 1 < stages) {
+      do_stage(s + 1, ab, H1{}, H0{});
+      ab = ring_next(ab);
+      if (s + 2 < stages) do_stage(s + 2, ab, H0{}, H1{});
+    }
+  }
 
   // ---- epilogue: D[m = 8*(r/4) + 4*(lane>>5) + r%4][n = lane&31] of each 32x32 tile ---------------------
 #pragma unroll
@@ -290,7 +310,7 @@ int launch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const
                 int K, hipStream_t stream) {
   constexpr int BM = 32 * WMT * WAVES_M, BN = 32 * WNT * WAVES_N;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-  const size_t lds = (size_t)2 * (BM / 8 + BN / 8) * 1024;
+  const size_t lds = (size_t)(3 * (BM / 8) + 2 * (BN / 8)) * 1024;
   auto kern = gemm_kernel<WAVES_M, WAVES_N, WMT, WNT, W4>;
   if (lds > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
