@@ -144,6 +144,63 @@ def test_b16_linear(dev, M, N, K):
     assert torch.allclose(y, ref, rtol=2 ** -8, atol=2 ** -8 * ref.abs().max().item())
 
 
+def _force_gemm_tile(width):
+    # test-only hook of the library (not part of the declared interface): 0 = choose by shape
+    from olmo_amd import _lib
+    _lib.lib().olmo355_debug_set_gemm_tile(int(width))
+
+
+@pytest.mark.parametrize("width", [256, 192, 128])
+@pytest.mark.parametrize("M,N,K", [(65, 208, 128), (300, 1008, 384), (513, 400, 1408), (256, 768, 256), (1, 16, 640)])
+def test_w4_gemm_every_tile_width(dev, width, M, N, K):
+    """Ragged M and N against every tile shape, and K whose stage count leaves 0..3 stages after the
+    four-stage main loop (int4 stages come in pairs: K = 128, 384, 1408 leave two, 256 none, 640 two)."""
+    say("w4_gemm_tile", width, M, N, K)
+    ops = _ops()
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=M + N + K)
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(7)).to(torch.bfloat16)
+    ref = ow4.linear_fp32(x, ow4.dequantize(qw, qz, sc, 128))
+    t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    xd = x.to(dev)
+    from olmo_amd import _lib
+    _force_gemm_tile(width)
+    try:
+        st = _lib.lib().olmo355_w4_gemm(xd.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y.data_ptr(),
+                                        M, N, K, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+    finally:
+        _force_gemm_tile(0)
+    assert st == 0
+    scale = ref.abs().max().item()
+    assert (y.float().cpu() - ref).abs().max().item() <= 2 ** -7 * scale
+
+
+@pytest.mark.parametrize("width", [256, 192, 128])
+@pytest.mark.parametrize("M,N,K", [(65, 208, 64), (300, 1008, 192), (513, 400, 320), (256, 768, 448), (40, 48, 1024)])
+def test_b16_gemm_every_tile_width(dev, width, M, N, K):
+    """Dense weights: stage counts 1, 3, 5, 7, 16 cover every tail length of the four-stage loop."""
+    say("b16_gemm_tile", width, M, N, K)
+    ops = _ops()
+    gen = torch.Generator().manual_seed(M + N + K)
+    w = (torch.randn(N, K, generator=gen) * 0.02).to(torch.bfloat16)
+    x = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    ref = x.float() @ w.float().t()
+    t = ops.b16_repack(w.to(dev))
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    xd = x.to(dev)
+    from olmo_amd import _lib
+    _force_gemm_tile(width)
+    try:
+        st = _lib.lib().olmo355_b16_gemm(xd.data_ptr(), t.wt.data_ptr(), y.data_ptr(), M, N, K,
+                                         torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+    finally:
+        _force_gemm_tile(0)
+    assert st == 0
+    assert torch.allclose(y.float().cpu(), ref, rtol=2 ** -8, atol=2 ** -8 * ref.abs().max().item())
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 50304, 256), (2048, 768, 256), (77, 130, 1024)])
 def test_f32_linear(dev, M, N, K):
     ops = _ops()
