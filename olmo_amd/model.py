@@ -351,29 +351,15 @@ class OLMo(nn.Module):
 
     def _block_decode_fused(self, blk, x, pend, kc, vc, B, past_len, key_bias, graph_pos, n_keys_max):
         eps = self.config.layer_norm_eps
-        import os
-        mode = os.environ.get("O355_FUSE", "both")
         if pend is None:
             qkv = self._linear(blk.att_proj, x)
-        elif mode in ("both", "pro"):
-            qkv, x = ops.linear_fused(pend[0], self._tiled(blk.att_proj), resid=x, norm_w=pend[1], eps=eps)
         else:
-            x = ops.rmsnorm(pend[0], pend[1], eps, residual=x)
-            qkv = self._linear(blk.att_proj, x)
+            # x := x + norm(previous block's MLP output) happens in the projection's prologue
+            qkv, x = ops.linear_fused(pend[0], self._tiled(blk.att_proj), resid=x, norm_w=pend[1], eps=eps)
         att = self._attention(blk, qkv, kc, vc, B, 1, past_len, key_bias, graph_pos, n_keys_max)
         a = self._linear(blk.attn_out, att)
-        if mode == "both":
-            u, x = ops.linear_fused(a, self._tiled(blk.ff_proj), resid=x, norm_w=blk.attn_norm.weight.data, eps=eps,
-                                    swiglu_out=True)
-        elif mode == "pro":
-            u, x = ops.linear_fused(a, self._tiled(blk.ff_proj), resid=x, norm_w=blk.attn_norm.weight.data, eps=eps)
-            u = ops.swiglu(u)
-        elif mode == "epi":
-            x = ops.rmsnorm(a, blk.attn_norm.weight.data, eps, residual=x)
-            u, _ = ops.linear_fused(x, self._tiled(blk.ff_proj), swiglu_out=True)
-        else:
-            x = ops.rmsnorm(a, blk.attn_norm.weight.data, eps, residual=x)
-            u = ops.swiglu(self._linear(blk.ff_proj, x))
+        u, x = ops.linear_fused(a, self._tiled(blk.ff_proj), resid=x, norm_w=blk.attn_norm.weight.data, eps=eps,
+                                swiglu_out=True)
         f = self._linear(blk.ff_out, u)
         return x, (f, blk.ff_norm.weight.data)
 
