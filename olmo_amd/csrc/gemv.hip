@@ -35,12 +35,24 @@ struct GemvArgs {
   int M, N, K;
 };
 
-__device__ __forceinline__ bf16x8 unpack_w4_bias128(uint32_t w) {
+// The two constants of the unpack, made opaque to the optimiser (empty asm, no instruction): as
+// literals the compiler emits v_and + v_or per pair, from registers it selects the single
+// v_and_or_b32.  (An asm *instruction* here would be unsafe: the hazard recogniser does not see an
+// asm's result feeding an MFMA and leaves out the wait states.)
+struct UnpackConsts {
+  uint32_t mask, bias;
+  __device__ __forceinline__ UnpackConsts() : mask(0x000f000fu), bias(0x43004300u) {
+    asm volatile("" : "+s"(mask));
+    asm volatile("" : "+v"(bias));
+  }
+};
+
+__device__ __forceinline__ bf16x8 unpack_w4_bias128(uint32_t w, const UnpackConsts& c) {
   u32x4 r;
-  r.x = (w & 0x000f000fu) | 0x43004300u;
-  r.y = ((w >> 4) & 0x000f000fu) | 0x43004300u;
-  r.z = ((w >> 8) & 0x000f000fu) | 0x43004300u;
-  r.w = ((w >> 12) & 0x000f000fu) | 0x43004300u;
+  r.x = (w & c.mask) | c.bias;
+  r.y = ((w >> 4) & c.mask) | c.bias;
+  r.z = ((w >> 8) & c.mask) | c.bias;
+  r.w = ((w >> 12) & c.mask) | c.bias;
   return __builtin_bit_cast(bf16x8, r);
 }
 
@@ -67,10 +79,30 @@ __device__ __forceinline__ void unpack8(const u32x4& v, float (&f)[8]) {
 // finish(), after the weight loads have been issued; the barrier orders LDS only.
 constexpr int kXStageRegs = 4;  // plain copy: 16-byte pieces per thread held across the weight prologue
 
+// sum over an aligned row of 16 lanes; every lane gets it
+__device__ __forceinline__ float row16_sum(float v) {
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 16);
+  return v;
+}
+
+// Per-group sums of the staged activations, xs[g][rp] (rp rows per group, row m of group g): 16
+// consecutive 16-byte pieces are one group of 128, i.e. one row of 16 lanes.  `v` is the piece as
+// it went into LDS; all 64 lanes call this, `valid` per lane (whole rows of lanes are valid or not).
+__device__ __forceinline__ void group_sum_to_lds(const u32x4& v, bool valid, int idx, int nvec, float* xs, int rp) {
+  float f[8], s = 0.f;
+  unpack8(v, f);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) s += f[e];
+  s = row16_sum(valid ? s : 0.f);
+  if (valid && (threadIdx.x & 15) == 0) xs[((idx % nvec) >> 4) * rp + idx / nvec] = s;
+}
+
 template <int WAVES, bool XLDS, int PRO>
 struct XStage {
   __device__ __forceinline__ void begin(const GemvArgs&) {}
-  __device__ __forceinline__ void finish(const GemvArgs&, uint16_t*, float*) {}
+  template <bool XSUM = false>
+  __device__ __forceinline__ void finish(const GemvArgs&, uint16_t*, float*, float* = nullptr, int = 0) {}
 };
 
 template <int WAVES>
@@ -84,15 +116,20 @@ struct XStage<WAVES, true, 0> {
       if (idx < total) xr[i] = reinterpret_cast<const u32x4*>(a.x)[idx];
     }
   }
-  __device__ __forceinline__ void finish(const GemvArgs& a, uint16_t* xl, float*) {
-    const int total = (a.M * a.K) >> 3;
+  template <bool XSUM = false>
+  __device__ __forceinline__ void finish(const GemvArgs& a, uint16_t* xl, float*, float* xs = nullptr, int rp = 0) {
+    const int total = (a.M * a.K) >> 3, nvec = a.K >> 3;
 #pragma unroll
     for (int i = 0; i < kXStageRegs; ++i) {
       const int idx = threadIdx.x + i * WAVES * 64;
       if (idx < total) reinterpret_cast<u32x4*>(xl)[idx] = xr[i];
+      if constexpr (XSUM) group_sum_to_lds(xr[i], idx < total, idx, nvec, xs, rp);
     }
-    for (int idx = threadIdx.x + kXStageRegs * WAVES * 64; idx < total; idx += WAVES * 64)
-      reinterpret_cast<u32x4*>(xl)[idx] = reinterpret_cast<const u32x4*>(a.x)[idx];
+    for (int idx = threadIdx.x + kXStageRegs * WAVES * 64; idx < total; idx += WAVES * 64) {
+      const u32x4 v = reinterpret_cast<const u32x4*>(a.x)[idx];
+      reinterpret_cast<u32x4*>(xl)[idx] = v;
+      if constexpr (XSUM) group_sum_to_lds(v, true, idx, nvec, xs, rp);
+    }
     for (int i = threadIdx.x; i < (a.K >> 3); i += WAVES * 64)
       reinterpret_cast<u32x4*>(xl + (int64_t)a.M * a.K)[i] = u32x4{0u, 0u, 0u, 0u};
     lds_barrier();
@@ -118,7 +155,9 @@ struct NormStage {
       }
     }
   }
-  __device__ __forceinline__ void finish(const GemvArgs& a, uint16_t* xl, float* part /* [VPT*WAVES] */) {
+  template <bool XSUM = false>
+  __device__ __forceinline__ void finish(const GemvArgs& a, uint16_t* xl, float* part /* [VPT*WAVES] */, float* xs = nullptr,
+                                         int rp = 0) {
     const int nvec = a.K >> 3, total = a.M * nvec;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
@@ -134,8 +173,10 @@ struct NormStage {
       if (lane == 0) part[i * WAVES + wave] = ss;
     }
     lds_barrier();
+    u32x4 ov[VPT];
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
+      ov[i] = u32x4{0u, 0u, 0u, 0u};
       const int idx = threadIdx.x + i * WAVES * 64;
       if (idx < total) {
         const int m = idx / nvec;
@@ -158,6 +199,14 @@ struct NormStage {
         }
         reinterpret_cast<u32x4*>(xl)[idx] = o;
         if (blockIdx.x == 0) reinterpret_cast<u32x4*>(a.x_out)[idx] = o;
+        ov[i] = o;
+      }
+    }
+    if constexpr (XSUM) {
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        const int idx = threadIdx.x + i * WAVES * 64;
+        group_sum_to_lds(ov[i], idx < total, idx, nvec, xs, rp);
       }
     }
     for (int i = threadIdx.x; i < nvec; i += WAVES * 64)
@@ -241,6 +290,7 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_kernel(GemvArgs args, cons
   const int g_begin = (int)((int64_t)G * wave / WAVES), g_end = (int)((int64_t)G * (wave + 1) / WAVES);
   const bf16x8 ones = ones_bf16x8();
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  const UnpackConsts uc;
   const uint16_t* xrow = xl + (col < M ? col : M) * K;  // this lane's row in LDS (XLDS)
 
   f32x4 acc[MT][NT];
@@ -302,7 +352,7 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_kernel(GemvArgs args, cons
           }
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) {
-            const bf16x8 b = unpack_w4_bias128(w[u][nt][j]);
+            const bf16x8 b = unpack_w4_bias128(w[u][nt][j], uc);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
               t[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[mt], b, t[mt][nt], 0, 0, 0);
@@ -311,17 +361,159 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_kernel(GemvArgs args, cons
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
           const float sc = (float)__builtin_bit_cast(_Float16, s16[u][nt]);
-          const float zc = (float)(129 + (int)((z8[u][nt] >> (4 * (col & 1))) & 15u));  // 128 + (stored + 1)
+          const float nzc = -(float)(129 + (int)((z8[u][nt] >> (4 * (col & 1))) & 15u));  // -(128 + (stored + 1))
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) acc[mt][nt][r] += sc * (t[mt][nt][r] - zc * xsum[mt][r]);
+            for (int r = 0; r < 4; ++r)
+              acc[mt][nt][r] = __builtin_fmaf(sc, __builtin_fmaf(nzc, xsum[mt][r], t[mt][nt][r]), acc[mt][nt][r]);
         }
         if (g + U < g_end) issue(u, g + U);  // refill the slot just consumed
       }
     }
   }
   gemv_epilogue<MT, NT, WAVES, EPI>(acc, red, args, tile, ntiles);
+}
+
+// ---- int4, M <= 16: several groups share one accumulator --------------------------------------------------
+// With M <= 4 only rows 0..3 of the 16-row MFMA tile carry data.  GPA = 4 consecutive groups of 128
+// rows then use the *same* accumulator: group u of the four puts its activations in operand rows
+// 4u..4u+3, so its products land in the lanes of row block u (lane = 16 u + column) while the other
+// row blocks receive zeros.  The lanes of block u hold the scale and zero of group u, the sums of
+// the activations per group come from LDS (computed once while staging), and the fp32 correction
+// acc += scale * (T - (128 + zero) * X) is applied once per four groups instead of once per group.
+// M <= 8 shares an accumulator between GPA = 2 groups; M <= 16 (GPA = 1) is the plain scheme.
+template <int GPA, int NT, int WAVES, int PRO, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void w4_gemv_rot_kernel(GemvArgs args, const u32x4* __restrict__ wt,
+                                                                 const uint16_t* __restrict__ st,
+                                                                 const uint8_t* __restrict__ zt) {
+  constexpr int RP = 16 / GPA;   // operand rows per group
+  constexpr int KQS = 4 / GPA;   // lane row blocks (kq) per group
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int M = args.M, K = args.K;
+  const int G = K >> 7, ntiles = args.N >> 4;
+  float* red = reinterpret_cast<float*>(smem);                                           // [WAVES][NT*256]
+  uint16_t* xl = reinterpret_cast<uint16_t*>(smem + WAVES * NT * 256 * sizeof(float));   // [M+1][K]
+  float* xs = reinterpret_cast<float*>(xl + (int64_t)(M + 1) * K);                       // [G][RP]
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int col = lane & 15, kq = lane >> 4;
+  const int ul = kq / KQS;  // the group (of the GPA) whose results this lane holds
+  int tile[NT];
+  owned_tiles<NT, EPI>(tile, ntiles);
+  const int g_begin = (int)((int64_t)G * wave / WAVES), g_end = (int)((int64_t)G * (wave + 1) / WAVES);
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  const UnpackConsts uc;
+
+  // operand row `col` of group slot u is activation row col - u*RP when that is in [0, M), else zeros
+  int xoff[GPA];
+#pragma unroll
+  for (int u = 0; u < GPA; ++u) {
+    const int rel = col - u * RP;
+    xoff[u] = ((rel >= 0 && rel < M) ? rel : M) * K + 8 * kq;
+  }
+
+  f32x4 acc[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) acc[nt] = zero4;
+  u32x4 w[GPA][NT];
+  uint32_t s16c[NT], z8c[NT], s16n[NT], z8n[NT];
+  int64_t tbase[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) tbase[nt] = (int64_t)min(tile[nt], ntiles - 1) * G;  // out-of-range tiles: computed, dropped
+
+  auto issue_w = [&](int u, int g) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) w[u][nt] = __builtin_nontemporal_load(&wt[(tbase[nt] + g) * 64 + lane]);
+  };
+  auto issue_sz = [&](uint32_t (&s16)[NT], uint32_t (&z8)[NT], int base) {
+    const int g = max(min(base + ul, g_end - 1), 0);  // a wave without groups still reads valid memory
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      s16[nt] = st[(tbase[nt] + g) * 16 + col];
+      z8[nt] = zt[(tbase[nt] + g) * 8 + (col >> 1)];
+    }
+  };
+
+  XStage<WAVES, true, PRO> stage;
+  stage.begin(args);
+#pragma unroll
+  for (int u = 0; u < GPA; ++u)
+    if (g_begin + u < g_end) issue_w(u, g_begin + u);
+  issue_sz(s16c, z8c, g_begin);
+  stage.template finish<true>(args, xl, red, xs, RP);
+
+  for (int base = g_begin; base < g_end; base += GPA) {
+    const bool more = base + GPA < g_end;
+    if (more) issue_sz(s16n, z8n, base + GPA);
+    f32x4 t[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) t[nt] = zero4;
+#pragma unroll
+    for (int u = 0; u < GPA; ++u) {
+      const int g = base + u;
+      if (g < g_end) {
+        const uint16_t* xp = xl + xoff[u] + 128 * g;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const bf16x8 af = *reinterpret_cast<const bf16x8*>(xp + 32 * j);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            t[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, unpack_w4_bias128(w[u][nt][j], uc), t[nt], 0, 0, 0);
+        }
+        if (g + GPA < g_end) issue_w(u, g + GPA);  // refill the slot just consumed
+      }
+    }
+    // correction for this lane's group
+    const int gl = base + ul;
+    const f32x4 xg = *reinterpret_cast<const f32x4*>(xs + min(gl, g_end - 1) * RP + (4 * kq) % RP);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const float sc = gl < g_end ? (float)__builtin_bit_cast(_Float16, (uint16_t)s16c[nt]) : 0.f;
+      const float nzc = -(float)(129 + (int)((z8c[nt] >> (4 * (col & 1))) & 15u));  // -(128 + (stored + 1))
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[nt][r] = __builtin_fmaf(sc, __builtin_fmaf(nzc, xg[r], t[nt][r]), acc[nt][r]);
+    }
+    if (more) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) s16c[nt] = s16n[nt], z8c[nt] = z8n[nt];
+    }
+  }
+
+  // ---- reduce over waves and over the GPA row blocks, in fixed order ---------------------------------
+  constexpr int PER_WAVE = NT * 256;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave * PER_WAVE + (nt * 4 + r) * 64 + lane] = acc[nt][r];
+  __syncthreads();
+  // output element (m = 4 kqs + r, column c) of tile nt: lanes c + 16 (u KQS + kqs), u = 0..GPA-1
+  auto total_of = [&](int nt, int r, int kqs, int c) {
+    float v = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv)
+#pragma unroll
+      for (int u = 0; u < GPA; ++u) v += red[wv * PER_WAVE + (nt * 4 + r) * 64 + c + 16 * (u * KQS + kqs)];
+    return v;
+  };
+  if constexpr (EPI == 0) {
+    for (int i = threadIdx.x; i < NT * RP * 16; i += WAVES * 64) {
+      const int c = i & 15, m = (i >> 4) % RP, nt = i / (16 * RP);
+      if (tile[nt] < ntiles && m < M)
+        args.y[(int64_t)m * args.N + tile[nt] * 16 + c] = f32_to_bf16_bits(total_of(nt, m & 3, m >> 2, c));
+    }
+  } else {
+    static_assert(EPI == 0 || NT == 2, "the SwiGLU epilogue owns one up tile and one gate tile");
+    const int half_n = args.N >> 1;
+    for (int i = threadIdx.x; i < RP * 16; i += WAVES * 64) {
+      const int c = i & 15, m = i >> 4;
+      if (m < M) {
+        const float up = round_bf16(total_of(0, m & 3, m >> 2, c));  // the Linear's bf16 output
+        const float gate = round_bf16(total_of(1, m & 3, m >> 2, c));
+        const float sg = round_bf16(gate / (1.f + expf(-gate)));
+        args.y[(int64_t)m * half_n + tile[0] * 16 + c] = f32_to_bf16_bits(sg * up);
+      }
+    }
+  }
 }
 
 // ---- dense bf16 --------------------------------------------------------------------------------------------
@@ -449,19 +641,41 @@ int check_fused(const GemvArgs& a, bool pro, bool epi) {
   GEMV_CASE(KERNEL, MTv, NTv, 8, Uv, Xv, Pv, Ev, __VA_ARGS__)    \
   GEMV_CASE(KERNEL, MTv, NTv, 16, Uv, Xv, Pv, Ev, __VA_ARGS__)
 
+template <typename Kern>
+int launch_rot(Kern kern, int gpa, const GemvPlan& p, const GemvArgs& a, hipStream_t stream, const u32x4* w,
+               const uint16_t* st, const uint8_t* zt) {
+  const size_t lds = (size_t)p.waves * p.nt * 256 * 4 + (size_t)(a.M + 1) * a.K * 2 + (size_t)(a.K >> 7) * (16 / gpa) * 4;
+  if (lds > 48 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return O355_ELAUNCH;
+  const int ntiles = a.N >> 4;
+  const unsigned blocks = p.epi ? (unsigned)(ntiles >> 1) : (unsigned)ntiles;
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(p.waves * 64), lds, stream, a, w, st, zt);
+  O355_CHECK_LAUNCH();
+}
+
+#define ROT_CASE(GPAv, NTv, Wv, Pv, Ev)                                                   \
+  if (gpa == GPAv && p.nt == NTv && p.waves == Wv && p.pro == Pv && p.epi == Ev)          \
+    return launch_rot(w4_gemv_rot_kernel<GPAv, NTv, Wv, Pv, Ev>, gpa, p, a, as_stream(stream), w, st, zt);
+#define ROT_WAVES(GPAv, NTv, Pv, Ev) ROT_CASE(GPAv, NTv, 4, Pv, Ev) ROT_CASE(GPAv, NTv, 8, Pv, Ev) ROT_CASE(GPAv, NTv, 16, Pv, Ev)
+#define ROT_FORMS(GPAv)                                                                        \
+  ROT_WAVES(GPAv, 1, 0, 0) ROT_WAVES(GPAv, 1, 1, 0) ROT_WAVES(GPAv, 1, 4, 0) ROT_WAVES(GPAv, 2, 0, 1) \
+  ROT_WAVES(GPAv, 2, 1, 1) ROT_WAVES(GPAv, 2, 4, 1)
+
 int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, bool pro, bool epi,
                      void* stream) {
   const GemvPlan p = plan_gemv(a.M, a.N, a.K, true, pro, epi);
   const u32x4* w = (const u32x4*)wt;
-  GEMV_WAVES(w4_gemv_kernel, 1, 1, 2, true, 0, 0, w, st, zt)
+  if (p.mt == 1 && p.xlds) {  // M <= 16 with the activations in LDS: accumulators shared between groups
+    const int gpa = a.M <= 4 ? 4 : (a.M <= 8 ? 2 : 1);
+    ROT_FORMS(4)
+    ROT_FORMS(2)
+    ROT_FORMS(1)
+    return O355_EUNSUPPORTED;
+  }
   GEMV_WAVES(w4_gemv_kernel, 1, 1, 2, false, 0, 0, w, st, zt)
   GEMV_WAVES(w4_gemv_kernel, 2, 1, 2, false, 0, 0, w, st, zt)
   GEMV_WAVES(w4_gemv_kernel, 4, 1, 2, false, 0, 0, w, st, zt)
-  GEMV_WAVES(w4_gemv_kernel, 1, 1, 2, true, 1, 0, w, st, zt)
-  GEMV_WAVES(w4_gemv_kernel, 1, 1, 2, true, 4, 0, w, st, zt)
-  GEMV_WAVES(w4_gemv_kernel, 1, 2, 2, true, 0, 1, w, st, zt)
-  GEMV_WAVES(w4_gemv_kernel, 1, 2, 2, true, 1, 1, w, st, zt)
-  GEMV_WAVES(w4_gemv_kernel, 1, 2, 2, true, 4, 1, w, st, zt)
   return O355_EUNSUPPORTED;
 }
 
