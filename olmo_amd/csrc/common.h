@@ -66,6 +66,19 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// ---- buffer addressing ----------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// buffer resource over [base, base + bytes): loads past the end return zero
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int64_t bytes) {
+  const int64_t cap = 0xffffffffll;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)(uint32_t)(bytes < cap ? (bytes < 0 ? 0 : bytes) : cap),
+                                           0x00020000);
+}
+
+// s_waitcnt immediate: at most `vm` vector-memory operations outstanding (and, with lds, no LDS ones)
+constexpr int waitcnt_imm(int vm, bool lds) { return (vm & 15) | ((vm >> 4) << 14) | 0x0070 | (lds ? 0 : 0x0f00); }
+
 // ---- wave64 reductions ------------------------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -53,16 +53,6 @@ __device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& 
   }
 }
 
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-
-// buffer resource over [base, base + bytes): loads past the end return zero, which is what pads
-// ragged M and N edges
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, int64_t bytes) {
-  const int64_t cap = 0xffffffffll;
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)(uint32_t)(bytes < cap ? (bytes < 0 ? 0 : bytes) : cap),
-                                           0x00020000);
-}
-
 template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4>  // wave grid, 32x32 MFMA tiles per wave
 __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wt,
                                           const uint16_t* __restrict__ st, const uint8_t* __restrict__ zt,

@@ -21,6 +21,8 @@
 //             its first weight pieces are in flight; workgroup 0 also writes x to memory;
 //   epilogue  y := silu(gate) * up              SwiGLU (olmo/model.py:365-368) on the two column
 //             tiles a workgroup owns (tile p of the first half and tile p of the second half).
+#include <algorithm>
+
 #include "common.h"
 
 namespace {
@@ -516,6 +518,253 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_rot_kernel(GemvArgs args, 
   }
 }
 
+// ---- norm prologue for M <= 4 ---------------------------------------------------------------------------
+// Same arithmetic and rounding points as NormStage, written for few instructions: buffer loads
+// with the thread index as offset, rows found by comparison instead of division (M <= 4 and a wave's
+// 64 pieces lie in one row, K % 512 == 0), sums over a wave with DPP.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+template <int WAVES, int VPT>
+struct SmallNorm {
+  u32x4 av[VPT], rv[VPT], wv[VPT];
+  int row[VPT];  // row of this wave's pieces in pass i (wave-uniform), -1 past the end
+  __device__ __forceinline__ void begin(const GemvArgs& a, int wave) {
+    const int nvec = a.K >> 3, total = a.M * nvec;
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(a.x, (int64_t)total * 16), rr = make_rsrc(a.resid, (int64_t)total * 16),
+                                 rn = make_rsrc(a.norm_w, (int64_t)nvec * 16);
+    const int voff = (threadIdx.x & 63) * 16;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int first = (wave + i * WAVES) * 64;  // first piece of this wave in pass i
+      const int m = (first >= nvec) + (first >= 2 * nvec) + (first >= 3 * nvec);
+      row[i] = first < total ? m : -1;
+      av[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, voff, first * 16, 0));  // past the end: zeros
+      rv[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, voff, first * 16, 0));
+      wv[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rn, voff, (first - m * nvec) * 16, 0));
+    }
+  }
+  // part: [VPT*WAVES] floats of LDS
+  __device__ __forceinline__ void finish(const GemvArgs& a, uint16_t* xl, float* part, int wave) {
+    const int nvec = a.K >> 3, total = a.M * nvec;
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      float f[8], ss = 0.f;
+      unpack8(av[i], f);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+      ss = wave_sum_dpp(ss);
+      if (lane == 0) part[i * WAVES + wave] = ss;
+    }
+    lds_barrier();
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      if (row[i] >= 0) {  // wave-uniform
+        float ss = 0.f;   // partials of this row, in (pass, wave) order
+#pragma unroll
+        for (int j = 0; j < VPT * WAVES; ++j) {
+          const int first = ((j % WAVES) + (j / WAVES) * WAVES) * 64;
+          const int mj = (first >= nvec) + (first >= 2 * nvec) + (first >= 3 * nvec);
+          if (first < total && mj == row[i]) ss += part[j];
+        }
+        const float rstd = 1.f / sqrtf(ss / (float)a.K + a.eps);
+        float f[8], r[8], w[8];
+        unpack8(av[i], f);
+        unpack8(rv[i], r);
+        unpack8(wv[i], w);
+        u32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float y0 = round_bf16(w[2 * e] * round_bf16(f[2 * e] * rstd));
+          const float y1 = round_bf16(w[2 * e + 1] * round_bf16(f[2 * e + 1] * rstd));
+          o[e] = pack_bf16x2(r[2 * e] + y0, r[2 * e + 1] + y1);
+        }
+        const int idx = (wave + i * WAVES) * 64 + lane;
+        reinterpret_cast<u32x4*>(xl)[idx] = o;
+        if (blockIdx.x == 0) reinterpret_cast<u32x4*>(a.x_out)[idx] = o;
+      }
+    }
+    for (int i = threadIdx.x; i < nvec; i += WAVES * 64)
+      reinterpret_cast<u32x4*>(xl + (int64_t)a.M * a.K)[i] = u32x4{0u, 0u, 0u, 0u};
+    lds_barrier();
+  }
+};
+
+// ---- int4, M <= 4: the lean decode kernel ---------------------------------------------------------------
+// A decode launch lives for a few microseconds and every SIMD interleaves several waves, so each
+// instruction of the per-wave preamble costs (waves per SIMD) x 4 cycles before the first weight
+// request leaves.  This variant keeps the preamble short: buffer loads with scalar offsets (no
+// per-lane 64-bit address arithmetic), the activations copied memory -> LDS directly (no registers,
+// no VALU), all weight requests of the wave issued before anything else is waited for, the sums of
+// the activations from the matrix cores (B = ones) instead of a staging pass.  Four groups share an
+// accumulator as in w4_gemv_rot_kernel (GPA = 4).
+template <int NT, int WAVES, int PRO, int EPI>
+__device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u32x4* __restrict__ wt,
+                                                   const uint16_t* __restrict__ st, const uint8_t* __restrict__ zt) {
+  constexpr int GPA = 4;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int M = args.M, K = args.K;
+  const int G = K >> 7, ntiles = args.N >> 4, nvec = K >> 3;
+  const int xbytes = M * K * 2;
+  // LDS: x rows [M][K] (the direct copy works in whole KiB), a zero row [K], then the reduction area
+  const int red_off = max((xbytes + 1023) & ~1023, xbytes + K * 2);
+  uint16_t* xl = reinterpret_cast<uint16_t*>(smem);
+  float* red = reinterpret_cast<float*>(smem + red_off);  // [WAVES][NT*4][16]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 15, kq = lane >> 4;
+  const int g_begin = (G * wave) / WAVES, g_end = (G * (wave + 1)) / WAVES;
+  int tile[NT], tg[NT];
+  owned_tiles<NT, EPI>(tile, ntiles);
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) tg[nt] = min(tile[nt], ntiles - 1) * G;  // out-of-range tiles: computed, dropped
+
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(wt, (int64_t)ntiles * G * 1024);
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(st, (int64_t)ntiles * G * 32);
+  const __amdgpu_buffer_rsrc_t rz = make_rsrc(zt, (int64_t)ntiles * G * 8);
+  const int wvoff = lane * 16, svoff = lane * 2, zvoff = lane >> 1;
+
+  u32x4 w[GPA][NT];
+  uint32_t s16c[NT], z8c[NT], s16n[NT], z8n[NT];
+  // slot u of a quad is group base+u, clamped into the matrix so that every request is valid and
+  // the number of requests per wave is fixed
+  auto issue_w = [&](int u, int g) {
+    const int gc = min(g, G - 1);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+      w[u][nt] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, wvoff, (tg[nt] + gc) * 1024, 2));
+  };
+  // the lanes of row block kq hold the scale and zero of group base+kq: one contiguous request each
+  auto issue_sz = [&](uint32_t (&s16)[NT], uint32_t (&z8)[NT], int base) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      s16[nt] = __builtin_amdgcn_raw_buffer_load_b16(rs, svoff, (tg[nt] + base) * 32, 0);
+      z8[nt] = __builtin_amdgcn_raw_buffer_load_b8(rz, zvoff, (tg[nt] + base) * 8, 0);
+    }
+  };
+
+  // ---- activations first (they are needed first and come from L2), then the whole first quad ----
+  if constexpr (PRO == 0) {
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(args.x, xbytes);
+    for (int off = wave * 1024; off < xbytes; off += WAVES * 1024)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(smem + off), 16, wvoff, off, 0, 0);
+  }
+  SmallNorm<WAVES, PRO == 0 ? 1 : PRO> norm;
+  if constexpr (PRO != 0) norm.begin(args, wave);
+#pragma unroll
+  for (int u = 0; u < GPA; ++u) issue_w(u, g_begin + u);
+  issue_sz(s16c, z8c, g_begin);
+  if constexpr (PRO == 0) {
+    for (int i = tid; i < nvec; i += WAVES * 64) reinterpret_cast<u32x4*>(xl + (int64_t)M * K)[i] = u32x4{0u, 0u, 0u, 0u};
+    // everything but the GPA*NT weight and 2*NT scale/zero requests has arrived: x is in LDS
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(GPA * NT + 2 * NT, true));
+    __builtin_amdgcn_s_barrier();
+  } else {
+    norm.finish(args, xl, red, wave);
+  }
+
+  // operand row `col` of slot u is activation row col - 4u when that is in [0, M), else the zero row
+  int xoff[GPA];
+#pragma unroll
+  for (int u = 0; u < GPA; ++u) {
+    const int rel = col - 4 * u;
+    xoff[u] = ((rel >= 0 && rel < M) ? rel : M) * K + 8 * kq;
+  }
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  const bf16x8 ones = ones_bf16x8();
+  const UnpackConsts uc;
+  f32x4 acc[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) acc[nt] = zero4;
+
+  for (int base = g_begin; base < g_end; base += GPA) {
+    const bool more = base + GPA < g_end;
+    if (more) issue_sz(s16n, z8n, base + GPA);
+    f32x4 t[NT], xsum = zero4;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) t[nt] = zero4;
+#pragma unroll
+    for (int u = 0; u < GPA; ++u) {
+      const int g = base + u;
+      if (g < g_end) {
+        const uint16_t* xp = xl + xoff[u] + 128 * g;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const bf16x8 af = *reinterpret_cast<const bf16x8*>(xp + 32 * j);
+          xsum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, ones, xsum, 0, 0, 0);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            t[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, unpack_w4_bias128(w[u][nt][j], uc), t[nt], 0, 0, 0);
+        }
+        if (g + GPA < g_end) issue_w(u, g + GPA);  // refill the slot just consumed
+      }
+    }
+    // fp32 correction; rows of a slot whose group lies past the wave's range are all zero
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const float sc = (float)__builtin_bit_cast(_Float16, (uint16_t)s16c[nt]);
+      const float nzc = -(float)(129 + (int)((z8c[nt] >> (4 * (col & 1))) & 15u));  // -(128 + (stored + 1))
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[nt][r] = __builtin_fmaf(sc, __builtin_fmaf(nzc, xsum[r], t[nt][r]), acc[nt][r]);
+    }
+    if (more) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) s16c[nt] = s16n[nt], z8c[nt] = z8n[nt];
+    }
+  }
+
+  // ---- reduce: the four row blocks inside the wave, then the waves through LDS, in fixed order ----
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (r < M) {
+        float v = acc[nt][r];
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        if (lane < 16) red[(wave * NT * 4 + nt * 4 + r) * 16 + lane] = v;
+      }
+  __syncthreads();
+  auto total_of = [&](int nt, int m, int c) {
+    float v = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv) v += red[(wv * NT * 4 + nt * 4 + m) * 16 + c];
+    return v;
+  };
+  if constexpr (EPI == 0) {
+    if (tid < NT * 64) {
+      const int c = tid & 15, m = (tid >> 4) & 3, nt = tid >> 6;
+      if (tile[nt] < ntiles && m < M) args.y[(int64_t)m * args.N + tile[nt] * 16 + c] = f32_to_bf16_bits(total_of(nt, m, c));
+    }
+  } else {
+    static_assert(EPI == 0 || NT == 2, "the SwiGLU epilogue owns one up tile and one gate tile");
+    if (tid < 64) {
+      const int c = tid & 15, m = tid >> 4;
+      if (m < M) {
+        const float up = round_bf16(total_of(0, m, c));  // the Linear's bf16 output
+        const float gate = round_bf16(total_of(1, m, c));
+        const float sg = round_bf16(gate / (1.f + expf(-gate)));
+        args.y[(int64_t)m * (args.N >> 1) + tile[0] * 16 + c] = f32_to_bf16_bits(sg * up);
+      }
+    }
+  }
+}
+
+template <int NT, int WAVES, int PRO, int EPI>
+__global__ __launch_bounds__(WAVES * 64) void w4_gemv_small_kernel(GemvArgs args, const u32x4* __restrict__ wt,
+                                                                   const uint16_t* __restrict__ st,
+                                                                   const uint8_t* __restrict__ zt) {
+  w4_gemv_small_body<NT, WAVES, PRO, EPI>(args, wt, st, zt);
+}
+
 // ---- dense bf16 --------------------------------------------------------------------------------------------
 template <int MT, int NT, int WAVES, int U, bool XLDS, int PRO, int EPI>
 __global__ __launch_bounds__(WAVES * 64) void b16_gemv_kernel(GemvArgs args, const bf16x8* __restrict__ wt) {
@@ -584,7 +833,7 @@ struct GemvPlan {
 };
 
 // Experiment hook (not part of the public interface): overrides waves / xlds when >= 0.
-int g_dbg_waves = -1, g_dbg_xlds = -1;
+int g_dbg_waves = -1, g_dbg_xlds = -1, g_dbg_small = 1;
 
 constexpr int kXldsMaxBytes = 64 * 1024;
 
@@ -654,6 +903,29 @@ int launch_rot(Kern kern, int gpa, const GemvPlan& p, const GemvArgs& a, hipStre
   O355_CHECK_LAUNCH();
 }
 
+template <typename Kern>
+int launch_small(Kern kern, const GemvPlan& p, const GemvArgs& a, hipStream_t stream, const u32x4* w, const uint16_t* st,
+                 const uint8_t* zt) {
+  const int xbytes = a.M * a.K * 2;
+  const int red_off = std::max((xbytes + 1023) & ~1023, xbytes + a.K * 2);
+  const size_t lds = (size_t)red_off + (size_t)p.waves * p.nt * 4 * 16 * 4;
+  if (lds > 48 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return O355_ELAUNCH;
+  const int ntiles = a.N >> 4;
+  const unsigned blocks = p.epi ? (unsigned)(ntiles >> 1) : (unsigned)ntiles;
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(p.waves * 64), lds, stream, a, w, st, zt);
+  O355_CHECK_LAUNCH();
+}
+
+#define SMALL_CASE(NTv, Wv, Pv, Ev)                                        \
+  if (p.nt == NTv && p.waves == Wv && p.pro == Pv && p.epi == Ev)          \
+    return launch_small(w4_gemv_small_kernel<NTv, Wv, Pv, Ev>, p, a, as_stream(stream), w, st, zt);
+#define SMALL_WAVES(NTv, Pv, Ev) SMALL_CASE(NTv, 4, Pv, Ev) SMALL_CASE(NTv, 8, Pv, Ev) SMALL_CASE(NTv, 16, Pv, Ev)
+#define SMALL_FORMS                                                                              \
+  SMALL_WAVES(1, 0, 0) SMALL_WAVES(1, 1, 0) SMALL_WAVES(1, 4, 0) SMALL_WAVES(2, 0, 1) \
+  SMALL_WAVES(2, 1, 1) SMALL_WAVES(2, 4, 1)
+
 #define ROT_CASE(GPAv, NTv, Wv, Pv, Ev)                                                   \
   if (gpa == GPAv && p.nt == NTv && p.waves == Wv && p.pro == Pv && p.epi == Ev)          \
     return launch_rot(w4_gemv_rot_kernel<GPAv, NTv, Wv, Pv, Ev>, gpa, p, a, as_stream(stream), w, st, zt);
@@ -666,6 +938,10 @@ int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, 
                      void* stream) {
   const GemvPlan p = plan_gemv(a.M, a.N, a.K, true, pro, epi);
   const u32x4* w = (const u32x4*)wt;
+  if (p.mt == 1 && p.xlds && a.M <= 4 && (int64_t)(a.N >> 4) * (a.K >> 7) * 1024 < (1ll << 31) && g_dbg_small && p.pro >= 0) {
+    SMALL_FORMS
+    return O355_EUNSUPPORTED;
+  }
   if (p.mt == 1 && p.xlds) {  // M <= 16 with the activations in LDS: accumulators shared between groups
     const int gpa = a.M <= 4 ? 4 : (a.M <= 8 ? 2 : 1);
     ROT_FORMS(4)
@@ -697,6 +973,7 @@ int b16_gemv_dispatch(const GemvArgs& a, const uint16_t* wt, bool pro, bool epi,
 }  // namespace
 
 extern "C" void olmo355_debug_set_gemv_plan(int waves, int xlds) { g_dbg_waves = waves, g_dbg_xlds = xlds; }
+extern "C" void olmo355_debug_set_gemv_small(int on) { g_dbg_small = on; }
 
 extern "C" int olmo355_w4_gemv(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
                                uint16_t* y, int M, int N, int K, void* stream) {
