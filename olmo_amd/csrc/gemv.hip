@@ -614,8 +614,8 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
   const int M = args.M, K = args.K;
   const int G = K >> 7, ntiles = args.N >> 4, nvec = K >> 3;
   const int xbytes = M * K * 2;
-  // LDS: x rows [M][K] (the direct copy works in whole KiB), a zero row [K], then the reduction area
-  const int red_off = max((xbytes + 1023) & ~1023, xbytes + K * 2);
+  // LDS: x rows [M][K], a zero row [K], then the reduction area
+  const int red_off = xbytes + max(K * 2, 1024);  // a direct copy may run up to 1 KiB past the rows (zeros)
   uint16_t* xl = reinterpret_cast<uint16_t*>(smem);
   float* red = reinterpret_cast<float*>(smem + red_off);  // [WAVES][NT*4][16]
   const int tid = threadIdx.x, lane = tid & 63;
@@ -652,10 +652,19 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
   };
 
   // ---- activations first (they are needed first and come from L2), then the whole first quad ----
+  // Without a norm prologue every wave stages just the columns of x it will multiply (its own
+  // groups), so no workgroup barrier is needed before the main loop.
+  int n_x = 0;  // direct-to-LDS requests of this wave (wave-uniform)
   if constexpr (PRO == 0) {
     const __amdgpu_buffer_rsrc_t rx = make_rsrc(args.x, xbytes);
-    for (int off = wave * 1024; off < xbytes; off += WAVES * 1024)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(smem + off), 16, wvoff, off, 0, 0);
+    const int lo = g_begin * 256, hi = g_end * 256;  // byte range of the wave's slice within a row
+    for (int m = 0; m < M; ++m)
+      for (int off = lo; off < hi; off += 1024) {
+        // lanes past the slice (or the row) read past the buffer or into the next wave's slice: harmless,
+        // the LDS rows are laid out like memory and neighbours write the same bytes
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(smem + m * K * 2 + off), 16, wvoff, m * K * 2 + off, 0, 0);
+        ++n_x;
+      }
   }
   SmallNorm<WAVES, PRO == 0 ? 1 : PRO> norm;
   if constexpr (PRO != 0) norm.begin(args, wave);
@@ -663,10 +672,11 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
   for (int u = 0; u < GPA; ++u) issue_w(u, g_begin + u);
   issue_sz(s16c, z8c, g_begin);
   if constexpr (PRO == 0) {
-    for (int i = tid; i < nvec; i += WAVES * 64) reinterpret_cast<u32x4*>(xl + (int64_t)M * K)[i] = u32x4{0u, 0u, 0u, 0u};
-    // everything but the GPA*NT weight and 2*NT scale/zero requests has arrived: x is in LDS
+    // zero row, this wave's slice of it
+    for (int off = g_begin * 256 + lane * 16; off < g_end * 256; off += 1024)
+      *reinterpret_cast<u32x4*>(smem + xbytes + off) = u32x4{0u, 0u, 0u, 0u};
+    // everything but the GPA*NT weight and 2*NT scale/zero requests has arrived: the slice is in LDS
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(GPA * NT + 2 * NT, true));
-    __builtin_amdgcn_s_barrier();
   } else {
     norm.finish(args, xl, red, wave);
   }
@@ -907,7 +917,7 @@ template <typename Kern>
 int launch_small(Kern kern, const GemvPlan& p, const GemvArgs& a, hipStream_t stream, const u32x4* w, const uint16_t* st,
                  const uint8_t* zt) {
   const int xbytes = a.M * a.K * 2;
-  const int red_off = std::max((xbytes + 1023) & ~1023, xbytes + a.K * 2);
+  const int red_off = xbytes + std::max(a.K * 2, 1024);
   const size_t lds = (size_t)red_off + (size_t)p.waves * p.nt * 4 * 16 * 4;
   if (lds > 48 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
