@@ -86,6 +86,17 @@ int olmo355_w4_gemv_fused(const uint16_t* x, const uint16_t* resid, const uint16
                           uint16_t* x_out, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
                           int M, int N, int K, int swiglu, void* stream);
 
+/* olmo355_w4_gemv_fused for M <= 4 with the norms chained between launches: RMSNorm needs the sum
+ * of squares of a whole row, and the launch that *produces* that row can leave it behind per 16-column
+ * tile, so the consumer's prologue neither re-reads the row nor synchronises its workgroup.
+ *   ssq_out != NULL (swiglu == 0): ssq_out[m][N/16] = sum of squares of the bf16 outputs of row m, per tile;
+ *   resid != NULL: ssq_in[m][K/16] (left by the launch that wrote x) must be given; x' as above.
+ * Used for the three norms of a decode block (olmo/model.py:786-794 attention/MLP post-norms and the
+ * full-width QK-norm of :711-716 via olmo355_attn_decode_fused).  O355_EUNSUPPORTED: use the calls above. */
+int olmo355_w4_gemv_chain(const uint16_t* x, const uint16_t* resid, const uint16_t* norm_w, float eps, uint16_t* x_out,
+                          const float* ssq_in, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
+                          float* ssq_out, int M, int N, int K, int swiglu, void* stream);
+
 /* Large-M path: dequantise tiles into LDS as bf16 and multiply on the matrix cores.  Stands
  * in for the reference's dequantise-then-matmul branch (AGQ qlinear_cuda_old.py:236-287) and
  * exllama's reconstruct + cublasHgemm (exllama/cuda_func/q4_matmul.cu:222-260). */
@@ -151,12 +162,14 @@ int olmo355_attn_decode(const void* q, const void* kcache, const void* vcache, c
 
 /* olmo355_qknorm_rope_kvwrite (T == 1) and olmo355_attn_decode in one pass over the new token's
  * fused projection qkv [B, (H+2*Hkv)*hd]: bf16, hd 64 or 128; O355_EUNSUPPORTED otherwise (the caller
- * then issues the two separate calls).  Same workspace as olmo355_attn_decode. */
+ * then issues the two separate calls).  Same workspace as olmo355_attn_decode.
+ * qk_ssq: NULL, or the per-tile sums of squares [B][(H+2*Hkv)*hd/16] that olmo355_w4_gemv_chain left for
+ * qkv (the q and k norms then do not re-read the rows). */
 int olmo355_attn_decode_fused(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
                               const float* cos_tab, void* kcache, void* vcache, const float* key_bias, void* out,
                               void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos, int past_len,
-                              const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps, int dtype,
-                              void* stream);
+                              const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps,
+                              const float* qk_ssq, int dtype, void* stream);
 
 /* ---- MLP activation: SwiGLU.forward (olmo/model.py:365-368) --------------------------------
  * x [rows, 2h]: first half "up", second half "gate"; out [rows, h] = silu(gate) * up. */

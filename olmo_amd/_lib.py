@@ -38,6 +38,7 @@ EXPORTS = {
     "olmo355_w4t_dequant_fp16": (I, [P, P, P, P, I, I, P]),
     "olmo355_w4_gemv": (I, [P, P, P, P, P, I, I, I, P]),
     "olmo355_w4_gemv_fused": (I, [P, P, P, F, P, P, P, P, P, I, I, I, I, P]),
+    "olmo355_w4_gemv_chain": (I, [P, P, P, F, P, P, P, P, P, P, P, I, I, I, I, P]),
     "olmo355_b16_gemv_fused": (I, [P, P, P, F, P, P, P, I, I, I, I, P]),
     "olmo355_w4_gemm": (I, [P, P, P, P, P, I, I, I, P]),
     "olmo355_b16_repack": (I, [P, P, I, I, P]),
@@ -50,7 +51,7 @@ EXPORTS = {
     "olmo355_attn_prefill": (I, [P, P, P, P, P, I, I, I, I, I, I, I, I, I, P]),
     "olmo355_attn_decode_workspace_bytes": (L, [I, I, I, I]),
     "olmo355_attn_decode": (I, [P, P, P, P, P, P, I, I, I, I, I, I, P, I, I, I, P]),
-    "olmo355_attn_decode_fused": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, I, P]),
+    "olmo355_attn_decode_fused": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, I, P]),
     "olmo355_swiglu": (I, [P, P, I, I, I, P]),
     "olmo355_embedding": (I, [P, P, P, I, I, I, I, P]),
     "olmo355_add": (I, [P, P, P, L, I, P]),

@@ -476,7 +476,8 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     const uint16_t* __restrict__ qkv, const uint16_t* __restrict__ qw, const uint16_t* __restrict__ kw,
     const float* __restrict__ sin_t, const float* __restrict__ cos_t, uint16_t* __restrict__ kc,
     uint16_t* __restrict__ vc, const float* __restrict__ key_bias, float* __restrict__ ws, int H, int Hkv, int Lmax,
-    int n_pos, int past_len, const int32_t* __restrict__ past_dev, int nchunks_max, int bias_stride, float eps) {
+    int n_pos, int past_len, const int32_t* __restrict__ past_dev, int nchunks_max, int bias_stride, float eps,
+    const float* __restrict__ qk_ssq) {
   constexpr int LPK = HD / 8, KPI = 64 / LPK, ITERS = kDecodeKeysPerWave / KPI;
   constexpr int HALF = HD / 2, CPH = HD / 16;  // pair chunks per head
   __shared__ float red_o[4][HD];
@@ -510,14 +511,22 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     vreg[it] = reinterpret_cast<const u32x4*>(vc)[(cbase + (int64_t)keyc * HD + sub * 8) >> 3];
     bias[it] = key_bias ? key_bias[(int64_t)b * bias_stride + keyc] : 0.f;
   }
+  // sums of squares of the q and k rows: from the projection's per-tile partials when it left them
+  // (qk_ssq[b][(dq + 2 dk) / 16], q tiles first), else from the rows themselves
+  const bool norm = (qw != nullptr);
+  float sq_part = 0.f, sk_part = 0.f;
+  if (norm && qk_ssq) {
+    const float* pr = qk_ssq + (int64_t)b * ((dq + 2 * dk) >> 4);
+    for (int i = tid; i < (dq >> 4); i += 256) sq_part += pr[i];
+    for (int i = tid; i < (dk >> 4); i += 256) sk_part += pr[(dq >> 4) + i];
+  }
   const int pos = past_dev ? *past_dev : past_len;
   const int L = pos + 1;
   if (chunk * kDecodeChunk >= L || pos >= Lmax || pos >= n_pos || pos > kmax) return;
   const bool owns_new = (pos / kDecodeChunk == chunk);
   // ---- 2. the token's q and k rows (sums of squares) and this head's pieces ------------------------------
-  const bool norm = (qw != nullptr);
   u32x4 qrow[QV], krow[QV];
-  if (norm) {
+  if (norm && !qk_ssq) {
 #pragma unroll
     for (int i = 0; i < QV; ++i) {
       const int idx = tid + i * 256;
@@ -553,9 +562,9 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
 
   float rq = 1.f, rk = 1.f;
   if (norm) {
-    float sq = 0.f, sk = 0.f;
+    float sq = sq_part, sk = sk_part;
 #pragma unroll
-    for (int i = 0; i < QV; ++i) {
+    for (int i = 0; i < (qk_ssq ? 0 : QV); ++i) {
       const int idx = tid + i * 256;
       float f[8];
       if (idx < (dq >> 3)) {
@@ -1009,7 +1018,7 @@ extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const 
                                          const float* cos_tab, void* kcache, void* vcache, const float* key_bias,
                                          void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
                                          int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride,
-                                         float eps, int dtype, void* stream) {
+                                         float eps, const float* qk_ssq, int dtype, void* stream) {
   if (!qkv || !sin_tab || !cos_tab || !kcache || !vcache || !out || !ws) return O355_EINVAL;
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || past_len < 0 || n_keys_max <= 0 || n_keys_max > Lmax)
     return O355_EINVAL;
@@ -1040,7 +1049,7 @@ extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const 
 #define FUSED(HDv, QVv)                                                                                                 \
   hipLaunchKernelGGL((attn_decode_fused_kernel<HDv, QVv>), dim3(nch, H, B), dim3(256), 0, s, (const uint16_t*)qkv,   \
                      (const uint16_t*)qw, (const uint16_t*)kw, sin_tab, cos_tab, (uint16_t*)kcache, (uint16_t*)vcache, \
-                     key_bias, (float*)ws, H, Hkv, Lmax, n_pos, past_len, past_len_dev, nch, bias_stride, eps);       \
+                     key_bias, (float*)ws, H, Hkv, Lmax, n_pos, past_len, past_len_dev, nch, bias_stride, eps, qk_ssq); \
   hipLaunchKernelGGL((attn_decode_combine_kernel<O355_BF16, HDv>), dim3(H, B), dim3(HDv), 0, s, (const float*)ws, out, \
                      H, past_len, past_len_dev, nch)
   const int qv = (H * hd / 8 + 255) / 256;

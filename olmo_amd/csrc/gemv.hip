@@ -35,6 +35,10 @@ struct GemvArgs {
   uint16_t* y;             // [M,N], or [M,N/2] with the SwiGLU epilogue
   float eps;
   int M, N, K;
+  // chained norms: the launch that produced x left the sum of squares of each 16-column tile of its
+  // (bf16-rounded) output rows in ssq_in[M][K/16]; this launch leaves its own in ssq_out[M][N/16]
+  const float* ssq_in = nullptr;
+  float* ssq_out = nullptr;
 };
 
 // The two constants of the unpack, made opaque to the optimiser (empty asm, no instruction): as
@@ -598,6 +602,92 @@ struct SmallNorm {
   }
 };
 
+// ---- norm prologue fed by the producer's sums of squares --------------------------------------------------
+// mean(a^2) of a row is the sum of K/16 per-tile partials that the launch which wrote `a` left behind,
+// so a wave needs no other wave: it adds the partials (fixed order: lane-strided, then the DPP tree),
+// normalises just its own slice of the row and goes on without a workgroup barrier.
+constexpr int kChainPieces = 4;  // at most: 16-byte pieces per lane = rows x KiB of slice
+
+template <int P>  // pieces per lane (1, 2 or 4); also bounds the rows
+struct ChainNorm {
+  u32x4 av[P], rv[P], wv[P];
+  f32x4 pv[P][4];  // partial sums: row, chunk of 256
+  __device__ __forceinline__ static void piece_of(int p, int per_row, int& m, int& k) {
+    m = per_row == 1 ? p : (per_row == 2 ? p >> 1 : (per_row == 3 ? p / 3 : p >> 2));
+    k = p - m * per_row;
+  }
+  // lo, hi: byte range of the wave's slice within a row
+  __device__ __forceinline__ void begin(const GemvArgs& a, int lo, int hi) {
+    const int lane = threadIdx.x & 63, n_ssq = a.K >> 4, per_row = (hi - lo + 1023) >> 10;
+#pragma unroll
+    for (int m = 0; m < P; ++m) {
+      const __amdgpu_buffer_rsrc_t rp = make_rsrc(a.ssq_in + (int64_t)min(m, a.M - 1) * n_ssq, (int64_t)n_ssq * 4);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        pv[m][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (m < a.M && c * 256 < n_ssq)
+          pv[m][c] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rp, lane * 16, c * 1024, 0));
+      }
+    }
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(a.x, (int64_t)a.M * a.K * 2), rr = make_rsrc(a.resid, (int64_t)a.M * a.K * 2),
+                                 rn = make_rsrc(a.norm_w, (int64_t)a.K * 2);
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      int m, k;
+      piece_of(p, per_row, m, k);
+      if (m < a.M) {  // wave-uniform
+        const int off = lo + k * 1024;
+        av[p] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, lane * 16, m * a.K * 2 + off, 0));
+        rv[p] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, lane * 16, m * a.K * 2 + off, 0));
+        wv[p] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rn, lane * 16, off, 0));
+      }
+    }
+  }
+  __device__ __forceinline__ void finish(const GemvArgs& a, unsigned char* smem, int lo, int hi) {
+    const int lane = threadIdx.x & 63, per_row = (hi - lo + 1023) >> 10;
+    const int n_ssq = a.K >> 4;
+    float rstd[P];
+#pragma unroll
+    for (int m = 0; m < P; ++m) {
+      rstd[m] = 0.f;
+      if (m < a.M) {  // wave-uniform
+        float ss = (pv[m][0][0] + pv[m][0][1]) + (pv[m][0][2] + pv[m][0][3]);
+#pragma unroll
+        for (int c = 1; c < 4; ++c)
+          if (c * 256 < n_ssq) ss += (pv[m][c][0] + pv[m][c][1]) + (pv[m][c][2] + pv[m][c][3]);
+        ss = wave_sum_dpp(ss);
+        rstd[m] = 1.f / sqrtf(ss / (float)a.K + a.eps);
+      }
+    }
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      int m, k;
+      piece_of(p, per_row, m, k);
+      if (m < a.M) {
+        const int off = lo + k * 1024 + lane * 16;
+        float rs = rstd[0];
+#pragma unroll
+        for (int q = 1; q < P; ++q) rs = m == q ? rstd[q] : rs;
+        float f[8], r[8], w[8];
+        unpack8(av[p], f);
+        unpack8(rv[p], r);
+        unpack8(wv[p], w);
+        u32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float y0 = round_bf16(w[2 * e] * round_bf16(f[2 * e] * rs));
+          const float y1 = round_bf16(w[2 * e + 1] * round_bf16(f[2 * e + 1] * rs));
+          o[e] = pack_bf16x2(r[2 * e] + y0, r[2 * e + 1] + y1);
+        }
+        if (off < hi) {  // lanes past the slice would mix rows
+          *reinterpret_cast<u32x4*>(smem + m * a.K * 2 + off) = o;
+          if (blockIdx.x == 0) *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(a.x_out) + m * a.K * 2 + off) = o;
+        }
+      }
+    }
+  }
+};
+
 // ---- int4, M <= 4: the lean decode kernel ---------------------------------------------------------------
 // A decode launch lives for a few microseconds and every SIMD interleaves several waves, so each
 // instruction of the per-wave preamble costs (waves per SIMD) x 4 cycles before the first weight
@@ -666,15 +756,19 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
         ++n_x;
       }
   }
-  SmallNorm<WAVES, PRO == 0 ? 1 : PRO> norm;
-  if constexpr (PRO != 0) norm.begin(args, wave);
+  constexpr bool CHAIN = PRO >= 8;  // 8, 9, 10: chained norm with 1, 2, 4 pieces per lane
+  SmallNorm<WAVES, (PRO == 0 || CHAIN) ? 1 : PRO> norm;
+  ChainNorm<CHAIN ? (1 << (PRO - 8)) : 1> chain;
+  if constexpr (CHAIN) chain.begin(args, g_begin * 256, g_end * 256);
+  else if constexpr (PRO != 0) norm.begin(args, wave);
 #pragma unroll
   for (int u = 0; u < GPA; ++u) issue_w(u, g_begin + u);
   issue_sz(s16c, z8c, g_begin);
-  if constexpr (PRO == 0) {
+  if constexpr (PRO == 0 || CHAIN) {
     // zero row, this wave's slice of it
     for (int off = g_begin * 256 + lane * 16; off < g_end * 256; off += 1024)
       *reinterpret_cast<u32x4*>(smem + xbytes + off) = u32x4{0u, 0u, 0u, 0u};
+    if constexpr (CHAIN) chain.finish(args, smem, g_begin * 256, g_end * 256);
     // everything but the GPA*NT weight and 2*NT scale/zero requests has arrived: the slice is in LDS
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(GPA * NT + 2 * NT, true));
   } else {
@@ -752,7 +846,13 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
   if constexpr (EPI == 0) {
     if (tid < NT * 64) {
       const int c = tid & 15, m = (tid >> 4) & 3, nt = tid >> 6;
-      if (tile[nt] < ntiles && m < M) args.y[(int64_t)m * args.N + tile[nt] * 16 + c] = f32_to_bf16_bits(total_of(nt, m, c));
+      const bool live = tile[nt] < ntiles && m < M;
+      const float v = live ? round_bf16(total_of(nt, m, c)) : 0.f;
+      if (live) args.y[(int64_t)m * args.N + tile[nt] * 16 + c] = f32_to_bf16_bits(v);
+      if (args.ssq_out) {  // sum of squares of the 16 outputs of (row, tile): one row of 16 lanes
+        const float q = row16_sum(v * v);
+        if (live && c == 0) args.ssq_out[(int64_t)m * ntiles + tile[nt]] = q;
+      }
     }
   } else {
     static_assert(EPI == 0 || NT == 2, "the SwiGLU epilogue owns one up tile and one gate tile");
@@ -934,7 +1034,8 @@ int launch_small(Kern kern, const GemvPlan& p, const GemvArgs& a, hipStream_t st
 #define SMALL_WAVES(NTv, Pv, Ev) SMALL_CASE(NTv, 4, Pv, Ev) SMALL_CASE(NTv, 8, Pv, Ev) SMALL_CASE(NTv, 16, Pv, Ev)
 #define SMALL_FORMS                                                                              \
   SMALL_WAVES(1, 0, 0) SMALL_WAVES(1, 1, 0) SMALL_WAVES(1, 4, 0) SMALL_WAVES(2, 0, 1) \
-  SMALL_WAVES(2, 1, 1) SMALL_WAVES(2, 4, 1)
+  SMALL_WAVES(2, 1, 1) SMALL_WAVES(2, 4, 1) SMALL_WAVES(1, 8, 0) SMALL_WAVES(2, 8, 1) \
+  SMALL_WAVES(1, 9, 0) SMALL_WAVES(2, 9, 1) SMALL_WAVES(1, 10, 0) SMALL_WAVES(2, 10, 1)
 
 #define ROT_CASE(GPAv, NTv, Wv, Pv, Ev)                                                   \
   if (gpa == GPAv && p.nt == NTv && p.waves == Wv && p.pro == Pv && p.epi == Ev)          \
@@ -946,9 +1047,19 @@ int launch_small(Kern kern, const GemvPlan& p, const GemvArgs& a, hipStream_t st
 
 int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, bool pro, bool epi,
                      void* stream) {
-  const GemvPlan p = plan_gemv(a.M, a.N, a.K, true, pro, epi);
+  GemvPlan p = plan_gemv(a.M, a.N, a.K, true, pro, epi);
   const u32x4* w = (const u32x4*)wt;
-  if (p.mt == 1 && p.xlds && a.M <= 4 && (int64_t)(a.N >> 4) * (a.K >> 7) * 1024 < (1ll << 31) && g_dbg_small && p.pro >= 0) {
+  const bool small_ok = p.mt == 1 && p.xlds && a.M <= 4 && (int64_t)(a.N >> 4) * (a.K >> 7) * 1024 < (1ll << 31) && g_dbg_small;
+  if (a.ssq_in || a.ssq_out) {  // chained norms: only the lean kernel speaks that protocol
+    if (!small_ok || (a.ssq_out && epi)) return O355_EUNSUPPORTED;
+    if (a.ssq_in) {
+      const int slice_kib = ((((a.K >> 7) + p.waves - 1) / p.waves) * 256 + 1023) >> 10;  // per row, largest wave
+      const int pieces = a.M * slice_kib;
+      if (!pro || pieces > kChainPieces || (a.K >> 4) > 1024) return O355_EUNSUPPORTED;
+      p.pro = pieces <= 1 ? 8 : (pieces <= 2 ? 9 : 10);
+    }
+  }
+  if (small_ok && p.pro >= 0) {
     SMALL_FORMS
     return O355_EUNSUPPORTED;
   }
@@ -1007,6 +1118,21 @@ extern "C" int olmo355_w4_gemv_fused(const uint16_t* x, const uint16_t* resid, c
   if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
   if (M > 64 || (K & 127) || (N & 15)) return O355_EUNSUPPORTED;
   const GemvArgs a{x, resid, norm_w, x_out, y, eps, M, N, K};
+  const bool pro = resid != nullptr, epi = swiglu != 0;
+  const int chk = check_fused(a, pro, epi);
+  if (chk != O355_OK) return chk;
+  return w4_gemv_dispatch(a, wt, st, zt, pro, epi, stream);
+}
+
+extern "C" int olmo355_w4_gemv_chain(const uint16_t* x, const uint16_t* resid, const uint16_t* norm_w, float eps,
+                                     uint16_t* x_out, const float* ssq_in, const uint32_t* wt, const uint16_t* st,
+                                     const uint8_t* zt, uint16_t* y, float* ssq_out, int M, int N, int K, int swiglu,
+                                     void* stream) {
+  if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
+  if ((resid != nullptr) != (ssq_in != nullptr)) return O355_EINVAL;  // the prologue here is the chained one
+  if (M > 4 || (K & 127) || (N & 15)) return O355_EUNSUPPORTED;
+  GemvArgs a{x, resid, norm_w, x_out, y, eps, M, N, K};
+  a.ssq_in = ssq_in, a.ssq_out = ssq_out;
   const bool pro = resid != nullptr, epi = swiglu != 0;
   const int chk = check_fused(a, pro, epi);
   if (chk != O355_OK) return chk;

@@ -227,6 +227,7 @@ class OLMo(nn.Module):
         c = self.config
         n_pos = max(self.max_cache_len, c.max_sequence_length)
         self._rope = ops.rope_tables(c.head_dim, float(c.rope_theta), n_pos, self.device)
+        self._chain_ok = {}  # rows -> whether the chained decode block covers this model
         self._prepared = True
         return self
 
@@ -302,7 +303,7 @@ class OLMo(nn.Module):
     def _linear(self, m: nn.Module, x: torch.Tensor) -> torch.Tensor:
         return m(x)
 
-    def _attention(self, blk, qkv, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max):
+    def _attention(self, blk, qkv, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max, qk_ssq=None):
         c = self.config
         H, Hkv, hd = c.n_heads, c.effective_n_kv_heads, c.head_dim
         sin, cos = self._rope
@@ -312,7 +313,7 @@ class OLMo(nn.Module):
         if decode:
             att = ops.attn_decode_fused(qkv, qw, kw, sin, cos, kc, vc, self._decode_ws(B, n_keys_max), B, H, Hkv, hd,
                                         past_len, n_keys_max, c.layer_norm_eps, key_bias=key_bias,
-                                        past_len_dev=graph_pos)
+                                        past_len_dev=graph_pos, qk_ssq=qk_ssq)
             if att is not None:
                 return att
         q = ops.qknorm_rope_kvwrite(qkv, qw, kw, sin, cos, kc, vc, B, T, H, Hkv, hd, past_len, c.layer_norm_eps,
@@ -362,6 +363,51 @@ class OLMo(nn.Module):
                                 swiglu_out=True)
         f = self._linear(blk.ff_out, u)
         return x, (f, blk.ff_norm.weight.data)
+
+    # The same block for at most 4 rows of int4 weights, with the three norms *chained*: the launch that
+    # produces a tensor also leaves the sums of squares of its 16-column tiles, and the launch that
+    # normalises the tensor (att_proj / ff_proj prologue, QK-norm inside attention) adds those up instead
+    # of re-reading the row and synchronising its workgroup.
+    #   pend   (f_prev, ff_norm weight, ssq of f_prev) or None
+    def _block_decode_chain(self, blk, x, pend, kc, vc, B, past_len, key_bias, graph_pos, n_keys_max):
+        eps = self.config.layer_norm_eps
+        qknorm = blk.q_norm is not None
+        if pend is None:
+            qkv, _, ssq_qkv = ops.w4_linear_chain(x, blk.att_proj.tiled, want_ssq=qknorm)
+        else:
+            qkv, x, ssq_qkv = ops.w4_linear_chain(pend[0], blk.att_proj.tiled, resid=x, norm_w=pend[1], eps=eps,
+                                                  ssq_in=pend[2], want_ssq=qknorm)
+        att = self._attention(blk, qkv, kc, vc, B, 1, past_len, key_bias, graph_pos, n_keys_max, qk_ssq=ssq_qkv)
+        a, _, ssq_a = ops.w4_linear_chain(att, blk.attn_out.tiled, want_ssq=True)
+        u, x, _ = ops.w4_linear_chain(a, blk.ff_proj.tiled, resid=x, norm_w=blk.attn_norm.weight.data, eps=eps,
+                                      ssq_in=ssq_a, swiglu_out=True)
+        f, _, ssq_f = ops.w4_linear_chain(u, blk.ff_out.tiled, want_ssq=True)
+        return x, (f, blk.ff_norm.weight.data, ssq_f)
+
+    def _chain_decode_ok(self, M: int) -> bool:
+        """Whether :meth:`_block_decode_chain` covers this model at ``M`` rows: decided once per ``M`` by
+        issuing block 0's four linears in chained form on scratch inputs (outside any graph capture)."""
+        cached = self._chain_ok.get(M)
+        if cached is not None:
+            return cached
+        blk = self.transformer["blocks"][0]
+        lin = (blk.att_proj, blk.attn_out, blk.ff_proj, blk.ff_out)
+        ok = M <= 4 and all(isinstance(m, QuantLinear) for m in lin) and not torch.cuda.is_current_stream_capturing()
+        if ok:
+            d = self.config.d_model
+            x = torch.zeros(M, 1, d, dtype=torch.bfloat16, device=self.device)
+            nw = blk.attn_norm.weight.data
+            s_in = torch.zeros(M, d // 16, dtype=torch.float32, device=self.device)
+            r1 = ops.w4_linear_chain(x, blk.att_proj.tiled, resid=x, norm_w=nw, eps=1e-6, ssq_in=s_in, want_ssq=True)
+            r2 = ops.w4_linear_chain(x, blk.attn_out.tiled, want_ssq=True)
+            r3 = ops.w4_linear_chain(x, blk.ff_proj.tiled, resid=x, norm_w=nw, eps=1e-6, ssq_in=s_in, swiglu_out=True)
+            ok = r1 is not None and r2 is not None and r3 is not None
+            if ok:
+                ok = ops.w4_linear_chain(r3[0], blk.ff_out.tiled, want_ssq=True) is not None
+        elif torch.cuda.is_current_stream_capturing():
+            return False  # not decided yet: do not record a probe into the graph
+        self._chain_ok[M] = ok
+        return ok
 
     # ------------------------------------------------------------------------------------------
     # forward: olmo/model.py:1253-1465
@@ -441,6 +487,7 @@ class OLMo(nn.Module):
         n_keys_max = cache.capacity if graph_pos is not None else past_len + T
         hidden: List[torch.Tensor] = []
         fused = T == 1 and cache is not None and self._fused_decode_ok(B, collect_hidden)
+        chain = fused and self._chain_decode_ok(B)
         pend = None
         for i, blk in enumerate(self.transformer["blocks"]):
             if collect_hidden:
@@ -449,7 +496,9 @@ class OLMo(nn.Module):
                 kc, vc = cache.k[i], cache.v[i]
             else:
                 kc, vc = self._scratch_cache(B, T)
-            if fused:
+            if chain:
+                x, pend = self._block_decode_chain(blk, x, pend, kc, vc, B, past_len, key_bias, graph_pos, n_keys_max)
+            elif fused:
                 x, pend = self._block_decode_fused(blk, x, pend, kc, vc, B, past_len, key_bias, graph_pos, n_keys_max)
             else:
                 x = self._block(blk, x, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max)

@@ -205,6 +205,33 @@ def linear_fused(x: torch.Tensor, w, resid: Optional[torch.Tensor] = None, norm_
     return (swiglu(y) if swiglu_out else y), x_new
 
 
+def w4_linear_chain(x: torch.Tensor, w: "W4Tiled", resid: Optional[torch.Tensor] = None,
+                    norm_w: Optional[torch.Tensor] = None, eps: float = 0.0, ssq_in: Optional[torch.Tensor] = None,
+                    swiglu_out: bool = False, want_ssq: bool = False):
+    """Decode-step int4 linear (at most 4 rows) with the norms chained between launches.  Returns
+    ``(y, x_new, ssq)`` or ``None`` when the kernel does not cover the shape.  ``ssq`` (float32
+    ``[M, N/16]``, only with ``want_ssq``) holds the sum of squares of every 16-column tile of ``y``: hand
+    it to the launch that normalises ``y`` (``ssq_in`` here, ``qk_ssq`` of :func:`attn_decode_fused`).
+    With ``resid``: ``x_new = resid + rmsnorm(x; norm_w, eps)`` using ``ssq_in`` for the mean square."""
+    _dev(x, resid, norm_w, ssq_in)
+    if x.dtype != torch.bfloat16 or not isinstance(w, W4Tiled):
+        return None
+    M = x.numel() // w.K
+    if M < 1 or M > 4 or (resid is None) != (ssq_in is None) or (want_ssq and swiglu_out):
+        return None
+    n_out = w.N // 2 if swiglu_out else w.N
+    y = torch.empty(*x.shape[:-1], n_out, dtype=torch.bfloat16, device=x.device)
+    x_new = torch.empty_like(x) if resid is not None else x
+    ssq = torch.empty(M, w.N // 16, dtype=torch.float32, device=x.device) if want_ssq else None
+    st = lib().olmo355_w4_gemv_chain(_p(x), _p(resid), _p(norm_w), float(eps), _p(x_new) if resid is not None else None,
+                                     _p(ssq_in), _p(w.wt), _p(w.st), _p(w.zt), _p(y), _p(ssq), M, w.N, w.K,
+                                     int(swiglu_out), _stream())
+    if st == 2:
+        return None
+    check("olmo355_w4_gemv_chain", st)
+    return y, x_new, ssq
+
+
 def f32_linear(x: torch.Tensor, weight_nk: torch.Tensor) -> torch.Tensor:
     _dev(x, weight_nk)
     if x.dtype != torch.float32 or weight_nk.dtype != torch.float32:
@@ -364,12 +391,15 @@ def attn_decode(q, kcache, vcache, ws, B: int, H: int, Hkv: int, hd: int, past_l
 
 def attn_decode_fused(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, ws, B: int, H: int, Hkv: int, hd: int,
                       past_len: int, n_keys_max: int, eps: float, key_bias: Optional[torch.Tensor] = None,
-                      past_len_dev: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+                      past_len_dev: Optional[torch.Tensor] = None,
+                      qk_ssq: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """One new token per sequence: QK-norm, rotary, cache append and attention in one pass.  Returns
     ``None`` when the fused kernel does not cover the shape (use the separate calls then)."""
-    _dev(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, ws, key_bias, past_len_dev)
+    _dev(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, ws, key_bias, past_len_dev, qk_ssq)
     if qkv.dtype != torch.bfloat16 or hd not in (64, 128):
         return None
+    if qk_ssq is not None and (qk_ssq.dtype != torch.float32 or qk_ssq.numel() != B * (H + 2 * Hkv) * hd // 16):
+        raise ValueError("qk_ssq: float32 [B, (H + 2 Hkv) hd / 16] expected")
     if qkv.numel() != B * (H + 2 * Hkv) * hd or kcache.shape != vcache.shape or kcache.shape[1] != Hkv or kcache.shape[3] != hd:
         raise ValueError("qkv / cache shape mismatch")
     Lmax, n_pos = kcache.shape[2], sin_tab.shape[0]
@@ -380,7 +410,7 @@ def attn_decode_fused(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache,
     st = lib().olmo355_attn_decode_fused(_p(qkv), _p(q_weight), _p(k_weight), _p(sin_tab), _p(cos_tab), _p(kcache),
                                          _p(vcache), _p(key_bias), _p(out), _p(ws), B, H, Hkv, hd, Lmax, n_pos, past_len,
                                          _p(past_len_dev), n_keys_max, key_bias.shape[1] if key_bias is not None else 0,
-                                         float(eps), _dt(qkv), _stream())
+                                         float(eps), _p(qk_ssq), _dt(qkv), _stream())
     if st == 2:
         return None
     check("olmo355_attn_decode_fused", st)

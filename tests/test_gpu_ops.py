@@ -503,3 +503,58 @@ def test_attn_decode_fused(dev, qknorm, B, past, H, Hkv, hd):
         assert torch.allclose(out3.cpu().float(), ref3.float(), rtol=2 ** -7, atol=2 ** -7)
     else:
         assert torch.allclose(out3.float(), out.float(), rtol=2 ** -8, atol=2 ** -10)
+    # the q and k sums of squares handed over per 16-column tile instead of being recomputed from the rows
+    if qknorm:
+        kc4, vc4 = fresh()
+        ssq = (qkv.float() ** 2).view(B, -1, 16).sum(-1)
+        out4 = ops.attn_decode_fused(qkv.to(dev), d(qw), d(kw), sin, cos, kc4, vc4, ws, B, H, Hkv, hd, past, past + 1, eps,
+                                     qk_ssq=ssq.to(dev))
+        assert torch.allclose(out4.float(), out.float(), rtol=2 ** -7, atol=2 ** -7)
+        assert torch.allclose(kc4[:, :, past].float(), kc[:, :, past].float(), rtol=2 ** -7, atol=2 ** -7)
+
+
+@pytest.mark.parametrize("M", [1, 2, 4])
+@pytest.mark.parametrize("N,K,epi", [(4096, 4096, False), (12288, 4096, False), (22016, 4096, True), (768, 512, False),
+                                     (4096, 11264, False), (1024, 1024, True)])
+def test_w4_gemv_chain(dev, M, N, K, epi):
+    """Norms chained between launches: the producer's per-tile sums of squares equal those of its output,
+    and a consumer fed with them gives the same x' and y as the oracle's norm + linear (+ SwiGLU)."""
+    say("w4_gemv_chain", M, N, K, epi)
+    ops = _ops()
+    gen = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    resid = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    nw = (1 + 0.1 * torch.randn(K, generator=gen)).to(torch.bfloat16)
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=N + K)
+    Wf = ow4.dequantize(qw, qz, sc, 128).float()
+    w = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    if (M + 1) * K * 2 > 64 * 1024:
+        # the activations (plus a zero row) no longer fit the kernel's LDS budget: the call declines
+        assert ops.w4_linear_chain(a.to(dev), w, want_ssq=not epi, swiglu_out=epi) is None
+        return
+    # producer side: plain product, sums of squares of its own output
+    if not epi:
+        r = ops.w4_linear_chain(a.to(dev), w, want_ssq=True)
+        assert r is not None
+        y0, _, ssq0 = r
+        assert torch.equal(y0, ops.w4_linear(a.to(dev), w)) or torch.allclose(y0.float(), ops.w4_linear(a.to(dev), w).float(),
+                                                                              rtol=2 ** -7, atol=2 ** -7 * y0.float().abs().max().item())
+        want = (y0.float().cpu() ** 2).view(M, -1, 16).sum(-1)
+        assert torch.allclose(ssq0.cpu(), want, rtol=1e-5, atol=1e-6 * want.max().item())
+    # consumer side
+    ssq_in = (a.float() ** 2).view(M, -1, 16).sum(-1)
+    r = ops.w4_linear_chain(a.to(dev), w, resid=resid.to(dev), norm_w=nw.to(dev), eps=1e-6, ssq_in=ssq_in.to(dev),
+                            swiglu_out=epi, want_ssq=not epi)
+    assert r is not None
+    y, x_new, ssq = r
+    x_ref = resid + om.rms_norm(a, nw, 1e-6)
+    y_ref = (x_ref.float() @ Wf).to(torch.bfloat16)
+    if epi:
+        y_ref = om.swiglu(y_ref)
+    dx = (x_new.cpu().float() - x_ref.float()).abs()
+    assert (dx <= 2.0 ** (torch.floor(torch.log2(x_ref.float().abs().clamp_min(1e-30))) - 7)).all()
+    scale = y_ref.float().abs().max().item()
+    assert (y.cpu().float() - y_ref.float()).abs().max().item() <= 2 ** -6 * scale
+    if ssq is not None:
+        want = (y.float().cpu() ** 2).view(M, -1, 16).sum(-1)
+        assert torch.allclose(ssq.cpu(), want, rtol=1e-5, atol=1e-6 * want.max().item())
