@@ -477,7 +477,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     const float* __restrict__ sin_t, const float* __restrict__ cos_t, uint16_t* __restrict__ kc,
     uint16_t* __restrict__ vc, const float* __restrict__ key_bias, float* __restrict__ ws, int H, int Hkv, int Lmax,
     int n_pos, int past_len, const int32_t* __restrict__ past_dev, int nchunks_max, int bias_stride, float eps,
-    const float* __restrict__ qk_ssq) {
+    const float* __restrict__ qk_ssq, uint16_t* __restrict__ out, int* __restrict__ tickets) {
   constexpr int LPK = HD / 8, KPI = 64 / LPK, ITERS = kDecodeKeysPerWave / KPI;
   constexpr int HALF = HD / 2, CPH = HD / 16;  // pair chunks per head
   __shared__ float red_o[4][HD];
@@ -679,19 +679,70 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
 #pragma unroll
   for (int w = 1; w < 4; ++w) mm = fmaxf(mm, red_ml[w][0]);
   float* dst = ws + (((int64_t)b * H + h) * nchunks_max + chunk) * (HD + 2);
+  float ov = 0.f, lv = 0.f;
   if (tid < HD) {
-    float ov = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) ov += red_o[w][tid] * __expf(red_ml[w][0] - mm);
-    dst[tid] = ov;
   }
   if (tid == 0) {
-    float lv = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) lv += red_ml[w][1] * __expf(red_ml[w][0] - mm);
-    dst[HD] = mm;
-    dst[HD + 1] = lv;
   }
+  if (!tickets) {  // partials merged by attn_decode_combine_kernel
+    if (tid < HD) dst[tid] = ov;
+    if (tid == 0) dst[HD] = mm, dst[HD + 1] = lv;
+    return;
+  }
+  // ---- 4. the last workgroup of a (batch, head) to finish merges the partials itself ---------------------
+  // Partials are published with device-scope stores (they bypass the per-XCD L2), each wave waits
+  // until its stores are acknowledged, then one thread takes a ticket with a device-scope atomic;
+  // whoever draws the last ticket reads all partials back with device-scope loads.  No workgroup
+  // ever waits for another one.
+  if (tid < HD) __hip_atomic_store(dst + tid, ov, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (tid == 0) {
+    __hip_atomic_store(dst + HD, mm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(dst + HD + 1, lv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, false));  // vmcnt(0): this wave's stores have landed
+  __syncthreads();
+  __shared__ int s_last;
+  const int nact = min((L + kDecodeChunk - 1) / kDecodeChunk, nchunks_max);
+  if (tid == 0) {
+    int* tk = tickets + b * H + h;
+    const int t = __hip_atomic_fetch_add(tk, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = (t == nact - 1);
+    if (t == nact - 1) __hip_atomic_store(tk, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+  }
+  __syncthreads();
+  if (!s_last || tid >= HD) return;
+  const float* src = ws + ((int64_t)b * H + h) * nchunks_max * (HD + 2);
+  constexpr int UN = 16;
+  float gm = -INFINITY, go = 0.f, gl = 0.f;
+  for (int c0 = 0; c0 < nact; c0 += UN) {
+    float m[UN], l[UN], o[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u)
+      if (c0 + u < nact) {
+        const float* pp = src + (c0 + u) * (HD + 2);
+        m[u] = __hip_atomic_load(pp + HD, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        l[u] = __hip_atomic_load(pp + HD + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        o[u] = __hip_atomic_load(pp + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    float rm = gm;
+#pragma unroll
+    for (int u = 0; u < UN; ++u)
+      if (c0 + u < nact) rm = fmaxf(rm, m[u]);
+    const float a = __expf(gm - rm);  // exp(-inf) = 0 on the first round
+    go *= a, gl *= a;
+#pragma unroll
+    for (int u = 0; u < UN; ++u)
+      if (c0 + u < nact) {
+        const float wgt = __expf(m[u] - rm);
+        go += o[u] * wgt, gl += l[u] * wgt;
+      }
+    gm = rm;
+  }
+  out[((int64_t)b * H + h) * HD + tid] = f32_to_bf16_bits(go / gl);
 }
 
 template <int DT, int HD>
@@ -751,7 +802,7 @@ extern "C" int olmo355_attn_prefill(const void* q, const void* kcache, const voi
 extern "C" int64_t olmo355_attn_decode_workspace_bytes(int B, int H, int hd, int n_keys_max) {
   if (B <= 0 || H <= 0 || hd <= 0 || n_keys_max <= 0) return 0;
   const int64_t nch = (n_keys_max + kDecodeChunk - 1) / kDecodeChunk;
-  return (int64_t)B * H * nch * (hd + 2) * 4;
+  return (int64_t)B * H * 4 + (int64_t)B * H * nch * (hd + 2) * 4;  // ticket counters, then the partials
 }
 
 extern "C" int olmo355_attn_decode(const void* q, const void* kcache, const void* vcache, const float* key_bias,
@@ -765,7 +816,7 @@ extern "C" int olmo355_attn_decode(const void* q, const void* kcache, const void
   if (key_bias && bias_stride < n_keys_max) return O355_EINVAL;
   hipStream_t s = as_stream(stream);
 #define DECODE(DTv, HDv)                                                                                          \
-  return launch_decode<DTv, HDv>(q, kcache, vcache, key_bias, out, (float*)ws, B, H, Hkv, Lmax, past_len, \
+  return launch_decode<DTv, HDv>(q, kcache, vcache, key_bias, out, (float*)ws + (int64_t)B * H, B, H, Hkv, Lmax, past_len, \
                                  past_len_dev, n_keys_max, bias_stride, s)
   if (dtype == O355_BF16) {
     if (hd == 128) DECODE(O355_BF16, 128);
@@ -1049,9 +1100,15 @@ extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const 
 #define FUSED(HDv, QVv)                                                                                                 \
   hipLaunchKernelGGL((attn_decode_fused_kernel<HDv, QVv>), dim3(nch, H, B), dim3(256), 0, s, (const uint16_t*)qkv,   \
                      (const uint16_t*)qw, (const uint16_t*)kw, sin_tab, cos_tab, (uint16_t*)kcache, (uint16_t*)vcache, \
-                     key_bias, (float*)ws, H, Hkv, Lmax, n_pos, past_len, past_len_dev, nch, bias_stride, eps, qk_ssq); \
+                     key_bias, (float*)ws, H, Hkv, Lmax, n_pos, past_len, past_len_dev, nch, bias_stride, eps, qk_ssq, \
+                     (uint16_t*)out, tickets);                                                                         \
+  if (!tickets)                                                                                                        \
   hipLaunchKernelGGL((attn_decode_combine_kernel<O355_BF16, HDv>), dim3(H, B), dim3(HDv), 0, s, (const float*)ws, out, \
                      H, past_len, past_len_dev, nch)
+  // the workspace starts with one ticket counter per (batch, head): zero on entry (zeroed at allocation,
+  // reset by the workgroup that draws the last ticket), then the partials
+  int* tickets = g_dbg_attn_mode == 2 ? nullptr : reinterpret_cast<int*>(ws);
+  ws = reinterpret_cast<float*>(ws) + (int64_t)B * H;
   const int qv = (H * hd / 8 + 255) / 256;
   if (hd == 128) {
     if (qv <= 1) { FUSED(128, 1); } else if (qv <= 2) { FUSED(128, 2); } else { FUSED(128, 4); }
