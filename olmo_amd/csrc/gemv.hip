@@ -694,12 +694,14 @@ struct ChainNorm {
 // request leaves.  This variant keeps the preamble short: buffer loads with scalar offsets (no
 // per-lane 64-bit address arithmetic), the activations copied memory -> LDS directly (no registers,
 // no VALU), all weight requests of the wave issued before anything else is waited for, the sums of
-// the activations from the matrix cores (B = ones) instead of a staging pass.  Four groups share an
-// accumulator as in w4_gemv_rot_kernel (GPA = 4).
-template <int NT, int WAVES, int PRO, int EPI>
+// the activations from the matrix cores (B = ones) instead of a staging pass.  GPA = 4, 2 or 1 groups
+// share an accumulator as in w4_gemv_rot_kernel (M <= 4, 8, 16); the norm prologues exist for GPA = 4.
+template <int GPA, int NT, int WAVES, int PRO, int EPI>
 __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u32x4* __restrict__ wt,
                                                    const uint16_t* __restrict__ st, const uint8_t* __restrict__ zt) {
-  constexpr int GPA = 4;
+  constexpr int RP = 16 / GPA;  // operand rows per group slot
+  constexpr int KQS = 4 / GPA;  // lane row blocks per slot
+  static_assert(PRO == 0 || GPA == 4, "the norm prologues are written for M <= 4");
   extern __shared__ __align__(16) unsigned char smem[];
   const int M = args.M, K = args.K;
   const int G = K >> 7, ntiles = args.N >> 4, nvec = K >> 3;
@@ -707,7 +709,7 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
   // LDS: x rows [M][K], a zero row [K], then the reduction area
   const int red_off = xbytes + max(K * 2, 1024);  // a direct copy may run up to 1 KiB past the rows (zeros)
   uint16_t* xl = reinterpret_cast<uint16_t*>(smem);
-  float* red = reinterpret_cast<float*>(smem + red_off);  // [WAVES][NT*4][16]
+  float* red = reinterpret_cast<float*>(smem + red_off);  // [WAVES][NT][RP rows][16 columns]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, kq = lane >> 4;
@@ -720,7 +722,8 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
   const __amdgpu_buffer_rsrc_t rw = make_rsrc(wt, (int64_t)ntiles * G * 1024);
   const __amdgpu_buffer_rsrc_t rs = make_rsrc(st, (int64_t)ntiles * G * 32);
   const __amdgpu_buffer_rsrc_t rz = make_rsrc(zt, (int64_t)ntiles * G * 8);
-  const int wvoff = lane * 16, svoff = lane * 2, zvoff = lane >> 1;
+  const int ul = kq / KQS;  // the slot whose results this lane holds
+  const int wvoff = lane * 16, svoff = (ul * 16 + col) * 2, zvoff = ul * 8 + (col >> 1);
 
   u32x4 w[GPA][NT];
   uint32_t s16c[NT], z8c[NT], s16n[NT], z8n[NT];
@@ -732,7 +735,7 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
     for (int nt = 0; nt < NT; ++nt)
       w[u][nt] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, wvoff, (tg[nt] + gc) * 1024, 2));
   };
-  // the lanes of row block kq hold the scale and zero of group base+kq: one contiguous request each
+  // the lanes of slot ul hold the scale and zero of group base+ul: one contiguous request each
   auto issue_sz = [&](uint32_t (&s16)[NT], uint32_t (&z8)[NT], int base) {
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -775,11 +778,11 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
     norm.finish(args, xl, red, wave);
   }
 
-  // operand row `col` of slot u is activation row col - 4u when that is in [0, M), else the zero row
+  // operand row `col` of slot u is activation row col - u*RP when that is in [0, M), else the zero row
   int xoff[GPA];
 #pragma unroll
   for (int u = 0; u < GPA; ++u) {
-    const int rel = col - 4 * u;
+    const int rel = col - RP * u;
     xoff[u] = ((rel >= 0 && rel < M) ? rel : M) * K + 8 * kq;
   }
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -825,27 +828,28 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
     }
   }
 
-  // ---- reduce: the four row blocks inside the wave, then the waves through LDS, in fixed order ----
+  // ---- reduce: the slots inside the wave, then the waves through LDS, in fixed order ----------------
+  // this lane's rows are m = 4 (kq % KQS) + r; lanes kq and kq + KQS, ... hold the other slots' shares
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      if (r < M) {
-        float v = acc[nt][r];
-        v += __shfl_xor(v, 16, 64);
-        v += __shfl_xor(v, 32, 64);
-        if (lane < 16) red[(wave * NT * 4 + nt * 4 + r) * 16 + lane] = v;
-      }
+    for (int r = 0; r < 4; ++r) {
+      if (GPA == 4 && r >= M) continue;  // rows past M hold nothing (uniform: with GPA = 4 a lane's rows are r)
+      float v = acc[nt][r];
+      if constexpr (GPA == 4) v += __shfl_xor(v, 16, 64);
+      if constexpr (GPA >= 2) v += __shfl_xor(v, 32, 64);
+      if (kq < KQS) red[((wave * NT + nt) * RP + 4 * kq + r) * 16 + col] = v;
+    }
   __syncthreads();
   auto total_of = [&](int nt, int m, int c) {
     float v = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < WAVES; ++wv) v += red[(wv * NT * 4 + nt * 4 + m) * 16 + c];
+    for (int wv = 0; wv < WAVES; ++wv) v += red[((wv * NT + nt) * RP + m) * 16 + c];
     return v;
   };
   if constexpr (EPI == 0) {
-    if (tid < NT * 64) {
-      const int c = tid & 15, m = (tid >> 4) & 3, nt = tid >> 6;
+    for (int i = tid; i < NT * RP * 16; i += WAVES * 64) {  // whole waves: 16 lanes = one (row, tile)
+      const int c = i & 15, m = (i >> 4) % RP, nt = (i >> 4) / RP;
       const bool live = tile[nt] < ntiles && m < M;
       const float v = live ? round_bf16(total_of(nt, m, c)) : 0.f;
       if (live) args.y[(int64_t)m * args.N + tile[nt] * 16 + c] = f32_to_bf16_bits(v);
@@ -856,7 +860,7 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
     }
   } else {
     static_assert(EPI == 0 || NT == 2, "the SwiGLU epilogue owns one up tile and one gate tile");
-    if (tid < 64) {
+    if (tid < RP * 16) {
       const int c = tid & 15, m = tid >> 4;
       if (m < M) {
         const float up = round_bf16(total_of(0, m, c));  // the Linear's bf16 output
@@ -868,11 +872,11 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
   }
 }
 
-template <int NT, int WAVES, int PRO, int EPI>
+template <int GPA, int NT, int WAVES, int PRO, int EPI>
 __global__ __launch_bounds__(WAVES * 64) void w4_gemv_small_kernel(GemvArgs args, const u32x4* __restrict__ wt,
                                                                    const uint16_t* __restrict__ st,
                                                                    const uint8_t* __restrict__ zt) {
-  w4_gemv_small_body<NT, WAVES, PRO, EPI>(args, wt, st, zt);
+  w4_gemv_small_body<GPA, NT, WAVES, PRO, EPI>(args, wt, st, zt);
 }
 
 // ---- dense bf16 --------------------------------------------------------------------------------------------
@@ -945,7 +949,8 @@ struct GemvPlan {
 // Experiment hook (not part of the public interface): overrides waves / xlds when >= 0.
 int g_dbg_waves = -1, g_dbg_xlds = -1, g_dbg_small = 1;
 
-constexpr int kXldsMaxBytes = 64 * 1024;
+constexpr int kXldsMaxBytes = 64 * 1024;     // activations (+ zero row) in LDS, kernels for M <= 16
+constexpr int kSmallMaxBytes = 128 * 1024;   // the same for the lean M <= 4 kernel (160 KiB of LDS per CU)
 
 // u (pieces in flight per wave) is fixed per format: 2 KiB-groups for int4, 8 (4 for M > 16) 32-row steps for bf16
 inline GemvPlan plan_gemv(int M, int N, int K, bool w4, bool pro, bool epi) {
@@ -987,7 +992,7 @@ int launch_gemv(Kern kern, const GemvPlan& p, const GemvArgs& a, hipStream_t str
 
 int check_fused(const GemvArgs& a, bool pro, bool epi) {
   if (pro && (!a.resid || !a.norm_w || !a.x_out || a.M > 16 || (a.K & 511))) return O355_EUNSUPPORTED;
-  if ((pro || epi) && (int64_t)(a.M + 1) * a.K * 2 > kXldsMaxBytes) return O355_EUNSUPPORTED;
+  if ((pro || epi) && (int64_t)(a.M + 1) * a.K * 2 > ((a.M <= 4 || !pro) ? kSmallMaxBytes : kXldsMaxBytes)) return O355_EUNSUPPORTED;
   if (epi && ((a.N & 31) || a.M > 16)) return O355_EUNSUPPORTED;
   return O355_OK;
 }
@@ -1018,7 +1023,7 @@ int launch_small(Kern kern, const GemvPlan& p, const GemvArgs& a, hipStream_t st
                  const uint8_t* zt) {
   const int xbytes = a.M * a.K * 2;
   const int red_off = xbytes + std::max(a.K * 2, 1024);
-  const size_t lds = (size_t)red_off + (size_t)p.waves * p.nt * 4 * 16 * 4;
+  const size_t lds = (size_t)red_off + (size_t)p.waves * p.nt * (a.M <= 4 ? 4 : (a.M <= 8 ? 8 : 16)) * 16 * 4;
   if (lds > 48 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
     return O355_ELAUNCH;
@@ -1028,9 +1033,13 @@ int launch_small(Kern kern, const GemvPlan& p, const GemvArgs& a, hipStream_t st
   O355_CHECK_LAUNCH();
 }
 
-#define SMALL_CASE(NTv, Wv, Pv, Ev)                                        \
-  if (p.nt == NTv && p.waves == Wv && p.pro == Pv && p.epi == Ev)          \
-    return launch_small(w4_gemv_small_kernel<NTv, Wv, Pv, Ev>, p, a, as_stream(stream), w, st, zt);
+#define SMALL_CASE_G(GPAv, NTv, Wv, Pv, Ev)                                                 \
+  if (sgpa == GPAv && p.nt == NTv && p.waves == Wv && p.pro == Pv && p.epi == Ev)           \
+    return launch_small(w4_gemv_small_kernel<GPAv, NTv, Wv, Pv, Ev>, p, a, as_stream(stream), w, st, zt);
+#define SMALL_CASE(NTv, Wv, Pv, Ev) SMALL_CASE_G(4, NTv, Wv, Pv, Ev)
+#define SMALL_PLAIN(GPAv)                                                                                        \
+  SMALL_CASE_G(GPAv, 1, 4, 0, 0) SMALL_CASE_G(GPAv, 1, 8, 0, 0) SMALL_CASE_G(GPAv, 1, 16, 0, 0)                   \
+  SMALL_CASE_G(GPAv, 2, 4, 0, 1) SMALL_CASE_G(GPAv, 2, 8, 0, 1) SMALL_CASE_G(GPAv, 2, 16, 0, 1)
 #define SMALL_WAVES(NTv, Pv, Ev) SMALL_CASE(NTv, 4, Pv, Ev) SMALL_CASE(NTv, 8, Pv, Ev) SMALL_CASE(NTv, 16, Pv, Ev)
 #define SMALL_FORMS                                                                              \
   SMALL_WAVES(1, 0, 0) SMALL_WAVES(1, 1, 0) SMALL_WAVES(1, 4, 0) SMALL_WAVES(2, 0, 1) \
@@ -1049,9 +1058,10 @@ int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, 
                      void* stream) {
   GemvPlan p = plan_gemv(a.M, a.N, a.K, true, pro, epi);
   const u32x4* w = (const u32x4*)wt;
-  const bool small_ok = p.mt == 1 && p.xlds && a.M <= 4 && (int64_t)(a.N >> 4) * (a.K >> 7) * 1024 < (1ll << 31) && g_dbg_small;
+  const int sgpa = a.M <= 4 ? 4 : (a.M <= 8 ? 2 : 1);
+  const bool small_ok = a.M <= 16 && (a.M <= 4 || p.pro == 0) && (int64_t)(a.M + 1) * a.K * 2 <= kSmallMaxBytes && (int64_t)(a.N >> 4) * (a.K >> 7) * 1024 < (1ll << 31) && g_dbg_small;
   if (a.ssq_in || a.ssq_out) {  // chained norms: only the lean kernel speaks that protocol
-    if (!small_ok || (a.ssq_out && epi)) return O355_EUNSUPPORTED;
+    if (!small_ok || a.M > 4 || (a.ssq_out && epi)) return O355_EUNSUPPORTED;
     if (a.ssq_in) {
       const int slice_kib = ((((a.K >> 7) + p.waves - 1) / p.waves) * 256 + 1023) >> 10;  // per row, largest wave
       const int pieces = a.M * slice_kib;
@@ -1061,6 +1071,8 @@ int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, 
   }
   if (small_ok && p.pro >= 0) {
     SMALL_FORMS
+    SMALL_PLAIN(2)
+    SMALL_PLAIN(1)
     return O355_EUNSUPPORTED;
   }
   if (p.mt == 1 && p.xlds) {  // M <= 16 with the activations in LDS: accumulators shared between groups

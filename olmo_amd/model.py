@@ -331,8 +331,10 @@ class OLMo(nn.Module):
         att = self._linear(blk.attn_out, att)
         x = blk.attn_norm(att, residual=x) if c.norm_after else ops.add(x, att)
         h = x if c.norm_after else blk.ff_norm(x)
-        h = self._linear(blk.ff_proj, h)
-        h = ops.swiglu(h)
+        if B * T <= 16 and self.dtype == torch.bfloat16:  # few rows: SwiGLU rides in the projection's epilogue
+            h, _ = ops.linear_fused(h, self._tiled(blk.ff_proj), swiglu_out=True)
+        else:
+            h = ops.swiglu(self._linear(blk.ff_proj, h))
         h = self._linear(blk.ff_out, h)
         return blk.ff_norm(h, residual=x) if c.norm_after else ops.add(x, h)
 

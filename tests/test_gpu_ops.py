@@ -528,7 +528,7 @@ def test_w4_gemv_chain(dev, M, N, K, epi):
     qw, qz, sc = ow4.random_quantized(K, N, 128, seed=N + K)
     Wf = ow4.dequantize(qw, qz, sc, 128).float()
     w = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
-    if (M + 1) * K * 2 > 64 * 1024:
+    if (M + 1) * K * 2 > 128 * 1024:
         # the activations (plus a zero row) no longer fit the kernel's LDS budget: the call declines
         assert ops.w4_linear_chain(a.to(dev), w, want_ssq=not epi, swiglu_out=epi) is None
         return
@@ -545,7 +545,10 @@ def test_w4_gemv_chain(dev, M, N, K, epi):
     ssq_in = (a.float() ** 2).view(M, -1, 16).sum(-1)
     r = ops.w4_linear_chain(a.to(dev), w, resid=resid.to(dev), norm_w=nw.to(dev), eps=1e-6, ssq_in=ssq_in.to(dev),
                             swiglu_out=epi, want_ssq=not epi)
-    assert r is not None
+    if r is None:
+        # a consumer may decline (more than 4 pieces of the row per lane); never for the 7B decode shapes
+        assert K > 4096
+        return
     y, x_new, ssq = r
     x_ref = resid + om.rms_norm(a, nw, 1e-6)
     y_ref = (x_ref.float() @ Wf).to(torch.bfloat16)
