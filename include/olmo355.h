@@ -164,12 +164,19 @@ int olmo355_attn_decode(const void* q, const void* kcache, const void* vcache, c
  * fused projection qkv [B, (H+2*Hkv)*hd]: bf16, hd 64 or 128; O355_EUNSUPPORTED otherwise (the caller
  * then issues the two separate calls).  Same workspace as olmo355_attn_decode.
  * qk_ssq: NULL, or the per-tile sums of squares [B][(H+2*Hkv)*hd/16] that olmo355_w4_gemv_chain left for
- * qkv (the q and k norms then do not re-read the rows). */
+ * qkv (the q and k norms then do not re-read the rows).
+ * rope_now: NULL, or the rotary rows of the current position, float [2*hd] = sin row | cos row, as kept
+ * by olmo355_rope_advance: with the position in device memory (past_len_dev) the table lookup would be a
+ * dependent load behind the whole cache stream. */
 int olmo355_attn_decode_fused(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
                               const float* cos_tab, void* kcache, void* vcache, const float* key_bias, void* out,
                               void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos, int past_len,
                               const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps,
-                              const float* qk_ssq, int dtype, void* stream);
+                              const float* qk_ssq, const float* rope_now, int dtype, void* stream);
+/* Between captured decode steps: *pos += delta, then rope_now [2*hd] = sin_tab[*pos] | cos_tab[*pos]
+ * (rows of get_rotary_embedding's tables, olmo/model.py:285-296).  delta 0 initialises rope_now. */
+int olmo355_rope_advance(int32_t* pos, int delta, const float* sin_tab, const float* cos_tab, float* rope_now, int hd,
+                         int n_pos, void* stream);
 
 /* ---- MLP activation: SwiGLU.forward (olmo/model.py:365-368) --------------------------------
  * x [rows, 2h]: first half "up", second half "gate"; out [rows, h] = silu(gate) * up. */

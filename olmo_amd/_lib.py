@@ -51,7 +51,8 @@ EXPORTS = {
     "olmo355_attn_prefill": (I, [P, P, P, P, P, I, I, I, I, I, I, I, I, I, P]),
     "olmo355_attn_decode_workspace_bytes": (L, [I, I, I, I]),
     "olmo355_attn_decode": (I, [P, P, P, P, P, P, I, I, I, I, I, I, P, I, I, I, P]),
-    "olmo355_attn_decode_fused": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, I, P]),
+    "olmo355_attn_decode_fused": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, P, I, P]),
+    "olmo355_rope_advance": (I, [P, I, P, P, P, I, I, P]),
     "olmo355_swiglu": (I, [P, P, I, I, I, P]),
     "olmo355_embedding": (I, [P, P, P, I, I, I, I, P]),
     "olmo355_add": (I, [P, P, P, L, I, P]),

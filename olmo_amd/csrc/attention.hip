@@ -477,16 +477,20 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     const float* __restrict__ sin_t, const float* __restrict__ cos_t, uint16_t* __restrict__ kc,
     uint16_t* __restrict__ vc, const float* __restrict__ key_bias, float* __restrict__ ws, int H, int Hkv, int Lmax,
     int n_pos, int past_len, const int32_t* __restrict__ past_dev, int nchunks_max, int bias_stride, float eps,
-    const float* __restrict__ qk_ssq, uint16_t* __restrict__ out, int* __restrict__ tickets) {
+    const float* __restrict__ qk_ssq, const float* __restrict__ rope_now, uint16_t* __restrict__ out,
+    int* __restrict__ tickets) {
   constexpr int LPK = HD / 8, KPI = 64 / LPK, ITERS = kDecodeKeysPerWave / KPI;
   constexpr int HALF = HD / 2, CPH = HD / 16;  // pair chunks per head
-  __shared__ float red_o[4][HD];
-  __shared__ float red_ml[4][2];
+  constexpr int ROWS = 4 * KPI;                 // partial results of the workgroup: one per (wave, key slot)
+  __shared__ __align__(16) float red_o[ROWS][HD];
+  __shared__ float red_ml[ROWS][2];
   __shared__ float red2[2][4];
   __shared__ __align__(16) float qs[HD];
   __shared__ __align__(16) u32x4 knew[HD / 8], vnew[HD / 8];
+  __shared__ int s_last;
   const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z, gsz = H / Hkv, hk = h / gsz;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int sub = lane % LPK, kslot = lane / LPK;
   const float scale = 1.f / sqrtf((float)HD);
   const float lowest = -3.3895313892515355e38f;
@@ -495,94 +499,106 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   const int kmax = min(nchunks_max * kDecodeChunk, Lmax) - 1;  // last row the launch may touch
   const int dq = H * HD, dk = Hkv * HD;
   const uint16_t* row = qkv + (int64_t)b * (dq + 2 * dk);
-
-  // ---- 1. cache loads of this wave, at addresses that do not depend on the position (rows at and
-  // past the new position are unwritten: the new one is replaced from LDS, later ones are discarded) --
-  u32x4 kreg[ITERS], vreg[ITERS];
-  float bias[ITERS];
-#pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
-    const int keyc = min(kbase + it * KPI + kslot, kmax);
-    kreg[it] = reinterpret_cast<const u32x4*>(kc)[(cbase + (int64_t)keyc * HD + sub * 8) >> 3];
-  }
-#pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
-    const int keyc = min(kbase + it * KPI + kslot, kmax);
-    vreg[it] = reinterpret_cast<const u32x4*>(vc)[(cbase + (int64_t)keyc * HD + sub * 8) >> 3];
-    bias[it] = key_bias ? key_bias[(int64_t)b * bias_stride + keyc] : 0.f;
-  }
-  // sums of squares of the q and k rows: from the projection's per-tile partials when it left them
-  // (qk_ssq[b][(dq + 2 dk) / 16], q tiles first), else from the rows themselves
   const bool norm = (qw != nullptr);
-  float sq_part = 0.f, sk_part = 0.f;
-  if (norm && qk_ssq) {
-    const float* pr = qk_ssq + (int64_t)b * ((dq + 2 * dk) >> 4);
-    for (int i = tid; i < (dq >> 4); i += 256) sq_part += pr[i];
-    for (int i = tid; i < (dk >> 4); i += 256) sk_part += pr[(dq >> 4) + i];
-  }
+
+  // ---- 0. the position.  Read from device memory (graph replay) it arrives late: every request issued
+  // after the cache rows below queues behind 30+ MB of them.  So nothing on the way to the rotated query
+  // may depend on it: the rotary rows of the current position are then taken from rope_now ([sin | cos],
+  // refreshed once per decode step by olmo355_rope_advance) rather than looked up by position, and the
+  // position itself is first needed for masking, long after it has arrived.
   const int pos = past_dev ? *past_dev : past_len;
-  const int L = pos + 1;
-  if (chunk * kDecodeChunk >= L || pos >= Lmax || pos >= n_pos || pos > kmax) return;
-  const bool owns_new = (pos / kDecodeChunk == chunk);
-  // ---- 2. the token's q and k rows (sums of squares) and this head's pieces ------------------------------
-  u32x4 qrow[QV], krow[QV];
-  if (norm && !qk_ssq) {
-#pragma unroll
-    for (int i = 0; i < QV; ++i) {
-      const int idx = tid + i * 256;
-      if (idx < (dq >> 3)) qrow[i] = reinterpret_cast<const u32x4*>(row)[idx];
-      if (idx < (dk >> 3)) krow[i] = reinterpret_cast<const u32x4*>(row + dq)[idx];
-    }
-  }
+
+  // ---- 1. this head's q / new-k pieces, norm weights, rotary rows, sums of squares; then the cache rows
+  // of this wave.  Cache rows come through a buffer resource with a scalar offset per request and the
+  // lane index as address (a wave's 64 pieces are contiguous); rows past the last one the launch may
+  // touch read as zero, rows at and past the new position are unwritten: the new one is replaced from
+  // LDS, later ones are discarded.
   // roles: threads [0,CPH) rotate q of head h; [32,32+CPH) the new key of head hk; [64,64+HD/8) copy v
-  const bool role_q = tid < CPH, role_k = owns_new && tid >= 32 && tid < 32 + CPH;
-  const bool role_v = owns_new && tid >= 64 && tid < 64 + HD / 8;
+  const bool role_q = tid < CPH, role_k = tid >= 32 && tid < 32 + CPH, role_v = tid >= 64 && tid < 64 + HD / 8;
   const int c = role_q ? tid : tid - 32, j = c * 8;
-  u32x4 x1, x2, w1, w2;
+  u32x4 x1, x2, w1, w2, vrow;
   f32x4 cs1[2], cs2[2], sn1[2], sn2[2];
   if (role_q || role_k) {
     const uint16_t* src = role_q ? row + h * HD : row + dq + hk * HD;
-    const uint16_t* wsrc = role_q ? qw + h * HD : kw + hk * HD;
     x1 = reinterpret_cast<const u32x4*>(src + j)[0];
     x2 = reinterpret_cast<const u32x4*>(src + j + HALF)[0];
     if (norm) {
+      const uint16_t* wsrc = role_q ? qw + h * HD : kw + hk * HD;
       w1 = reinterpret_cast<const u32x4*>(wsrc + j)[0];
       w2 = reinterpret_cast<const u32x4*>(wsrc + j + HALF)[0];
     }
-    const float* cp = cos_t + (int64_t)pos * HD;
-    const float* sp = sin_t + (int64_t)pos * HD;
+    const float* sp = rope_now ? rope_now : sin_t + (int64_t)min(pos, n_pos - 1) * HD;
+    const float* cp = rope_now ? rope_now + HD : cos_t + (int64_t)min(pos, n_pos - 1) * HD;
 #pragma unroll
     for (int v4 = 0; v4 < 2; ++v4) {
       cs1[v4] = reinterpret_cast<const f32x4*>(cp + j)[v4], cs2[v4] = reinterpret_cast<const f32x4*>(cp + j + HALF)[v4];
       sn1[v4] = reinterpret_cast<const f32x4*>(sp + j)[v4], sn2[v4] = reinterpret_cast<const f32x4*>(sp + j + HALF)[v4];
     }
   }
-  u32x4 vrow;
   if (role_v) vrow = reinterpret_cast<const u32x4*>(row + dq + dk + hk * HD)[tid - 64];
-
-  float rq = 1.f, rk = 1.f;
+  float sq = 0.f, sk = 0.f;
+  u32x4 qrow[QV], krow[QV];
   if (norm) {
-    float sq = sq_part, sk = sk_part;
-#pragma unroll
-    for (int i = 0; i < (qk_ssq ? 0 : QV); ++i) {
-      const int idx = tid + i * 256;
-      float f[8];
-      if (idx < (dq >> 3)) {
-        Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(qrow[i]), f);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) sq += f[e] * f[e];
+    if (qk_ssq) {  // per-tile partials left by the projection: wave 0 alone adds them up
+      if (wave == 0) {
+        const float* pr = qk_ssq + (int64_t)b * ((dq + 2 * dk) >> 4);
+        for (int i = lane; i < (dq >> 4); i += 64) sq += pr[i];
+        for (int i = lane; i < (dk >> 4); i += 64) sk += pr[(dq >> 4) + i];
       }
-      if (idx < (dk >> 3)) {
-        Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(krow[i]), f);
+    } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) sk += f[e] * f[e];
+      for (int i = 0; i < QV; ++i) {
+        const int idx = tid + i * 256;
+        if (idx < (dq >> 3)) qrow[i] = reinterpret_cast<const u32x4*>(row)[idx];
+        if (idx < (dk >> 3)) krow[i] = reinterpret_cast<const u32x4*>(row + dq)[idx];
       }
     }
-    sq = wave_sum(sq), sk = wave_sum(sk);
-    if (lane == 0) red2[0][wave] = sq, red2[1][wave] = sk;
-    lds_barrier();
-    rq = 1.f / sqrtf((red2[0][0] + red2[0][1] + red2[0][2] + red2[0][3]) / (float)dq + eps);
-    rk = 1.f / sqrtf((red2[1][0] + red2[1][1] + red2[1][2] + red2[1][3]) / (float)dk + eps);
+  }
+  const __amdgpu_buffer_rsrc_t rk = make_rsrc(kc + cbase, (int64_t)(kmax + 1) * HD * 2);
+  const __amdgpu_buffer_rsrc_t rv = make_rsrc(vc + cbase, (int64_t)(kmax + 1) * HD * 2);
+  u32x4 kreg[ITERS], vreg[ITERS];
+  float bias[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it)
+    kreg[it] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rk, lane * 16, (kbase + it * KPI) * HD * 2, 0));
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    vreg[it] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rv, lane * 16, (kbase + it * KPI) * HD * 2, 0));
+    bias[it] = key_bias ? key_bias[(int64_t)b * bias_stride + min(kbase + it * KPI + kslot, kmax)] : 0.f;
+  }
+
+  // ---- 2. QK-norm scale factors, rotary, the new cache row --------------------------------------------------
+  float rq = 1.f, rk_ = 1.f;
+  u32x4 pk1, pk2;
+  if (norm) {
+    if (qk_ssq) {
+      if (wave == 0) {
+        sq = wave_sum(sq), sk = wave_sum(sk);
+        rq = 1.f / sqrtf(sq / (float)dq + eps);
+        rk_ = 1.f / sqrtf(sk / (float)dk + eps);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < QV; ++i) {
+        const int idx = tid + i * 256;
+        float f[8];
+        if (idx < (dq >> 3)) {
+          Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(qrow[i]), f);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) sq += f[e] * f[e];
+        }
+        if (idx < (dk >> 3)) {
+          Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(krow[i]), f);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) sk += f[e] * f[e];
+        }
+      }
+      sq = wave_sum(sq), sk = wave_sum(sk);
+      if (lane == 0) red2[0][wave] = sq, red2[1][wave] = sk;
+      lds_barrier();
+      rq = 1.f / sqrtf((red2[0][0] + red2[0][1] + red2[0][2] + red2[0][3]) / (float)dq + eps);
+      rk_ = 1.f / sqrtf((red2[1][0] + red2[1][1] + red2[1][2] + red2[1][3]) / (float)dk + eps);
+    }
   }
   if (role_q || role_k) {
     float a1[8], a2[8], ww1[8], ww2[8];
@@ -592,7 +608,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
       Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(w1), ww1);
       Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(w2), ww2);
     }
-    const float r = role_q ? rq : rk;
+    const float r = role_q ? rq : rk_;
     float o1[8], o2[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -608,34 +624,36 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
 #pragma unroll
       for (int e = 0; e < 8; ++e) qs[j + e] = o1[e], qs[j + HALF + e] = o2[e];
     } else {
-      u32x4 p1, p2;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) p1[e] = pack_bf16x2(o1[2 * e], o1[2 * e + 1]), p2[e] = pack_bf16x2(o2[2 * e], o2[2 * e + 1]);
-      knew[c] = p1, knew[c + CPH] = p2;
-      if (h % gsz == 0) {
-        const int64_t o = cbase + (int64_t)pos * HD + j;
-        reinterpret_cast<u32x4*>(kc)[o >> 3] = p1;
-        reinterpret_cast<u32x4*>(kc)[(o + HALF) >> 3] = p2;
-      }
+      for (int e = 0; e < 4; ++e) pk1[e] = pack_bf16x2(o1[2 * e], o1[2 * e + 1]), pk2[e] = pack_bf16x2(o2[2 * e], o2[2 * e + 1]);
+      knew[c] = pk1, knew[c + CPH] = pk2;
     }
   }
-  if (role_v) {
-    vnew[tid - 64] = vrow;
-    if (h % gsz == 0) reinterpret_cast<u32x4*>(vc)[(cbase + (int64_t)pos * HD + (tid - 64) * 8) >> 3] = vrow;
+  if (role_v) vnew[tid - 64] = vrow;
+  // ---- the position is needed from here on ----------------------------------------------------------------
+  const int L = pos + 1;
+  if (chunk * kDecodeChunk >= L || pos >= Lmax || pos >= n_pos || pos > kmax) return;  // whole workgroup
+  if (pos / kDecodeChunk == chunk && h % gsz == 0) {  // the chunk that holds the new position appends it
+    if (role_k) {
+      const int64_t o = cbase + (int64_t)pos * HD + j;
+      reinterpret_cast<u32x4*>(kc)[o >> 3] = pk1;
+      reinterpret_cast<u32x4*>(kc)[(o + HALF) >> 3] = pk2;
+    }
+    if (role_v) reinterpret_cast<u32x4*>(vc)[(cbase + (int64_t)pos * HD + (tid - 64) * 8) >> 3] = vrow;
   }
   lds_barrier();
   float qr[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) qr[i] = qs[sub * 8 + i];
 
-  // ---- 3. scores, softmax partial, P.V -------------------------------------------------------------------
+  // ---- 3. scores, softmax partial and P.V per key slot (the LPK lanes that share a key) ------------
   float s[ITERS];
-  float wmax = -INFINITY;
+  float smax = -INFINITY;
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const int key = kbase + it * KPI + kslot;
     if (key == pos) kreg[it] = knew[sub], vreg[it] = vnew[sub];
-    if (key >= L) vreg[it] = u32x4{0u, 0u, 0u, 0u};  // clamped duplicates may be unwritten rows: 0 * NaN
+    if (key >= L) vreg[it] = u32x4{0u, 0u, 0u, 0u};  // unwritten rows: 0 * NaN
     float kf[8];
     Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(kreg[it]), kf);
     float d = 0.f;
@@ -645,48 +663,43 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     float v = bias[it] <= kMaskThreshold ? lowest : d * scale + bias[it];
     v = key < L ? v : -INFINITY;
     s[it] = v;
-    wmax = fmaxf(wmax, v);
+    smax = fmaxf(smax, v);
   }
-#pragma unroll
-  for (int o = LPK; o < 64; o <<= 1) wmax = fmaxf(wmax, __shfl_xor(wmax, o, 64));
-  const bool empty = (kbase >= L);
+  // a slot whose keys all lie beyond L contributes nothing
+  const bool empty = (kbase + kslot >= L);
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float lsum = 0.f;
   if (!empty) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      const float p = __expf(s[it] - wmax);
-      lsum += p;
+      const float pw = __expf(s[it] - smax);
+      lsum += pw;
       float vf[8];
       Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(vreg[it]), vf);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, vf[i], acc[i]);
-    }
-#pragma unroll
-    for (int o = LPK; o < 64; o <<= 1) {
-      lsum += __shfl_xor(lsum, o, 64);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] += __shfl_xor(acc[i], o, 64);
+      for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(pw, vf[i], acc[i]);
     }
   }
-  if (lane < LPK) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) red_o[wave][sub * 8 + i] = acc[i];
+  {
+    const int rrow = wave * KPI + kslot;
+    f32x4* ro = reinterpret_cast<f32x4*>(&red_o[rrow][sub * 8]);
+    ro[0] = f32x4{acc[0], acc[1], acc[2], acc[3]};
+    ro[1] = f32x4{acc[4], acc[5], acc[6], acc[7]};
+    if (sub == 0) red_ml[rrow][0] = empty ? -INFINITY : smax, red_ml[rrow][1] = empty ? 0.f : lsum;
   }
-  if (lane == 0) red_ml[wave][0] = empty ? -INFINITY : wmax, red_ml[wave][1] = empty ? 0.f : lsum;
   __syncthreads();
   float mm = red_ml[0][0];
 #pragma unroll
-  for (int w = 1; w < 4; ++w) mm = fmaxf(mm, red_ml[w][0]);
+  for (int w = 1; w < ROWS; ++w) mm = fmaxf(mm, red_ml[w][0]);
   float* dst = ws + (((int64_t)b * H + h) * nchunks_max + chunk) * (HD + 2);
   float ov = 0.f, lv = 0.f;
   if (tid < HD) {
 #pragma unroll
-    for (int w = 0; w < 4; ++w) ov += red_o[w][tid] * __expf(red_ml[w][0] - mm);
+    for (int w = 0; w < ROWS; ++w) ov += red_o[w][tid] * __expf(red_ml[w][0] - mm);
   }
   if (tid == 0) {
 #pragma unroll
-    for (int w = 0; w < 4; ++w) lv += red_ml[w][1] * __expf(red_ml[w][0] - mm);
+    for (int w = 0; w < ROWS; ++w) lv += red_ml[w][1] * __expf(red_ml[w][0] - mm);
   }
   if (!tickets) {  // partials merged by attn_decode_combine_kernel
     if (tid < HD) dst[tid] = ov;
@@ -705,7 +718,6 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, false));  // vmcnt(0): this wave's stores have landed
   __syncthreads();
-  __shared__ int s_last;
   const int nact = min((L + kDecodeChunk - 1) / kDecodeChunk, nchunks_max);
   if (tid == 0) {
     int* tk = tickets + b * H + h;
@@ -797,6 +809,29 @@ extern "C" int olmo355_attn_prefill(const void* q, const void* kcache, const voi
   }
 #undef GENERIC
   return O355_EUNSUPPORTED;
+}
+
+namespace {
+// *pos += delta, then rope_now = [sin_tab[*pos] | cos_tab[*pos]] (the last table row when *pos runs past it)
+__global__ void rope_advance_kernel(int32_t* __restrict__ pos, int delta, const float* __restrict__ sin_t,
+                                    const float* __restrict__ cos_t, float* __restrict__ rope_now, int hd, int n_pos) {
+  const int p = *pos + delta;
+  __syncthreads();  // every thread has read the old value
+  if (threadIdx.x == 0) *pos = p;
+  const int r = min(max(p, 0), n_pos - 1);
+  for (int i = threadIdx.x; i < hd; i += blockDim.x) {
+    rope_now[i] = sin_t[(int64_t)r * hd + i];
+    rope_now[hd + i] = cos_t[(int64_t)r * hd + i];
+  }
+}
+}  // namespace
+
+extern "C" int olmo355_rope_advance(int32_t* pos, int delta, const float* sin_tab, const float* cos_tab, float* rope_now,
+                                    int hd, int n_pos, void* stream) {
+  if (!pos || !sin_tab || !cos_tab || !rope_now || hd <= 0 || n_pos <= 0) return O355_EINVAL;
+  hipLaunchKernelGGL(rope_advance_kernel, dim3(1), dim3(128), 0, as_stream(stream), pos, delta, sin_tab, cos_tab, rope_now,
+                     hd, n_pos);
+  O355_CHECK_LAUNCH();
 }
 
 extern "C" int64_t olmo355_attn_decode_workspace_bytes(int B, int H, int hd, int n_keys_max) {
@@ -1069,7 +1104,8 @@ extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const 
                                          const float* cos_tab, void* kcache, void* vcache, const float* key_bias,
                                          void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
                                          int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride,
-                                         float eps, const float* qk_ssq, int dtype, void* stream) {
+                                         float eps, const float* qk_ssq, const float* rope_now, int dtype,
+                                         void* stream) {
   if (!qkv || !sin_tab || !cos_tab || !kcache || !vcache || !out || !ws) return O355_EINVAL;
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || past_len < 0 || n_keys_max <= 0 || n_keys_max > Lmax)
     return O355_EINVAL;
@@ -1079,10 +1115,8 @@ extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const 
   if (dtype != O355_BF16 || (hd != 128 && hd != 64) || H * hd > 8 * 4 * 256) return O355_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
   const int nch = (n_keys_max + kDecodeChunk - 1) / kDecodeChunk;
-  // one workgroup per (batch, head) when that already fills the chip
-  // (measured at 7B shapes, context 2048: 5 % faster at batch 8, 40 % slower at batch 1, where only
-  // 32 CUs would pull data)
-  bool onepass = H * hd <= 8 * 1024 && (int64_t)B * H >= 256;
+  // one workgroup per (batch, head) is kept as an experiment only: never faster than the chunked form
+  bool onepass = false;
   if (g_dbg_attn_mode >= 0) onepass = g_dbg_attn_mode == 1 && H * hd <= 8 * 1024;
   if (onepass) {
 #define ONEPASS(HDv)                                                                                                  \
@@ -1101,13 +1135,17 @@ extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const 
   hipLaunchKernelGGL((attn_decode_fused_kernel<HDv, QVv>), dim3(nch, H, B), dim3(256), 0, s, (const uint16_t*)qkv,   \
                      (const uint16_t*)qw, (const uint16_t*)kw, sin_tab, cos_tab, (uint16_t*)kcache, (uint16_t*)vcache, \
                      key_bias, (float*)ws, H, Hkv, Lmax, n_pos, past_len, past_len_dev, nch, bias_stride, eps, qk_ssq, \
-                     (uint16_t*)out, tickets);                                                                         \
+                     rope_now, (uint16_t*)out, tickets);                                                                         \
   if (!tickets)                                                                                                        \
   hipLaunchKernelGGL((attn_decode_combine_kernel<O355_BF16, HDv>), dim3(H, B), dim3(HDv), 0, s, (const float*)ws, out, \
                      H, past_len, past_len_dev, nch)
   // the workspace starts with one ticket counter per (batch, head): zero on entry (zeroed at allocation,
   // reset by the workgroup that draws the last ticket), then the partials
-  int* tickets = g_dbg_attn_mode == 2 ? nullptr : reinterpret_cast<int*>(ws);
+  // (measured at the 7B shapes, context 2048: the in-kernel merge wins while the launch is a single round of
+  // workgroups -- 17.0 against 20.4 us at batch 1 -- and loses once workgroups queue up -- 69.7 against 61.6 us
+  // at batch 8, where one workgroup per (batch, head) takes 66.9)
+  const bool merge_in_kernel = g_dbg_attn_mode == 0 || (g_dbg_attn_mode < 0 && (int64_t)B * H * nch <= 1536);
+  int* tickets = merge_in_kernel ? reinterpret_cast<int*>(ws) : nullptr;
   ws = reinterpret_cast<float*>(ws) + (int64_t)B * H;
   const int qv = (H * hd / 8 + 255) / 256;
   if (hd == 128) {

@@ -33,6 +33,10 @@ class DecodeSession:
         self.key_bias = key_bias_full
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
+        # rotary rows of the position about to be written, refreshed on the device after every step
+        sin, cos = model._rope
+        cache.rope_now = torch.empty(2 * sin.shape[1], dtype=torch.float32, device=sin.device)
+        ops.rope_advance(cache.length_dev, 0, sin, cos, cache.rope_now)
 
     def _step_kernels(self) -> None:
         m = self.model
@@ -40,7 +44,7 @@ class DecodeSession:
         logits, _ = m._forward_tokens(x, self.cache, self.B, 1, 0, self.key_bias, self.cache.length_dev, False)
         self.logits = logits
         ops.argmax(logits.view(self.B, -1), out=self.ids.view(self.B))
-        ops.incr_i32(self.cache.length_dev)
+        ops.rope_advance(self.cache.length_dev, 1, *m._rope, self.cache.rope_now)
 
     def step(self) -> None:
         """Advance by one token: afterwards ``self.ids`` holds the new token of every sequence."""

@@ -56,6 +56,8 @@ class KVCache:
         self.B, self.capacity, self.length = B, capacity, 0
         # device copy of the number of cached positions, for captured decode steps
         self.length_dev = torch.zeros(1, dtype=torch.int32, device=device)
+        # rotary rows [sin | cos] of position `length`, kept current by a decode session (None otherwise)
+        self.rope_now: Optional[torch.Tensor] = None
 
     def views(self) -> List["LayerKV"]:
         L = self.length
@@ -228,6 +230,7 @@ class OLMo(nn.Module):
         n_pos = max(self.max_cache_len, c.max_sequence_length)
         self._rope = ops.rope_tables(c.head_dim, float(c.rope_theta), n_pos, self.device)
         self._chain_ok = {}  # rows -> whether the chained decode block covers this model
+        self._rope_now = None  # rotary rows of the current position during a captured decode step
         self._prepared = True
         return self
 
@@ -313,7 +316,8 @@ class OLMo(nn.Module):
         if decode:
             att = ops.attn_decode_fused(qkv, qw, kw, sin, cos, kc, vc, self._decode_ws(B, n_keys_max), B, H, Hkv, hd,
                                         past_len, n_keys_max, c.layer_norm_eps, key_bias=key_bias,
-                                        past_len_dev=graph_pos, qk_ssq=qk_ssq)
+                                        past_len_dev=graph_pos, qk_ssq=qk_ssq,
+                                        rope_now=self._rope_now if graph_pos is not None else None)
             if att is not None:
                 return att
         q = ops.qknorm_rope_kvwrite(qkv, qw, kw, sin, cos, kc, vc, B, T, H, Hkv, hd, past_len, c.layer_norm_eps,
@@ -487,6 +491,7 @@ class OLMo(nn.Module):
         int32 holding the number of cached positions) the launch arguments do not depend on the
         position, so the call can be captured once and replayed; it requires ``T == 1``."""
         n_keys_max = cache.capacity if graph_pos is not None else past_len + T
+        self._rope_now = cache.rope_now if (cache is not None and graph_pos is not None) else None
         hidden: List[torch.Tensor] = []
         fused = T == 1 and cache is not None and self._fused_decode_ok(B, collect_hidden)
         chain = fused and self._chain_decode_ok(B)

@@ -391,11 +391,13 @@ def attn_decode(q, kcache, vcache, ws, B: int, H: int, Hkv: int, hd: int, past_l
 
 def attn_decode_fused(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, ws, B: int, H: int, Hkv: int, hd: int,
                       past_len: int, n_keys_max: int, eps: float, key_bias: Optional[torch.Tensor] = None,
-                      past_len_dev: Optional[torch.Tensor] = None,
-                      qk_ssq: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+                      past_len_dev: Optional[torch.Tensor] = None, qk_ssq: Optional[torch.Tensor] = None,
+                      rope_now: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """One new token per sequence: QK-norm, rotary, cache append and attention in one pass.  Returns
     ``None`` when the fused kernel does not cover the shape (use the separate calls then)."""
-    _dev(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, ws, key_bias, past_len_dev, qk_ssq)
+    _dev(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, ws, key_bias, past_len_dev, qk_ssq, rope_now)
+    if rope_now is not None and (rope_now.dtype != torch.float32 or rope_now.numel() != 2 * hd):
+        raise ValueError("rope_now: float32 [2 * hd] expected")
     if qkv.dtype != torch.bfloat16 or hd not in (64, 128):
         return None
     if qk_ssq is not None and (qk_ssq.dtype != torch.float32 or qk_ssq.numel() != B * (H + 2 * Hkv) * hd // 16):
@@ -410,11 +412,24 @@ def attn_decode_fused(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache,
     st = lib().olmo355_attn_decode_fused(_p(qkv), _p(q_weight), _p(k_weight), _p(sin_tab), _p(cos_tab), _p(kcache),
                                          _p(vcache), _p(key_bias), _p(out), _p(ws), B, H, Hkv, hd, Lmax, n_pos, past_len,
                                          _p(past_len_dev), n_keys_max, key_bias.shape[1] if key_bias is not None else 0,
-                                         float(eps), _p(qk_ssq), _dt(qkv), _stream())
+                                         float(eps), _p(qk_ssq), _p(rope_now), _dt(qkv), _stream())
     if st == 2:
         return None
     check("olmo355_attn_decode_fused", st)
     return out
+
+
+def rope_advance(pos_dev: torch.Tensor, delta: int, sin_tab: torch.Tensor, cos_tab: torch.Tensor,
+                 rope_now: torch.Tensor) -> None:
+    """``pos_dev += delta`` (device int32) and ``rope_now = [sin_tab[pos] | cos_tab[pos]]``: run between
+    captured decode steps so that the attention kernel never looks the rotary rows up by position."""
+    _dev(pos_dev, sin_tab, cos_tab, rope_now)
+    hd = sin_tab.shape[1]
+    if pos_dev.dtype != torch.int32 or rope_now.dtype != torch.float32 or rope_now.numel() != 2 * hd:
+        raise TypeError("pos_dev int32, rope_now float32 [2 * hd] expected")
+    check("olmo355_rope_advance",
+          lib().olmo355_rope_advance(_p(pos_dev), int(delta), _p(sin_tab), _p(cos_tab), _p(rope_now), hd, sin_tab.shape[0],
+                                     _stream()))
 
 
 def rope_tables(head_dim: int, theta: float, n_pos: int, device) -> Tuple[torch.Tensor, torch.Tensor]:
