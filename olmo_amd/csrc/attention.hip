@@ -127,13 +127,17 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const uint16_t* 
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, kq = lane >> 4;
-  // heavier (later) query blocks first: they have the most key tiles
-  const int qblock = gridDim.x - 1 - blockIdx.x;
+  // Causal work grows with the query block, so a workgroup takes a complementary pair: block
+  // nqb-1-x (many key tiles) and then block x (few); every workgroup does the same amount.
+  const int nqb = (T + 127) / 128;
   const int b = blockIdx.z, h = blockIdx.y, hk = h / (H / Hkv);
-  const int q0 = qblock * 128 + wave * 32;
   const float scale = 1.f / sqrtf((float)HD);
   const float lowest = -3.3895313892515355e38f;
   const int64_t cbase = ((int64_t)b * Hkv + hk) * Lmax * HD;
+  for (int pass = 0; pass < 2; ++pass) {
+  const int qblock = pass == 0 ? nqb - 1 - (int)blockIdx.x : (int)blockIdx.x;
+  if (pass == 1 && qblock >= nqb - 1 - (int)blockIdx.x) break;  // the middle block of an odd count is its own pair
+  const int q0 = qblock * 128 + wave * 32;
 
   // Q^T fragments: lane (query col, hd 32*step + 8*kq ..)
   bf16x8 qf[QT][STEPS];
@@ -279,6 +283,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const uint16_t* 
       *reinterpret_cast<u32x2*>(dst + 16 * ht + 4 * kq) = w;
     }
   }
+  }  // pass
 }
 
 // =====================================================================================================
@@ -787,7 +792,7 @@ extern "C" int olmo355_attn_prefill(const void* q, const void* kcache, const voi
   if (key_bias && bias_stride < past_len + T) return O355_EINVAL;
   hipStream_t s = as_stream(stream);
   if (dtype == O355_BF16 && (hd == 128 || hd == 64)) {
-    const dim3 grid((T + 127) / 128, H, B);
+    const dim3 grid(((T + 127) / 128 + 1) / 2, H, B);  // pairs of query blocks
     if (hd == 128)
       hipLaunchKernelGGL(attn_prefill_mfma_kernel<128>, grid, dim3(256), 0, s, (const uint16_t*)q,
                          (const uint16_t*)kcache, (const uint16_t*)vcache, key_bias, (uint16_t*)out, T, H, Hkv, Lmax,
