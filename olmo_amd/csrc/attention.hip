@@ -161,39 +161,56 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const uint16_t* 
 
   const int last_pos = past_len + min(qblock * 128 + 127, T - 1);   // workgroup-uniform loop bound
   const int wave_last = past_len + min(q0 + 31, T - 1);             // last position this wave needs
-  for (int k0 = 0; k0 <= last_pos; k0 += KT) {
-    __syncthreads();
-    // ---- stage K: 64 keys x HD, 16-byte chunks ------------------------------------------------------
-    constexpr int CPR = HD / 8;  // chunks per key row
-    for (int e = tid; e < KT * CPR; e += 256) {
-      const int kk = e / CPR, c = e % CPR;
-      const int key = min(k0 + kk, last_pos);
-      const u32x4 v = *reinterpret_cast<const u32x4*>(kc + cbase + (int64_t)key * HD + 8 * c);
-      lds_k[((kk >> 4) * STEPS + (c >> 2)) * 64 + (kk & 15) + 16 * (c & 3)] = v;
+  // K / V of a tile travel memory -> registers -> LDS; the registers of tile k0+KT are requested right
+  // after tile k0 has been written to LDS, so the requests are in flight while tile k0 is multiplied.
+  constexpr int CPR = HD / 8;                     // 16-byte chunks per key row
+  constexpr int KPT = KT * CPR / 256;             // K chunks per thread per tile
+  constexpr int VPT = (KT / 2) * CPR / 256;       // V chunk pairs (two consecutive keys) per thread per tile
+  u32x4 rkk[KPT], rv0[VPT], rv1[VPT];
+  float rbias = 0.f;
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
+      rkk[i] = *reinterpret_cast<const u32x4*>(kc + cbase + (int64_t)min(k0 + kk, last_pos) * HD + 8 * c);
     }
-    // ---- stage V^T: key pairs (kk, kk+1) x 8 hd values -> 8 dword writes -------------------------------
-    for (int e = tid; e < (KT / 2) * CPR; e += 256) {
-      const int kp = e / CPR, c = e % CPR;
-      const int kk = 2 * kp;
-      const int key0 = min(k0 + kk, last_pos), key1 = min(k0 + kk + 1, last_pos);
-      const u32x4 v0 = *reinterpret_cast<const u32x4*>(vc + cbase + (int64_t)key0 * HD + 8 * c);
-      const u32x4 v1 = *reinterpret_cast<const u32x4*>(vc + cbase + (int64_t)key1 * HD + 8 * c);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int e = tid + i * 256, kk = 2 * (e / CPR), c = e % CPR;
+      rv0[i] = *reinterpret_cast<const u32x4*>(vc + cbase + (int64_t)min(k0 + kk, last_pos) * HD + 8 * c);
+      rv1[i] = *reinterpret_cast<const u32x4*>(vc + cbase + (int64_t)min(k0 + kk + 1, last_pos) * HD + 8 * c);
+    }
+    if (tid < KT) rbias = key_bias ? key_bias[(int64_t)b * bias_stride + min(k0 + tid, last_pos)] : 0.f;
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
+      lds_k[((kk >> 4) * STEPS + (c >> 2)) * 64 + (kk & 15) + 16 * (c & 3)] = rkk[i];
+    }
+    // V^T: key pairs (kk, kk+1) x 8 hd values -> 8 dword writes
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int e = tid + i * 256, kk = 2 * (e / CPR), c = e % CPR;
       const int kt = kk >> 4, s2 = kt >> 1, hf = kt & 1, k16 = kk & 15;
       const int kq_ = k16 >> 2, e0 = (k16 & 3) + 4 * hf;  // e0 even
       uint32_t* dst = reinterpret_cast<uint32_t*>(lds_v);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int hd_ = 8 * c + i;
+      for (int x = 0; x < 8; ++x) {
+        const int hd_ = 8 * c + x;
         const int ht = hd_ >> 4, lo = hd_ & 15;
-        const uint32_t a = (i & 1) ? (v0[i >> 1] >> 16) : (v0[i >> 1] & 0xffffu);
-        const uint32_t bb = (i & 1) ? (v1[i >> 1] >> 16) : (v1[i >> 1] & 0xffffu);
+        const uint32_t a = (x & 1) ? (rv0[i][x >> 1] >> 16) : (rv0[i][x >> 1] & 0xffffu);
+        const uint32_t bb = (x & 1) ? (rv1[i][x >> 1] >> 16) : (rv1[i][x >> 1] & 0xffffu);
         dst[(((ht * 2 + s2) * 64 + kq_ * 16 + lo) * 8 + e0) >> 1] = a | (bb << 16);
       }
     }
-    if (tid < KT) {
-      const int key = min(k0 + tid, last_pos);
-      lds_bias[tid] = key_bias ? key_bias[(int64_t)b * bias_stride + key] : 0.f;
-    }
+    if (tid < KT) lds_bias[tid] = rbias;
+  };
+  fetch(0);
+  for (int k0 = 0; k0 <= last_pos; k0 += KT) {
+    __syncthreads();  // the previous tile has been read
+    stash();
+    if (k0 + KT <= last_pos) fetch(k0 + KT);
     __syncthreads();
     if (k0 > wave_last) continue;  // nothing visible to this wave in the tile (barriers stay uniform)
 
