@@ -23,6 +23,12 @@ import time
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
 MFMA_BF16_PEAK_TF = 2500.0  # MI355X dense bf16, published
 W4_BYTES_PER_WEIGHT = 0.5 + 2.0 / 128 + 0.5 / 128  # nibble + fp16 scale and 4-bit zero per group of 128
+# HBM bytes per launch of the int4 small-M linear, averaged over the four 7B block shapes, from two
+# rocprofv3 --pmc runs of `bench.py --traffic-probe` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each
+# scaled by what the same counter reads for a 256 MiB device copy (FETCH_SIZE reads half the bytes: factor
+# 2.0; WRITE_SIZE factor 1.0).  Per shape, read: 26.29 / 8.92 / 46.99 / 23.74 MB against 26.15 / 8.72 /
+# 46.85 / 23.43 MB of packed weights, scales and zeros; written: the output rows.
+GEMV_TRAFFIC_BYTES_7B = 26.51e6
 
 
 def log(*a):
@@ -42,6 +48,9 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=2048)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bs8", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: one plain copy of known size, then the four "
+                         "int4 linears of a layer at one row; nothing is timed or printed")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this build runs the whole model on ONE GPU; --gpus N with N > 1 is not supported.")
@@ -60,6 +69,8 @@ def main() -> int:
         return 2
     dev = torch.device("cuda:0")
     cfg = PRESETS["olmo2-7b"]
+    if args.traffic_probe:
+        return traffic_probe(cfg, dev)
     ctx, K, W = args.context, args.steps, args.warmup
     cap = ctx + K + W + 8
     t0 = time.time()
@@ -125,9 +136,9 @@ def main() -> int:
     avg_s = e0.elapsed_time(e1) * 1e-3 / (reps * n_launch)
     bytes_per_launch = sum(n * k * W4_BYTES_PER_WEIGHT + 2 * k + 2 * n for n, k in shapes) * cfg.n_layers / n_launch
     achieved = bytes_per_launch / avg_s / 1e9
-    roofline = {"bound": "hbm", "kernel": "w4_gemv_kernel (M=1, the 4 block Linears x 32 layers)",
+    roofline = {"bound": "hbm", "kernel": "w4_gemv_small_kernel (M=1, the 4 block Linears x 32 layers)",
                 "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                "traffic": None, "avg_launch_us": avg_s * 1e6, "bytes_per_launch": bytes_per_launch}
+                "traffic": GEMV_TRAFFIC_BYTES_7B, "avg_launch_us": avg_s * 1e6, "bytes_per_launch": bytes_per_launch}
     log(f"[bench] int4 GEMV: {avg_s * 1e6:.2f} us/launch avg, {achieved:.0f} GB/s = {achieved / HBM_PEAK_GBS:.1%} of HBM peak")
 
     # ---- prefill GEMMs (M = context): TFLOP/s against the bf16 MFMA peak ---------------------------
@@ -172,6 +183,35 @@ def main() -> int:
         "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
     }
     print(json.dumps(line), flush=True)
+    return 0
+
+
+def traffic_probe(cfg, dev) -> int:
+    """Launches whose HBM traffic the hardware counters are read for: a 256 MiB device copy (the
+    yardstick: 256 MiB read, 256 MiB written) and the four int4 block linears at one row, three
+    times each over distinct weights."""
+    import torch
+
+    from olmo_amd import ops
+    from olmo_amd.qlinear import QuantLinear
+    from olmo_amd.synthetic import fill_random_int4
+
+    gen = torch.Generator(device=dev).manual_seed(0)
+    src = torch.randint(0, 255, (256 << 20,), dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    for n, k in linear_shapes(cfg):
+        x = torch.randn(1, k, device=dev).to(torch.bfloat16)
+        for _ in range(3):
+            q = QuantLinear(4, 128, k, n, True, device=dev)
+            fill_random_int4(q, gen)
+            q.post_init(free_checkpoint_buffers=True)
+            torch.cuda.synchronize()
+            ops.w4_linear(x, q.tiled)
+            torch.cuda.synchronize()
+            del q
     return 0
 
 
