@@ -48,6 +48,8 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=2048)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bs8", action="store_true")
+    ap.add_argument("--sweep", action="store_true",
+                    help="isolated int4 linear sweep (M x shapes): prints a table on stderr and a JSON list on stdout")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: one plain copy of known size, then the four "
                          "int4 linears of a layer at one row; nothing is timed or printed")
@@ -71,6 +73,8 @@ def main() -> int:
     cfg = PRESETS["olmo2-7b"]
     if args.traffic_probe:
         return traffic_probe(cfg, dev)
+    if args.sweep:
+        return linear_sweep(dev)
     ctx, K, W = args.context, args.steps, args.warmup
     cap = ctx + K + W + 8
     t0 = time.time()
@@ -183,6 +187,65 @@ def main() -> int:
         "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
     }
     print(json.dumps(line), flush=True)
+    return 0
+
+
+def linear_sweep(dev) -> int:
+    """The isolated int4 linear over M x (N, K): launches over distinct weight copies (>= 2 GB or 64 copies,
+    so no cache level can serve them) timed inside a captured graph.  (The bit-exactness of the dequantised
+    table for such shapes is a test, tests/test_gpu_ops.py, not part of the timing.)
+    M <= 64 is reported as GB/s of algorithmic bytes against the HBM peak, M >= 512 as TFLOP/s against the
+    bf16 MFMA peak."""
+    import torch
+
+    from olmo_amd import ops
+    from olmo_amd.qlinear import QuantLinear
+    from olmo_amd.synthetic import fill_random_int4
+
+    gen = torch.Generator(device=dev).manual_seed(0)
+    rows = []
+    for n, k in [(4096, 4096), (11008, 4096), (4096, 11008), (13824, 5120), (100352, 4096)]:
+        per = n * k * W4_BYTES_PER_WEIGHT
+        ncopy = int(min(64, max(4, -(-2e9 // per))))
+        tiles = []
+        for i in range(ncopy):
+            q = QuantLinear(4, 128, k, n, True, device=dev)
+            fill_random_int4(q, gen)
+            q.post_init(free_checkpoint_buffers=True)
+            tiles.append(q.tiled)
+        for m in (1, 8, 64, 512, 4096):
+            x = torch.randn(m, k, device=dev).to(torch.bfloat16)
+
+            def run():
+                for t in tiles:
+                    ops.w4_linear(x, t)
+
+            run()
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                run()
+            g.replay()
+            torch.cuda.synchronize()
+            reps = 5 if m <= 64 else 2
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / (reps * ncopy)
+            by = per + 2 * m * k + 2 * m * n
+            fl = 2.0 * m * n * k
+            row = {"M": m, "N": n, "K": k, "us": us, "copies": ncopy}
+            if m <= 64:
+                row.update(bound="hbm", achieved=by / us / 1e3, unit="GB/s", frac=by / us / 1e3 / HBM_PEAK_GBS)
+            else:
+                row.update(bound="mfma", achieved=fl / us / 1e6, unit="TFLOP/s", frac=fl / us / 1e6 / MFMA_BF16_PEAK_TF)
+            rows.append(row)
+            log(f"[sweep] M={m:5d} N={n:6d} K={k:5d}: {us:9.2f} us  {row['achieved']:8.1f} {row['unit']:8s} {row['frac']:6.1%}")
+        del tiles
+    print(json.dumps(rows))
     return 0
 
 

@@ -312,28 +312,37 @@ int launch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const
   O355_CHECK_LAUNCH();
 }
 
-int g_force_tile = 0;  // debug: 0 = choose, else 256 / 192 / 128 = the tile's width
+int g_force_tile = 0;  // debug: 0 = choose, else 1000 * rows + columns of the tile (rows 0 = 256)
 
-// Tiles are 256 rows by 256, 192 or 128 columns.  A launch runs in rounds of one tile per CU, so the
-// width is picked to minimise rounds x width (narrow tiles cost a little more per column: more
-// operand traffic per MFMA).
+// Tiles are 256 rows by 256, 192 or 128 columns, or 128 rows by 128 or 64 columns.  A launch runs in
+// rounds of one tile per CU (two for the smallest tile, whose LDS fits twice), and the time of a round
+// is far from proportional to the tile's area: a K-stage costs about 0.5 us of latency however small
+// the tile.  The table holds measured microseconds per round at K = 4096 with int4 weights (the ratios
+// are what matters); the shape with the smallest rounds x time wins.
 template <bool W4>
 int dispatch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M,
                   int N, int K, hipStream_t stream) {
-  int cus = 256;
-  const int64_t tm = (M + 255) / 256;
-  auto cost = [&](int bn, double penalty) {
-    const int64_t tiles = tm * ((N + bn - 1) / bn);
-    return (double)((tiles + cus - 1) / cus) * bn * penalty;
-  };
-  int best = 256;
-  double c = cost(256, 1.0);
-  if (cost(192, 1.04) < c) best = 192, c = cost(192, 1.04);
-  if (cost(128, 1.10) < c) best = 128, c = cost(128, 1.10);
-  if (g_force_tile) best = g_force_tile;
-  if (best == 256) return launch_gemm<2, 4, 4, 2, W4>(x, wt, st, zt, y, M, N, K, stream);
-  if (best == 192) return launch_gemm<4, 2, 2, 3, W4>(x, wt, st, zt, y, M, N, K, stream);
-  return launch_gemm<4, 2, 2, 2, W4>(x, wt, st, zt, y, M, N, K, stream);
+  const int cus = 256;
+  struct Shape { int bm, bn, per_cu; double round_us; };
+  static const Shape shapes[] = {{256, 256, 1, 95.}, {256, 192, 1, 80.}, {256, 128, 1, 55.}, {128, 128, 1, 37.}, {128, 64, 2, 47.}};
+  int best = 0;
+  double c = 1e300;
+  for (const Shape& sh : shapes) {
+    const int64_t tiles = (int64_t)((M + sh.bm - 1) / sh.bm) * ((N + sh.bn - 1) / sh.bn);
+    const int64_t slots = cus * sh.per_cu;
+    double ci = (double)((tiles + slots - 1) / slots) * sh.round_us;
+    if (sh.per_cu == 2 && tiles <= cus) ci = 32.;  // one tile per CU: no sharing of the CU
+    if (ci < c) c = ci, best = 1000 * sh.bm + sh.bn;
+  }
+  if (g_force_tile) best = g_force_tile < 1000 ? 256000 + g_force_tile : g_force_tile;
+  switch (best) {
+    case 256256: return launch_gemm<2, 4, 4, 2, W4>(x, wt, st, zt, y, M, N, K, stream);
+    case 256192: return launch_gemm<4, 2, 2, 3, W4>(x, wt, st, zt, y, M, N, K, stream);
+    case 256128: return launch_gemm<4, 2, 2, 2, W4>(x, wt, st, zt, y, M, N, K, stream);
+    case 128128: return launch_gemm<2, 4, 2, 1, W4>(x, wt, st, zt, y, M, N, K, stream);
+    case 128064: return launch_gemm<4, 2, 1, 1, W4>(x, wt, st, zt, y, M, N, K, stream);
+  }
+  return O355_EINVAL;
 }
 
 }  // namespace

@@ -51,6 +51,25 @@ def test_w4_dequant_bit_exact(dev, K, N, g):
         assert torch.equal(out2.view(torch.int16), ref.view(torch.int16))
 
 
+@pytest.mark.parametrize("N,K", [(4096, 4096), (11008, 4096), (4096, 11008), (13824, 5120), (100352, 4096)])
+def test_w4_dequant_bit_exact_sweep_shapes(dev, N, K):
+    """The shapes of the isolated linear sweep (`bench.py --sweep`): the fp16 table from the GPTQ tensors and
+    from the tiled layout the timed kernels read, both bit-exact against the oracle."""
+    say("w4_dequant sweep shape", N, K)
+    ops = _ops()
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=N + K)
+    # the oracle runs on column bands (all of them unless N is the vocabulary-sized one: first, middle, last)
+    bands = [(0, N)] if N <= 20000 else [(0, 4096), (N // 2 - 2048, N // 2 + 2048), (N - 4096, N)]
+    a = ops.w4_dequant_fp16(qw.to(dev), qz.to(dev), sc.to(dev), 128).view(torch.int16)
+    b = ops.w4t_dequant_fp16(ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)).view(torch.int16)
+    assert a.shape == b.shape == (K, N)
+    for lo, hi in bands:
+        ref = ow4.dequantize(qw[:, lo:hi].contiguous(), qz[:, lo // 8 : hi // 8].contiguous(), sc[:, lo:hi].contiguous(), 128)
+        ref = ref.view(torch.int16)
+        assert torch.equal(a[:, lo:hi].cpu(), ref), (lo, hi)
+        assert torch.equal(b[:, lo:hi].cpu(), ref), (lo, hi)
+
+
 def test_w4_dequant_g_idx_general(dev):
     ops = _ops()
     K, N, g = 256, 32, 128
@@ -150,7 +169,7 @@ def _force_gemm_tile(width):
     _lib.lib().olmo355_debug_set_gemm_tile(int(width))
 
 
-@pytest.mark.parametrize("width", [256, 192, 128])
+@pytest.mark.parametrize("width", [256, 192, 128, 128128, 128064])
 @pytest.mark.parametrize("M,N,K", [(65, 208, 128), (300, 1008, 384), (513, 400, 1408), (256, 768, 256), (1, 16, 640)])
 def test_w4_gemm_every_tile_width(dev, width, M, N, K):
     """Ragged M and N against every tile shape, and K whose stage count leaves 0..3 stages after the
@@ -176,7 +195,7 @@ def test_w4_gemm_every_tile_width(dev, width, M, N, K):
     assert (y.float().cpu() - ref).abs().max().item() <= 2 ** -7 * scale
 
 
-@pytest.mark.parametrize("width", [256, 192, 128])
+@pytest.mark.parametrize("width", [256, 192, 128, 128128, 128064])
 @pytest.mark.parametrize("M,N,K", [(65, 208, 64), (300, 1008, 192), (513, 400, 320), (256, 768, 448), (40, 48, 1024)])
 def test_b16_gemm_every_tile_width(dev, width, M, N, K):
     """Dense weights: stage counts 1, 3, 5, 7, 16 cover every tail length of the four-stage loop."""
