@@ -24,6 +24,10 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 static inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
+// int4 linear for 17..64 rows (gemv_mid.hip); arguments as olmo355_w4_gemv, already validated
+int o355_w4_mid_dispatch(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
+                         int M, int N, int K, void* stream);
+
 // ---- scalar conversions -------------------------------------------------------------------
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 __device__ __forceinline__ float bf16lo_to_f32(uint32_t pair) { return __uint_as_float(pair << 16); }
@@ -102,3 +106,26 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   for (int i = 0; i < nw; ++i) t += red[i];
   return t;
 }
+
+// ---- int4 unpack -----------------------------------------------------------------------------
+// The two constants of the unpack, made opaque to the optimiser (empty asm, no instruction): as
+// literals the compiler emits v_and + v_or per pair, from registers it selects the single
+// v_and_or_b32.  (An asm *instruction* here would be unsafe: the hazard recogniser does not see an
+// asm's result feeding an MFMA and leaves out the wait states.)
+struct UnpackConsts {
+  uint32_t mask, bias;
+  __device__ __forceinline__ UnpackConsts() : mask(0x000f000fu), bias(0x43004300u) {
+    asm volatile("" : "+s"(mask));
+    asm volatile("" : "+v"(bias));
+  }
+};
+
+__device__ __forceinline__ bf16x8 unpack_w4_bias128(uint32_t w, const UnpackConsts& c) {
+  u32x4 r;
+  r.x = (w & c.mask) | c.bias;
+  r.y = ((w >> 4) & c.mask) | c.bias;
+  r.z = ((w >> 8) & c.mask) | c.bias;
+  r.w = ((w >> 12) & c.mask) | c.bias;
+  return __builtin_bit_cast(bf16x8, r);
+}
+

@@ -41,27 +41,6 @@ struct GemvArgs {
   float* ssq_out = nullptr;
 };
 
-// The two constants of the unpack, made opaque to the optimiser (empty asm, no instruction): as
-// literals the compiler emits v_and + v_or per pair, from registers it selects the single
-// v_and_or_b32.  (An asm *instruction* here would be unsafe: the hazard recogniser does not see an
-// asm's result feeding an MFMA and leaves out the wait states.)
-struct UnpackConsts {
-  uint32_t mask, bias;
-  __device__ __forceinline__ UnpackConsts() : mask(0x000f000fu), bias(0x43004300u) {
-    asm volatile("" : "+s"(mask));
-    asm volatile("" : "+v"(bias));
-  }
-};
-
-__device__ __forceinline__ bf16x8 unpack_w4_bias128(uint32_t w, const UnpackConsts& c) {
-  u32x4 r;
-  r.x = (w & c.mask) | c.bias;
-  r.y = ((w >> 4) & c.mask) | c.bias;
-  r.z = ((w >> 8) & c.mask) | c.bias;
-  r.w = ((w >> 12) & c.mask) | c.bias;
-  return __builtin_bit_cast(bf16x8, r);
-}
-
 __device__ __forceinline__ bf16x8 ones_bf16x8() {
   u32x4 r = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
   return __builtin_bit_cast(bf16x8, r);
@@ -1060,6 +1039,14 @@ int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, 
   const u32x4* w = (const u32x4*)wt;
   const int sgpa = a.M <= 4 ? 4 : (a.M <= 8 ? 2 : 1);
   const bool small_ok = a.M <= 16 && (a.M <= 4 || p.pro == 0) && (int64_t)(a.M + 1) * a.K * 2 <= kSmallMaxBytes && (int64_t)(a.N >> 4) * (a.K >> 7) * 1024 < (1ll << 31) && g_dbg_small;
+  // Plain products with many columns: from 9 rows (5 for wide outputs) the staged-activation kernel
+  // wins over the kernels below, which keep all rows of x in LDS per workgroup (measured).
+  const bool plain = !pro && !epi && !a.ssq_in && !a.ssq_out;
+  const bool mid_wins = a.M > 16 || (a.M > 8 && a.N >= 8192) || (a.M > 4 && a.N >= 12288);
+  if (plain && g_dbg_small && (mid_wins || g_dbg_small == 2)) {
+    const int st_mid = o355_w4_mid_dispatch(a.x, wt, st, zt, a.y, a.M, a.N, a.K, stream);
+    if (st_mid != O355_EUNSUPPORTED) return st_mid;  // else: sizes beyond its 32-bit offsets
+  }
   if (a.ssq_in || a.ssq_out) {  // chained norms: only the lean kernel speaks that protocol
     if (!small_ok || a.M > 4 || (a.ssq_out && epi)) return O355_EUNSUPPORTED;
     if (a.ssq_in) {
