@@ -188,6 +188,11 @@ int olmo355_swiglu(const void* x, void* out, int rows, int h, int dtype, void* s
 /* wte lookup (olmo/model.py:1318): out[r,:] = table[ids[r],:]; ids int64. */
 int olmo355_embedding(const int64_t* ids, const void* table, void* out, int rows, int d, int vocab, int dtype,
                       void* stream);
+/* Act-order (desc_act) int4 weights: the rows of W are sorted by group once at load and the activation
+ * columns follow at run time, out[m][k] = x[m][perm[k]], 16-bit elements, K even, M <= 65535 -- the column
+ * remap of the reference's exllama back-end (AGQ/autogptq_extension/exllama/cuda_func/column_remap.cu:9-63,
+ * q4_matrix.cu:105-169); perm int32 [K], a permutation of 0..K-1 (not checked). */
+int olmo355_gather_columns(const uint16_t* x, const int32_t* perm, uint16_t* out, int M, int K, void* stream);
 /* out = a + b (residual add of the pre-norm block, olmo/model.py:794,821). */
 int olmo355_add(const void* a, const void* b, void* out, int64_t n, int dtype, void* stream);
 /* Greedy step (olmo/beam_search.py:102-113 with beam 1): first index of the row maximum,

@@ -55,6 +55,7 @@ EXPORTS = {
     "olmo355_rope_advance": (I, [P, I, P, P, P, I, I, P]),
     "olmo355_swiglu": (I, [P, P, I, I, I, P]),
     "olmo355_embedding": (I, [P, P, P, I, I, I, I, P]),
+    "olmo355_gather_columns": (I, [P, P, P, I, I, P]),
     "olmo355_add": (I, [P, P, P, L, I, P]),
     "olmo355_argmax": (I, [P, P, I, I, I, P]),
     "olmo355_incr_i32": (I, [P, P]),

@@ -513,6 +513,32 @@ extern "C" int olmo355_embedding(const int64_t* ids, const void* table, void* ou
   O355_CHECK_LAUNCH();
 }
 
+// Activation column gather for act-order int4 weights: out[m][k] = x[m][perm[k]] (16-bit elements).
+namespace {
+__global__ __launch_bounds__(256) void gather_columns_kernel(const uint16_t* __restrict__ x,
+                                                             const int32_t* __restrict__ perm,
+                                                             uint16_t* __restrict__ out, int K) {
+  const uint16_t* xr = x + (int64_t)blockIdx.y * K;
+  uint16_t* orow = out + (int64_t)blockIdx.y * K;
+  const int k = (blockIdx.x * 256 + threadIdx.x) * 2;  // two outputs per thread: one 32-bit store
+  if (k + 1 < K) {
+    const uint32_t lo = xr[perm[k]], hi = xr[perm[k + 1]];
+    *reinterpret_cast<uint32_t*>(orow + k) = lo | (hi << 16);
+  } else if (k < K) {
+    orow[k] = xr[perm[k]];
+  }
+}
+}  // namespace
+
+extern "C" int olmo355_gather_columns(const uint16_t* x, const int32_t* perm, uint16_t* out, int M, int K,
+                                      void* stream) {
+  if (!x || !perm || !out || M <= 0 || K <= 0) return O355_EINVAL;
+  if (M > 65535 || (K & 1)) return O355_EUNSUPPORTED;
+  hipLaunchKernelGGL(gather_columns_kernel, dim3((unsigned)((K / 2 + 255) / 256), (unsigned)M), dim3(256), 0,
+                     as_stream(stream), x, perm, out, K);
+  O355_CHECK_LAUNCH();
+}
+
 extern "C" int olmo355_add(const void* a, const void* b, void* out, int64_t n, int dtype, void* stream) {
   if (!a || !b || !out || n <= 0) return O355_EINVAL;
   DT_SWITCH(dtype, hipLaunchKernelGGL(add_kernel<DT>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,

@@ -193,6 +193,7 @@ class OLMo(nn.Module):
             ff_out=DenseLinear(config.d_model, V, device, dtype),
         ))
         self._prepared = False
+        self._act_order = False
         self._rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
         self._attn_ws: Dict[Tuple[int, int], torch.Tensor] = {}
         self._scratch_kv: Dict[Tuple[int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
@@ -229,6 +230,9 @@ class OLMo(nn.Module):
         c = self.config
         n_pos = max(self.max_cache_len, c.max_sequence_length)
         self._rope = ops.rope_tables(c.head_dim, float(c.rope_theta), n_pos, self.device)
+        # act-order int4 layers gather their activation columns in QuantLinear.forward: the fused decode forms
+        # (which hand the tiled weights to the kernels directly) are not used for such models
+        self._act_order = any(isinstance(m, QuantLinear) and m._perm is not None for m in self.modules())
         self._chain_ok = {}  # rows -> whether the chained decode block covers this model
         self._rope_now = None  # rotary rows of the current position during a captured decode step
         self._prepared = True
@@ -335,7 +339,7 @@ class OLMo(nn.Module):
         att = self._linear(blk.attn_out, att)
         x = blk.attn_norm(att, residual=x) if c.norm_after else ops.add(x, att)
         h = x if c.norm_after else blk.ff_norm(x)
-        if B * T <= 16 and self.dtype == torch.bfloat16:  # few rows: SwiGLU rides in the projection's epilogue
+        if B * T <= 16 and self.dtype == torch.bfloat16 and not self._act_order:  # few rows: SwiGLU rides in the projection's epilogue
             h, _ = ops.linear_fused(h, self._tiled(blk.ff_proj), swiglu_out=True)
         else:
             h = ops.swiglu(self._linear(blk.ff_proj, h))
@@ -350,7 +354,7 @@ class OLMo(nn.Module):
     def _fused_decode_ok(self, M: int, collect_hidden: bool) -> bool:
         c = self.config
         return (M <= 16 and self.dtype == torch.bfloat16 and c.norm_after and c.layer_norm_type == "rms"
-                and not collect_hidden and c.d_model * 2 * (M + 1) <= 64 * 1024 and c.d_model <= 5120)
+                and not collect_hidden and not self._act_order and c.d_model * 2 * (M + 1) <= 64 * 1024 and c.d_model <= 5120)
 
     @staticmethod
     def _tiled(m: nn.Module):

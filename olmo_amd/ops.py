@@ -287,6 +287,21 @@ def swiglu(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def gather_columns(x: torch.Tensor, perm: torch.Tensor) -> torch.Tensor:
+    """``x[..., perm]`` for 16-bit activations (the column remap in front of an act-order int4 linear)."""
+    _dev(x, perm)
+    if x.element_size() != 2 or perm.dtype != torch.int32:
+        raise TypeError("gather_columns takes 16-bit activations and an int32 permutation")
+    K = x.shape[-1]
+    if perm.numel() != K:
+        raise ValueError(f"permutation of {perm.numel()} for {K} columns")
+    out = torch.empty_like(x)
+    M = x.numel() // K
+    if M:
+        check("olmo355_gather_columns", lib().olmo355_gather_columns(_p(x), _p(perm), _p(out), M, K, _stream()))
+    return out
+
+
 def embedding(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     _dev(ids, table)
     if ids.dtype != torch.int64:

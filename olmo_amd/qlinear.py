@@ -14,8 +14,10 @@ Differences, on purpose:
   * ``post_init`` derives a re-tiled copy of the weight for the matrix-core kernels, the way the
     reference's exllama back-end rewrites ``qweight`` in its own ``post_init``
     (``qlinear_exllama.py:85-98``);
-  * only ``bits=4``, ``group_size=128``, sequential ``g_idx`` run through the linear kernels
-    (the dequantise table kernel also handles other group sizes and any ``g_idx``).
+  * only ``bits=4``, ``group_size=128`` run through the linear kernels (the dequantise table kernel
+    also handles other group sizes); act-order checkpoints (non-sequential ``g_idx``) get their rows
+    sorted by group in ``post_init`` and their activation columns gathered in ``forward``, as the
+    reference's exllama back-end does (``qlinear_exllama.py:85-98``, ``q4_matrix.cu:105-169``).
 """
 
 from __future__ import annotations
@@ -61,6 +63,7 @@ class QuantLinear(nn.Module):
         self.kernel_switch_threshold = kernel_switch_threshold
         self.trainable = trainable
         self._tiled: Optional[ops.W4Tiled] = None
+        self._perm: Optional[torch.Tensor] = None  # act-order: row order of the tiled copy (int32 [K])
 
     # -- one-time preparation ------------------------------------------------------------------
     def post_init(self, free_checkpoint_buffers: bool = False):
@@ -71,12 +74,22 @@ class QuantLinear(nn.Module):
             raise RuntimeError("QuantLinear.post_init needs the buffers on the GPU; there is no CPU path")
         K = self.infeatures
         seq = torch.arange(K, dtype=torch.int32, device=self.g_idx.device) // self.group_size
+        qweight = self.qweight
+        self._perm = None
         if not torch.equal(self.g_idx.to(torch.int32), seq):
-            raise NotImplementedError(
-                "non-sequential g_idx (act-order / desc_act checkpoints) is not supported by the linear kernels")
+            # act-order: sort the rows of W by group once (stable, so rows keep their order inside a group);
+            # forward() gathers the activation columns to match -- what the reference's exllama back-end does
+            # (q4_matrix.cu:105-169 make_sequential, column_remap.cu:9-63)
+            perm = torch.argsort(self.g_idx.to(torch.int64), stable=True)
+            if not torch.equal(self.g_idx.to(torch.int32)[perm], seq):
+                raise NotImplementedError("g_idx whose groups do not hold exactly group_size rows each is not supported")
+            sh = torch.arange(0, 32, 4, dtype=torch.int32, device=qweight.device).view(1, 8, 1)
+            q = ((qweight.unsqueeze(1) >> sh) & 15).reshape(K, self.outfeatures)[perm]  # nibbles, rows sorted
+            qweight = (q.view(K // 8, 8, self.outfeatures) << sh).sum(1, dtype=torch.int32)  # nibble 7 lands in the sign bit
+            self._perm = perm.to(torch.int32).contiguous()
         if self.bias is not None and bool(self.bias.any()):
             raise NotImplementedError("a non-zero QuantLinear bias is not implemented")
-        self._tiled = ops.w4_repack(self.qweight, self.qzeros, self.scales, self.group_size)
+        self._tiled = ops.w4_repack(qweight, self.qzeros, self.scales, self.group_size)
         if free_checkpoint_buffers:
             empty = torch.empty(0, dtype=torch.int32, device=self.qweight.device)
             self.qweight, self.qzeros = empty, empty.clone()
@@ -96,8 +109,13 @@ class QuantLinear(nn.Module):
     def dequantize(self) -> torch.Tensor:
         """fp16 ``[K, N]`` table (the reference's torch dequantize, bit for bit)."""
         if self._tiled is not None:
-            return ops.w4t_dequant_fp16(self._tiled)
-        return ops.w4_dequant_fp16(self.qweight, self.qzeros, self.scales, self.group_size)
+            t = ops.w4t_dequant_fp16(self._tiled)
+            if self._perm is None:
+                return t
+            out = torch.empty_like(t)
+            out[self._perm.long()] = t  # row i of the sorted table is row perm[i] of W
+            return out
+        return ops.w4_dequant_fp16(self.qweight, self.qzeros, self.scales, self.group_size, self.g_idx)
 
     # -- quantise a dense layer with given parameters ----------------------------------------------
     def pack(self, linear, scales, zeros, g_idx=None):
@@ -130,7 +148,11 @@ class QuantLinear(nn.Module):
         in_dtype = x.dtype
         if in_dtype != torch.bfloat16:
             x = x.to(torch.bfloat16)  # the reference casts to float16 here (qlinear_cuda_old.py:287)
-        y = ops.w4_linear(x.contiguous(), self.tiled)
+        t = self.tiled
+        x = x.contiguous()
+        if self._perm is not None:
+            x = ops.gather_columns(x, self._perm)
+        y = ops.w4_linear(x, t)
         return y if in_dtype == torch.bfloat16 else y.to(in_dtype)
 
     def extra_repr(self):
@@ -156,8 +178,6 @@ def make_quant(module: nn.Module, names: Iterable[str], bits: int, group_size: i
     layers that replace meta-device Linears."""
     if use_triton:
         raise NotImplementedError("no Triton back-end here")
-    if desc_act and group_size != -1:
-        raise NotImplementedError("desc_act (act-order) checkpoints are not supported")
     names = set(names)
     if isinstance(module, QuantLinear):
         return
@@ -175,13 +195,74 @@ def make_quant(module: nn.Module, names: Iterable[str], bits: int, group_size: i
 
 
 class OLMoGPTQForCausalLM:
-    """Wiring constants of ``inference/compression/olmo_gptq_class.py:4-17`` plus the swap itself
-    (step 2 of ``from_quantized``, ``AGQ/auto_gptq/modeling/_base.py:863-880``)."""
+    """``OLMoGPTQForCausalLM`` (``inference/compression/olmo_gptq_class.py:4-17``) on top of the parts of
+    ``BaseGPTQForCausalLM`` the inference path uses (``AGQ/auto_gptq/modeling/_base.py:85-100,450-460,
+    534-603,784-918``): the wiring constants, the Linear -> ``QuantLinear`` swap, ``from_quantized`` /
+    ``save_quantized`` for local AutoGPTQ directories, and ``forward`` / ``generate`` passed through to the
+    wrapped HF-style model.  Calibration (``quantize``) is outside this path."""
 
+    layer_type = "OLMoBlock"
     layers_block_name = "model.transformer.blocks"
     outside_layer_modules = ["model.transformer.wte", "model.transformer.ln_f"]
     inside_layer_modules = [["att_proj"], ["attn_out"], ["ff_proj"], ["ff_out"]]
     lm_head_name = "model.transformer.ff_out"
+
+    def __init__(self, model: nn.Module, quantized: bool, quantize_config):
+        self.model = model
+        self._quantized = quantized
+        self.quantize_config = quantize_config
+        self.config = model.config
+
+    @property
+    def quantized(self) -> bool:
+        return self._quantized
+
+    @property
+    def device(self) -> torch.device:
+        return next(self.model.parameters()).device
+
+    def to(self, device):
+        self.model.to(device)
+        return self
+
+    def forward(self, *args, **kwargs):
+        return self.model(*args, **kwargs)
+
+    __call__ = forward
+
+    def generate(self, **kwargs):
+        with torch.inference_mode():
+            return self.model.generate(**kwargs)
+
+    def prepare_inputs_for_generation(self, *args, **kwargs):
+        return self.model.prepare_inputs_for_generation(*args, **kwargs)
+
+    def quantize(self, *args, **kwargs):
+        raise NotImplementedError("GPTQ calibration is not part of the inference path; load a quantized directory")
+
+    def save_quantized(self, save_dir: str, use_safetensors: bool = False, safetensors_metadata=None):
+        if not self.quantized:
+            raise EnvironmentError("can only save quantized model, please execute .quantize first.")  # _base.py:540-541
+        from .checkpoint import save_quantized
+
+        return save_quantized(self.model, self.quantize_config, save_dir, use_safetensors, safetensors_metadata)
+
+    def save_pretrained(self, save_dir: str, use_safetensors: bool = False, safetensors_metadata=None, **kwargs):
+        return self.save_quantized(save_dir, use_safetensors, safetensors_metadata)  # _base.py:605-614
+
+    @classmethod
+    def from_quantized(cls, model_name_or_path: str, device="cuda:0", use_safetensors: Optional[bool] = None,
+                       quantize_config=None, model_basename: Optional[str] = None, use_triton: bool = False,
+                       trainable: bool = False, **kwargs) -> "OLMoGPTQForCausalLM":
+        if use_triton:
+            raise NotImplementedError("no Triton back-end here")
+        if trainable:
+            raise NotImplementedError("trainable=True is not implemented (inference only)")
+        from .checkpoint import from_quantized
+
+        hf, qc = from_quantized(model_name_or_path, device=device, use_safetensors=use_safetensors,
+                                quantize_config=quantize_config, model_basename=model_basename, **kwargs)
+        return cls(hf, True, qc)
 
     @classmethod
     def quantize_modules(cls, hf_model: nn.Module, bits: int = 4, group_size: int = 128) -> nn.Module:

@@ -133,7 +133,8 @@ class OracleModel:
             w = self.w[prefix + ".weight"].to(torch.float32).t()
         else:
             w = w4.dequantize(
-                self.w[prefix + ".qweight"], self.w[prefix + ".qzeros"], self.w[prefix + ".scales"], self.group_size
+                self.w[prefix + ".qweight"], self.w[prefix + ".qzeros"], self.w[prefix + ".scales"], self.group_size,
+                self.w.get(prefix + ".g_idx"),
             ).to(torch.float32)
         if self.cache_weights:
             self._wf32[prefix] = w = w.contiguous()

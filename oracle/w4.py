@@ -16,6 +16,8 @@ of the fp16 product (subnormal scales, zero scales).
 
 from __future__ import annotations
 
+from typing import Optional
+
 import numpy as np
 import torch
 
@@ -49,9 +51,12 @@ def unpack_qzeros(qzeros: torch.Tensor) -> torch.Tensor:
     return out.reshape(z.shape[0], z.shape[1] * 8)
 
 
-def dequantize(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor, group_size: int) -> torch.Tensor:
-    """The reference's torch dequantize (``AGQ:qlinear_cuda_old.py:241-285``), sequential
-    ``g_idx`` (``k // group_size``): ``W[k,n] = fp16(scales[g,n] * int8(q[k,n] - zero[g,n]))``.
+def dequantize(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor, group_size: int,
+               g_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The reference's torch dequantize (``AGQ:qlinear_cuda_old.py:241-285``):
+    ``W[k,n] = fp16(scales[g,n] * int8(q[k,n] - zero[g,n]))`` with ``g = k // group_size``, or
+    ``g = g_idx[k]`` when an act-order ``g_idx`` is given (the per-row gather of scale and zero,
+    ``AGQ:qlinear_cuda.py:253-265``).
 
     The int8 difference lies in [-16, 14]; fp16 x int8 in torch promotes the int8 to fp16
     (exact) and multiplies in fp16, i.e. the exact product rounded once to nearest-even
@@ -61,7 +66,7 @@ def dequantize(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor
     q = unpack_qweight(qweight)  # [K,N]
     z = unpack_qzeros(qzeros)  # [G,N]
     K, N = q.shape
-    g = torch.arange(K) // group_size
+    g = torch.arange(K) // group_size if g_idx is None else g_idx.to(torch.int64)
     diff = (q - z[g]).to(torch.float32)
     w = scales.to(torch.float16).to(torch.float32)[g] * diff
     return w.to(torch.float16)

@@ -297,3 +297,115 @@ def test_config2_1b_bf16_prefill_and_256_greedy_steps(dev):
     say(f"  softmax max-abs err {e:.3e}; greedy agreement over 256 steps: strict {strict:.4f} ulp {loose:.4f}")
     assert e <= 2e-2
     assert loose >= 0.99
+
+
+# ------------------------------------------------------------------------------------------------
+# checkpoint formats either side of the path
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("use_safetensors", [True, False])
+def test_gptq_directory_round_trip(dev, tmp_path, use_safetensors):
+    """save_quantized -> from_quantized (AutoGPTQ directory layout): same files, same logits, bit for bit."""
+    say("gptq directory", use_safetensors)
+    import json
+    import os
+
+    from olmo_amd.checkpoint import BaseQuantizeConfig
+    from olmo_amd.hf import OLMoConfig, OLMoForCausalLM
+    from olmo_amd.qlinear import OLMoGPTQForCausalLM, QuantLinear
+
+    cfg = small_cfg("olmo2")
+    model, _ = build_pair(cfg, torch.bfloat16, dev, quantized=True, seed=3)
+    hf = OLMoForCausalLM(OLMoConfig.from_model_config(cfg, use_cache=True), model=model)
+    qc = BaseQuantizeConfig(bits=4, group_size=128, desc_act=False)
+    wrapped = OLMoGPTQForCausalLM(hf, True, qc)
+    d = str(tmp_path / "q")
+    wrapped.save_quantized(d, use_safetensors=use_safetensors)
+    names = sorted(os.listdir(d))
+    assert names == sorted(["config.json", "quantize_config.json",
+                            "gptq_model-4bit-128g" + (".safetensors" if use_safetensors else ".bin")])
+    assert json.load(open(os.path.join(d, "quantize_config.json")))["group_size"] == 128
+    loaded = OLMoGPTQForCausalLM.from_quantized(d, device=str(dev), use_safetensors=use_safetensors)
+    assert loaded.quantized and loaded.quantize_config.model_file_base_name == "gptq_model-4bit-128g"
+    n_q = sum(isinstance(m, QuantLinear) for m in loaded.model.modules())
+    assert n_q == 4 * cfg.n_layers
+    ids = torch.randint(0, cfg.vocab_size, (2, 33), generator=torch.Generator().manual_seed(5)).to(dev)
+    a = hf(ids).logits
+    b = loaded.forward(ids).logits
+    assert torch.equal(a, b)
+    out = loaded.generate(input_ids=ids[:, :8], max_new_tokens=4)
+    assert out.shape == (2, 12)
+
+
+def test_gptq_directory_act_order(dev, tmp_path):
+    """A desc_act directory (non-sequential g_idx in every int4 layer) against the oracle on the same tensors."""
+    say("gptq directory act-order")
+    from olmo_amd.checkpoint import BaseQuantizeConfig, save_quantized
+    from olmo_amd.hf import OLMoConfig, OLMoForCausalLM
+    from olmo_amd.model import OLMo
+    from olmo_amd.qlinear import OLMoGPTQForCausalLM, make_quant
+    from oracle import w4 as ow4
+
+    cfg = small_cfg("olmo2")
+    w = om.random_weights(cfg, torch.bfloat16, seed=4, quantized=True, norm_weight_std=0.1)
+    gen = torch.Generator().manual_seed(7)
+    for key in [k for k in w if k.endswith(".qweight")]:  # scatter the rows of every int4 matrix, g_idx follows
+        q = ow4.unpack_qweight(w[key])
+        K = q.shape[0]
+        perm = torch.randperm(K, generator=gen)
+        q2 = torch.empty_like(q)
+        q2[perm] = q
+        g2 = torch.empty(K, dtype=torch.int32)
+        g2[perm] = (torch.arange(K) // 128).to(torch.int32)
+        w[key] = ow4.pack_nibbles(q2, 0)
+        w[key[:-len("qweight")] + "g_idx"] = g2
+    oracle = om.OracleModel(cfg, w, torch.bfloat16)
+    model = OLMo(cfg, device=dev, dtype=torch.bfloat16, block_weight_device="meta")
+    names = [f"transformer.blocks.{i}.{n}" for i in range(cfg.n_layers) for (n,) in OLMoGPTQForCausalLM.inside_layer_modules]
+    make_quant(model, names, 4, 128, desc_act=True, device=dev)
+    model.load_reference_state_dict(w)
+    hf = OLMoForCausalLM(OLMoConfig.from_model_config(cfg), model=model)
+    d = str(tmp_path / "q")
+    save_quantized(hf, BaseQuantizeConfig(bits=4, group_size=128, desc_act=True), d, use_safetensors=True)
+    loaded = OLMoGPTQForCausalLM.from_quantized(d, device=str(dev))
+    assert loaded.model.model._act_order
+    ids = torch.randint(0, cfg.vocab_size, (2, 40), generator=torch.Generator().manual_seed(6))
+    ref, _ = oracle.forward(ids)
+    lg = loaded.forward(ids.to(dev)).logits.cpu()
+    err = softmax_err(lg, ref)
+    say("  act-order softmax err", err)
+    assert err <= 2e-2
+    # decode steps with a cache go through the same layers
+    out = loaded.generate(input_ids=ids[:, :8].to(dev), max_new_tokens=4)
+    full, _ = oracle.forward(out.cpu())
+    strict, loose = agreement(out[:, 8:].cpu(), full[:, 7:-1])
+    assert loose == 1.0
+
+
+def test_unsharded_checkpoint_and_hf_layout(dev, tmp_path):
+    """config.yaml + model.pt (OLMo.from_checkpoint's unsharded layout) and the HF Olmo2 tensor layout both
+    lead back to the same logits."""
+    say("unsharded checkpoint / HF layout")
+    import yaml
+    from dataclasses import asdict
+
+    from olmo_amd.checkpoint import (hf_olmo2_to_olmo_state_dict, load_unsharded_checkpoint,
+                                     olmo_to_hf_olmo2_state_dict)
+    from olmo_amd.model import OLMo
+
+    cfg = small_cfg("olmo2-gqa")
+    model, _ = build_pair(cfg, torch.bfloat16, dev, seed=9)
+    ids = torch.randint(0, cfg.vocab_size, (2, 21), generator=torch.Generator().manual_seed(2)).to(dev)
+    ref = model(ids).logits
+    sd = {k: v.cpu() for k, v in model.state_dict().items()}
+    d = tmp_path / "ckpt"
+    d.mkdir()
+    mc = asdict(cfg)
+    mc.pop("extra", None)
+    (d / "config.yaml").write_text(yaml.safe_dump({"model": mc, "run_name": "x"}))
+    torch.save({"_fsdp_wrapped_module." + k: v for k, v in sd.items()}, d / "model.pt")  # an FSDP-era key prefix
+    m2 = load_unsharded_checkpoint(str(d), device=str(dev))
+    assert torch.equal(m2(ids).logits, ref)
+    hf_sd = olmo_to_hf_olmo2_state_dict(sd, cfg)
+    m3 = OLMo(cfg, device=dev, dtype=torch.bfloat16)
+    m3.load_reference_state_dict(hf_olmo2_to_olmo_state_dict(hf_sd, cfg))
+    assert torch.equal(m3.post_init()(ids).logits, ref)

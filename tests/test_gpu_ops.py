@@ -591,3 +591,55 @@ def test_w4_gemv_chain(dev, M, N, K, epi):
     if ssq is not None:
         want = (y.float().cpu() ** 2).view(M, -1, 16).sum(-1)
         assert torch.allclose(ssq.cpu(), want, rtol=1e-5, atol=1e-6 * want.max().item())
+
+
+# ------------------------------------------------------------------------------------------------
+# act-order (desc_act) int4 layers
+# ------------------------------------------------------------------------------------------------
+def _act_order_case(K, N, seed):
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=seed)
+    perm = torch.randperm(K, generator=torch.Generator().manual_seed(seed))
+    g_idx = torch.empty(K, dtype=torch.int32)
+    g_idx[perm] = (torch.arange(K) // 128).to(torch.int32)  # what GPTQ writes with desc_act (quantization/gptq.py order)
+    q, z = ow4.unpack_qweight(qw), ow4.unpack_qzeros(qz)
+    W = (sc.float()[g_idx.long()] * (q - z[g_idx.long()]).float()).half()  # qlinear_cuda_old.py:253-265 semantics
+    return qw, qz, sc, g_idx, W
+
+
+@pytest.mark.parametrize("M", [1, 7, 40, 300])
+@pytest.mark.parametrize("K,N,free", [(512, 256, False), (4096, 1024, True)])
+def test_qlinear_act_order(dev, M, K, N, free):
+    """Non-sequential g_idx: rows sorted by group at post_init, activation columns gathered in forward."""
+    say("qlinear act-order", M, K, N, free)
+    from olmo_amd.qlinear import QuantLinear
+
+    qw, qz, sc, g_idx, W = _act_order_case(K, N, seed=K + N)
+    m = QuantLinear(4, 128, K, N, True, device=dev)
+    m.qweight.copy_(qw), m.qzeros.copy_(qz), m.scales.copy_(sc), m.g_idx.copy_(g_idx)
+    assert torch.equal(m.dequantize().cpu().view(torch.int16), W.view(torch.int16))  # table straight from the buffers
+    m.post_init(free_checkpoint_buffers=free)
+    assert m._perm is not None
+    assert torch.equal(m.dequantize().cpu().view(torch.int16), W.view(torch.int16))  # and from the sorted, tiled copy
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(M)).to(torch.bfloat16)
+    ref = ow4.linear_fp32(x, W)
+    y = m(x.to(dev)).float().cpu()
+    assert (y - ref).abs().max().item() <= 2 ** -7 * ref.abs().max().item()
+
+
+def test_qlinear_act_order_uneven_groups_rejected(dev):
+    from olmo_amd.qlinear import QuantLinear
+
+    m = QuantLinear(4, 128, 256, 32, True, device=dev)
+    g = torch.zeros(256, dtype=torch.int32)
+    g[200:] = 1  # 200 rows in group 0, 56 in group 1
+    m.g_idx.copy_(g)
+    with pytest.raises(NotImplementedError):
+        m.post_init()
+
+
+def test_gather_columns(dev):
+    ops = _ops()
+    x = torch.randn(5, 1026, generator=torch.Generator().manual_seed(0)).to(torch.bfloat16)
+    perm = torch.randperm(1026, generator=torch.Generator().manual_seed(1)).to(torch.int32)
+    out = ops.gather_columns(x.to(dev), perm.to(dev)).cpu()
+    assert torch.equal(out.view(torch.int16), x[:, perm.long()].view(torch.int16))

@@ -88,3 +88,22 @@ def test_pack_linear_quantises_back_to_grid():
     assert torch.equal(w4.unpack_qzeros(qz), zeros.t().to(torch.int32))
     Wd = w4.dequantize(qw, qz, s16, g)
     assert torch.allclose(Wd.float().t(), W, rtol=1e-3, atol=1e-6)
+
+
+def test_dequant_act_order_g_idx_matches_bruteforce():
+    """Per-row gather of scale and zero (``AGQ:qlinear_cuda.py:253-265``) against a scalar loop."""
+    import numpy as np
+
+    K, N, g = 256, 16, 128
+    qw, qz, sc = w4.random_quantized(K, N, g, seed=3)
+    g_idx = (torch.randperm(K, generator=torch.Generator().manual_seed(0)) // g).to(torch.int32)
+    out = w4.dequantize(qw, qz, sc, g, g_idx)
+    qwn, qzn = qw.numpy().astype(np.int64) & 0xFFFFFFFF, qz.numpy().astype(np.int64) & 0xFFFFFFFF
+    scn = sc.numpy()
+    for k in range(0, K, 7):
+        gi = int(g_idx[k])
+        for n in range(N):
+            q = (int(qwn[k >> 3, n]) >> (4 * (k & 7))) & 15
+            z = ((int(qzn[gi, n >> 3]) >> (4 * (n & 7))) & 15) + 1
+            assert out[k, n].item() == float(np.float16(np.float32(scn[gi, n]) * np.float32(q - z)))
+    assert torch.equal(w4.dequantize(qw, qz, sc, g, torch.arange(K) // g), w4.dequantize(qw, qz, sc, g))
