@@ -106,12 +106,13 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const void* __restrict
 // Workgroup: 4 waves x 32 queries = 128 queries of one (batch, head); KV tile: 64 keys.
 // LDS  K  : [key-tile 4][hd-step HD/32][64 lanes][8 bf16]   A operand of S^T = K . Q^T
 //      V^T: [hd-tile HD/16][key-step 2][64 lanes][8 bf16]   A operand of O^T = V^T . P^T
+//      (plus pad slots, see the declarations)
 // In the second product the 8 key slots of lane group kq in key-step s are
 //   e<4 : key 32s + 4kq + e        e>=4 : key 32s + 16 + 4kq + (e-4)
 // which is exactly how the S^T accumulators of the two 16-key tiles 2s, 2s+1 sit in a lane, so
 // P goes from accumulator registers to the B operand without leaving the lane.
 template <int HD>
-__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const uint16_t* __restrict__ q,
+__global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_t* __restrict__ q,
                                                                 const uint16_t* __restrict__ kc,
                                                                 const uint16_t* __restrict__ vc,
                                                                 const float* __restrict__ key_bias,
@@ -121,22 +122,25 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const uint16_t* 
   constexpr int STEPS = HD / 32;     // hd steps of the first product
   constexpr int HT = HD / 16;        // hd tiles of the second product
   constexpr int QT = 2;              // 16-query tiles per wave
-  __shared__ __align__(16) u32x4 lds_k[4 * STEPS * 64];
-  __shared__ __align__(16) u32x4 lds_v[HT * 2 * 64];
+  // 16-byte slots; a pad slot after every 16 (K) / every 128 (V) spreads the staging writes over the banks
+  __shared__ __align__(16) u32x4 lds_k[4 * STEPS * 4 * 17];
+  __shared__ __align__(16) u32x4 lds_v[HT * 129];
   __shared__ float lds_bias[KT];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, kq = lane >> 4;
-  // Causal work grows with the query block, so a workgroup takes a complementary pair: block
-  // nqb-1-x (many key tiles) and then block x (few); every workgroup does the same amount.
+  // One 128-query block per workgroup, two workgroups per CU.  Causal work grows with the block index;
+  // blockIdx.y is the rank in this order: the heaviest half of the blocks (descending), then the
+  // lightest half (ascending), so the two workgroups a CU holds -- rank r and rank r + nqb/2 when the
+  // grid just fills the chip, heads varying fastest -- add up to about the same number of key tiles.
   const int nqb = (T + 127) / 128;
-  const int b = blockIdx.z, h = blockIdx.y, hk = h / (H / Hkv);
-  const float scale = 1.f / sqrtf((float)HD);
+  const int b = blockIdx.z, h = blockIdx.x, hk = h / (H / Hkv);
   const float lowest = -3.3895313892515355e38f;
+  const float c2 = 1.4426950408889634f / sqrtf((float)HD);  // scores live in the log2 domain: exp2(s*c2 + bias*log2e - m)
   const int64_t cbase = ((int64_t)b * Hkv + hk) * Lmax * HD;
-  for (int pass = 0; pass < 2; ++pass) {
-  const int qblock = pass == 0 ? nqb - 1 - (int)blockIdx.x : (int)blockIdx.x;
-  if (pass == 1 && qblock >= nqb - 1 - (int)blockIdx.x) break;  // the middle block of an odd count is its own pair
+  const int half = (nqb + 1) / 2, rank = blockIdx.y;
+  const int qblock = rank < half ? nqb - 1 - rank : rank - half;
+  {
   const int q0 = qblock * 128 + wave * 32;
 
   // Q^T fragments: lane (query col, hd 32*step + 8*kq ..)
@@ -168,25 +172,30 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const uint16_t* 
   constexpr int VPT = (KT / 2) * CPR / 256;       // V chunk pairs (two consecutive keys) per thread per tile
   u32x4 rkk[KPT], rv0[VPT], rv1[VPT];
   float rbias = 0.f;
+  const uint16_t* kbase = kc + cbase;
+  const uint16_t* vbase = vc + cbase;
   auto fetch = [&](int k0) {
+    const bool tail = k0 + KT - 1 > last_pos;  // only the last tile can reach past the last visible key
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
       const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
-      rkk[i] = *reinterpret_cast<const u32x4*>(kc + cbase + (int64_t)min(k0 + kk, last_pos) * HD + 8 * c);
+      const uint32_t row = tail ? min(k0 + kk, last_pos) : k0 + kk;
+      rkk[i] = *reinterpret_cast<const u32x4*>(kbase + (row * HD + 8 * c));
     }
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
       const int e = tid + i * 256, kk = 2 * (e / CPR), c = e % CPR;
-      rv0[i] = *reinterpret_cast<const u32x4*>(vc + cbase + (int64_t)min(k0 + kk, last_pos) * HD + 8 * c);
-      rv1[i] = *reinterpret_cast<const u32x4*>(vc + cbase + (int64_t)min(k0 + kk + 1, last_pos) * HD + 8 * c);
+      const uint32_t r0 = tail ? min(k0 + kk, last_pos) : k0 + kk, r1 = tail ? min(k0 + kk + 1, last_pos) : k0 + kk + 1;
+      rv0[i] = *reinterpret_cast<const u32x4*>(vbase + (r0 * HD + 8 * c));
+      rv1[i] = *reinterpret_cast<const u32x4*>(vbase + (r1 * HD + 8 * c));
     }
-    if (tid < KT) rbias = key_bias ? key_bias[(int64_t)b * bias_stride + min(k0 + tid, last_pos)] : 0.f;
+    if (key_bias && tid < KT) rbias = key_bias[(int64_t)b * bias_stride + min(k0 + tid, last_pos)];
   };
   auto stash = [&]() {
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
       const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
-      lds_k[((kk >> 4) * STEPS + (c >> 2)) * 64 + (kk & 15) + 16 * (c & 3)] = rkk[i];
+      lds_k[(((kk >> 4) * STEPS + (c >> 2)) * 4 + (c & 3)) * 17 + (kk & 15)] = rkk[i];
     }
     // V^T: key pairs (kk, kk+1) x 8 hd values -> 8 dword writes
 #pragma unroll
@@ -201,7 +210,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const uint16_t* 
         const int ht = hd_ >> 4, lo = hd_ & 15;
         const uint32_t a = (x & 1) ? (rv0[i][x >> 1] >> 16) : (rv0[i][x >> 1] & 0xffffu);
         const uint32_t bb = (x & 1) ? (rv1[i][x >> 1] >> 16) : (rv1[i][x >> 1] & 0xffffu);
-        dst[(((ht * 2 + s2) * 64 + kq_ * 16 + lo) * 8 + e0) >> 1] = a | (bb << 16);
+        dst[((ht * 129 + s2 * 64 + kq_ * 16 + lo) * 8 + e0) >> 1] = a | (bb << 16);
       }
     }
     if (tid < KT) lds_bias[tid] = rbias;
@@ -222,49 +231,63 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const uint16_t* 
       for (int qt = 0; qt < QT; ++qt) s[qt][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int st = 0; st < STEPS; ++st) {
-        const bf16x8 kf = __builtin_bit_cast(bf16x8, lds_k[(kt * STEPS + st) * 64 + lane]);
+        const bf16x8 kf = __builtin_bit_cast(bf16x8, lds_k[((kt * STEPS + st) * 4 + kq) * 17 + col]);
 #pragma unroll
         for (int qt = 0; qt < QT; ++qt) s[qt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qt][st], s[qt][kt], 0, 0, 0);
       }
     }
-    // ---- online softmax per query column ----------------------------------------------------------------
+    // ---- online softmax per query column, in the log2 domain -----------------------------------------------
+    // Only tiles that reach past the wave's first query need the causal compare, and only calls with a
+    // padding bias need the bias terms: the common tile costs a max, one fma and one exp2 per score.
+    const bool masked = key_bias != nullptr || k0 + KT - 1 > past_len + q0;  // wave-uniform
+    const float cs = masked ? 1.f : c2;  // the masked path leaves its scores already scaled
     bf16x8 pf[QT][2];
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
       float tmax = -INFINITY;
+      if (masked) {
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt)
+        for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int kk = kt * 16 + 4 * kq + r;
-          const int key = k0 + kk;
-          const float bias = lds_bias[kk];
-          float v = bias <= kMaskThreshold ? lowest : s[qt][kt][r] * scale + bias;
-          v = key > qpos[qt] ? -INFINITY : v;
-          s[qt][kt][r] = v;
-          tmax = fmaxf(tmax, v);
-        }
+          for (int r = 0; r < 4; ++r) {
+            const int kk = kt * 16 + 4 * kq + r;
+            const float bias = lds_bias[kk];
+            float v = bias <= kMaskThreshold ? lowest : __builtin_fmaf(s[qt][kt][r], c2, bias * 1.4426950408889634f);
+            v = k0 + kk > qpos[qt] ? -INFINITY : v;
+            s[qt][kt][r] = v;
+            tmax = fmaxf(tmax, v);
+          }
+      } else {
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) tmax = fmaxf(tmax, s[qt][kt][r]);
+        tmax *= c2;  // c2 > 0: the maximum commutes with the scaling
+      }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
       const float mn = fmaxf(m[qt], tmax);  // finite: key 0 of the first tile is visible to every query
-      const float alpha = __expf(m[qt] - mn);
       float psum = 0.f;
       float p[4][4];
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          p[kt][r] = __expf(s[qt][kt][r] - mn);
+          p[kt][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qt][kt][r], cs, -mn));
           psum += p[kt][r];
         }
       psum += __shfl_xor(psum, 16, 64);
       psum += __shfl_xor(psum, 32, 64);
-      l[qt] = l[qt] * alpha + psum;
-      m[qt] = mn;
+      if (__builtin_amdgcn_ballot_w64(mn != m[qt]) != 0) {  // the running maximum moved for some query of the wave
+        const float alpha = __builtin_amdgcn_exp2f(m[qt] - mn);
+        l[qt] *= alpha;
 #pragma unroll
-      for (int ht = 0; ht < HT; ++ht)
+        for (int ht = 0; ht < HT; ++ht)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o[qt][ht][r] *= alpha;
+          for (int r = 0; r < 4; ++r) o[qt][ht][r] *= alpha;
+        m[qt] = mn;
+      }
+      l[qt] += psum;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         u32x4 w;
@@ -280,7 +303,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const uint16_t* 
     for (int ht = 0; ht < HT; ++ht)
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
-        const bf16x8 vf = __builtin_bit_cast(bf16x8, lds_v[(ht * 2 + s2) * 64 + lane]);
+        const bf16x8 vf = __builtin_bit_cast(bf16x8, lds_v[ht * 129 + s2 * 64 + lane]);
 #pragma unroll
         for (int qt = 0; qt < QT; ++qt) o[qt][ht] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[qt][s2], o[qt][ht], 0, 0, 0);
       }
@@ -300,7 +323,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const uint16_t* 
       *reinterpret_cast<u32x2*>(dst + 16 * ht + 4 * kq) = w;
     }
   }
-  }  // pass
+  }
 }
 
 // =====================================================================================================
@@ -808,8 +831,8 @@ extern "C" int olmo355_attn_prefill(const void* q, const void* kcache, const voi
   if (B <= 0 || T <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || past_len < 0 || past_len + T > Lmax) return O355_EINVAL;
   if (key_bias && bias_stride < past_len + T) return O355_EINVAL;
   hipStream_t s = as_stream(stream);
-  if (dtype == O355_BF16 && (hd == 128 || hd == 64)) {
-    const dim3 grid(((T + 127) / 128 + 1) / 2, H, B);  // pairs of query blocks
+  if (dtype == O355_BF16 && (hd == 128 || hd == 64) && (int64_t)Lmax * hd < (1ll << 31)) {  // 32-bit offsets within a head
+    const dim3 grid(H, (T + 127) / 128, B);  // heads fastest, then query blocks by rank (see the kernel)
     if (hd == 128)
       hipLaunchKernelGGL(attn_prefill_mfma_kernel<128>, grid, dim3(256), 0, s, (const uint16_t*)q,
                          (const uint16_t*)kcache, (const uint16_t*)vcache, key_bias, (uint16_t*)out, T, H, Hkv, Lmax,
