@@ -162,6 +162,60 @@ def main() -> int:
     extra["prefill_gemm"] = {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
                              "frac": tf / MFMA_BF16_PEAK_TF, "M": ctx}
     log(f"[bench] int4 prefill GEMMs (M={ctx}): {tf:.0f} TFLOP/s = {tf / MFMA_BF16_PEAK_TF:.1%} of bf16 MFMA peak")
+    # ---- what this box gives a kernel that only streams the same weights / only issues MFMAs ----------
+    # Same launches as above (one per block Linear, distinct buffers, one captured graph), but the kernel reads
+    # the tiled weight bytes and does nothing else: the distance from here to the published 8 TB/s is not the
+    # linear kernel's to close.  The matrix-core probe runs v_mfma_f32_32x32x16_bf16 on random operands.
+    from olmo_amd._lib import check as _check, lib as _lib
+
+    sink = torch.zeros(1024, dtype=torch.int32, device=dev)
+
+    def stream_all():
+        st_ = torch.cuda.current_stream().cuda_stream
+        for q in qls:
+            t = q.tiled
+            _check("olmo355_probe_stream_read",
+                   _lib().olmo355_probe_stream_read(t.wt.data_ptr(), t.wt.numel() * t.wt.element_size(), sink.data_ptr(), st_))
+
+    stream_all()
+    torch.cuda.synchronize()
+    gs = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gs):
+        stream_all()
+    gs.replay()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        gs.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    s_avg = e0.elapsed_time(e1) * 1e-3 / (reps * n_launch)
+    wt_bytes = sum(q.tiled.wt.numel() * q.tiled.wt.element_size() for q in qls) / n_launch
+    assert int(sink.abs().sum().item()) == 0
+    extra["ceilings"] = {
+        "stream_read": {"what": "a kernel that only reads the same int4 weight tiles, same 128 launches in one graph",
+                        "avg_launch_us": s_avg * 1e6, "bytes_per_launch": wt_bytes, "achieved": wt_bytes / s_avg / 1e9,
+                        "unit": "GB/s", "linear_time_over_stream_time": avg_s / s_avg},
+    }
+    log(f"[bench] ceiling on this box: streaming the same weights {s_avg * 1e6:.2f} us/launch = {wt_bytes / s_avg / 1e9:.0f} GB/s "
+        f"(linear / stream = {avg_s / s_avg:.2f})")
+
+    # matrix cores alone, after the GEMM timing (a sustained MFMA burst lowers the clocks of what follows)
+    import ctypes
+
+    fl = ctypes.c_double(0.0)
+    _check("olmo355_probe_mfma_bf16", _lib().olmo355_probe_mfma_bf16(2000, sink.data_ptr(), ctypes.byref(fl),
+                                                                     torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    e0.record()
+    _check("olmo355_probe_mfma_bf16", _lib().olmo355_probe_mfma_bf16(20000, sink.data_ptr(), ctypes.byref(fl),
+                                                                     torch.cuda.current_stream().cuda_stream))
+    e1.record()
+    torch.cuda.synchronize()
+    mfma_tf = fl.value / (e0.elapsed_time(e1) * 1e-3) / 1e12
+    extra["ceilings"]["mfma_bf16_random_operands"] = {"achieved": mfma_tf, "unit": "TFLOP/s",
+                                                      "frac_of_peak": mfma_tf / MFMA_BF16_PEAK_TF}
+    log(f"[bench] ceiling on this box: MFMA-only bf16 (32x32x16, random operands, all CUs): {mfma_tf:.0f} TFLOP/s")
     del xp
 
     # ---- batch 8 ------------------------------------------------------------------------------------

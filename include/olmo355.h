@@ -201,6 +201,14 @@ int olmo355_argmax(const void* logits, int64_t* out, int rows, int n, int dtype,
 /* *p += 1 for a device int32 (advances the position between captured decode steps). */
 int olmo355_incr_i32(int32_t* p, void* stream);
 
+/* ---- measuring probes (no counterpart in the reference; used by bench.py only) -------------------
+ * What a kernel that only streams `bytes` from HBM takes (16-byte non-temporal loads per lane, launch shaped
+ * like the small-M linears; nothing is written), and what the matrix cores sustain on random bf16 operands
+ * (256 workgroups x 8 waves x iters x 8 v_mfma_f32_32x32x16_bf16; *flops = total floating-point operations).
+ * `sink` is a device buffer of at least 2 KiB that stays unwritten. */
+int olmo355_probe_stream_read(const void* src, int64_t bytes, void* sink, void* stream);
+int olmo355_probe_mfma_bf16(int iters, void* sink, double* flops, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -56,6 +56,8 @@ EXPORTS = {
     "olmo355_swiglu": (I, [P, P, I, I, I, P]),
     "olmo355_embedding": (I, [P, P, P, I, I, I, I, P]),
     "olmo355_gather_columns": (I, [P, P, P, I, I, P]),
+    "olmo355_probe_stream_read": (I, [P, L, P, P]),
+    "olmo355_probe_mfma_bf16": (I, [I, P, P, P]),
     "olmo355_add": (I, [P, P, P, L, I, P]),
     "olmo355_argmax": (I, [P, P, I, I, I, P]),
     "olmo355_incr_i32": (I, [P, P]),

@@ -1,0 +1,90 @@
+// Two measuring probes, not part of the forward pass: what this GPU gives a kernel that only streams bytes
+// from HBM, and one that only issues bf16 MFMAs on random operands.  bench.py reports them beside the
+// achieved figures so that "fraction of the published peak" can be read against what is reachable at the
+// same launch sizes on the same box.
+#include "common.h"
+
+namespace {
+
+// Every wave reads 1 KiB pieces (16 bytes per lane, non-temporal) round-robin with U requests in flight and
+// folds them into one word; nothing is written unless the fold hits a value it cannot predict.
+template <int U>
+__global__ __launch_bounds__(512) void stream_read_kernel(const u32x4* __restrict__ src, int64_t pieces,
+                                                          uint32_t* __restrict__ sink) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 6), nw = (int64_t)gridDim.x * 8;
+  uint32_t acc = 0;
+  for (int64_t p = wave; p < pieces; p += nw * U) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t q = p + u * nw;
+      v[u] = q < pieces ? __builtin_nontemporal_load(&src[q * 64 + lane]) : u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  if (acc == 0x9e3779b9u) sink[threadIdx.x] = acc;
+}
+
+// 8 waves per workgroup, 8 independent 32x32 accumulators per wave, operands drawn once from a generator
+// (random mantissas and signs, exponents near 1: constant operands run faster than a real product does).
+__global__ __launch_bounds__(512) void mfma_bf16_kernel(float* __restrict__ sink, int iters, uint32_t seed) {
+  typedef float f32x16 __attribute__((ext_vector_type(16)));
+  f32x16 acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+  uint32_t r = seed + (blockIdx.x * 512 + threadIdx.x) * 2654435761u;
+  auto draw = [&]() {
+    u32x4 v;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      r = r * 1664525u + 1013904223u;
+      v[j] = (r & 0x807f807fu) | 0x3f003f00u;  // +-[0.5, 1)
+    }
+    return __builtin_bit_cast(bf16x8, v);
+  };
+  bf16x8 a[4], b[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) a[i] = draw();
+#pragma unroll
+  for (int i = 0; i < 2; ++i) b[i] = draw();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i * 2 + j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i * 2 + j], 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s += acc[i][0];
+  if (s == 12345.678f) sink[threadIdx.x] = s;
+}
+
+}  // namespace
+
+extern "C" int olmo355_probe_stream_read(const void* src, int64_t bytes, void* sink, void* stream) {
+  if (!src || !sink || bytes < 1024) return O355_EINVAL;
+  const int64_t pieces = bytes >> 10;
+  // as in the small-M linears: enough waves that none holds more than a few pieces
+  if (pieces >= 8 * 8 * 512) {
+    const unsigned grid = (unsigned)std::min<int64_t>((pieces + 63) / 64, 4096);
+    hipLaunchKernelGGL(stream_read_kernel<8>, dim3(grid), dim3(512), 0, as_stream(stream), (const u32x4*)src, pieces,
+                       (uint32_t*)sink);
+  } else {
+    const unsigned grid = (unsigned)std::max<int64_t>((pieces + 15) / 16, 1);
+    hipLaunchKernelGGL(stream_read_kernel<2>, dim3(grid), dim3(512), 0, as_stream(stream), (const u32x4*)src, pieces,
+                       (uint32_t*)sink);
+  }
+  O355_CHECK_LAUNCH();
+}
+
+// 256 workgroups x 8 waves x iters x 8 MFMAs of 32x32x16 (32768 flop each); *flops receives the total.
+extern "C" int olmo355_probe_mfma_bf16(int iters, void* sink, double* flops, void* stream) {
+  if (iters <= 0 || !sink) return O355_EINVAL;
+  hipLaunchKernelGGL(mfma_bf16_kernel, dim3(256), dim3(512), 0, as_stream(stream), (float*)sink, iters, 77u);
+  if (flops) *flops = 256.0 * 8.0 * (double)iters * 8.0 * 32768.0;
+  O355_CHECK_LAUNCH();
+}

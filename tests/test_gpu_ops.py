@@ -643,3 +643,23 @@ def test_gather_columns(dev):
     perm = torch.randperm(1026, generator=torch.Generator().manual_seed(1)).to(torch.int32)
     out = ops.gather_columns(x.to(dev), perm.to(dev)).cpu()
     assert torch.equal(out.view(torch.int16), x[:, perm.long()].view(torch.int16))
+
+
+def test_measuring_probes(dev):
+    """The two probes bench.py reports beside the achieved figures run and leave their sink untouched."""
+    import ctypes
+
+    from olmo_amd import _lib
+
+    h = _lib.lib()
+    src = torch.randint(-2 ** 31, 2 ** 31 - 1, (3 * 1024 * 1024 + 512,), dtype=torch.int32, device=dev)  # not a KiB multiple
+    sink = torch.zeros(1024, dtype=torch.int32, device=dev)
+    s = torch.cuda.current_stream().cuda_stream
+    for nbytes in (1024, 70 * 1024, src.numel() * 4, 40 * 2 ** 20 // 4 * 0 + 2048):
+        assert h.olmo355_probe_stream_read(src.data_ptr(), nbytes, sink.data_ptr(), s) == 0
+    assert h.olmo355_probe_stream_read(src.data_ptr(), 100, sink.data_ptr(), s) == 1  # less than one piece
+    fl = ctypes.c_double(0.0)
+    assert h.olmo355_probe_mfma_bf16(10, sink.data_ptr(), ctypes.byref(fl), s) == 0
+    torch.cuda.synchronize()
+    assert fl.value == 256 * 8 * 10 * 8 * 32768.0
+    assert int(sink.abs().sum().item()) == 0
