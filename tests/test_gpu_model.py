@@ -252,11 +252,14 @@ def test_quantlinear_module_surface(dev):
     ql2.pack(lin, scales, zeros)
     assert torch.equal(ow4.unpack_qweight(ql2.qweight.cpu()), qtrue.t().to(torch.int32))
     assert torch.equal(ow4.unpack_qzeros(ql2.qzeros.cpu()), zeros.t().to(torch.int32))
-    # act-order checkpoints are rejected explicitly
+    # a non-sequential g_idx (act-order) is taken: rows sorted by group, columns gathered in forward
     ql3 = QuantLinear(4, 128, K, N, True).to(dev)
-    ql3.g_idx = ql3.g_idx.flip(0).contiguous()
-    with pytest.raises(NotImplementedError):
-        ql3.post_init()
+    ql3.load_state_dict({"qweight": qw, "qzeros": qz, "scales": sc, "g_idx": (torch.arange(K, dtype=torch.int32) // 128).flip(0),
+                         "bias": torch.zeros(N, dtype=torch.float16)})
+    ql3.post_init()
+    assert ql3._perm is not None
+    W3 = ow4.dequantize(qw, qz, sc, 128, (torch.arange(K) // 128).flip(0))
+    assert torch.equal(ql3.dequantize().cpu().view(torch.int16), W3.view(torch.int16))
 
 
 def test_config1_fp32_20m_full(dev):
