@@ -102,6 +102,11 @@ int olmo355_w4_gemv_chain(const uint16_t* x, const uint16_t* resid, const uint16
  * exllama's reconstruct + cublasHgemm (exllama/cuda_func/q4_matmul.cu:222-260). */
 int olmo355_w4_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
                     int M, int N, int K, void* stream);
+/* The same product for an ff_proj weight ([up | gate] column halves) with SwiGLU (olmo/model.py:365-368,813-819)
+ * in the epilogue: y [M, N/2] = silu(gate) * up, each factor rounded to bf16 first as the separate Linear and
+ * activation would.  N a multiple of 256; O355_EUNSUPPORTED otherwise: olmo355_w4_gemm + olmo355_swiglu. */
+int olmo355_w4_gemm_swiglu(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
+                           int M, int N, int K, void* stream);
 
 /* ---- dense Linear (nn.Linear without bias: olmo/model.py:452-462,695-701,1129-1139) -------
  * bf16: weight pre-tiled by olmo355_b16_repack into [N/16][K/32][64 lanes][8 bf16]

@@ -41,6 +41,7 @@ EXPORTS = {
     "olmo355_w4_gemv_chain": (I, [P, P, P, F, P, P, P, P, P, P, P, I, I, I, I, P]),
     "olmo355_b16_gemv_fused": (I, [P, P, P, F, P, P, P, I, I, I, I, P]),
     "olmo355_w4_gemm": (I, [P, P, P, P, P, I, I, I, P]),
+    "olmo355_w4_gemm_swiglu": (I, [P, P, P, P, P, I, I, I, P]),
     "olmo355_b16_repack": (I, [P, P, I, I, P]),
     "olmo355_b16_gemv": (I, [P, P, P, I, I, I, P]),
     "olmo355_b16_gemm": (I, [P, P, P, I, I, I, P]),

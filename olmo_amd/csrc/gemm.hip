@@ -53,7 +53,10 @@ __device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& 
   }
 }
 
-template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4>  // wave grid, 32x32 MFMA tiles per wave
+// SWIGLU (int4, WNT == 2): the weight holds [up | gate] column halves of N/2 each; a tile's first 32-column
+// block per wave comes from the up half and its second from the matching gate columns, so both land in
+// the same lanes and the epilogue writes silu(gate) * up, [M, N/2] (SwiGLU.forward, olmo/model.py:365-368).
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false>  // wave grid, 32x32 MFMA tiles per wave
 __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wt,
                                           const uint16_t* __restrict__ st, const uint8_t* __restrict__ zt,
                                           uint16_t* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n) {
@@ -76,8 +79,15 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   int tile_m, tile_n;
   tile_of(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
-  const int m0 = tile_m * BM, nt0 = tile_n * (BN / 16);
+  static_assert(!SWIGLU || (W4 && WNT == 2), "fused SwiGLU: int4 weights, two column blocks per wave");
+  const int m0 = tile_m * BM, nt0 = SWIGLU ? 0 : tile_n * (BN / 16);  // fused: absolute tile indices, see tile_abs
   const int ntiles = N >> 4;
+  // 16-column tile of the weight behind local tile ntl (32-column block ntl/2 = wave column wn = ntl/4, block j)
+  auto tile_abs = [&](int ntl) {
+    if constexpr (!SWIGLU) return ntl;
+    const int ct = ntl >> 1, j = ct & 1, wn_ = ct >> 1;
+    return (j ? (ntiles >> 1) : 0) + tile_n * (BN / 32) + wn_ * 2 + (ntl & 1);
+  };
   const int G = K >> 7, KS = K >> 5;
   const int stages = K / BK;
   const int row32 = lane & 31, kh = lane >> 5;
@@ -126,10 +136,10 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   if constexpr (W4) {
 #pragma unroll
     for (int i = 0; i < B_ITEMS; ++i) {
-      const int ntl = wave + NW * i, col = lane & 15;
-      bw_voff[i] = (ntl * G * 64 + lane) * 16;
-      bs_voff[i] = (ntl * G * 16 + col) * 2;
-      bz_voff[i] = ntl * G * 8 + (col >> 1);
+      const int nta = tile_abs(wave + NW * i), col = lane & 15;
+      bw_voff[i] = (nta * G * 64 + lane) * 16;
+      bs_voff[i] = (nta * G * 16 + col) * 2;
+      bz_voff[i] = nta * G * 8 + (col >> 1);
     }
   }
   auto fetch_b = [&](int g, int set, int part = -1) {  // part: as for the activations
@@ -271,6 +281,20 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   }
 
   // ---- epilogue: D[m = 8*(r/4) + 4*(lane>>5) + r%4][n = lane&31] of each 32x32 tile ---------------------
+  if constexpr (SWIGLU) {
+    const int half_n = N >> 1;
+    const int n = tile_n * (BN / 2) + wn * 32 + (lane & 31);  // no ragged columns: N/2 is a multiple of BN/2
+#pragma unroll
+    for (int i = 0; i < WMT; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + (wm * WMT + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const float up = round_bf16(acc[i][0][r]), gate = round_bf16(acc[i][1][r]);  // the Linear's bf16 output
+        const float sg = round_bf16(gate / (1.f + expf(-gate)));
+        if (m < M) y[(int64_t)m * half_n + n] = f32_to_bf16_bits(sg * up);
+      }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < WMT; ++i)
 #pragma unroll
@@ -285,23 +309,23 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     }
 }
 
-template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4>
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const uint16_t* __restrict__ x,
                                                                      const uint32_t* __restrict__ wt,
                                                                      const uint16_t* __restrict__ st,
                                                                      const uint8_t* __restrict__ zt,
                                                                      uint16_t* __restrict__ y, int M, int N, int K,
                                                                      int tiles_m, int tiles_n) {
-  gemm_body<WAVES_M, WAVES_N, WMT, WNT, W4>(x, wt, st, zt, y, M, N, K, tiles_m, tiles_n);
+  gemm_body<WAVES_M, WAVES_N, WMT, WNT, W4, SWIGLU>(x, wt, st, zt, y, M, N, K, tiles_m, tiles_n);
 }
 
-template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4>
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false>
 int launch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M, int N,
                 int K, hipStream_t stream) {
   constexpr int BM = 32 * WMT * WAVES_M, BN = 32 * WNT * WAVES_N;
-  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;  // fused SwiGLU: N/2 divides by BN/2
   const size_t lds = (size_t)(3 * (BM / 8) + 2 * (BN / 8)) * 1024;
-  auto kern = gemm_kernel<WAVES_M, WAVES_N, WMT, WNT, W4>;
+  auto kern = gemm_kernel<WAVES_M, WAVES_N, WMT, WNT, W4, SWIGLU>;
   if (lds > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
         hipSuccess)
@@ -354,6 +378,17 @@ extern "C" int olmo355_w4_gemm(const uint16_t* x, const uint32_t* wt, const uint
   if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
   if ((K & 127) || (N & 15)) return O355_EUNSUPPORTED;
   return dispatch_gemm<true>(x, wt, st, zt, y, M, N, K, as_stream(stream));
+}
+
+extern "C" int olmo355_w4_gemm_swiglu(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
+                                      uint16_t* y, int M, int N, int K, void* stream) {
+  if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
+  if ((K & 127) || (N & 255) || (int64_t)(N >> 4) * (K >> 7) * 1024 >= (1ll << 32)) return O355_EUNSUPPORTED;
+  // rounds of one tile per CU, as in dispatch_gemm: 256 or 128 virtual columns (half up, half gate) per tile
+  const int64_t tm = (M + 255) / 256;
+  const double c256 = (double)((tm * (N / 256) + 255) / 256) * 95., c128 = (double)((tm * (N / 128) + 255) / 256) * 55.;
+  if (c128 < c256) return launch_gemm<4, 2, 2, 2, true, true>(x, wt, st, zt, y, M, N, K, as_stream(stream));
+  return launch_gemm<2, 4, 4, 2, true, true>(x, wt, st, zt, y, M, N, K, as_stream(stream));
 }
 
 extern "C" int olmo355_b16_gemm(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K,

@@ -1007,7 +1007,7 @@ int launch_small(Kern kern, const GemvPlan& p, const GemvArgs& a, hipStream_t st
       hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
     return O355_ELAUNCH;
   const int ntiles = a.N >> 4;
-  const unsigned blocks = p.epi ? (unsigned)(ntiles >> 1) : (unsigned)ntiles;
+  const unsigned blocks = p.epi ? (unsigned)(ntiles >> 1) : (unsigned)((ntiles + p.nt - 1) / p.nt);
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(p.waves * 64), lds, stream, a, w, st, zt);
   O355_CHECK_LAUNCH();
 }

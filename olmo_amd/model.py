@@ -339,7 +339,10 @@ class OLMo(nn.Module):
         att = self._linear(blk.attn_out, att)
         x = blk.attn_norm(att, residual=x) if c.norm_after else ops.add(x, att)
         h = x if c.norm_after else blk.ff_norm(x)
-        if B * T <= 16 and self.dtype == torch.bfloat16 and not self._act_order:  # few rows: SwiGLU rides in the projection's epilogue
+        rows = B * T
+        if (self.dtype == torch.bfloat16 and not self._act_order
+                and (rows <= 16 or (rows > ops.GEMV_MAX_M and isinstance(blk.ff_proj, QuantLinear)))):
+            # SwiGLU rides in the projection's epilogue (few rows: the GEMV's; many rows: the int4 GEMM's)
             h, _ = ops.linear_fused(h, self._tiled(blk.ff_proj), swiglu_out=True)
         else:
             h = ops.swiglu(self._linear(blk.ff_proj, h))

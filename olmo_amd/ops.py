@@ -201,6 +201,13 @@ def linear_fused(x: torch.Tensor, w, resid: Optional[torch.Tensor] = None, norm_
         if st != 2:
             check(name, st)
     x_new = rmsnorm(x, norm_w, eps, residual=resid) if resid is not None else x
+    if swiglu_out and isinstance(w, W4Tiled) and M > GEMV_MAX_M:  # many rows: SwiGLU in the GEMM's epilogue
+        y = torch.empty(*x.shape[:-1], n_out, dtype=torch.bfloat16, device=x.device)
+        st = lib().olmo355_w4_gemm_swiglu(_p(x_new), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream())
+        if st == 0:
+            return y, x_new
+        if st != 2:
+            check("olmo355_w4_gemm_swiglu", st)
     y = w4_linear(x_new, w) if isinstance(w, W4Tiled) else b16_linear(x_new, w)
     return (swiglu(y) if swiglu_out else y), x_new
 

@@ -663,3 +663,22 @@ def test_measuring_probes(dev):
     torch.cuda.synchronize()
     assert fl.value == 256 * 8 * 10 * 8 * 32768.0
     assert int(sink.abs().sum().item()) == 0
+
+
+@pytest.mark.parametrize("M,N,K", [(65, 256, 128), (300, 1024, 384), (2048, 2816, 512), (513, 22016, 256)])
+def test_w4_gemm_swiglu_epilogue(dev, M, N, K):
+    """int4 GEMM with SwiGLU in its epilogue == the separate GEMM then the SwiGLU kernel, bit for bit (the
+    epilogue rounds up and gate to bf16 first), and both match the oracle."""
+    say("w4_gemm_swiglu", M, N, K)
+    ops = _ops()
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=M + N + K)
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    fused, _ = ops.linear_fused(x.to(dev), t, swiglu_out=True)
+    sep = ops.swiglu(ops.w4_linear(x.to(dev), t))
+    assert fused.shape == (M, N // 2)
+    assert torch.equal(fused, sep)
+    lin = ow4.linear_fp32(x, ow4.dequantize(qw, qz, sc, 128)).to(torch.bfloat16).float()
+    up, gate = lin[:, : N // 2], lin[:, N // 2:]
+    ref = (torch.nn.functional.silu(gate).to(torch.bfloat16).float() * up)
+    assert (fused.float().cpu() - ref).abs().max().item() <= 2 ** -6 * ref.abs().max().item()
