@@ -203,6 +203,16 @@ int olmo355_add(const void* a, const void* b, void* out, int64_t n, int dtype, v
 /* Greedy step (olmo/beam_search.py:102-113 with beam 1): first index of the row maximum,
  * written as int64 to out[r], and the same value appended at ids_next when non-NULL. */
 int olmo355_argmax(const void* logits, int64_t* out, int rows, int n, int dtype, void* stream);
+/* One sampled step (olmo/beam_search.py:117-277 with beam size 1): z = logits / temperature; top_k > 0 keeps the
+ * k largest, then top_p < 1 keeps the most probable tokens up to and including the one at which the cumulative
+ * probability reaches top_p (of what top-k kept); the draw is from what remains, renormalised.  top_k = 0 and
+ * top_p = 1 is MultinomialSampler.  out[r] = token (int64), logprob[r] = log_softmax(logits)[token] at
+ * temperature 1, as the reference's samplers return.  The uniform number comes from (seed, counter, row), with the
+ * counter read from *counter_dev when that is non-NULL (e.g. the device-side position, so that a captured step
+ * draws a fresh number on every replay).  Tokens tied with a filter's threshold are all kept.  The reference's
+ * random stream (torch.multinomial) is not reproduced.  temperature > 0, 0 <= top_p <= 1. */
+int olmo355_sample(const void* logits, int rows, int n, float temperature, int top_k, float top_p, uint64_t seed,
+                   const int32_t* counter_dev, int counter, int64_t* out, float* logprob, int dtype, void* stream);
 /* *p += 1 for a device int32 (advances the position between captured decode steps). */
 int olmo355_incr_i32(int32_t* p, void* stream);
 

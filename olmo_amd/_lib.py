@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_uint64, c_void_p
 from typing import Optional
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -57,6 +57,7 @@ EXPORTS = {
     "olmo355_swiglu": (I, [P, P, I, I, I, P]),
     "olmo355_embedding": (I, [P, P, P, I, I, I, I, P]),
     "olmo355_gather_columns": (I, [P, P, P, I, I, P]),
+    "olmo355_sample": (I, [P, I, I, F, I, F, c_uint64, P, I, P, P, I, P]),
     "olmo355_probe_stream_read": (I, [P, L, P, P]),
     "olmo355_probe_mfma_bf16": (I, [I, P, P, P]),
     "olmo355_add": (I, [P, P, P, L, I, P]),

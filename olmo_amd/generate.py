@@ -19,14 +19,19 @@ import torch
 
 from . import ops
 
-__all__ = ["greedy_generate", "DecodeSession"]
+__all__ = ["greedy_generate", "DecodeSession"]  # greedy_generate also samples (its ``sampling`` argument)
 
 
 class DecodeSession:
-    """State of one batched greedy decode after its prefill."""
+    """State of one batched decode after its prefill: greedy, or sampled when ``sampling`` holds
+    ``temperature`` / ``top_k`` / ``top_p`` / ``seed`` (the draw then runs on the device inside the step, with
+    the device-side position as the random-number counter, so a captured step draws afresh on every replay)."""
 
-    def __init__(self, model, cache, first_ids: torch.Tensor, key_bias_full: Optional[torch.Tensor]):
+    def __init__(self, model, cache, first_ids: torch.Tensor, key_bias_full: Optional[torch.Tensor],
+                 sampling: Optional[dict] = None):
         self.model = model
+        self.sampling = sampling
+        self.logprob = torch.zeros(first_ids.shape[0], dtype=torch.float32, device=first_ids.device)
         self.cache = cache
         self.B = first_ids.shape[0]
         self.ids = first_ids.view(self.B, 1).contiguous()  # token to feed next; rewritten by every step
@@ -43,7 +48,11 @@ class DecodeSession:
         x = m.transformer["wte"](self.ids)
         logits, _ = m._forward_tokens(x, self.cache, self.B, 1, 0, self.key_bias, self.cache.length_dev, False)
         self.logits = logits
-        ops.argmax(logits.view(self.B, -1), out=self.ids.view(self.B))
+        if self.sampling is None:
+            ops.argmax(logits.view(self.B, -1), out=self.ids.view(self.B))
+        else:
+            ops.sample(logits.view(self.B, -1), counter_dev=self.cache.length_dev, out=self.ids.view(self.B),
+                       logprob=self.logprob, **self.sampling)
         ops.rope_advance(self.cache.length_dev, 1, *m._rope, self.cache.rope_now)
 
     def step(self) -> None:
@@ -65,11 +74,14 @@ class DecodeSession:
         self.graph = g
 
 
-def _prefill(model, input_ids, attention_mask):
+def _prefill(model, input_ids, attention_mask, sampling: Optional[dict] = None):
     out = model(input_ids, attention_mask=attention_mask, use_cache=True, last_logits_only=True)
     cache = out.attn_key_values[0].cache
     B = input_ids.shape[0]
-    first = ops.argmax(out.logits.view(B, -1))
+    if sampling is None:
+        first = ops.argmax(out.logits.view(B, -1))
+    else:  # counter: the position of the token being drawn, as in the decode steps
+        first, _ = ops.sample(out.logits.view(B, -1), counter=input_ids.shape[1], **sampling)
     key_bias_full = None
     if attention_mask is not None:
         am = attention_mask.to(model.device, torch.float32).view(B, -1)
@@ -81,18 +93,20 @@ def _prefill(model, input_ids, attention_mask):
 @torch.no_grad()
 def greedy_generate(model, input_ids: torch.Tensor, attention_mask: Optional[torch.Tensor], max_new_tokens: int,
                     use_graph: bool = True, eos_token_id: Optional[int] = None, pad_token_id: Optional[int] = None,
-                    return_scores: bool = False, return_logits: bool = False):
+                    return_scores: bool = False, return_logits: bool = False, sampling: Optional[dict] = None):
     """Returns ``tokens [B, max_new_tokens]`` (and, on request, the summed log-probabilities of the
     chosen tokens and / or the per-step logits).  Always runs ``max_new_tokens`` steps; with
-    ``eos_token_id`` the tokens after a sequence's first EOS are replaced by ``pad_token_id``."""
+    ``eos_token_id`` the tokens after a sequence's first EOS are replaced by ``pad_token_id``.
+    ``sampling`` (``temperature``, ``top_k``, ``top_p``, ``seed``) draws the tokens instead of taking the
+    arg-max; the same seed and prompt give the same tokens."""
     if max_new_tokens < 1:
         raise ValueError("max_new_tokens must be >= 1")
     input_ids = input_ids.to(model.device)
     B, T0 = input_ids.shape
     if T0 + max_new_tokens - 1 > model.max_cache_len:
         raise ValueError(f"prompt {T0} + {max_new_tokens} new tokens exceeds max_cache_len {model.max_cache_len}")
-    out, cache, first, key_bias_full = _prefill(model, input_ids, attention_mask)
-    sess = DecodeSession(model, cache, first, key_bias_full)
+    out, cache, first, key_bias_full = _prefill(model, input_ids, attention_mask, sampling)
+    sess = DecodeSession(model, cache, first, key_bias_full, sampling)
     tokens = torch.empty(B, max_new_tokens, dtype=torch.int64, device=model.device)
     tokens[:, 0] = sess.ids.view(B)
     all_logits = [out.logits[:, -1].clone()] if (return_scores or return_logits) else None

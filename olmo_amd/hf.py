@@ -146,12 +146,16 @@ class OLMoForCausalLM(nn.Module):
     def generate(self, input_ids: torch.LongTensor, attention_mask: Optional[torch.Tensor] = None,
                  max_new_tokens: int = 20, do_sample: bool = False, num_beams: int = 1,
                  eos_token_id: Optional[int] = None, pad_token_id: Optional[int] = None, use_graph: bool = True,
+                 temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0,
                  **unused) -> torch.Tensor:
-        """Greedy continuation: returns ``[B, prompt + max_new_tokens]`` token ids like HF ``generate``."""
-        if do_sample or num_beams != 1:
-            raise NotImplementedError("only greedy decoding (do_sample=False, num_beams=1) is implemented")
+        """Greedy or sampled continuation: returns ``[B, prompt + max_new_tokens]`` token ids like HF ``generate``.
+        With ``do_sample`` the logits go through temperature, top-k and top-p in HF's order and one token is
+        drawn per step on the device (``top_k=0`` / ``top_p=1.0`` switch a filter off); ``seed`` fixes the draw."""
+        if num_beams != 1:
+            raise NotImplementedError("beam search (num_beams > 1) is not implemented")
+        sampling = dict(temperature=temperature, top_k=top_k or 0, top_p=top_p, seed=seed) if do_sample else None
         new = greedy_generate(self.model, input_ids, attention_mask, max_new_tokens, use_graph=use_graph,
-                              eos_token_id=eos_token_id, pad_token_id=pad_token_id)
+                              eos_token_id=eos_token_id, pad_token_id=pad_token_id, sampling=sampling)
         return torch.cat((input_ids.to(new.device), new), dim=1)
 
     def get_input_embeddings(self):

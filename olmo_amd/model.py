@@ -533,14 +533,23 @@ class OLMo(nn.Module):
     @torch.no_grad()
     def generate(self, input_ids: torch.LongTensor, attention_mask: Optional[torch.Tensor] = None,
                  max_steps: int = 10, beam_size: int = 1, use_graph: bool = True,
-                 stop_at_eos: bool = False) -> OLMoGenerateOutput:
+                 stop_at_eos: bool = False, sampler=None, seed: int = 0) -> OLMoGenerateOutput:
+        """``OLMo.generate`` (``olmo/model.py:1603-1728``) with beam size 1: greedy by default
+        (``DeterministicSampler``), or one draw per step on the device with the ``MultinomialSampler`` /
+        ``TopKSampler`` / ``TopPSampler`` of ``olmo_amd.beam_search``.  ``scores`` is the summed log-probability
+        of the chosen tokens under the unfiltered distribution, as the reference's samplers report it."""
         if beam_size != 1:
-            raise NotImplementedError("only greedy search (beam_size=1) is implemented")
+            raise NotImplementedError("only beam_size=1 is implemented")
         from .generate import greedy_generate
 
+        sampling = None
+        if sampler is not None and not getattr(sampler, "greedy", False):
+            if hasattr(sampler, "check"):
+                sampler.check(self.config.logits_size)
+            sampling = dict(sampler.params(), seed=seed)
         toks, scores = greedy_generate(self, input_ids, attention_mask, max_steps, use_graph=use_graph,
                                        eos_token_id=self.config.eos_token_id if stop_at_eos else None,
-                                       return_scores=True)
+                                       return_scores=True, sampling=sampling)
         return OLMoGenerateOutput(token_ids=toks.unsqueeze(1), scores=scores.unsqueeze(1))
 
     @property

@@ -341,6 +341,33 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Te
     return out
 
 
+def sample(logits: torch.Tensor, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0,
+           counter: int = 0, counter_dev: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+           logprob: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One sampled token per row of ``logits``: temperature, then top-k, then top-p, then the draw.  Returns
+    ``(tokens int64, log-probabilities float32)``; the log-probability is the chosen token's under the unscaled,
+    unfiltered distribution.  The random number is a function of ``(seed, counter, row)``; ``counter_dev``
+    (a device int32) overrides ``counter``."""
+    _dev(logits, counter_dev, out, logprob)
+    if not temperature > 0:
+        raise ValueError("temperature must be positive")
+    if top_k < 0 or not 0.0 <= top_p <= 1.0:
+        raise ValueError("top_k must be >= 0 and top_p in [0, 1]")
+    n = logits.shape[-1]
+    rows = logits.numel() // n
+    if out is None:
+        out = torch.empty(logits.shape[:-1], dtype=torch.int64, device=logits.device)
+    if logprob is None:
+        logprob = torch.empty(logits.shape[:-1], dtype=torch.float32, device=logits.device)
+    if counter_dev is not None and counter_dev.dtype != torch.int32:
+        raise TypeError("counter_dev must be int32")
+    check("olmo355_sample",
+          lib().olmo355_sample(_p(logits), rows, n, float(temperature), int(top_k), float(top_p),
+                               int(seed) & 0xFFFFFFFFFFFFFFFF, _p(counter_dev), int(counter), _p(out), _p(logprob),
+                               _dt(logits), _stream()))
+    return out, logprob
+
+
 def incr_i32(p: torch.Tensor) -> None:
     _dev(p)
     if p.dtype != torch.int32:

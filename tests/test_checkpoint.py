@@ -87,3 +87,16 @@ def test_hf_olmo2_layout_split_orders_and_round_trip():
     # tied head: the embedding stands in (convert_olmo2_to_hf.py:160-162)
     sd.pop("transformer.ff_out.weight")
     assert torch.equal(olmo_to_hf_olmo2_state_dict(sd, cfg)["lm_head.weight"], sd["transformer.wte.weight"])
+
+
+def test_sampler_classes_mirror_reference_arguments():
+    from olmo_amd.beam_search import DeterministicSampler, MultinomialSampler, TopKSampler, TopPSampler
+
+    assert DeterministicSampler().greedy
+    assert MultinomialSampler(temperature=0.5).params() == {"temperature": 0.5, "top_k": 0, "top_p": 1.0}
+    assert TopKSampler().params() == {"temperature": 1.0, "top_k": 1, "top_p": 1.0}  # defaults of olmo/beam_search.py:163-172
+    assert TopPSampler().params() == {"temperature": 1.0, "top_k": 0, "top_p": 0.9}  # :217-231
+    with pytest.raises(ValueError, match="p must be a positive float no greater than 1.0"):
+        TopPSampler(p=1.5)
+    with pytest.raises(ValueError, match="k must be a postive integer"):
+        TopKSampler(k=0).check(100)

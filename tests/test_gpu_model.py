@@ -412,3 +412,33 @@ def test_unsharded_checkpoint_and_hf_layout(dev, tmp_path):
     m3 = OLMo(cfg, device=dev, dtype=torch.bfloat16)
     m3.load_reference_state_dict(hf_olmo2_to_olmo_state_dict(hf_sd, cfg))
     assert torch.equal(m3.post_init()(ids).logits, ref)
+
+
+def test_sampled_generation(dev):
+    """Sampling inside the decode step: the captured graph draws the same tokens as eager launches (the random
+    number is a function of seed and device-side position), a seed reproduces, and top_k=1 is greedy."""
+    say("sampled generation")
+    from olmo_amd.beam_search import TopKSampler, TopPSampler
+    from olmo_amd.hf import OLMoConfig, OLMoForCausalLM
+
+    cfg = small_cfg("olmo2")
+    model, _ = build_pair(cfg, torch.bfloat16, dev, seed=11)
+    hf = OLMoForCausalLM(OLMoConfig.from_model_config(cfg), model=model)
+    ids = torch.randint(0, cfg.vocab_size, (3, 9), generator=torch.Generator().manual_seed(1)).to(dev)
+    kw = dict(max_new_tokens=12, do_sample=True, temperature=1.5, top_k=50, top_p=0.95, seed=42)
+    a = hf.generate(ids, use_graph=True, **kw)
+    b = hf.generate(ids, use_graph=False, **kw)
+    assert a.shape == (3, 21) and torch.equal(a, b)
+    c = hf.generate(ids, use_graph=True, **dict(kw, seed=43))
+    assert not torch.equal(a, c)
+    # top_k = 1 keeps the maximum (and whatever ties with it in bf16): every drawn token has the row's largest logit
+    from olmo_amd.generate import greedy_generate
+
+    toks, lg = greedy_generate(model, ids, None, 12, return_logits=True,
+                               sampling=dict(temperature=1.0, top_k=1, top_p=1.0, seed=1))
+    assert torch.equal(lg.float().gather(-1, toks.unsqueeze(-1)).squeeze(-1), lg.float().max(-1).values)
+    out = model.generate(ids, max_steps=6, sampler=TopPSampler(p=0.9, temperature=1.2), seed=7)
+    assert out.token_ids.shape == (3, 1, 6) and out.scores.shape == (3, 1) and bool((out.scores < 0).all())
+    assert model.generate(ids, max_steps=3, sampler=TopKSampler(k=1)).token_ids.shape == (3, 1, 3)
+    with pytest.raises(ValueError):
+        model.generate(ids, max_steps=2, sampler=TopKSampler(k=0))

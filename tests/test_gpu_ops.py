@@ -682,3 +682,83 @@ def test_w4_gemm_swiglu_epilogue(dev, M, N, K):
     up, gate = lin[:, : N // 2], lin[:, N // 2:]
     ref = (torch.nn.functional.silu(gate).to(torch.bfloat16).float() * up)
     assert (fused.float().cpu() - ref).abs().max().item() <= 2 ** -6 * ref.abs().max().item()
+
+
+# ------------------------------------------------------------------------------------------------
+# sampling step
+# ------------------------------------------------------------------------------------------------
+def _reference_filter(logits_f32, temperature, top_k, top_p):
+    """The kept set and its renormalised probabilities by the reference's recipe (olmo/beam_search.py:149-277:
+    topk then softmax; sort descending, cumulative sum, exclusion mask shifted by one), in float64."""
+    z = logits_f32.double() / temperature
+    p = torch.softmax(z, -1)
+    keep = torch.ones_like(p, dtype=torch.bool)
+    if 0 < top_k < p.numel():
+        kth = torch.topk(p, top_k).values[-1]
+        keep &= p >= kth
+    if top_p < 1.0:
+        q = torch.where(keep, p, torch.zeros_like(p))
+        q = q / q.sum()
+        srt, idx = torch.sort(q, descending=True)
+        cum = torch.cumsum(srt, -1)
+        excl = cum >= top_p
+        excl[1:] = excl[:-1].clone()
+        excl[0] = False
+        thr = srt[~excl][-1]
+        keep &= q >= thr
+    q = torch.where(keep, p, torch.zeros_like(p))
+    return keep, q / q.sum()
+
+
+@pytest.mark.parametrize("temperature,top_k,top_p", [(1.0, 0, 1.0), (0.7, 5, 1.0), (1.3, 0, 0.8), (1.0, 12, 0.6),
+                                                      (2.0, 0, 0.0), (1.0, 1, 1.0)])
+def test_sample_distribution_small_vocab(dev, temperature, top_k, top_p):
+    """65536 draws from one 40-token distribution (one per row): every token lies in the reference's kept set,
+    the frequencies fit its renormalised probabilities (chi-square), and the returned log-probability is the
+    unfiltered log-softmax of the chosen token."""
+    say("sample small", temperature, top_k, top_p)
+    ops = _ops()
+    n, rows = 40, 65536
+    row = torch.randn(n, generator=torch.Generator().manual_seed(4)) * 2.0
+    logits = row.repeat(rows, 1).to(dev)
+    tok, lp = ops.sample(logits, temperature, top_k, top_p, seed=123, counter=7)
+    tok, lp = tok.cpu(), lp.cpu()
+    keep, q = _reference_filter(row, temperature, top_k, top_p)
+    assert bool(keep[tok].all())
+    assert torch.allclose(lp, torch.log_softmax(row, -1)[tok], atol=1e-5)
+    obs = torch.bincount(tok, minlength=n).double()
+    exp = q * rows
+    m = exp > 0
+    chi2 = float((((obs - exp) ** 2)[m] / exp[m]).sum())
+    dof = int(m.sum()) - 1
+    say("  chi2", chi2, "dof", dof)
+    assert chi2 <= dof + 6.0 * (2.0 * max(dof, 1)) ** 0.5 + 1e-9
+    if dof == 0:
+        assert int(obs.max()) == rows and int(tok[0]) == int(row.argmax())
+    # same (seed, counter) -> same draws; another counter -> other draws
+    tok2, _ = ops.sample(logits, temperature, top_k, top_p, seed=123, counter=7)
+    assert torch.equal(tok2.cpu(), tok)
+    if dof > 0:
+        cd = torch.tensor([8], dtype=torch.int32, device=dev)
+        tok3, _ = ops.sample(logits, temperature, top_k, top_p, seed=123, counter_dev=cd)
+        assert not torch.equal(tok3.cpu(), tok)
+
+
+@pytest.mark.parametrize("scale,top_k,top_p", [(3.0, 50, 0.9), (3.0, 0, 0.95), (0.3, 40, 1.0), (0.3, 0, 0.5), (6.0, 20000, 0.999)])
+def test_sample_large_vocab_bf16(dev, scale, top_k, top_p):
+    """Vocabulary-sized bf16 rows: peaked rows are decided among the tokens near the maximum, flat ones
+    (scale 0.3: every token within 2^-14 of the maximum) and very large k by the search over the whole row."""
+    say("sample large", scale, top_k, top_p)
+    ops = _ops()
+    n, rows = 100352, 64
+    logits = (torch.randn(rows, n, generator=torch.Generator().manual_seed(9)) * scale).to(torch.bfloat16)
+    tok, lp = ops.sample(logits.to(dev), 1.0, top_k, top_p, seed=5, counter=3)
+    tok, lp = tok.cpu(), lp.cpu()
+    for r in range(0, rows, 7):
+        row = logits[r].float()
+        keep, q = _reference_filter(row, 1.0, top_k, top_p)
+        p = torch.softmax(row.double(), -1)
+        # membership up to rounding at the boundary: the kernel sums fp32 exponentials in fixed point
+        assert p[tok[r]] >= p[keep].min() * (1 - 1e-4), (r, int(tok[r]))
+        assert abs(float(lp[r]) - float(torch.log_softmax(row, -1)[tok[r]])) <= 1e-3
+    assert len(set(tok.tolist())) > 1
