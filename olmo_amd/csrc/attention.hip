@@ -1140,7 +1140,7 @@ __global__ __launch_bounds__(1024) void attn_decode_onepass_kernel(
   }
 }
 
-int g_dbg_attn_mode = -1;  // experiment hook: 0 = chunked + combine, 1 = one workgroup per (batch, head)
+int g_dbg_attn_mode = -1;  // test hook (include/olmo355_debug.h); -1 = choose
 }  // namespace
 
 extern "C" void olmo355_debug_set_attn_mode(int mode) { g_dbg_attn_mode = mode; }

@@ -1,4 +1,7 @@
-// Small-M linear layers (decode): y[M,N] = x[M,K] . W[K,N], M <= 64, bandwidth-bound.
+// Small-M int4 / bf16 linear layers (decode): y[M,N] = x[M,K] . W[K,N], bandwidth-bound.  This file holds the
+// kernels that keep all rows of x in LDS (or registers) per workgroup -- the lean kernel of the decode step
+// (M <= 16, with the norm / SwiGLU fusions) and its older forms -- and the dispatcher of olmo355_w4_gemv*;
+// plain products with 5..64 rows mostly go to gemv_mid.hip (see w4_gemv_dispatch).
 //
 // The weight stream is read once with 128-bit loads per lane, already in MFMA operand order,
 // and multiplied on the matrix cores (v_mfma_f32_16x16x32_bf16) with the activations as the

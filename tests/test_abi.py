@@ -22,6 +22,19 @@ def test_header_symbols_are_exported_and_bound():
     assert b"unsupported" in h.olmo355_status_string(2)
 
 
+def test_debug_header_symbols_are_exported():
+    import ctypes
+
+    from olmo_amd import _lib
+
+    hdr = open(os.path.join(ROOT, "include", "olmo355_debug.h")).read()
+    declared = set(re.findall(r"\b(olmo355_debug_\w+)\s*\(", hdr))
+    assert len(declared) == 5
+    h = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert getattr(h, name) is not None
+
+
 def test_argument_checks_return_status_without_launching():
     from olmo_amd import _lib
 
