@@ -442,3 +442,70 @@ def test_sampled_generation(dev):
     assert model.generate(ids, max_steps=3, sampler=TopKSampler(k=1)).token_ids.shape == (3, 1, 3)
     with pytest.raises(ValueError):
         model.generate(ids, max_steps=2, sampler=TopKSampler(k=0))
+
+
+# ------------------------------------------------------------------------------------------------
+# the 7B / 13B int4 configurations at their real widths
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("preset", ["olmo2-7b", "olmo2-13b"])
+def test_full_width_int4_two_layers_against_oracle(dev, preset):
+    """BASELINE configs 3 and 4 at full width (d_model, heads, MLP width, vocabulary; int4-g128 block Linears),
+    cut to two layers so that the CPU oracle finishes in seconds: prefill logits and greedy steps."""
+    say("full width, two layers", preset)
+    import copy
+
+    from olmo_amd.generate import greedy_generate
+
+    cfg = copy.deepcopy(PRESETS[preset])
+    cfg.n_layers, cfg.max_sequence_length = 2, 512
+    model, oracle = build_pair(cfg, torch.bfloat16, dev, quantized=True, seed=5, max_cache_len=160)
+    ids = torch.randint(0, cfg.vocab_size, (2, 96), generator=torch.Generator().manual_seed(8))
+    ref, _ = oracle.forward(ids)
+    lg = model(ids.to(dev)).logits.cpu()
+    e = softmax_err(lg, ref)
+    say(f"  prefill softmax max-abs err {e:.3e}")
+    assert e <= 2e-2
+    toks, logits = greedy_generate(model, ids.to(dev), None, 8, use_graph=True, return_logits=True)
+    toks, logits = toks.cpu(), logits.cpu()
+    full, _ = oracle.forward(torch.cat((ids, toks), dim=1))
+    refd = full[:, ids.shape[1] - 1:-1]
+    e2 = softmax_err(logits, refd)
+    strict, loose = agreement(toks, refd)
+    say(f"  decode softmax max-abs err {e2:.3e}; agreement strict {strict:.3f} ulp {loose:.3f}")
+    assert e2 <= 2e-2 and loose == 1.0
+
+
+@pytest.mark.parametrize("preset", ["olmo2-7b", "olmo2-13b"])
+def test_full_depth_int4_invariants(dev, preset):
+    """Configs 3 and 4 at full depth and width, device only (the oracle would take hours): decoding with the
+    cache reproduces the rows of a full forward, a sequence's logits do not depend on its batch, and the
+    captured decode step draws the same tokens as eager launches."""
+    say("full depth invariants", preset)
+    from olmo_amd.generate import greedy_generate
+    from olmo_amd.synthetic import build_random_model
+
+    cfg = PRESETS[preset]
+    T, steps = 200, 6
+    model = build_random_model(cfg, torch.bfloat16, quantized=True, seed=1, device=dev, max_cache_len=T + 16,
+                               free_checkpoint_buffers=True)
+    ids = torch.randint(0, cfg.vocab_size, (2, T), generator=torch.Generator().manual_seed(3)).to(dev)
+    full = model(ids).logits  # [2, T, V]
+    # (1) cache: prefill T - steps tokens, then feed the remaining ones one at a time
+    out = model(ids[:, : T - steps], use_cache=True, last_logits_only=True)
+    assert softmax_err(out.logits[:, -1].cpu(), full[:, T - steps - 1].cpu()) <= 2e-2
+    past = out.attn_key_values
+    for i in range(steps):
+        o = model(ids[:, T - steps + i: T - steps + i + 1], past_key_values=past, use_cache=True)
+        past = o.attn_key_values
+        e = softmax_err(o.logits[:, -1].cpu(), full[:, T - steps + i].cpu())
+        assert e <= 2e-2, (i, e)
+        assert bool((o.logits[:, -1].argmax(-1) == full[:, T - steps + i].argmax(-1)).all()) or e <= 2e-3
+    # (2) batch invariance (different row counts take different kernels: tolerance, not equality)
+    single = model(ids[1:2]).logits
+    assert softmax_err(single[0].cpu(), full[1].cpu()) <= 2e-2
+    # (3) graph replay == eager
+    a = greedy_generate(model, ids[:, :64], None, 8, use_graph=True)
+    b = greedy_generate(model, ids[:, :64], None, 8, use_graph=False)
+    assert torch.equal(a, b)
+    del model, full, past
+    torch.cuda.empty_cache()
