@@ -50,6 +50,9 @@ def main() -> int:
     ap.add_argument("--no-bs8", action="store_true")
     ap.add_argument("--sweep", action="store_true",
                     help="isolated int4 linear sweep (M x shapes): prints a table on stderr and a JSON list on stdout")
+    ap.add_argument("--config4", action="store_true",
+                    help="BASELINE config 4 instead of the default line: OLMo-2 13B int4-g128, prefill 4 x 4096, "
+                         "decode batch 16 at KV context 4096; prints one JSON object on stdout")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: one plain copy of known size, then the four "
                          "int4 linears of a layer at one row; nothing is timed or printed")
@@ -75,6 +78,8 @@ def main() -> int:
         return traffic_probe(cfg, dev)
     if args.sweep:
         return linear_sweep(dev)
+    if args.config4:
+        return config4(dev, args.steps if args.steps != 128 else 32)
     ctx, K, W = args.context, args.steps, args.warmup
     cap = ctx + K + W + 8
     t0 = time.time()
@@ -300,6 +305,59 @@ def linear_sweep(dev) -> int:
             log(f"[sweep] M={m:5d} N={n:6d} K={k:5d}: {us:9.2f} us  {row['achieved']:8.1f} {row['unit']:8s} {row['frac']:6.1%}")
         del tiles
     print(json.dumps(rows))
+    return 0
+
+
+def config4(dev, steps: int) -> int:
+    """OLMo-2 13B int4-g128 (random weights): prefill 4 x 4096 (16384 rows), then greedy decode of 16 sequences
+    at KV context 4096, graph-replayed.  Algorithmic work: 415.8 TFLOP in the block GEMMs of the prefill;
+    per decode step 6.59 GB of int4 weights + 1.03 GB bf16 head + 53.7 GB of KV cache."""
+    import torch
+
+    from olmo_amd.config import PRESETS
+    from olmo_amd.generate import DecodeSession, _prefill
+    from olmo_amd.synthetic import build_random_model
+
+    cfg = PRESETS["olmo2-13b"]
+    ctx = 4096
+    model = build_random_model(cfg, torch.bfloat16, quantized=True, seed=0, device=dev, max_cache_len=ctx + steps + 16,
+                               free_checkpoint_buffers=True)
+    gen = torch.Generator().manual_seed(0)
+    ids4 = torch.randint(0, cfg.vocab_size, (4, ctx), generator=gen).to(dev)
+    for _ in range(2):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        _prefill(model, ids4, None)
+        torch.cuda.synchronize()
+        t_prefill = time.perf_counter() - t0
+    d, h, L = cfg.d_model, cfg.hidden_size, cfg.n_layers
+    gemm_flop = 2.0 * 4 * ctx * L * (d * 3 * d + d * d + d * h + (h // 2) * d)
+    log(f"[config4] prefill 4x{ctx}: {t_prefill * 1e3:.1f} ms = {4 * ctx / t_prefill:.0f} tok/s "
+        f"({gemm_flop / t_prefill / 1e12:.0f} TFLOP/s counting the block GEMMs only)")
+    ids16 = torch.randint(0, cfg.vocab_size, (16, ctx), generator=gen).to(dev)
+    out, cache, first, kb = _prefill(model, ids16, None)
+    sess = DecodeSession(model, cache, first, kb)
+    sess.step()
+    sess.step()
+    sess.capture()
+    for _ in range(4):
+        sess.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        sess.step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    kv_bytes = 2.0 * 16 * L * cfg.effective_n_kv_heads * cfg.head_dim * 2 * (ctx + 6 + steps / 2)
+    w_bytes = L * (d * 3 * d + d * d + d * h + (h // 2) * d) * W4_BYTES_PER_WEIGHT + 2.0 * d * cfg.logits_size
+    log(f"[config4] decode batch 16 at context {ctx}: {dt * 1e3:.2f} ms/step = {16 / dt:.0f} tok/s; "
+        f"{(kv_bytes + w_bytes) / dt / 1e9:.0f} GB/s of KV cache + weights")
+    print(json.dumps({"workload": "olmo2-13b int4-g128: prefill 4x4096, decode batch 16 at KV context 4096",
+                      "prefill_ms": t_prefill * 1e3, "prefill_tokens_per_s": 4 * ctx / t_prefill,
+                      "prefill_block_gemm_tflops": gemm_flop / t_prefill / 1e12,
+                      "decode_ms_per_step": dt * 1e3, "decode_tokens_per_s": 16 / dt,
+                      "decode_bytes_per_step": kv_bytes + w_bytes, "decode_gbs": (kv_bytes + w_bytes) / dt / 1e9,
+                      "steps": steps}), flush=True)
     return 0
 
 
