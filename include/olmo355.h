@@ -198,6 +198,8 @@ int olmo355_embedding(const int64_t* ids, const void* table, void* out, int rows
  * remap of the reference's exllama back-end (AGQ/autogptq_extension/exllama/cuda_func/column_remap.cu:9-63,
  * q4_matrix.cu:105-169); perm int32 [K], a permutation of 0..K-1 (not checked). */
 int olmo355_gather_columns(const uint16_t* x, const int32_t* perm, uint16_t* out, int M, int K, void* stream);
+/* clip_qkv (olmo/model.py:756-757): x := clamp(x, -c, c) in place over n elements, c > 0. */
+int olmo355_clamp(void* x, int64_t n, float c, int dtype, void* stream);
 /* out = a + b (residual add of the pre-norm block, olmo/model.py:794,821). */
 int olmo355_add(const void* a, const void* b, void* out, int64_t n, int dtype, void* stream);
 /* Greedy step (olmo/beam_search.py:102-113 with beam 1): first index of the row maximum,

@@ -57,6 +57,7 @@ EXPORTS = {
     "olmo355_swiglu": (I, [P, P, I, I, I, P]),
     "olmo355_embedding": (I, [P, P, P, I, I, I, I, P]),
     "olmo355_gather_columns": (I, [P, P, P, I, I, P]),
+    "olmo355_clamp": (I, [P, L, F, I, P]),
     "olmo355_sample": (I, [P, I, I, F, I, F, c_uint64, P, I, P, P, I, P]),
     "olmo355_probe_stream_read": (I, [P, L, P, P]),
     "olmo355_probe_mfma_bf16": (I, [I, P, P, P]),

@@ -127,10 +127,10 @@ class ModelConfig:
             bad(f"activation_type={self.activation_type!r} is not implemented; only 'swiglu'")
         if self.include_bias:
             bad("include_bias=true is not implemented")
-        if self.weight_tying:
-            bad("weight_tying=true is not implemented")
-        if self.embedding_layer_norm or self.scale_logits or self.clip_qkv is not None:
-            bad("embedding_layer_norm / scale_logits / clip_qkv are not implemented")
+        if self.embedding_layer_norm or self.scale_logits:
+            bad("embedding_layer_norm / scale_logits are not implemented")
+        if self.clip_qkv is not None and not self.clip_qkv > 0:
+            bad("clip_qkv must be positive")  # olmo/model.py:444-445
         if self.layer_norm_type == "rms":
             if not self.layer_norm_with_affine:
                 bad("rms layer norm without affine is not implemented")

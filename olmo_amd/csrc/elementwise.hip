@@ -539,6 +539,22 @@ extern "C" int olmo355_gather_columns(const uint16_t* x, const int32_t* perm, ui
   O355_CHECK_LAUNCH();
 }
 
+// x := min(max(x, -c), c) in place (clip_qkv)
+namespace {
+template <int DT>
+__global__ __launch_bounds__(256) void clamp_kernel(void* __restrict__ x, int64_t n, float c) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) Act<DT>::st(x, i, fminf(fmaxf(Act<DT>::ld(x, i), -c), c));
+}
+}  // namespace
+
+extern "C" int olmo355_clamp(void* x, int64_t n, float c, int dtype, void* stream) {
+  if (!x || n <= 0 || !(c > 0.f)) return O355_EINVAL;
+  DT_SWITCH(dtype, hipLaunchKernelGGL(clamp_kernel<DT>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream),
+                                      x, n, c));
+  O355_CHECK_LAUNCH();
+}
+
 extern "C" int olmo355_add(const void* a, const void* b, void* out, int64_t n, int dtype, void* stream) {
   if (!a || !b || !out || n <= 0) return O355_EINVAL;
   DT_SWITCH(dtype, hipLaunchKernelGGL(add_kernel<DT>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,

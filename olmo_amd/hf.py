@@ -161,5 +161,7 @@ class OLMoForCausalLM(nn.Module):
     def get_input_embeddings(self):
         return self.model.transformer["wte"]
 
-    def get_output_embeddings(self):
+    def get_output_embeddings(self):  # modeling_olmo.py:171-175: the embedding itself when the weights are tied
+        if self.config.weight_tying:
+            return self.model.transformer["wte"]
         return self.model.transformer["ff_out"]

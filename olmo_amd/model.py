@@ -190,8 +190,10 @@ class OLMo(nn.Module):
             blocks=nn.ModuleList([OLMoSequentialBlock(i, config, device, dtype, block_weight_device)
                                   for i in range(config.n_layers)]),
             ln_f=_build_norm(config, config.d_model, device, dtype),
-            ff_out=DenseLinear(config.d_model, V, device, dtype),
         ))
+        if not config.weight_tying:  # olmo/model.py:1129-1137
+            self.transformer.update({"ff_out": DenseLinear(config.d_model, V, device, dtype)})
+        self._tied_head: Optional[ops.B16Tiled] = None  # weight tying, bf16: the embedding re-tiled as the output matrix
         self._prepared = False
         self._act_order = False
         self._rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
@@ -228,6 +230,8 @@ class OLMo(nn.Module):
                     raise RuntimeError("a block Linear is still on the meta device: swap it or load weights first")
                 m.post_init()
         c = self.config
+        if c.weight_tying and self.dtype == torch.bfloat16:
+            self._tied_head = ops.b16_repack(self.transformer["wte"].weight.data.contiguous())
         n_pos = max(self.max_cache_len, c.max_sequence_length)
         self._rope = ops.rope_tables(c.head_dim, float(c.rope_theta), n_pos, self.device)
         # act-order int4 layers gather their activation columns in QuantLinear.forward: the fused decode forms
@@ -335,6 +339,8 @@ class OLMo(nn.Module):
         c = self.config
         h = x if c.norm_after else blk.attn_norm(x)
         qkv = self._linear(blk.att_proj, h)
+        if c.clip_qkv is not None:
+            ops.clamp_(qkv, c.clip_qkv)
         att = self._attention(blk, qkv, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max)
         att = self._linear(blk.attn_out, att)
         x = blk.attn_norm(att, residual=x) if c.norm_after else ops.add(x, att)
@@ -357,7 +363,7 @@ class OLMo(nn.Module):
     def _fused_decode_ok(self, M: int, collect_hidden: bool) -> bool:
         c = self.config
         return (M <= 16 and self.dtype == torch.bfloat16 and c.norm_after and c.layer_norm_type == "rms"
-                and not collect_hidden and not self._act_order and c.d_model * 2 * (M + 1) <= 64 * 1024 and c.d_model <= 5120)
+                and not collect_hidden and not self._act_order and c.clip_qkv is None and c.d_model * 2 * (M + 1) <= 64 * 1024 and c.d_model <= 5120)
 
     @staticmethod
     def _tiled(m: nn.Module):
@@ -523,8 +529,17 @@ class OLMo(nn.Module):
         x = self.transformer["ln_f"](x)
         if collect_hidden:
             hidden.append(x)
-        logits = self._linear(self.transformer["ff_out"], x)
+        logits = self._head(x)
         return logits, (tuple(hidden) if collect_hidden else None)
+
+    def _head(self, x: torch.Tensor) -> torch.Tensor:
+        """Output projection; with weight tying the embedding matrix (``olmo/model.py:1454-1457``)."""
+        if not self.config.weight_tying:
+            return self._linear(self.transformer["ff_out"], x)
+        wte = self.transformer["wte"].weight.data
+        if wte.dtype == torch.float32:
+            return ops.f32_linear(x, wte)
+        return ops.b16_linear(x, self._tied_head)
 
     # ------------------------------------------------------------------------------------------
     # greedy generation: olmo/model.py:1603-1728 with beam_size 1 and the deterministic sampler

@@ -294,6 +294,14 @@ def swiglu(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def clamp_(x: torch.Tensor, c: float) -> torch.Tensor:
+    """In-place ``x.clamp_(-c, c)`` (``clip_qkv``)."""
+    _dev(x)
+    if x.numel():
+        check("olmo355_clamp", lib().olmo355_clamp(_p(x), x.numel(), float(c), _dt(x), _stream()))
+    return x
+
+
 def gather_columns(x: torch.Tensor, perm: torch.Tensor) -> torch.Tensor:
     """``x[..., perm]`` for 16-bit activations (the column remap in front of an act-order int4 linear)."""
     _dev(x, perm)

@@ -195,6 +195,8 @@ class OracleModel:
         hd = c.d_model // c.n_heads
         h = x if c.norm_after else self._norm(pre + "attn_norm", x)
         qkv = self.linear(pre + "att_proj", h)
+        if c.clip_qkv is not None:  # olmo/model.py:756-757
+            qkv = qkv.clamp(min=-c.clip_qkv, max=c.clip_qkv)
         dkv = c.effective_n_kv_heads * hd
         q, k, v = qkv.split((c.d_model, dkv, dkv), dim=-1)
         att, cache = self._attention(i, q, k, v, bias, layer_past, use_cache)
@@ -252,7 +254,8 @@ class OracleModel:
         if last_logits_only:
             x = x[:, -1, :].unsqueeze(1)
         x = self._norm("transformer.ln_f", x)
-        logits = self.linear("transformer.ff_out", x)
+        # weight tying: the embedding is the output matrix (olmo/model.py:1454-1457)
+        logits = self.linear("transformer.wte" if c.weight_tying else "transformer.ff_out", x)
         return logits, kvs
 
 
@@ -300,5 +303,6 @@ def random_weights(cfg, dtype: torch.dtype, seed: int = 0, quantized: bool = Fal
                 w[pre + "k_norm.weight"] = normw(dkv)
     if cfg.layer_norm_type == "rms":
         w["transformer.ln_f.weight"] = normw(cfg.d_model)
-    w["transformer.ff_out.weight"] = normal(cfg.embedding_size or cfg.vocab_size, cfg.d_model)
+    if not cfg.weight_tying:  # olmo/model.py:1129-1137: no separate output matrix when tied
+        w["transformer.ff_out.weight"] = normal(cfg.embedding_size or cfg.vocab_size, cfg.d_model)
     return w

@@ -48,6 +48,10 @@ def small_cfg(kind: str) -> ModelConfig:
                            layer_norm_type="default", layer_norm_with_affine=False, layer_norm_eps=1e-5,
                            attention_layer_norm=False, norm_after=False, attention_dropout=0.0, residual_dropout=0.0,
                            embedding_dropout=0.0)
+    if kind == "ln-tied-clip":  # OLMo-1 style extras: output matrix tied to the embedding, clip_qkv (small, so it bites)
+        c = small_cfg("ln")
+        c.weight_tying, c.clip_qkv = True, 0.05
+        return c
     raise KeyError(kind)
 
 
@@ -96,6 +100,8 @@ def agreement(dev_tokens, oracle_logits):
     ("olmo2-gqa", torch.bfloat16, False),
     ("ln", torch.float32, False),
     ("ln", torch.bfloat16, False),
+    ("ln-tied-clip", torch.float32, False),
+    ("ln-tied-clip", torch.bfloat16, False),
 ])
 def test_forward_parity_and_invariants(dev, kind, dtype, quantized):
     say("forward parity", kind, dtype, quantized)

@@ -173,3 +173,47 @@ def test_forward_quantised_linear_equals_dense_on_dequantised_weights():
     a, _ = om.OracleModel(cfg, wq, torch.bfloat16).forward(ids)
     b, _ = om.OracleModel(cfg, wd, torch.bfloat16).forward(ids)
     assert torch.equal(a, b)
+
+
+def test_weight_tying_and_clip_qkv_reduce_to_known_cases():
+    """Tied output matrix == an untied model whose ff_out holds the embedding (olmo/model.py:1454-1457);
+    clip_qkv above every |qkv| changes nothing, a small one equals clamping the projection by hand (:756-757)."""
+    cfg = tiny_cfg(olmo2=False)
+    w = om.random_weights(cfg, torch.float32, seed=3)
+    ids = torch.randint(0, cfg.vocab_size, (2, 12), generator=torch.Generator().manual_seed(0))
+    base, _ = om.OracleModel(cfg, w, torch.float32).forward(ids)
+    import copy
+
+    tied = copy.deepcopy(cfg)
+    tied.weight_tying = True
+    wt = {k: v for k, v in w.items() if k != "transformer.ff_out.weight"}
+    w2 = dict(w)
+    w2["transformer.ff_out.weight"] = w["transformer.wte.weight"]
+    a, _ = om.OracleModel(tied, wt, torch.float32).forward(ids)
+    b, _ = om.OracleModel(cfg, w2, torch.float32).forward(ids)
+    assert torch.equal(a, b) and not torch.equal(a, base)
+    assert "transformer.ff_out.weight" not in om.random_weights(tied, torch.float32, seed=3)
+    big = copy.deepcopy(cfg)
+    big.clip_qkv = 1e6
+    c, _ = om.OracleModel(big, w, torch.float32).forward(ids)
+    assert torch.equal(c, base)
+    # one layer, by hand: clamp the att_proj output of layer 0 and nothing else
+    one = copy.deepcopy(cfg)
+    one.n_layers, one.clip_qkv = 1, 0.02
+    m = om.OracleModel(one, w, torch.float32)
+    x = w["transformer.wte.weight"][ids]
+    h = m._norm("transformer.blocks.0.attn_norm", x)
+    qkv = (h @ w["transformer.blocks.0.att_proj.weight"].t())
+    assert float(qkv.abs().max()) > 0.02  # the clip bites
+    got, _ = m.forward(ids)
+    noclip = copy.deepcopy(one)
+    noclip.clip_qkv = None
+    ref_noclip, _ = om.OracleModel(noclip, w, torch.float32).forward(ids)
+    assert not torch.allclose(got, ref_noclip)
+    w3 = dict(w)
+    # a model without clipping whose att_proj output is already inside the range behaves like the clipped one:
+    # scale the projection down so that nothing exceeds the clip, on both sides
+    w3["transformer.blocks.0.att_proj.weight"] = w["transformer.blocks.0.att_proj.weight"] * (0.019 / float(qkv.abs().max()))
+    g1, _ = om.OracleModel(one, w3, torch.float32).forward(ids)
+    g2, _ = om.OracleModel(noclip, w3, torch.float32).forward(ids)
+    assert torch.equal(g1, g2)
