@@ -1,4 +1,5 @@
-// int4 linear for 17..64 activation rows: y[M,N] = x[M,K] . W[K,N], bf16 in and out.
+// int4 linear for up to 64 activation rows (the dispatcher sends it every product above 16 rows and the wide
+// ones from 5): y[M,N] = x[M,K] . W[K,N], bf16 in and out.
 //
 // At these sizes the weight stream (N*K/2 bytes from HBM) and the activations (M*K*2 bytes, which
 // every workgroup needs in full) are of the same order, and the vector ALU (unpacking nibbles,
@@ -6,7 +7,7 @@
 // stages of GS groups of 128.  The stage's activations go from memory (L2) straight into LDS
 // (buffer loads with the LDS destination, no registers, no ALU work), one stage ahead of their
 // use.  A wave owns one pair of column tiles and one group of the stage, for all rows, so a weight
-// word is unpacked once per workgroup; its weight pieces go from memory to registers D stages
+// word is unpacked once per workgroup; its weight pieces go from memory to registers two stages
 // ahead.  Per group the matrix cores give T[n][m] = sum_k (128+q[k][n]) * x[m][k]
 // (v_mfma_f32_16x16x32_bf16, weights as the A operand, 0x4300|q == 128+q exactly) and
 // X[m] = sum_k x[m][k] (A = all ones), and the fp32 update
@@ -212,13 +213,13 @@ int launch_mid(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const 
   O355_CHECK_LAUNCH();
 }
 
-int g_dbg_np = 0;  // debug: 0 = choose, 1 / 2 = column-tile pairs per workgroup
+int g_dbg_np = 0;  // test hook (include/olmo355_debug.h): 0 = choose, 1 / 2 = column-tile pairs per workgroup
 
 }  // namespace
 
 extern "C" void olmo355_debug_set_mid_pairs(int np) { g_dbg_np = np; }
 
-// 17..64 rows; the caller has checked pointers and that K is a multiple of 128 and N of 16.
+// 1..64 rows; the caller has checked pointers and that K is a multiple of 128 and N of 16.
 int o355_w4_mid_dispatch(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
                          int M, int N, int K, void* stream) {
   if (M < 1 || M > 64 || (int64_t)M * K * 2 >= (1ll << 31) || (int64_t)(N >> 4) * (K >> 7) * 1024 >= (1ll << 31))
