@@ -167,6 +167,18 @@ int olmo355_attn_decode(const void* q, const void* kcache, const void* vcache, c
                         void* ws, int B, int H, int Hkv, int hd, int Lmax, int past_len,
                         const int32_t* past_len_dev, int n_keys_max, int bias_stride, int dtype, void* stream);
 
+/* olmo355_attn_decode for beam search: the B rows are beam b % beam of sequence b / beam.  Where the
+ * reference keeps the beams' caches consistent by gathering every cache tensor along the batch axis after each
+ * step (olmo/beam_search.py:1062-1078, called at :1000), here no cache row moves: the keys and values of
+ * positions < prompt_len are read from row (b / beam) * beam (the prefill of the sequence), and those of
+ * position prompt_len + i from row beam_src[b * src_stride + i] (int32, the row whose beam wrote the i-th
+ * generated token of b's history; entries past the current length must still be valid row numbers).  The
+ * search updates beam_src with its backpointers.  Needs prompt_len + src_stride >= n_keys_max. */
+int olmo355_attn_decode_beam(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out,
+                             void* ws, int B, int H, int Hkv, int hd, int Lmax, int past_len,
+                             const int32_t* past_len_dev, int n_keys_max, int bias_stride, const int32_t* beam_src,
+                             int src_stride, int prompt_len, int beam, int dtype, void* stream);
+
 /* olmo355_qknorm_rope_kvwrite (T == 1) and olmo355_attn_decode in one pass over the new token's
  * fused projection qkv [B, (H+2*Hkv)*hd]: bf16, hd 64 or 128; O355_EUNSUPPORTED otherwise (the caller
  * then issues the two separate calls).  Same workspace as olmo355_attn_decode.
@@ -205,6 +217,15 @@ int olmo355_add(const void* a, const void* b, void* out, int64_t n, int dtype, v
 /* Greedy step (olmo/beam_search.py:102-113 with beam 1): first index of the row maximum,
  * written as int64 to out[r], and the same value appended at ids_next when non-NULL. */
 int olmo355_argmax(const void* logits, int64_t* out, int rows, int n, int dtype, void* stream);
+/* The two selections of a beam-search step (olmo/beam_search.py:813-1045 with the DeterministicSampler,
+ * :102-113), one workgroup per row.
+ * olmo355_log_softmax: F.log_softmax of the step function (olmo/model.py:1705) over rows of n logits in the
+ *   activation dtype; fp32 log-probabilities out [rows, n].
+ * olmo355_topk: torch.topk(x, k, dim=-1) of fp32 rows: out_vals / out_idx [rows, k], descending; equal values
+ *   in ascending index order (torch leaves that order open).  k <= n, k <= 1024; NaNs are not supported. */
+int olmo355_log_softmax(const void* logits, float* out, int rows, int n, int dtype, void* stream);
+int olmo355_topk(const float* x, int rows, int n, int k, float* out_vals, int64_t* out_idx, void* stream);
+
 /* One sampled step (olmo/beam_search.py:117-277 with beam size 1): z = logits / temperature; top_k > 0 keeps the
  * k largest, then top_p < 1 keeps the most probable tokens up to and including the one at which the cumulative
  * probability reaches top_p (of what top-k kept); the draw is from what remains, renormalised.  top_k = 0 and

@@ -357,7 +357,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const void* __restrict
                                                           const float* __restrict__ key_bias, float* __restrict__ ws,
                                                           int H, int Hkv, int Lmax, int past_len,
                                                           const int32_t* __restrict__ past_dev, int nchunks_max,
-                                                          int bias_stride) {
+                                                          int bias_stride, const int32_t* __restrict__ beam_src,
+                                                          int src_stride, int prompt_len, int beam) {
   constexpr int LPK = HD / 8;                        // lanes per key (8 channels each)
   constexpr int KPI = 64 / LPK;                      // keys per wave iteration
   constexpr int ITERS = kDecodeKeysPerWave / KPI;    // iterations per wave
@@ -378,17 +379,33 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const void* __restrict
   // the launch bound, may be unwritten, and are discarded below. ----------------------------------
   u32x4 kreg[ITERS][VW], vreg[ITERS][VW];
   float bias[ITERS];
+  // Beam search (beam_src given): row b is beam b % beam of sequence b / beam.  Its prompt rows are those of
+  // the sequence's first beam; the row of its i-th generated token lives in cache row beam_src[b][i] (where
+  // the beam that produced that token wrote it), so choosing parents moves table entries, not cache rows
+  // (olmo/beam_search.py:1062-1078 gathers every cache tensor instead).
+  int64_t kb[ITERS];
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const int keyc = min(kbase + it * KPI + kslot, kmax);
-    const int64_t e = cbase + (int64_t)keyc * HD + sub * 8;
+    int64_t cb = cbase;
+    if (beam_src) {
+      int slot = (b / beam) * beam;
+      if (keyc >= prompt_len) slot = beam_src[(int64_t)b * src_stride + min(keyc - prompt_len, src_stride - 1)];
+      slot = min(max(slot, 0), (int)gridDim.z - 1);
+      cb = ((int64_t)slot * Hkv + hk) * Lmax * HD;
+    }
+    kb[it] = cb + (int64_t)keyc * HD + sub * 8;
+  }
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int64_t e = kb[it];
 #pragma unroll
     for (int v = 0; v < VW; ++v) kreg[it][v] = reinterpret_cast<const u32x4*>(kc)[e * VW / 8 + v];
   }
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const int keyc = min(kbase + it * KPI + kslot, kmax);
-    const int64_t e = cbase + (int64_t)keyc * HD + sub * 8;
+    const int64_t e = kb[it];
 #pragma unroll
     for (int v = 0; v < VW; ++v) vreg[it][v] = reinterpret_cast<const u32x4*>(vc)[e * VW / 8 + v];
     bias[it] = key_bias ? key_bias[(int64_t)b * bias_stride + keyc] : 0.f;
@@ -806,10 +823,10 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
 template <int DT, int HD>
 int launch_decode(const void* q, const void* kc, const void* vc, const float* key_bias, void* out, float* ws, int B,
                   int H, int Hkv, int Lmax, int past_len, const int32_t* past_dev, int n_keys_max, int bias_stride,
-                  hipStream_t stream) {
+                  const int32_t* beam_src, int src_stride, int prompt_len, int beam, hipStream_t stream) {
   const int nch = (n_keys_max + kDecodeChunk - 1) / kDecodeChunk;
   hipLaunchKernelGGL((attn_decode_kernel<DT, HD>), dim3(nch, H, B), dim3(256), 0, stream, q, kc, vc, key_bias, ws, H,
-                     Hkv, Lmax, past_len, past_dev, nch, bias_stride);
+                     Hkv, Lmax, past_len, past_dev, nch, bias_stride, beam_src, src_stride, prompt_len, beam);
   hipLaunchKernelGGL((attn_decode_combine_kernel<DT, HD>), dim3(H, B), dim3(HD), 0, stream, ws, out, H, past_len,
                      past_dev, nch);
   O355_CHECK_LAUNCH();
@@ -886,19 +903,22 @@ extern "C" int64_t olmo355_attn_decode_workspace_bytes(int B, int H, int hd, int
   return (int64_t)B * H * 4 + (int64_t)B * H * nch * (hd + 2) * 4;  // ticket counters, then the partials
 }
 
-extern "C" int olmo355_attn_decode(const void* q, const void* kcache, const void* vcache, const float* key_bias,
-                                   void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int past_len,
-                                   const int32_t* past_len_dev, int n_keys_max, int bias_stride, int dtype,
-                                   void* stream) {
+namespace {
+int attn_decode_any(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out, void* ws,
+                    int B, int H, int Hkv, int hd, int Lmax, int past_len, const int32_t* past_len_dev,
+                    int n_keys_max, int bias_stride, const int32_t* beam_src, int src_stride, int prompt_len, int beam,
+                    int dtype, void* stream) {
   if (!q || !kcache || !vcache || !out || !ws) return O355_EINVAL;
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || past_len < 0 || n_keys_max <= 0 || n_keys_max > Lmax)
     return O355_EINVAL;
   if (!past_len_dev && past_len + 1 > n_keys_max) return O355_EINVAL;
   if (key_bias && bias_stride < n_keys_max) return O355_EINVAL;
+  if (beam_src && (beam <= 0 || B % beam || prompt_len < 0 || src_stride <= 0 || prompt_len + src_stride < n_keys_max))
+    return O355_EINVAL;
   hipStream_t s = as_stream(stream);
 #define DECODE(DTv, HDv)                                                                                          \
   return launch_decode<DTv, HDv>(q, kcache, vcache, key_bias, out, (float*)ws + (int64_t)B * H, B, H, Hkv, Lmax, past_len, \
-                                 past_len_dev, n_keys_max, bias_stride, s)
+                                 past_len_dev, n_keys_max, bias_stride, beam_src, src_stride, prompt_len, beam, s)
   if (dtype == O355_BF16) {
     if (hd == 128) DECODE(O355_BF16, 128);
     if (hd == 64) DECODE(O355_BF16, 64);
@@ -910,6 +930,25 @@ extern "C" int olmo355_attn_decode(const void* q, const void* kcache, const void
   }
 #undef DECODE
   return O355_EUNSUPPORTED;
+}
+}  // namespace
+
+extern "C" int olmo355_attn_decode(const void* q, const void* kcache, const void* vcache, const float* key_bias,
+                                   void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int past_len,
+                                   const int32_t* past_len_dev, int n_keys_max, int bias_stride, int dtype,
+                                   void* stream) {
+  return attn_decode_any(q, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd, Lmax, past_len, past_len_dev, n_keys_max,
+                         bias_stride, nullptr, 0, 0, 1, dtype, stream);
+}
+
+extern "C" int olmo355_attn_decode_beam(const void* q, const void* kcache, const void* vcache, const float* key_bias,
+                                        void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int past_len,
+                                        const int32_t* past_len_dev, int n_keys_max, int bias_stride,
+                                        const int32_t* beam_src, int src_stride, int prompt_len, int beam, int dtype,
+                                        void* stream) {
+  if (!beam_src) return O355_EINVAL;
+  return attn_decode_any(q, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd, Lmax, past_len, past_len_dev, n_keys_max,
+                         bias_stride, beam_src, src_stride, prompt_len, beam, dtype, stream);
 }
 
 

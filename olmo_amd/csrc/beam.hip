@@ -1,0 +1,112 @@
+// Beam search on the device (olmo/beam_search.py:813-1045 with the deterministic sampler, :102-113): the two
+// selections of a step, each one workgroup per row.
+//   log_softmax: the step function's normalisation (olmo/model.py:1705), activation-dtype logits in, fp32
+//                log-probabilities out (the reference keeps them in the activation dtype; fp32 loses nothing).
+//   topk:        the k largest of a row in descending order, equal values in ascending index order
+//                (torch.topk leaves the order of ties open; with k = 1 this is torch.argmax's rule).
+//                Used for the per-node candidates (rows = batch * beam, n = vocabulary) and for the
+//                beam-level cut (rows = batch, n = beam * per_node_beam_size).
+// Selection is k rounds of a lexicographic arg-max over the row, which stays in L2 between rounds: beam widths
+// are single digits, and the rounds are exact and independent of scheduling.
+#include <math.h>
+
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 1024, kWaves = kThreads / 64;
+
+__device__ __forceinline__ float block_max_f(float v, float* lds) {
+  v = wave_max(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = lds[0];
+  for (int i = 1; i < kWaves; ++i) t = fmaxf(t, lds[i]);
+  return t;
+}
+
+__device__ __forceinline__ float block_sum_f(float v, float* lds) {  // fixed order: result independent of timing
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = lds[0];
+  for (int i = 1; i < kWaves; ++i) t += lds[i];
+  return t;
+}
+
+template <int DT>
+__global__ __launch_bounds__(kThreads) void log_softmax_kernel(const void* __restrict__ x, float* __restrict__ out,
+                                                               int n) {
+  __shared__ float red[kWaves];
+  const int64_t base = (int64_t)blockIdx.x * n;
+  float m = -INFINITY;
+  for (int i = threadIdx.x; i < n; i += kThreads) m = fmaxf(m, Act<DT>::ld(x, base + i));
+  m = block_max_f(m, red);
+  float s = 0.f;
+  for (int i = threadIdx.x; i < n; i += kThreads) s += expf(Act<DT>::ld(x, base + i) - m);
+  s = block_sum_f(s, red);
+  const float lse = logf(s);
+  for (int i = threadIdx.x; i < n; i += kThreads) out[base + i] = (Act<DT>::ld(x, base + i) - m) - lse;
+}
+
+// (a, ia) before (b, ib) in the output order: larger value first, then smaller index
+__device__ __forceinline__ bool before(float a, int ia, float b, int ib) { return a > b || (a == b && ia < ib); }
+
+__global__ __launch_bounds__(kThreads) void topk_kernel(const float* __restrict__ x, int n, int k,
+                                                        float* __restrict__ out_v, int64_t* __restrict__ out_i) {
+  __shared__ float sv[kWaves];
+  __shared__ int si[kWaves];
+  __shared__ float pick_v;
+  __shared__ int pick_i;
+  const int64_t base = (int64_t)blockIdx.x * n;
+  float prev_v = INFINITY;
+  int prev_i = -1;
+  for (int r = 0; r < k; ++r) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;  // nothing yet
+    for (int i = threadIdx.x; i < n; i += kThreads) {
+      const float v = x[base + i];
+      // still to be emitted: strictly after the previous pick in the output order
+      if (before(prev_v, prev_i, v, i) && before(v, i, best, bi)) best = v, bi = i;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (before(ov, oi, best, bi)) best = ov, bi = oi;
+    }
+    if ((threadIdx.x & 63) == 0) sv[threadIdx.x >> 6] = best, si[threadIdx.x >> 6] = bi;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      for (int w = 1; w < kWaves; ++w)
+        if (before(sv[w], si[w], best, bi)) best = sv[w], bi = si[w];
+      pick_v = best, pick_i = bi;
+      out_v[(int64_t)blockIdx.x * k + r] = best;
+      out_i[(int64_t)blockIdx.x * k + r] = bi == 0x7fffffff ? 0 : bi;  // only when the row holds NaNs
+    }
+    __syncthreads();
+    prev_v = pick_v, prev_i = pick_i;
+  }
+}
+
+}  // namespace
+
+extern "C" int olmo355_log_softmax(const void* logits, float* out, int rows, int n, int dtype, void* stream) {
+  if (!logits || !out || rows <= 0 || n <= 0) return O355_EINVAL;
+  hipStream_t s = as_stream(stream);
+  switch (dtype) {
+    case O355_F32: hipLaunchKernelGGL(log_softmax_kernel<O355_F32>, dim3(rows), dim3(kThreads), 0, s, logits, out, n); break;
+    case O355_BF16: hipLaunchKernelGGL(log_softmax_kernel<O355_BF16>, dim3(rows), dim3(kThreads), 0, s, logits, out, n); break;
+    default: return O355_EUNSUPPORTED;
+  }
+  O355_CHECK_LAUNCH();
+}
+
+extern "C" int olmo355_topk(const float* x, int rows, int n, int k, float* out_vals, int64_t* out_idx, void* stream) {
+  if (!x || !out_vals || !out_idx || rows <= 0 || n <= 0 || k <= 0 || k > n) return O355_EINVAL;
+  if (k > 1024) return O355_EUNSUPPORTED;  // k passes over the row: meant for beam widths
+  hipLaunchKernelGGL(topk_kernel, dim3(rows), dim3(kThreads), 0, as_stream(stream), x, n, k, out_vals, out_idx);
+  O355_CHECK_LAUNCH();
+}

@@ -3,9 +3,9 @@
 
 ``forward`` passes through to ``OLMo.forward`` and returns a ``CausalLMOutputWithPast``-shaped
 object; ``prepare_inputs_for_generation`` keeps only the last token when a cache is given
-(``modeling_olmo.py:150-160``).  ``generate`` is this package's own greedy loop (the HF
+(``modeling_olmo.py:150-160``).  ``generate`` is this package's own loop (the HF
 ``GenerationMixin`` is third-party code and is not reimplemented): prefill, then one captured
-decode step per token.  The module tree is ``self.model.transformer...`` so the names AutoGPTQ
+decode step per token, greedy or sampled; ``num_beams > 1`` runs OLMo's own beam search.  The module tree is ``self.model.transformer...`` so the names AutoGPTQ
 addresses (``model.transformer.blocks.{i}.att_proj`` ...,
 ``inference/compression/olmo_gptq_class.py:6``) resolve.
 """
@@ -148,11 +148,19 @@ class OLMoForCausalLM(nn.Module):
                  eos_token_id: Optional[int] = None, pad_token_id: Optional[int] = None, use_graph: bool = True,
                  temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0,
                  **unused) -> torch.Tensor:
-        """Greedy or sampled continuation: returns ``[B, prompt + max_new_tokens]`` token ids like HF ``generate``.
+        """Greedy, sampled or beam-searched continuation: returns ``[B, prompt + new tokens]`` token ids like HF
+        ``generate`` (``num_beams > 1``: the best beam, fewer than ``max_new_tokens`` columns when every beam ended early).
         With ``do_sample`` the logits go through temperature, top-k and top-p in HF's order and one token is
         drawn per step on the device (``top_k=0`` / ``top_p=1.0`` switch a filter off); ``seed`` fixes the draw."""
         if num_beams != 1:
-            raise NotImplementedError("beam search (num_beams > 1) is not implemented")
+            # OLMo's own search (olmo/beam_search.py via OLMo.generate), not transformers' BeamSearchScorer:
+            # summed log-probabilities, no length penalty; the best beam of each sequence, padded with the
+            # end token once it has ended
+            if do_sample:
+                raise NotImplementedError("sampling inside a beam search is not implemented")
+            out = self.model.generate(input_ids, attention_mask=attention_mask, max_steps=max_new_tokens,
+                                      beam_size=num_beams)
+            return torch.cat((input_ids.to(out.token_ids.device), out.token_ids[:, 0]), dim=1)
         sampling = dict(temperature=temperature, top_k=top_k or 0, top_p=top_p, seed=seed) if do_sample else None
         new = greedy_generate(self.model, input_ids, attention_mask, max_new_tokens, use_graph=use_graph,
                               eos_token_id=eos_token_id, pad_token_id=pad_token_id, sampling=sampling)

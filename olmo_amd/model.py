@@ -68,6 +68,28 @@ class KVCache:
         self.length_dev.fill_(L)
 
 
+class BeamKVCache(KVCache):
+    """Cache of a beam search: row ``b`` is beam ``b % beam`` of sequence ``b // beam``.  The prompt's keys and
+    values live once per sequence, in the row of its first beam; generated token ``i`` of a beam's history lives
+    in row ``beam_src[b, i]``, the row of the beam that fed it.  Choosing parents (``reorder_beams``) rewrites
+    that small table; no cache row is ever copied, where ``olmo/beam_search.py:1062-1078`` gathers all
+    ``2 * n_layers`` cache tensors after every step."""
+
+    def __init__(self, n_layers: int, B: int, beam: int, Hkv: int, prompt_len: int, steps: int, hd: int, dtype, device):
+        super().__init__(n_layers, B * beam, Hkv, prompt_len + steps, hd, dtype, device)
+        self.beam, self.prompt_len = beam, prompt_len
+        self._own = torch.arange(B * beam, dtype=torch.int32, device=device).unsqueeze(1)
+        self.beam_src = self._own.expand(B * beam, steps).contiguous()
+        self._seq0 = (torch.arange(B, device=device) * beam).unsqueeze(1)
+
+    def reorder_beams(self, backpointer: torch.Tensor) -> None:
+        rows = (backpointer.to(self._seq0.device) + self._seq0).reshape(-1)
+        src = self.beam_src.index_select(0, rows)
+        written = self.length - self.prompt_len  # generated tokens already in the cache
+        src[:, written:] = self._own            # whatever a beam feeds next goes to its own row
+        self.beam_src = src.contiguous()
+
+
 class LayerKV(tuple):
     """``(k, v)`` views of one layer's cache, remembering the cache they belong to."""
 
@@ -239,6 +261,7 @@ class OLMo(nn.Module):
         self._act_order = any(isinstance(m, QuantLinear) and m._perm is not None for m in self.modules())
         self._chain_ok = {}  # rows -> whether the chained decode block covers this model
         self._rope_now = None  # rotary rows of the current position during a captured decode step
+        self._beam = None  # the beam cache while a beam-search step runs
         self._prepared = True
         return self
 
@@ -321,7 +344,8 @@ class OLMo(nn.Module):
         qw = blk.q_norm.weight.data if blk.q_norm is not None else None
         kw = blk.k_norm.weight.data if blk.k_norm is not None else None
         decode = T == 1 and (graph_pos is not None or past_len > 0)
-        if decode:
+        beam = self._beam
+        if decode and beam is None:
             att = ops.attn_decode_fused(qkv, qw, kw, sin, cos, kc, vc, self._decode_ws(B, n_keys_max), B, H, Hkv, hd,
                                         past_len, n_keys_max, c.layer_norm_eps, key_bias=key_bias,
                                         past_len_dev=graph_pos, qk_ssq=qk_ssq,
@@ -331,6 +355,10 @@ class OLMo(nn.Module):
         q = ops.qknorm_rope_kvwrite(qkv, qw, kw, sin, cos, kc, vc, B, T, H, Hkv, hd, past_len, c.layer_norm_eps,
                                     past_len_dev=graph_pos)
         if decode:
+            if beam is not None:
+                return ops.attn_decode(q, kc, vc, self._decode_ws(B, n_keys_max), B, H, Hkv, hd, past_len, n_keys_max,
+                                       key_bias=key_bias, past_len_dev=graph_pos, beam_src=beam.beam_src,
+                                       prompt_len=beam.prompt_len, beam=beam.beam)
             return ops.attn_decode(q, kc, vc, self._decode_ws(B, n_keys_max), B, H, Hkv, hd, past_len, n_keys_max,
                                    key_bias=key_bias, past_len_dev=graph_pos)
         return ops.attn_prefill(q, kc, vc, B, T, H, Hkv, hd, past_len, key_bias=key_bias)
@@ -506,7 +534,10 @@ class OLMo(nn.Module):
         n_keys_max = cache.capacity if graph_pos is not None else past_len + T
         self._rope_now = cache.rope_now if (cache is not None and graph_pos is not None) else None
         hidden: List[torch.Tensor] = []
-        fused = T == 1 and cache is not None and self._fused_decode_ok(B, collect_hidden)
+        self._beam = cache if isinstance(cache, BeamKVCache) else None
+        if self._beam is not None and T != 1:
+            raise ValueError("a beam cache takes one token per row")
+        fused = T == 1 and cache is not None and self._beam is None and self._fused_decode_ok(B, collect_hidden)
         chain = fused and self._chain_decode_ok(B)
         pend = None
         for i, blk in enumerate(self.transformer["blocks"]):
@@ -547,14 +578,23 @@ class OLMo(nn.Module):
     # ------------------------------------------------------------------------------------------
     @torch.no_grad()
     def generate(self, input_ids: torch.LongTensor, attention_mask: Optional[torch.Tensor] = None,
-                 max_steps: int = 10, beam_size: int = 1, use_graph: bool = True,
-                 stop_at_eos: bool = False, sampler=None, seed: int = 0) -> OLMoGenerateOutput:
-        """``OLMo.generate`` (``olmo/model.py:1603-1728``) with beam size 1: greedy by default
+                 max_steps: int = 10, beam_size: int = 1, per_node_beam_size: Optional[int] = None,
+                 sampler=None, min_steps: Optional[int] = None, final_sequence_scorer=None,
+                 constraints: Optional[list] = None, use_graph: bool = True, stop_at_eos: bool = False,
+                 seed: int = 0) -> OLMoGenerateOutput:
+        """``OLMo.generate`` (``olmo/model.py:1603-1728``).
+
+        Beam size 1 without constraints, ``min_steps`` or a scorer is the captured greedy loop
         (``DeterministicSampler``), or one draw per step on the device with the ``MultinomialSampler`` /
-        ``TopKSampler`` / ``TopPSampler`` of ``olmo_amd.beam_search``.  ``scores`` is the summed log-probability
-        of the chosen tokens under the unfiltered distribution, as the reference's samplers report it."""
-        if beam_size != 1:
-            raise NotImplementedError("only beam_size=1 is implemented")
+        ``TopKSampler`` / ``TopPSampler`` of ``olmo_amd.beam_search``; it always runs ``max_steps`` steps
+        (``stop_at_eos`` pads after the first end token).  Anything else is ``olmo_amd.beam_search.BeamSearch``
+        over a :class:`BeamKVCache`: it stops when every beam has ended, as the reference does.  ``scores`` is the
+        summed log-probability of the chosen tokens under the unfiltered distribution (passed through
+        ``final_sequence_scorer`` in a beam search)."""
+        plain = beam_size == 1 and not constraints and not min_steps and final_sequence_scorer is None
+        if not plain:
+            return self._generate_beam(input_ids, attention_mask, max_steps, beam_size, per_node_beam_size, sampler,
+                                       min_steps, final_sequence_scorer, constraints)
         from .generate import greedy_generate
 
         sampling = None
@@ -566,6 +606,62 @@ class OLMo(nn.Module):
                                        eos_token_id=self.config.eos_token_id if stop_at_eos else None,
                                        return_scores=True, sampling=sampling)
         return OLMoGenerateOutput(token_ids=toks.unsqueeze(1), scores=scores.unsqueeze(1))
+
+    def _generate_beam(self, input_ids, attention_mask, max_steps, beam_size, per_node_beam_size, sampler, min_steps,
+                       final_sequence_scorer, constraints) -> OLMoGenerateOutput:
+        """The step function of ``olmo/model.py:1677-1714`` for ``BeamSearch``: prefill once with the batch, then
+        one token per beam and step against a :class:`BeamKVCache`; log-softmax of the last position on the
+        device."""
+        from .beam_search import BeamSearch
+
+        search = BeamSearch(self.config.eos_token_id, max_steps=max_steps, beam_size=beam_size,
+                            per_node_beam_size=per_node_beam_size, sampler=sampler, min_steps=min_steps,
+                            final_sequence_scorer=final_sequence_scorer, constraints=constraints)
+        input_ids = input_ids.to(self.device)
+        B, P = input_ids.shape
+        if attention_mask is not None:
+            assert attention_mask.shape == (B, P)
+        if P + max_steps - 1 > self.max_cache_len:
+            raise ValueError(f"prompt {P} + {max_steps} new tokens exceeds max_cache_len {self.max_cache_len}")
+        model, c = self, self.config
+
+        class _Beams:  # the search's state: BeamSearch calls expand_beams once, reorder_beams after every step
+            cache = None
+            key_bias = None
+
+            def expand_beams(st, batch: int, beam: int) -> None:
+                pre = st.cache
+                bc = BeamKVCache(c.n_layers, batch, beam, c.effective_n_kv_heads, P, max_steps, c.head_dim,
+                                 model.dtype, model.device)
+                for i in range(c.n_layers):  # the prompt, once per sequence
+                    bc.k[i].view(batch, beam, *bc.k[i].shape[1:])[:, 0, :, :P] = pre.k[i][:, :, :P]
+                    bc.v[i].view(batch, beam, *bc.v[i].shape[1:])[:, 0, :, :P] = pre.v[i][:, :, :P]
+                bc.set_length(P)
+                if attention_mask is not None:
+                    am = attention_mask.to(model.device, torch.float32).view(batch, P)
+                    kb = torch.zeros(batch, beam, bc.capacity, dtype=torch.float32, device=model.device)
+                    kb[:, :, :P] = ((1.0 - am) * torch.finfo(torch.float32).min).unsqueeze(1)
+                    st.key_bias = kb.view(batch * beam, bc.capacity)
+                st.cache = bc
+
+            def reorder_beams(st, backpointer: torch.Tensor) -> None:
+                st.cache.reorder_beams(backpointer)
+
+        def step(last_predictions: torch.Tensor, state: dict, timestep: int):
+            st = state["beams"]
+            if timestep == 0:
+                out = model(input_ids, attention_mask=attention_mask, use_cache=True, last_logits_only=True)
+                st.cache = out.attn_key_values[0].cache
+                logits = out.logits[:, -1]
+            else:
+                bc, R = st.cache, last_predictions.numel()
+                x = model.transformer["wte"](last_predictions.view(R, 1))
+                logits, _ = model._forward_tokens(x, bc, R, 1, 0, st.key_bias, bc.length_dev, True)
+                bc.set_length(bc.length + 1)
+            return ops.log_softmax(logits.reshape(logits.shape[0], -1)), state
+
+        tokens, scores = search.search(input_ids.new_zeros((B,)), {"beams": _Beams()}, step)
+        return OLMoGenerateOutput(token_ids=tokens, scores=scores)
 
     @property
     def num_params(self) -> int:

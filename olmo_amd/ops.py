@@ -349,6 +349,30 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Te
     return out
 
 
+def log_softmax(logits: torch.Tensor) -> torch.Tensor:
+    """``F.log_softmax(logits, dim=-1)`` with float32 results (beam search's step normalisation)."""
+    _dev(logits)
+    logits = logits.contiguous()
+    n = logits.shape[-1]
+    out = torch.empty(logits.shape, dtype=torch.float32, device=logits.device)
+    check("olmo355_log_softmax", lib().olmo355_log_softmax(_p(logits), _p(out), logits.numel() // n, n, _dt(logits), _stream()))
+    return out
+
+
+def topk(x: torch.Tensor, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``torch.topk(x, k, dim=-1)`` of float32 rows, sorted; equal values come in ascending index order."""
+    _dev(x)
+    if x.dtype != torch.float32:
+        raise TypeError("topk: float32 expected")
+    x = x.contiguous()
+    n = x.shape[-1]
+    rows = x.numel() // n
+    vals = torch.empty(*x.shape[:-1], k, dtype=torch.float32, device=x.device)
+    idx = torch.empty(*x.shape[:-1], k, dtype=torch.int64, device=x.device)
+    check("olmo355_topk", lib().olmo355_topk(_p(x), rows, n, int(k), _p(vals), _p(idx), _stream()))
+    return vals, idx
+
+
 def sample(logits: torch.Tensor, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0,
            counter: int = 0, counter_dev: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
            logprob: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -430,8 +454,11 @@ def attn_decode_workspace(B: int, H: int, hd: int, n_keys_max: int, device) -> t
 
 
 def attn_decode(q, kcache, vcache, ws, B: int, H: int, Hkv: int, hd: int, past_len: int, n_keys_max: int,
-                key_bias: Optional[torch.Tensor] = None, past_len_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
-    _dev(q, kcache, vcache, ws, key_bias, past_len_dev)
+                key_bias: Optional[torch.Tensor] = None, past_len_dev: Optional[torch.Tensor] = None,
+                beam_src: Optional[torch.Tensor] = None, prompt_len: int = 0, beam: int = 1) -> torch.Tensor:
+    """``beam_src`` (int32 ``[B, steps]``) switches to the beam-search form: prompt rows from the first beam of
+    each sequence, the row of generated token ``i`` from cache row ``beam_src[b, i]``."""
+    _dev(q, kcache, vcache, ws, key_bias, past_len_dev, beam_src)
     Lmax = kcache.shape[2]
     if q.numel() != B * H * hd or kcache.dtype != q.dtype:
         raise ValueError("q shape / cache dtype mismatch")
@@ -439,6 +466,15 @@ def attn_decode(q, kcache, vcache, ws, B: int, H: int, Hkv: int, hd: int, past_l
     if ws.numel() * ws.element_size() < need:
         raise ValueError("attention workspace too small")
     out = torch.empty(B, 1, H * hd, dtype=q.dtype, device=q.device)
+    if beam_src is not None:
+        if beam_src.dtype != torch.int32 or beam_src.dim() != 2 or beam_src.shape[0] != B or not beam_src.is_contiguous():
+            raise ValueError("beam_src: contiguous int32 [B, steps] expected")
+        check("olmo355_attn_decode_beam",
+              lib().olmo355_attn_decode_beam(_p(q), _p(kcache), _p(vcache), _p(key_bias), _p(out), _p(ws), B, H, Hkv, hd,
+                                             Lmax, past_len, _p(past_len_dev), n_keys_max,
+                                             key_bias.shape[1] if key_bias is not None else 0, _p(beam_src),
+                                             beam_src.shape[1], int(prompt_len), int(beam), _dt(q), _stream()))
+        return out
     check("olmo355_attn_decode",
           lib().olmo355_attn_decode(_p(q), _p(kcache), _p(vcache), _p(key_bias), _p(out), _p(ws), B, H, Hkv, hd, Lmax,
                                     past_len, _p(past_len_dev), n_keys_max,

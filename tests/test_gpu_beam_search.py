@@ -1,0 +1,264 @@
+"""Beam search on the device: the selection kernels against torch, the search against the known-answer cases of
+the reference's own tests (``tests/golden/beam_search_kat.json``), the attention kernel that reads beam histories
+through a row table against the plain kernel on caches gathered the reference's way, and ``OLMo.generate`` with
+beams against the oracle's search driven by the oracle's forward pass."""
+import json
+import os
+import warnings
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import beam_search as obs
+from tests.test_gpu_model import build_pair, say, small_cfg
+
+pytestmark = pytest.mark.gpu
+
+KAT = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "beam_search_kat.json")))
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from olmo_amd import _lib
+
+    _lib.lib()
+    return torch.device("cuda:0")
+
+
+@pytest.mark.parametrize("rows,n", [(1, 6), (3, 1000), (4, 100352), (2, 50281)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_log_softmax(dev, rows, n, dtype):
+    say("log_softmax", rows, n, dtype)
+    from olmo_amd import ops
+
+    x = (torch.randn(rows, n, generator=torch.Generator().manual_seed(n)) * 4).to(dtype)
+    got = ops.log_softmax(x.to(dev)).cpu()
+    want = torch.log_softmax(x.double(), dim=-1)
+    assert got.dtype == torch.float32
+    assert (got.double() - want).abs().max().item() < 2e-5  # fp32 arithmetic on values up to ~30
+    assert abs(torch.exp(got.double()).sum(-1) - 1).max().item() < 1e-4
+
+
+@pytest.mark.parametrize("rows,n,k", [(1, 6, 3), (5, 6, 6), (3, 1000, 7), (6, 100352, 4), (2, 4097, 64), (4, 36, 6)])
+def test_topk_values_order_and_ties(dev, rows, n, k):
+    """Values equal torch's; indices follow the stated tie rule (ascending index among equals), checked against a
+    stable descending sort.  The rows hold few distinct values, -inf and the float minimum, so ties are the rule."""
+    say("topk", rows, n, k)
+    from olmo_amd import ops
+
+    g = torch.Generator().manual_seed(rows * n + k)
+    x = torch.randint(-6, 6, (rows, n), generator=g).float() * 0.25
+    x[torch.rand(rows, n, generator=g) < 0.1] = -float("inf")
+    x[torch.rand(rows, n, generator=g) < 0.1] = torch.finfo(torch.float32).min
+    v, i = ops.topk(x.to(dev), k)
+    wv, wi = obs.topk_stable(x, k)
+    assert torch.equal(v.cpu(), wv) and torch.equal(i.cpu(), wi)
+    assert torch.equal(v.cpu(), torch.topk(x, k, dim=-1).values)
+    y = torch.randn(rows, n, generator=g)  # all distinct: indices equal torch's too
+    v, i = ops.topk(y.to(dev), k)
+    tv, ti = torch.topk(y, k, dim=-1)
+    assert torch.equal(v.cpu(), tv) and torch.equal(i.cpu(), ti)
+
+
+def chain_step(matrix):
+    def step(last, state, timestep):
+        return torch.log(matrix[last]), state
+    return step
+
+
+@pytest.mark.parametrize("case", KAT["cases"], ids=[c["name"] for c in KAT["cases"]])
+def test_search_reference_known_answers(dev, case):
+    say("beam search known answer", case["name"])
+    from olmo_amd.beam_search import (BeamSearch, LengthNormalizedSequenceLogProbabilityScorer,
+                                      RepeatedNGramBlockingConstraint)
+
+    m = torch.tensor(KAT["matrices"][case["matrix"]], device=dev)
+    scorer = None if "length_penalty" not in case else LengthNormalizedSequenceLogProbabilityScorer(case["length_penalty"])
+    cons = [RepeatedNGramBlockingConstraint(case["ngram_size"])] if case.get("ngram_size") else None
+    bs = BeamSearch(KAT["end_index"], max_steps=case["max_steps"], beam_size=case["beam_size"],
+                    per_node_beam_size=case.get("per_node_beam_size"), min_steps=case.get("min_steps"),
+                    final_sequence_scorer=scorer, constraints=cons)
+    start = torch.full((case["batch_size"],), KAT["start_token"], device=dev)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore", RuntimeWarning)
+        top, scores = bs.search(start, {}, chain_step(m))
+    assert list(top.shape[:2]) == [case["batch_size"], case["beam_size"]]
+    np.testing.assert_array_equal(top[0].cpu().numpy(), np.array(case["expected_top_k"]))
+    expected = np.log(np.array(case["expected_probs"]))
+    if "length_norm" in case:
+        expected = expected / np.array(case["length_norm"])
+    np.testing.assert_allclose(scores[0].cpu().numpy(), expected, rtol=KAT["rtol"])
+    # every batch element started the same way
+    assert all(torch.equal(top[b], top[0]) for b in range(top.shape[0]))
+
+
+def test_search_argument_checks_state_and_warnings(dev):
+    """``tests/beam_search_test.py:149-180`` (a tensor in the state is expanded per beam and follows the
+    backpointers), ``:289-297`` (per-node width above the number of classes), ``:299-318`` (warnings), and a
+    two-argument step function (``:146``)."""
+    say("beam search state / checks")
+    from olmo_amd.beam_search import BeamSearch, TopPSampler
+
+    m = torch.tensor(KAT["matrices"]["T"], device=dev)
+    state = {"foo": torch.tensor([[1, 0, 1], [2, 0, 1], [0, 0, 1], [1, 1, 1], [0, 0, 0]], device=dev)}
+    want = state["foo"].repeat_interleave(3, dim=0)
+    BeamSearch(5, max_steps=10, beam_size=3).search(torch.zeros(5, dtype=torch.long, device=dev), state,
+                                                   lambda last, st: (torch.log(m[last]), st))
+    assert torch.equal(state["foo"], want)
+    with pytest.raises(ValueError):
+        BeamSearch(5, beam_size=20).search(torch.zeros(5, dtype=torch.long, device=dev), {}, chain_step(m))
+    start = torch.tensor([4, 4], device=dev)
+    with pytest.warns(RuntimeWarning, match="Negligible log probabilities"):
+        BeamSearch(5, max_steps=10, beam_size=3).search(start, {}, chain_step(m))
+    with pytest.warns(RuntimeWarning, match="Empty sequences predicted"):
+        p, lp = BeamSearch(5, beam_size=1).search(start, {}, chain_step(m))
+    assert list(p.shape) == [2, 1, 1] and bool((p == 5).all()) and bool((lp == 0).all())
+    for bad in (dict(max_steps=0), dict(beam_size=0), dict(per_node_beam_size=0), dict(min_steps=-1),
+                dict(min_steps=11, max_steps=10)):
+        with pytest.raises(ValueError):
+            BeamSearch(5, **bad)
+    with pytest.raises(NotImplementedError):
+        BeamSearch(5, beam_size=2, sampler=TopPSampler())
+
+
+@pytest.mark.parametrize("dtype,hd", [(torch.bfloat16, 128), (torch.float32, 32), (torch.bfloat16, 64)])
+def test_attn_decode_beam_equals_gathered_caches(dev, dtype, hd):
+    """The row table must give what the reference's per-step cache gather gives: the plain kernel on caches
+    materialised row by row from (prompt of the first beam, generated rows by table) -- bit for bit."""
+    say("attn_decode_beam", dtype, hd)
+    from olmo_amd import ops
+
+    g = torch.Generator().manual_seed(hd)
+    B, beam, H, Hkv, P, S = 2, 3, 4, 2, 150, 40
+    R, cap, t = B * beam, P + S, 23  # t generated tokens in the cache, the newest at position P + t - 1
+    kc = torch.randn(R, Hkv, cap, hd, generator=g).to(dtype).to(dev)
+    vc = torch.randn(R, Hkv, cap, hd, generator=g).to(dtype).to(dev)
+    q = torch.randn(R, H * hd, generator=g).to(dtype).to(dev)
+    src = torch.empty(R, S, dtype=torch.int32)
+    for b in range(R):  # any row of the same sequence may hold a step; entries past t stay valid rows
+        lo = (b // beam) * beam
+        src[b] = torch.randint(lo, lo + beam, (S,), generator=g)
+    src = src.to(dev)
+    L = P + t
+    ws = ops.attn_decode_workspace(R, H, hd, cap, dev)
+    bias = torch.zeros(R, cap, device=dev)
+    bias[1, 3:9] = torch.finfo(torch.float32).min
+    got = ops.attn_decode(q, kc, vc, ws, R, H, Hkv, hd, L - 1, cap, key_bias=bias, beam_src=src, prompt_len=P, beam=beam)
+    gk, gv = torch.empty_like(kc), torch.empty_like(vc)
+    for b in range(R):
+        first = (b // beam) * beam
+        gk[b, :, :P], gv[b, :, :P] = kc[first, :, :P], vc[first, :, :P]
+        for i in range(S):
+            gk[b, :, P + i], gv[b, :, P + i] = kc[src[b, i], :, P + i], vc[src[b, i], :, P + i]
+    want = ops.attn_decode(q, gk, gv, ws, R, H, Hkv, hd, L - 1, cap, key_bias=bias)
+    assert torch.equal(got, want)
+    pos = torch.tensor([L - 1], dtype=torch.int32, device=dev)  # position from device memory
+    got2 = ops.attn_decode(q, kc, vc, ws, R, H, Hkv, hd, 0, cap, key_bias=bias, past_len_dev=pos, beam_src=src,
+                           prompt_len=P, beam=beam)
+    assert torch.equal(got2, want)
+
+
+def oracle_generate(oracle, ids, mask, eos, **kw):
+    """The reference's step function (``olmo/model.py:1677-1714``) over the oracle's forward pass; the state is the
+    cache in the reference's form, gathered along the batch axis by the oracle's search."""
+    n_layers = oracle.cfg.n_layers
+
+    def step(last, state, timestep):
+        if timestep == 0:
+            logits, kvs = oracle.forward(ids, attention_mask=mask, use_cache=True, last_logits_only=True)
+            st = {}
+        else:
+            past = [(state[f"k{i}"], state[f"v{i}"]) for i in range(n_layers)]
+            am = None
+            if mask is not None:
+                am = torch.cat([state["mask"], torch.ones(last.shape[0], 1, dtype=state["mask"].dtype)], dim=1)
+            logits, kvs = oracle.forward(last.unsqueeze(1), attention_mask=am, past_key_values=past, use_cache=True,
+                                         last_logits_only=True)
+            st = {}
+            if am is not None:
+                st["mask"] = am
+        if timestep == 0 and mask is not None:
+            st["mask"] = mask
+        for i, (k, v) in enumerate(kvs):
+            st[f"k{i}"], st[f"v{i}"] = k, v
+        return torch.log_softmax(logits[:, -1].float(), dim=-1), st
+
+    return obs.beam_search(step, torch.zeros(ids.shape[0], dtype=torch.long), {}, eos, **kw)
+
+
+@pytest.mark.parametrize("kind,masked", [("ln", False), ("ln", True), ("ln-tied-clip", False)])
+def test_generate_with_beams_against_oracle_fp32(dev, kind, masked):
+    """fp32 model: same sequences as the oracle's search over the oracle's forward pass, scores within fp32
+    noise; with and without left padding, with n-gram blocking, ``min_steps`` and length normalisation."""
+    say("generate with beams vs oracle", kind, masked)
+    from olmo_amd.beam_search import LengthNormalizedSequenceLogProbabilityScorer, RepeatedNGramBlockingConstraint
+
+    cfg = small_cfg(kind)
+    cfg.eos_token_id = 7
+    model, oracle = build_pair(cfg, torch.float32, dev, seed=5)
+    g = torch.Generator().manual_seed(2)
+    ids = torch.randint(8, cfg.vocab_size, (3, 11), generator=g)
+    mask = None
+    if masked:
+        mask = torch.ones(3, 11)
+        mask[1, :4] = 0
+        mask[2, :1] = 0
+    for kw in (dict(beam_size=4, max_steps=9),
+               dict(beam_size=3, per_node_beam_size=2, max_steps=7, min_steps=3),
+               dict(beam_size=2, max_steps=8, ngram_size=2, length_penalty=0.7),
+               dict(beam_size=1, max_steps=5, min_steps=2)):
+        okw = dict(kw)
+        dkw = dict(kw)
+        if "ngram_size" in dkw:
+            dkw["constraints"] = [RepeatedNGramBlockingConstraint(dkw.pop("ngram_size"))]
+        if "length_penalty" in dkw:
+            dkw["final_sequence_scorer"] = LengthNormalizedSequenceLogProbabilityScorer(dkw.pop("length_penalty"))
+        out = model.generate(ids.to(dev), attention_mask=None if mask is None else mask.to(dev), **dkw)
+        want_t, want_s = oracle_generate(oracle, ids, mask, cfg.eos_token_id, **okw)
+        assert out.token_ids.shape == want_t.shape and out.scores.shape == want_s.shape
+        assert torch.equal(out.token_ids.cpu(), want_t), (kw, out.token_ids.cpu(), want_t)
+        assert (out.scores.cpu() - want_s).abs().max().item() < 2e-3, kw
+
+
+def test_generate_with_beams_bf16_consistency(dev):
+    """bf16 OLMo-2 wiring (QK-norm, GQA off / on).  Every returned sequence's score equals its teacher-forced
+    log-probability from a plain forward pass of the same model (so the row table handed each beam its own
+    history); scores are sorted; beam 1 through the search is the greedy loop up to near-ties in bf16 (the two
+    run different kernels: the search's step is not the fused decode block), so its score matches greedy's;
+    and the best of four beams scores at least that."""
+    say("generate with beams, bf16 consistency")
+    from olmo_amd import ops
+
+    for kind in ("olmo2", "olmo2-gqa"):
+        cfg = small_cfg(kind)
+        cfg.eos_token_id = 3
+        model, _ = build_pair(cfg, torch.bfloat16, dev, seed=9)
+        ids = torch.randint(4, cfg.vocab_size, (2, 140), generator=torch.Generator().manual_seed(4)).to(dev)
+
+        def teacher_forced(b, toks):
+            logits = model(torch.cat([ids[b], toks]).unsqueeze(0)).logits[0]
+            lp = ops.log_softmax(logits[ids.shape[1] - 1: -1].contiguous())
+            is_end = (toks == cfg.eos_token_id).long()
+            after_end = torch.cumsum(is_end, 0) - is_end > 0
+            return torch.where(after_end, torch.zeros_like(lp[:, 0]), lp.gather(1, toks.unsqueeze(1)).squeeze(1)).sum().item()
+
+        greedy = model.generate(ids, max_steps=6)
+        one = model._generate_beam(ids, None, 6, 1, None, None, None, None, None)
+        assert one.token_ids.shape[:2] == (2, 1)
+        assert torch.equal(one.token_ids[:, :, :2], greedy.token_ids[:, :, :2])
+        assert (one.scores - greedy.scores).abs().max().item() < 0.3
+        out = model.generate(ids, max_steps=6, beam_size=4)
+        B, K, T = out.token_ids.shape
+        assert (B, K) == (2, 4) and bool((out.scores[:, :-1] >= out.scores[:, 1:]).all())
+        assert bool((out.scores[:, 0] >= one.scores[:, 0] - 1e-3).all())
+        from olmo_amd.hf import OLMoConfig, OLMoForCausalLM
+
+        hf = OLMoForCausalLM(OLMoConfig.from_model_config(cfg), model=model)
+        assert torch.equal(hf.generate(ids, max_new_tokens=6, num_beams=4), torch.cat([ids, out.token_ids[:, 0]], dim=1))
+        for b in range(B):
+            assert abs(teacher_forced(b, one.token_ids[b, 0]) - one.scores[b, 0].item()) < 0.05 * T
+            for j in range(K):
+                tf = teacher_forced(b, out.token_ids[b, j])
+                assert abs(tf - out.scores[b, j].item()) < 0.05 * T, (kind, b, j, tf, out.scores[b, j].item())
