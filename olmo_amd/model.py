@@ -87,7 +87,7 @@ class BeamKVCache(KVCache):
         src = self.beam_src.index_select(0, rows)
         written = self.length - self.prompt_len  # generated tokens already in the cache
         src[:, written:] = self._own            # whatever a beam feeds next goes to its own row
-        self.beam_src = src.contiguous()
+        self.beam_src.copy_(src)                # in place: a captured step keeps reading the same table
 
 
 class LayerKV(tuple):
@@ -594,7 +594,7 @@ class OLMo(nn.Module):
         plain = beam_size == 1 and not constraints and not min_steps and final_sequence_scorer is None
         if not plain:
             return self._generate_beam(input_ids, attention_mask, max_steps, beam_size, per_node_beam_size, sampler,
-                                       min_steps, final_sequence_scorer, constraints)
+                                       min_steps, final_sequence_scorer, constraints, use_graph)
         from .generate import greedy_generate
 
         sampling = None
@@ -608,10 +608,11 @@ class OLMo(nn.Module):
         return OLMoGenerateOutput(token_ids=toks.unsqueeze(1), scores=scores.unsqueeze(1))
 
     def _generate_beam(self, input_ids, attention_mask, max_steps, beam_size, per_node_beam_size, sampler, min_steps,
-                       final_sequence_scorer, constraints) -> OLMoGenerateOutput:
+                       final_sequence_scorer, constraints, use_graph: bool = True) -> OLMoGenerateOutput:
         """The step function of ``olmo/model.py:1677-1714`` for ``BeamSearch``: prefill once with the batch, then
         one token per beam and step against a :class:`BeamKVCache`; log-softmax of the last position on the
-        device."""
+        device.  The model's part of a step (embedding to log-probabilities) is captured into a HIP graph after
+        two eager steps: tokens, position and the row table are read from fixed device buffers."""
         from .beam_search import BeamSearch
 
         search = BeamSearch(self.config.eos_token_id, max_steps=max_steps, beam_size=beam_size,
@@ -628,6 +629,10 @@ class OLMo(nn.Module):
         class _Beams:  # the search's state: BeamSearch calls expand_beams once, reorder_beams after every step
             cache = None
             key_bias = None
+            ids = None     # [rows, 1] tokens the step reads
+            graph = None
+            logp = None
+            eager_steps = 0
 
             def expand_beams(st, batch: int, beam: int) -> None:
                 pre = st.cache
@@ -655,9 +660,26 @@ class OLMo(nn.Module):
                 logits = out.logits[:, -1]
             else:
                 bc, R = st.cache, last_predictions.numel()
-                x = model.transformer["wte"](last_predictions.view(R, 1))
-                logits, _ = model._forward_tokens(x, bc, R, 1, 0, st.key_bias, bc.length_dev, True)
+                if st.ids is None:
+                    st.ids = torch.empty(R, 1, dtype=torch.int64, device=model.device)
+                st.ids.copy_(last_predictions.view(R, 1))
+
+                def run():
+                    x = model.transformer["wte"](st.ids)
+                    lg, _ = model._forward_tokens(x, bc, R, 1, 0, st.key_bias, bc.length_dev, True)
+                    return ops.log_softmax(lg.reshape(R, -1))
+
+                if st.graph is None and use_graph and st.eager_steps >= 2:
+                    st.graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(st.graph):
+                        st.logp = run()
+                if st.graph is not None:
+                    st.graph.replay()
+                else:
+                    st.logp = run()
+                    st.eager_steps += 1
                 bc.set_length(bc.length + 1)
+                return st.logp, state
             return ops.log_softmax(logits.reshape(logits.shape[0], -1)), state
 
         tokens, scores = search.search(input_ids.new_zeros((B,)), {"beams": _Beams()}, step)
