@@ -572,9 +572,11 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
 
   // ---- 1. this head's q / new-k pieces, norm weights, rotary rows, sums of squares; then the cache rows
   // of this wave.  Cache rows come through a buffer resource with a scalar offset per request and the
-  // lane index as address (a wave's 64 pieces are contiguous); rows past the last one the launch may
-  // touch read as zero, rows at and past the new position are unwritten: the new one is replaced from
-  // LDS, later ones are discarded.
+  // lane index as address (a wave's 64 pieces are contiguous).  Requests stay inside the cache by
+  // construction, not by the resource's range check (what it does with a scalar offset beyond the range is
+  // not relied on): one that would start past the last row the launch may touch is moved back onto the last
+  // KPI rows; such rows, like every row at or past the new position, are discarded below (the new one is
+  // replaced from LDS).
   // roles: threads [0,CPH) rotate q of head h; [32,32+CPH) the new key of head hk; [64,64+HD/8) copy v
   const bool role_q = tid < CPH, role_k = tid >= 32 && tid < 32 + CPH, role_v = tid >= 64 && tid < 64 + HD / 8;
   const int c = role_q ? tid : tid - 32, j = c * 8;
@@ -616,6 +618,9 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
       }
     }
   }
+  // first row of the last request that fits; 0 for a cache shorter than one request, whose lanes past the end
+  // the range check then sees (the scalar offset is 0)
+  const int rowcap = max(kmax + 1 - KPI, 0);
   const __amdgpu_buffer_rsrc_t rk = make_rsrc(kc + cbase, (int64_t)(kmax + 1) * HD * 2);
   const __amdgpu_buffer_rsrc_t rv = make_rsrc(vc + cbase, (int64_t)(kmax + 1) * HD * 2);
   u32x4 kreg[ITERS], vreg[ITERS];
@@ -623,10 +628,10 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   // cache rows are read once per step: non-temporal (aux bit 1), 0.5 us less per launch at context 2048
 #pragma unroll
   for (int it = 0; it < ITERS; ++it)
-    kreg[it] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rk, lane * 16, (kbase + it * KPI) * HD * 2, 2));
+    kreg[it] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rk, lane * 16, min(kbase + it * KPI, rowcap) * HD * 2, 2));
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
-    vreg[it] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rv, lane * 16, (kbase + it * KPI) * HD * 2, 2));
+    vreg[it] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rv, lane * 16, min(kbase + it * KPI, rowcap) * HD * 2, 2));
     bias[it] = key_bias ? key_bias[(int64_t)b * bias_stride + min(kbase + it * KPI + kslot, kmax)] : 0.f;
   }
 

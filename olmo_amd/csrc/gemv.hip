@@ -529,10 +529,11 @@ struct SmallNorm {
     const int voff = (threadIdx.x & 63) * 16;
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-      const int first = (wave + i * WAVES) * 64;  // first piece of this wave in pass i
+      const int past = (wave + i * WAVES) * 64;  // first piece of this wave in pass i
+      const int first = min(past, total - 64);   // past the end: re-read the last pieces (nvec is a multiple of 64), unused
       const int m = (first >= nvec) + (first >= 2 * nvec) + (first >= 3 * nvec);
-      row[i] = first < total ? m : -1;
-      av[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, voff, first * 16, 0));  // past the end: zeros
+      row[i] = past < total ? m : -1;
+      av[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, voff, first * 16, 0));
       rv[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, voff, first * 16, 0));
       wv[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rn, voff, (first - m * nvec) * 16, 0));
     }
