@@ -325,10 +325,12 @@ class OLMo(nn.Module):
         return self._scratch_kv[key]
 
     def _decode_ws(self, B: int, n_keys_max: int) -> torch.Tensor:
-        key = (B, n_keys_max)
+        """Attention workspace for ``B`` rows and up to ``n_keys_max`` keys, sized in steps of 1024 keys so that
+        eager decoding (a new key count every step) reuses one buffer instead of allocating one per length."""
+        key = (B, -(-n_keys_max // 1024) * 1024)
         if key not in self._attn_ws:
             c = self.config
-            self._attn_ws[key] = ops.attn_decode_workspace(B, c.n_heads, c.head_dim, n_keys_max, self.device)
+            self._attn_ws[key] = ops.attn_decode_workspace(B, c.n_heads, c.head_dim, key[1], self.device)
         return self._attn_ws[key]
 
     # ------------------------------------------------------------------------------------------

@@ -450,7 +450,7 @@ def attn_prefill(q, kcache, vcache, B: int, T: int, H: int, Hkv: int, hd: int, p
 
 def attn_decode_workspace(B: int, H: int, hd: int, n_keys_max: int, device) -> torch.Tensor:
     n = int(lib().olmo355_attn_decode_workspace_bytes(B, H, hd, n_keys_max))
-    return torch.zeros(n // 4, dtype=torch.float32, device=device)  # the ticket counters at its end start at zero
+    return torch.zeros(n // 4, dtype=torch.float32, device=device)  # the ticket counters at its start begin at zero
 
 
 def attn_decode(q, kcache, vcache, ws, B: int, H: int, Hkv: int, hd: int, past_len: int, n_keys_max: int,
