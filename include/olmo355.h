@@ -102,6 +102,19 @@ int olmo355_w4_gemv_chain(const uint16_t* x, const uint16_t* resid, const uint16
  * exllama's reconstruct + cublasHgemm (exllama/cuda_func/q4_matmul.cu:222-260). */
 int olmo355_w4_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
                     int M, int N, int K, void* stream);
+/* Split-K forms of olmo355_w4_gemm / olmo355_b16_gemm for launches with fewer output tiles than CUs (prompts of
+ * 65 to a few hundred tokens): `splits` workgroups per 128 x 64 tile, each over its own run of K, fp32 partial
+ * sums in `workspace` (splits * M * N floats), added in split order and rounded once by a second kernel.  Same
+ * product as the plain entry up to the order of the fp32 additions (QuantLinear.forward's matmul,
+ * qlinear_cuda_old.py:287-290; F.linear of the dense layers, olmo/model.py:746-823).
+ * olmo355_gemm_splitk_plan returns the number of splits worth using for a shape (1: call the plain entry).
+ * Needs K % 256 == 0, N % 64 == 0, 2 <= splits <= K / 256. */
+int olmo355_gemm_splitk_plan(int M, int N, int K);
+int olmo355_w4_gemm_splitk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
+                           int M, int N, int K, int splits, float* workspace, void* stream);
+int olmo355_b16_gemm_splitk(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, int splits,
+                            float* workspace, void* stream);
+
 /* The same product for an ff_proj weight ([up | gate] column halves) with SwiGLU (olmo/model.py:365-368,813-819)
  * in the epilogue: y [M, N/2] = silu(gate) * up, each factor rounded to bf16 first as the separate Linear and
  * activation would.  N a multiple of 256; O355_EUNSUPPORTED otherwise: olmo355_w4_gemm + olmo355_swiglu. */

@@ -16,6 +16,7 @@
 //
 // The int4 operand is W = bf16(scale * (q - zero)) (fp32 product, one rounding).
 #include "common.h"
+#include <algorithm>
 #include <type_traits>
 
 namespace {
@@ -56,10 +57,16 @@ __device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& 
 // SWIGLU (int4, WNT == 2): the weight holds [up | gate] column halves of N/2 each; a tile's first 32-column
 // block per wave comes from the up half and its second from the matching gate columns, so both land in
 // the same lanes and the epilogue writes silu(gate) * up, [M, N/2] (SwiGLU.forward, olmo/model.py:365-368).
-template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false>  // wave grid, 32x32 MFMA tiles per wave
+//
+// SPLIT: the launch has gridDim.y workgroups per tile, each over its own run of K (whole units of 256, dealt
+// evenly), writing fp32 partial tiles to part[split][M][N]; splitk_reduce_kernel adds them in split order and
+// rounds once.  For launches with fewer tiles than CUs: the K loop is a serial chain of stages of about half a
+// microsecond each, so a tile count of 64 leaves three quarters of the chip idle for K / 64 such stages.
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false, bool SPLIT = false>  // wave grid, 32x32 MFMA tiles per wave
 __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wt,
                                           const uint16_t* __restrict__ st, const uint8_t* __restrict__ zt,
-                                          uint16_t* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n) {
+                                          uint16_t* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n,
+                                          float* __restrict__ part = nullptr) {
   constexpr int NW = WAVES_M * WAVES_N, NT = 64 * NW;
   constexpr int BM = 32 * WMT * WAVES_M, BN = 32 * WNT * WAVES_N;
   constexpr int A_BLK = BM / 8;        // 1 KiB blocks per stage: activations, 8 rows x 128 bytes each
@@ -88,8 +95,15 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     const int ct = ntl >> 1, j = ct & 1, wn_ = ct >> 1;
     return (j ? (ntiles >> 1) : 0) + tile_n * (BN / 32) + wn_ * 2 + (ntl & 1);
   };
-  const int G = K >> 7, KS = K >> 5;
-  const int stages = K / BK;
+  const int G = K >> 7, KS = K >> 5;  // strides of the tiled weight: always of the whole K
+  int k0 = 0, Kn = K;                 // this workgroup's run of K
+  if constexpr (SPLIT) {
+    const int units = K >> 8, z = blockIdx.y, nz = gridDim.y;
+    const int u0 = units * z / nz, u1 = units * (z + 1) / nz;
+    k0 = u0 << 8, Kn = (u1 - u0) << 8;
+  }
+  const int Gn = Kn >> 7;             // groups of 128 rows in the run
+  const int stages = Kn / BK;
   const int row32 = lane & 31, kh = lane >> 5;
 
   // ---- activations: memory -> LDS directly ------------------------------------------------------
@@ -98,7 +112,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   // position chunk ^ ((r >> 1) & 7), which makes the MFMA operand reads (32 rows, one chunk) hit
   // every bank once; the swizzle is applied on the memory side because the LDS side of these loads
   // is lane-linear.
-  const __amdgpu_buffer_rsrc_t rx = make_rsrc(x + (int64_t)m0 * K, (int64_t)(M - m0) * K * 2);
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(x + (int64_t)m0 * K + k0, ((int64_t)(M - m0) * K - k0) * 2);
   int a_voff[A_PW];
 #pragma unroll
   for (int i = 0; i < A_PW; ++i) {
@@ -120,11 +134,12 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   for (int ks = 0; ks < KSTEPS; ++ks) a_rd[ks] = row32 * 8 + ((2 * ks + kh) ^ a_swz);
 
   // ---- weights ---------------------------------------------------------------------------------
+  const int g0 = k0 >> 7, ks0 = k0 >> 5;  // first group / 32-row step of the run
   const __amdgpu_buffer_rsrc_t rw =
-      W4 ? make_rsrc(wt + (int64_t)nt0 * G * 256, (int64_t)(ntiles - nt0) * G * 1024)
-         : make_rsrc(wt + (int64_t)nt0 * KS * 256, (int64_t)(ntiles - nt0) * KS * 1024);
-  const __amdgpu_buffer_rsrc_t rs_ = make_rsrc(W4 ? st + (int64_t)nt0 * G * 16 : x, W4 ? (int64_t)(ntiles - nt0) * G * 32 : 0);
-  const __amdgpu_buffer_rsrc_t rz_ = make_rsrc(W4 ? zt + (int64_t)nt0 * G * 8 : (const uint8_t*)x, W4 ? (int64_t)(ntiles - nt0) * G * 8 : 0);
+      W4 ? make_rsrc(wt + ((int64_t)nt0 * G + g0) * 256, ((int64_t)(ntiles - nt0) * G - g0) * 1024)
+         : make_rsrc(wt + ((int64_t)nt0 * KS + ks0) * 256, ((int64_t)(ntiles - nt0) * KS - ks0) * 1024);
+  const __amdgpu_buffer_rsrc_t rs_ = make_rsrc(W4 ? st + ((int64_t)nt0 * G + g0) * 16 : x, W4 ? ((int64_t)(ntiles - nt0) * G - g0) * 32 : 0);
+  const __amdgpu_buffer_rsrc_t rz_ = make_rsrc(W4 ? zt + ((int64_t)nt0 * G + g0) * 8 : (const uint8_t*)x, W4 ? ((int64_t)(ntiles - nt0) * G - g0) * 8 : 0);
   // int4: one 16-byte piece (4 tiled words = the lane's share of a 128-row group), scale and zero per
   // item, fetched a group ahead into registers and dequantised on the way into LDS, fragment-major:
   // piece of lane l (column l&15 of its 16-column tile, rows 8*(l>>4).. of 32-row step j) goes to
@@ -227,7 +242,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
       load_frags(ab, h, ks);
       // requests are spread over the stage: a burst of them stalls the wave at issue
       load_a(s2, ab2, ks);
-      if constexpr (W4 && h == 1) fetch_b(min((s >> 1) + 2, G - 1), p, ks);
+      if constexpr (W4 && h == 1) fetch_b(min((s >> 1) + 2, Gn - 1), p, ks);
       __builtin_amdgcn_sched_barrier(0);
       mfmas();
       if constexpr (W4) {
@@ -250,7 +265,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     fetch_b(0, 0);
 #pragma unroll
     for (int i = 0; i < 2 * B_ITEMS; ++i) stash_b_word(0, 0, i >> 1, i & 1);
-    fetch_b(min(1, G - 1), 1);
+    fetch_b(min(1, Gn - 1), 1);
   } else {
     load_b_dense(0, 0);
   }
@@ -304,9 +319,36 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + (wm * WMT + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (m < M) y[(int64_t)m * N + n] = f32_to_bf16_bits(acc[i][j][r]);
+        if constexpr (SPLIT) {
+          if (m < M) part[((int64_t)blockIdx.y * M + m) * N + n] = acc[i][j][r];
+        } else {
+          if (m < M) y[(int64_t)m * N + n] = f32_to_bf16_bits(acc[i][j][r]);
+        }
       }
     }
+}
+
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_splitk_kernel(const uint16_t* __restrict__ x,
+                                                                            const uint32_t* __restrict__ wt,
+                                                                            const uint16_t* __restrict__ st,
+                                                                            const uint8_t* __restrict__ zt,
+                                                                            float* __restrict__ part, int M, int N, int K,
+                                                                            int tiles_m, int tiles_n) {
+  gemm_body<WAVES_M, WAVES_N, WMT, WNT, W4, false, true>(x, wt, st, zt, nullptr, M, N, K, tiles_m, tiles_n, part);
+}
+
+// y = bf16(part[0] + part[1] + ... ) in that order, four outputs per thread
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const f32x4* __restrict__ part, u32x2* __restrict__ y,
+                                                            int64_t n4, int splits) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n4) return;
+  f32x4 a = part[i];
+  for (int z = 1; z < splits; ++z) {
+    const f32x4 b = part[z * n4 + i];
+    a[0] += b[0], a[1] += b[1], a[2] += b[2], a[3] += b[3];
+  }
+  y[i] = u32x2{pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3])};
 }
 
 template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false>
@@ -333,6 +375,36 @@ int launch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(64 * WAVES_M * WAVES_N), lds, stream, x, wt, st, zt,
                      y, M, N, K, tiles_m, tiles_n);
+  O355_CHECK_LAUNCH();
+}
+
+// Split-K plan for 128 x 64 tiles (two workgroups per CU), from measurements at N = 4096 .. 22016, K = 4096 and
+// 11008, M = 96 .. 512: as many splits as keep the launch within two workgroups per CU and leave each at least
+// 1024 of K (16 stages); with every CU already holding a tile a split pays only for long K (the two workgroups
+// of a CU share its LDS bandwidth); 1 = do not split.  K must divide into units of 256 and N into whole tiles.
+int splitk_plan(int M, int N, int K) {
+  if (M <= 64 || (K & 255) || (N & 63) || ((int64_t)M * N & 3)) return 1;
+  const int64_t tiles = (int64_t)((M + 127) / 128) * (N / 64);
+  if (tiles > 256 || (tiles > 192 && K < 8192)) return 1;
+  const int z = std::min(std::min((int)(512 / tiles), K / 1024), 16);
+  return z < 2 ? 1 : z;
+}
+
+template <bool W4>
+int launch_splitk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M, int N,
+                  int K, int splits, float* part, hipStream_t stream) {
+  constexpr int BM = 128, BN = 64;
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = N / BN;
+  const size_t lds = (size_t)(3 * (BM / 8) + 2 * (BN / 8)) * 1024;
+  auto kern = gemm_splitk_kernel<4, 2, 1, 1, W4>;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
+      hipSuccess)
+    return O355_ELAUNCH;
+  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits), dim3(512),
+                     lds, stream, x, wt, st, zt, part, M, N, K, tiles_m, tiles_n);
+  const int64_t n4 = (int64_t)M * N / 4;
+  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream,
+                     reinterpret_cast<const f32x4*>(part), reinterpret_cast<u32x2*>(y), n4, splits);
   O355_CHECK_LAUNCH();
 }
 
@@ -378,6 +450,23 @@ extern "C" int olmo355_w4_gemm(const uint16_t* x, const uint32_t* wt, const uint
   if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
   if ((K & 127) || (N & 15)) return O355_EUNSUPPORTED;
   return dispatch_gemm<true>(x, wt, st, zt, y, M, N, K, as_stream(stream));
+}
+
+extern "C" int olmo355_gemm_splitk_plan(int M, int N, int K) { return splitk_plan(M, N, K); }
+
+extern "C" int olmo355_w4_gemm_splitk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
+                                      uint16_t* y, int M, int N, int K, int splits, float* workspace, void* stream) {
+  if (!x || !wt || !st || !zt || !y || !workspace || M <= 0 || N <= 0 || K <= 0 || splits < 2) return O355_EINVAL;
+  if ((K & 255) || (N & 63) || ((int64_t)M * N & 3) || splits > (K >> 8)) return O355_EUNSUPPORTED;
+  return launch_splitk<true>(x, wt, st, zt, y, M, N, K, splits, workspace, as_stream(stream));
+}
+
+extern "C" int olmo355_b16_gemm_splitk(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K,
+                                       int splits, float* workspace, void* stream) {
+  if (!x || !wt || !y || !workspace || M <= 0 || N <= 0 || K <= 0 || splits < 2) return O355_EINVAL;
+  if ((K & 255) || (N & 63) || ((int64_t)M * N & 3) || splits > (K >> 8)) return O355_EUNSUPPORTED;
+  return launch_splitk<false>(x, reinterpret_cast<const uint32_t*>(wt), nullptr, nullptr, y, M, N, K, splits, workspace,
+                              as_stream(stream));
 }
 
 extern "C" int olmo355_w4_gemm_swiglu(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,

@@ -129,9 +129,23 @@ def w4_linear(x: torch.Tensor, w: W4Tiled) -> torch.Tensor:
         check("olmo355_w4_gemv",
               lib().olmo355_w4_gemv(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream()))
     else:
-        check("olmo355_w4_gemm",
-              lib().olmo355_w4_gemm(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream()))
+        splits = _splitk(M, w.N, w.K)
+        if splits > 1:  # fewer tiles than CUs: several workgroups per tile along K, fp32 partials, one more kernel
+            part = torch.empty(splits, M, w.N, dtype=torch.float32, device=x.device)
+            check("olmo355_w4_gemm_splitk",
+                  lib().olmo355_w4_gemm_splitk(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, splits, _p(part),
+                                               _stream()))
+        else:
+            check("olmo355_w4_gemm",
+                  lib().olmo355_w4_gemm(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream()))
     return y
+
+
+SPLITK = True  # tests switch it off to compare the two forms
+
+
+def _splitk(M: int, N: int, K: int) -> int:
+    return int(lib().olmo355_gemm_splitk_plan(M, N, K)) if SPLITK else 1
 
 
 # ---------------------------------------------------------------------------------------------
@@ -169,7 +183,13 @@ def b16_linear(x: torch.Tensor, w: B16Tiled) -> torch.Tensor:
     if M <= GEMV_MAX_M:
         check("olmo355_b16_gemv", lib().olmo355_b16_gemv(_p(x), _p(w.wt), _p(y), M, w.N, w.K, _stream()))
     else:
-        check("olmo355_b16_gemm", lib().olmo355_b16_gemm(_p(x), _p(w.wt), _p(y), M, w.N, w.K, _stream()))
+        splits = _splitk(M, w.N, w.K)
+        if splits > 1:
+            part = torch.empty(splits, M, w.N, dtype=torch.float32, device=x.device)
+            check("olmo355_b16_gemm_splitk",
+                  lib().olmo355_b16_gemm_splitk(_p(x), _p(w.wt), _p(y), M, w.N, w.K, splits, _p(part), _stream()))
+        else:
+            check("olmo355_b16_gemm", lib().olmo355_b16_gemm(_p(x), _p(w.wt), _p(y), M, w.N, w.K, _stream()))
     return y
 
 

@@ -231,6 +231,72 @@ def test_b16_gemm_every_tile_width(dev, width, M, N, K):
     assert torch.allclose(y.float().cpu(), ref, rtol=2 ** -8, atol=2 ** -8 * ref.abs().max().item())
 
 
+@pytest.mark.parametrize("splits", [2, 3, 5])
+@pytest.mark.parametrize("M,N,K", [(65, 64, 1536), (128, 4096, 2816), (300, 1024, 1280), (512, 256, 4096)])
+def test_gemm_splitk(dev, splits, M, N, K):
+    """Several workgroups per tile along K (int4 and dense): uneven runs (K / 256 = 6, 11, 5, 16 units over 2, 3, 5
+    splits), ragged M, runs as short as one unit; against the oracle product and against the plain entry (same
+    products, other order of the fp32 additions: equal up to one rounding of the bf16 result)."""
+    say("gemm_splitk", splits, M, N, K)
+    ops = _ops()
+    from olmo_amd import _lib
+    L = _lib.lib()
+    s_ = torch.cuda.current_stream().cuda_stream
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=M + N + K)
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(7)).to(torch.bfloat16)
+    ref = ow4.linear_fp32(x, ow4.dequantize(qw, qz, sc, 128))
+    t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    xd = x.to(dev)
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    y0 = torch.empty_like(y)
+    part = torch.empty(splits, M, N, dtype=torch.float32, device=dev)
+    assert L.olmo355_w4_gemm_splitk(xd.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y.data_ptr(), M, N, K,
+                                    splits, part.data_ptr(), s_) == 0
+    assert L.olmo355_w4_gemm(xd.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y0.data_ptr(), M, N, K, s_) == 0
+    torch.cuda.synchronize()
+    scale = ref.abs().max().item()
+    assert (y.float().cpu() - ref).abs().max().item() <= 2 ** -7 * scale
+    assert (y.float() - y0.float()).abs().max().item() <= 2 ** -7 * scale
+    assert (y == y0).float().mean().item() > 0.9
+    # the partial sums add up to the product in fp32
+    assert (part.sum(0).cpu() - ref).abs().max().item() <= 2e-5 * scale * (K / 128) ** 0.5 + 2 ** -9 * scale
+    # dense
+    g = torch.Generator().manual_seed(M + N + K)
+    w = (torch.randn(N, K, generator=g) * 0.02).to(torch.bfloat16)
+    refd = x.float() @ w.float().t()
+    td = ops.b16_repack(w.to(dev))
+    assert L.olmo355_b16_gemm_splitk(xd.data_ptr(), td.wt.data_ptr(), y.data_ptr(), M, N, K, splits, part.data_ptr(), s_) == 0
+    torch.cuda.synchronize()
+    assert torch.allclose(y.float().cpu(), refd, rtol=2 ** -8, atol=2 ** -8 * refd.abs().max().item())
+    assert (part.sum(0).cpu() - refd).abs().max().item() <= 1e-4 * refd.abs().max().item()
+
+
+def test_gemm_splitk_plan_and_routing(dev):
+    """The plan splits only when tiles are scarce, and ops.w4_linear follows it."""
+    say("gemm_splitk plan")
+    ops = _ops()
+    from olmo_amd import _lib
+    plan = _lib.lib().olmo355_gemm_splitk_plan
+    assert plan(64, 4096, 4096) == 1 and plan(2048, 4096, 4096) == 1 and plan(128, 4096, 4000) == 1
+    assert plan(128, 4096, 4096) == 4 and plan(512, 4096, 4096) == 1 and plan(128, 4096, 11008) == 8
+    assert plan(512, 4096, 11008) == 2 and plan(256, 4096, 11008) == 4
+    assert plan(128, 22016, 4096) == 1 and plan(128, 12288, 4096) == 2 and plan(300, 4096, 4096) == 2
+    qw, qz, sc = ow4.random_quantized(2048, 1024, 128, seed=3)
+    t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    x = torch.randn(130, 2048, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(dev)
+    assert plan(130, 1024, 2048) == 2
+    a = ops.w4_linear(x, t)
+    ops.SPLITK = False
+    try:
+        b = ops.w4_linear(x, t)
+    finally:
+        ops.SPLITK = True
+    ref = ow4.linear_fp32(x.cpu(), ow4.dequantize(qw, qz, sc, 128))
+    scale = ref.abs().max().item()
+    assert (a.float().cpu() - ref).abs().max().item() <= 2 ** -7 * scale
+    assert (b.float().cpu() - ref).abs().max().item() <= 2 ** -7 * scale
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 50304, 256), (2048, 768, 256), (77, 130, 1024)])
 def test_f32_linear(dev, M, N, K):
     ops = _ops()
