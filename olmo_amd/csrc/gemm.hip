@@ -381,31 +381,42 @@ int launch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const
 // Split-K plan for 128 x 64 tiles (two workgroups per CU), from measurements at N = 4096 .. 22016, K = 4096 and
 // 11008, M = 96 .. 512: as many splits as keep the launch within two workgroups per CU and leave each at least
 // 1024 of K (16 stages); with every CU already holding a tile a split pays only for long K (the two workgroups
-// of a CU share its LDS bandwidth); 1 = do not split.  K must divide into units of 256 and N into whole tiles.
+// of a CU share its LDS bandwidth); 1 = do not split (for M <= 64: call the small-M entry).  K must divide into units of 256 and N into whole tiles.
 int splitk_plan(int M, int N, int K) {
-  if (M <= 64 || (K & 255) || (N & 63) || ((int64_t)M * N & 3)) return 1;
+  if ((K & 255) || (N & 63) || ((int64_t)M * N & 3)) return 1;
+  // 33 .. 64 rows belong to the staged-activation kernel except for narrow outputs over a long K (ff_out), where
+  // 64 x 128 tiles split eight ways take 20 us against its 35 (N = 4096, K = 11008)
+  if (M <= 64) return (M > 32 && (N & 127) == 0 && N <= 4096 && K >= 8192) ? 8 : 1;
   const int64_t tiles = (int64_t)((M + 127) / 128) * (N / 64);
   if (tiles > 256 || (tiles > 192 && K < 8192)) return 1;
   const int z = std::min(std::min((int)(512 / tiles), K / 1024), 16);
   return z < 2 ? 1 : z;
 }
 
-template <bool W4>
-int launch_splitk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M, int N,
-                  int K, int splits, float* part, hipStream_t stream) {
-  constexpr int BM = 128, BN = 64;
+template <int WAVES_M, int WAVES_N, bool W4>
+int launch_splitk_shape(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M,
+                        int N, int K, int splits, float* part, hipStream_t stream) {
+  constexpr int BM = 32 * WAVES_M, BN = 32 * WAVES_N;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = N / BN;
   const size_t lds = (size_t)(3 * (BM / 8) + 2 * (BN / 8)) * 1024;
-  auto kern = gemm_splitk_kernel<4, 2, 1, 1, W4>;
+  auto kern = gemm_splitk_kernel<WAVES_M, WAVES_N, 1, 1, W4>;
   if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
       hipSuccess)
     return O355_ELAUNCH;
-  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits), dim3(512),
-                     lds, stream, x, wt, st, zt, part, M, N, K, tiles_m, tiles_n);
+  hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), (unsigned)splits), dim3(512), lds, stream, x, wt, st, zt,
+                     part, M, N, K, tiles_m, tiles_n);
   const int64_t n4 = (int64_t)M * N / 4;
   hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream,
                      reinterpret_cast<const f32x4*>(part), reinterpret_cast<u32x2*>(y), n4, splits);
   O355_CHECK_LAUNCH();
+}
+
+// up to 64 rows: 64 x 128 tiles (no matrix-core work on rows that do not exist); otherwise 128 x 64
+template <bool W4>
+int launch_splitk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M, int N,
+                  int K, int splits, float* part, hipStream_t stream) {
+  if (M <= 64 && (N & 127) == 0) return launch_splitk_shape<2, 4, W4>(x, wt, st, zt, y, M, N, K, splits, part, stream);
+  return launch_splitk_shape<4, 2, W4>(x, wt, st, zt, y, M, N, K, splits, part, stream);
 }
 
 int g_force_tile = 0;  // debug: 0 = choose, else 1000 * rows + columns of the tile (rows 0 = 256)

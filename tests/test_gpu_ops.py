@@ -232,7 +232,8 @@ def test_b16_gemm_every_tile_width(dev, width, M, N, K):
 
 
 @pytest.mark.parametrize("splits", [2, 3, 5])
-@pytest.mark.parametrize("M,N,K", [(65, 64, 1536), (128, 4096, 2816), (300, 1024, 1280), (512, 256, 4096)])
+@pytest.mark.parametrize("M,N,K", [(65, 64, 1536), (128, 4096, 2816), (300, 1024, 1280), (512, 256, 4096), (33, 384, 1280),
+                                   (64, 4096, 2816)])
 def test_gemm_splitk(dev, splits, M, N, K):
     """Several workgroups per tile along K (int4 and dense): uneven runs (K / 256 = 6, 11, 5, 16 units over 2, 3, 5
     splits), ragged M, runs as short as one unit; against the oracle product and against the plain entry (same
@@ -278,6 +279,7 @@ def test_gemm_splitk_plan_and_routing(dev):
     from olmo_amd import _lib
     plan = _lib.lib().olmo355_gemm_splitk_plan
     assert plan(64, 4096, 4096) == 1 and plan(2048, 4096, 4096) == 1 and plan(128, 4096, 4000) == 1
+    assert plan(64, 4096, 11008) == 8 and plan(33, 4096, 11008) == 8 and plan(32, 4096, 11008) == 1 and plan(64, 12288, 11008) == 1
     assert plan(128, 4096, 4096) == 4 and plan(512, 4096, 4096) == 1 and plan(128, 4096, 11008) == 8
     assert plan(512, 4096, 11008) == 2 and plan(256, 4096, 11008) == 4
     assert plan(128, 22016, 4096) == 1 and plan(128, 12288, 4096) == 2 and plan(300, 4096, 4096) == 2
