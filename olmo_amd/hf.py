@@ -169,7 +169,22 @@ class OLMoForCausalLM(nn.Module):
     def get_input_embeddings(self):
         return self.model.transformer["wte"]
 
-    def get_output_embeddings(self):  # modeling_olmo.py:171-175: the embedding itself when the weights are tied
+    def set_input_embeddings(self, value: nn.Module) -> None:  # modeling_olmo.py:175-176
+        self.model.transformer["wte"] = value
+        self.model._prepared = False  # tiled copies of the head are rebuilt on the next forward
+
+    def get_output_embeddings(self):  # modeling_olmo.py:178-182: the embedding itself when the weights are tied
         if self.config.weight_tying:
             return self.model.transformer["wte"]
         return self.model.transformer["ff_out"]
+
+    def set_output_embeddings(self, value: nn.Module) -> None:  # modeling_olmo.py:184-188
+        self.model.transformer["wte" if self.config.weight_tying else "ff_out"] = value
+        self.model._prepared = False
+
+    def tie_weights(self) -> None:
+        """A no-op as in the reference (modeling_olmo.py:190-202): with ``weight_tying`` the model has no ``ff_out``
+        and multiplies by the embedding matrix itself."""
+
+    def resize_token_embeddings(self, new_num_tokens: Optional[int] = None, pad_to_multiple_of: Optional[int] = None):
+        raise NotImplementedError("resizing the embeddings (modeling_olmo.py:204-246) belongs to fine-tuning set-up")
