@@ -238,6 +238,12 @@ int olmo355_argmax(const void* logits, int64_t* out, int rows, int n, int dtype,
  *   in ascending index order (torch leaves that order open).  k <= n, k <= 1024; NaNs are not supported. */
 int olmo355_log_softmax(const void* logits, float* out, int rows, int n, int dtype, void* stream);
 int olmo355_topk(const float* x, int rows, int n, int k, float* out_vals, int64_t* out_idx, void* stream);
+/* Sampling inside a beam search (torch.multinomial of the MultinomialSampler / TopKSampler / TopPSampler,
+ * olmo/beam_search.py:135-146, 171-203, 238-289): out = x * inv_temp + Gumbel(0, 1) noise from
+ * (seed, counter, element), entries <= -1.7e38 -> -inf.  olmo355_topk(out, k) is then k draws without replacement
+ * from softmax(x * inv_temp); the reference's random stream is not reproduced. */
+int olmo355_gumbel_perturb(const float* x, float* out, int rows, int n, float inv_temp, uint64_t seed,
+                           uint64_t counter, void* stream);
 
 /* One sampled step (olmo/beam_search.py:117-277 with beam size 1): z = logits / temperature; top_k > 0 keeps the
  * k largest, then top_p < 1 keeps the most probable tokens up to and including the one at which the cumulative

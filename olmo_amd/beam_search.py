@@ -3,9 +3,9 @@
 
 Beam size 1: the samplers are parameter holders for the device-side sampling step (``olmo355_sample``);
 ``OLMo.generate(..., sampler=TopPSampler(p=0.9))`` draws one token per step on the GPU inside the captured
-decode step.  Beam sizes above 1: ``BeamSearch`` below, with the ``DeterministicSampler``.  The
-``GumbelSampler`` (``olmo/beam_search.py:280-421``) and stochastic samplers inside a beam search are not
-implemented.
+decode step.  Beam sizes above 1: ``BeamSearch`` below; the samplers' ``sample_nodes`` draw per-node candidates
+on the device (Gumbel-perturbed log-weights + top-k).  The ``GumbelSampler`` (``olmo/beam_search.py:291-421``)
+is not implemented.
 """
 
 from __future__ import annotations
@@ -17,63 +17,142 @@ from typing import Callable, List, Optional
 
 import torch
 
-__all__ = ["Sampler", "DeterministicSampler", "MultinomialSampler", "TopKSampler", "TopPSampler",
+__all__ = ["Sampler", "DeterministicSampler", "MultinomialSampler", "TopKSampler", "TopPSampler", "GumbelSampler",
            "FinalSequenceScorer", "SequenceLogProbabilityScorer", "LengthNormalizedSequenceLogProbabilityScorer",
            "Constraint", "RepeatedNGramBlockingConstraint", "BeamSearch"]
 
 
 class Sampler:
-    """Base class (``olmo/beam_search.py:72-99``); ``params()`` is what the device kernel takes."""
+    """Base class (``olmo/beam_search.py:44-99``).  Two uses: ``params()`` is what the device-side sampling step of
+    a beam-1 generation takes; ``sample_nodes`` / ``sample_beams`` are what :class:`BeamSearch` calls, on float32
+    device tensors ``[rows, examples]``, returning ``(log_probs, indices, state)`` like the reference.  Draws are
+    made by perturbing log-weights with Gumbel noise and taking the top k (k draws without replacement from the
+    softmax; the reference calls ``torch.multinomial``), with noise from ``(seed, draw number)``: a sampler
+    object reproduces its draws after ``init_state``; the reference's random stream is not reproduced."""
 
     temperature: float = 1.0
     top_k: int = 0
     top_p: float = 1.0
     greedy: bool = False
+    with_replacement: bool = False
+    seed: int = 0
+    _draws: int = 0
 
     def params(self) -> dict:
         return {"temperature": float(self.temperature or 1.0), "top_k": int(self.top_k), "top_p": float(self.top_p)}
 
+    def init_state(self, start_class_log_probabilities: torch.Tensor, batch_size: int, num_classes: int) -> dict:
+        self._draws = 0
+        return {}
+
+    def sample_nodes(self, log_probs: torch.Tensor, per_node_beam_size: int, state: dict):
+        raise NotImplementedError
+
+    def sample_beams(self, log_probs: torch.Tensor, beam_size: int, state: dict):
+        """The ``beam_size`` best, deterministically (``olmo/beam_search.py:94-99``)."""
+        from . import ops
+
+        v, i = ops.topk(log_probs, beam_size)
+        return v, i, {}
+
+    def _draw(self, log_weights: torch.Tensor, k: int, inv_temp: float = 1.0) -> torch.Tensor:
+        """Indices ``[rows, k]`` drawn from ``softmax(log_weights * inv_temp)``: without replacement the k largest
+        of one perturbed copy, with replacement the largest of k independent ones."""
+        from . import ops
+
+        self._draws += 1
+        if not self.with_replacement:
+            return ops.topk(ops.gumbel_perturb(log_weights, inv_temp, self.seed, self._draws << 16), k)[1]
+        return torch.cat([ops.topk(ops.gumbel_perturb(log_weights, inv_temp, self.seed, (self._draws << 16) + j + 1), 1)[1]
+                          for j in range(k)], dim=-1)
+
 
 class DeterministicSampler(Sampler):
-    """``topk(log_probs, 1)``: the arg-max (``olmo/beam_search.py:102-114``)."""
+    """``topk(log_probs, k)`` (``olmo/beam_search.py:102-114``)."""
 
     greedy = True
+
+    def sample_nodes(self, log_probs, per_node_beam_size, state):
+        from . import ops
+
+        v, i = ops.topk(log_probs, per_node_beam_size)
+        return v, i, state
 
 
 class MultinomialSampler(Sampler):
     """``olmo/beam_search.py:117-146``."""
 
-    def __init__(self, temperature: float = 1.0, with_replacement: bool = False) -> None:
+    def __init__(self, temperature: float = 1.0, with_replacement: bool = False, seed: int = 0) -> None:
         self.temperature = temperature
         self.with_replacement = with_replacement
+        self.seed = seed
+
+    def sample_nodes(self, log_probs, per_node_beam_size, state):
+        idx = self._draw(log_probs, per_node_beam_size, 1.0 / float(self.temperature or 1.0))
+        return log_probs.gather(1, idx), idx, state
 
 
 class TopKSampler(Sampler):
-    """``olmo/beam_search.py:149-196``."""
+    """``olmo/beam_search.py:149-203``."""
 
-    def __init__(self, k: int = 1, temperature: float = 1.0, with_replacement: bool = False):
+    def __init__(self, k: int = 1, temperature: float = 1.0, with_replacement: bool = False, seed: int = 0):
         self.k = k
         self.top_k = k
         self.temperature = temperature or 1.0
         self.with_replacement = with_replacement
+        self.seed = seed
 
-    def check(self, vocab: int) -> None:
-        if not 1 <= self.k <= vocab:
+    def check(self, vocab: int, at_least: int = 1) -> None:
+        if not at_least <= self.k <= vocab or self.k < 1:
             raise ValueError(
                 "k must be a postive integer no less than per_node_beam_size and no greater than vocabulary size"
-            )  # the reference's message, :178-181
+            )  # the reference's message, :175-178
+
+    def sample_nodes(self, log_probs, per_node_beam_size, state):
+        from . import ops
+
+        self.check(log_probs.size(1), per_node_beam_size)
+        top_lp, top_idx = ops.topk(log_probs, self.k)
+        idx = top_idx.gather(-1, self._draw(top_lp, per_node_beam_size, 1.0 / float(self.temperature)))
+        return log_probs.gather(1, idx), idx, state
 
 
 class TopPSampler(Sampler):
-    """``olmo/beam_search.py:199-277``."""
+    """``olmo/beam_search.py:205-289``."""
 
-    def __init__(self, p: float = 0.9, temperature: float = 1.0, with_replacement: bool = False):
+    def __init__(self, p: float = 0.9, temperature: float = 1.0, with_replacement: bool = False, seed: int = 0):
         if p < 0.0 or p > 1.0:
-            raise ValueError("p must be a positive float no greater than 1.0")  # :227-228
+            raise ValueError("p must be a positive float no greater than 1.0")  # :232-233
         self.p = p
         self.top_p = p
         self.temperature = temperature or 1.0
         self.with_replacement = with_replacement
+        self.seed = seed
+
+    def sample_nodes(self, log_probs, per_node_beam_size, state):
+        from . import ops
+
+        if not per_node_beam_size <= log_probs.size(1):
+            raise ValueError("per_node_beam_size cannot be greater than vocabulary size")
+        lp = log_probs if self.temperature == 1.0 else ops.log_softmax(log_probs * (1.0 / float(self.temperature)))
+        # the nucleus: sorted descending, everything up to and including the entry at which the cumulative
+        # probability reaches p (:252-268); sort and running sum are library calls, the draw is not
+        desc, order = torch.sort(lp, dim=-1, descending=True, stable=True)
+        reached = torch.cumsum(desc.exp(), dim=-1) >= self.p
+        excluded = torch.zeros_like(reached)
+        excluded[..., 1:] = reached[..., :-1]
+        if not self.with_replacement:
+            excluded[..., :per_node_beam_size] = False
+        desc = desc.masked_fill(excluded, torch.finfo(torch.float32).min)
+        idx = order.gather(-1, self._draw(desc, per_node_beam_size))
+        return log_probs.gather(1, idx), idx, state
+
+
+class GumbelSampler(Sampler):
+    """Stochastic beam search (``olmo/beam_search.py:291-421``): not implemented."""
+
+    def __init__(self, temperature: float = 1.0):
+        raise NotImplementedError("the GumbelSampler (stochastic beam search) is not implemented")
 
 
 # ---------------------------------------------------------------------------------------------------
@@ -179,8 +258,9 @@ class BeamSearch:
     ``[batch, beam]``-sized tensors with torch.  State values are either tensors ``[group, ...]``, gathered along
     the group axis as in the reference (``:1047-1078``), or objects with ``expand_beams(batch, beam)`` and
     ``reorder_beams(backpointer)`` that keep their own books (the KV cache of ``OLMo.generate`` does: it
-    updates a table of row numbers instead of moving cache rows).  Only the ``DeterministicSampler`` is
-    implemented for the search; the stochastic samplers apply to beam size 1 through ``OLMo.generate``."""
+    updates a table of row numbers instead of moving cache rows).  A finished beam's candidates are the end token
+    at no cost and others at the float minimum, whatever the sampler (the reference feeds the sampler a one-hot
+    row, ``:948-957``).  The ``GumbelSampler`` is not implemented."""
 
     def __init__(self, end_index: int, *, max_steps: int = 50, beam_size: int = 10,
                  per_node_beam_size: Optional[int] = None, sampler: Optional[Sampler] = None,
@@ -197,8 +277,6 @@ class BeamSearch:
                 raise ValueError("min_steps must be non-negative")
             if not min_steps <= max_steps:
                 raise ValueError("min_steps must be less than or equal to max_steps")
-        if sampler is not None and not getattr(sampler, "greedy", False):
-            raise NotImplementedError("beam search is implemented for the DeterministicSampler only")
         self._end_index = end_index
         self.max_steps = max_steps
         self.beam_size = beam_size
@@ -255,7 +333,8 @@ class BeamSearch:
             lp = c.apply(cs, lp.unsqueeze(1)).squeeze(1)
         if self.min_steps >= 1:
             lp[:, end] = fmin
-        last_lp, cls = ops.topk(lp, K)
+        sstate = self.sampler.init_state(lp, B, V)
+        last_lp, cls, sstate = self.sampler.sample_beams(lp, K, sstate)
         if K == 1 and bool((cls == end).all()):
             warnings.warn("Empty sequences predicted. You may want to increase the beam size or ensure "
                           "your step function is working properly.", RuntimeWarning)
@@ -282,11 +361,11 @@ class BeamSearch:
                 lp = c.apply(cs, lp.view(B, K, -1)).view(B * K, -1)
             if timestep + 2 <= self.min_steps:
                 lp[:, end] = fmin
-            node_lp, node_cls = ops.topk(lp, PN)
+            node_lp, node_cls, sstate = self.sampler.sample_nodes(lp, PN, sstate)
             node_lp = torch.where(finished.unsqueeze(1), after_v, node_lp)
             node_cls = torch.where(finished.unsqueeze(1), after_i, node_cls)
             summed = (node_lp.view(B, K, PN) + last_lp.unsqueeze(2)).reshape(B, K * PN)
-            last_lp, pick = ops.topk(summed, K)
+            last_lp, pick, sstate = self.sampler.sample_beams(summed, K, sstate)
             predictions.append(node_cls.reshape(B, K * PN).gather(1, pick))
             backpointer = torch.div(pick, PN, rounding_mode="trunc")
             backpointers.append(backpointer)

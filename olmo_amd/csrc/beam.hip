@@ -91,7 +91,43 @@ __global__ __launch_bounds__(kThreads) void topk_kernel(const float* __restrict_
   }
 }
 
+__device__ __forceinline__ uint64_t mix64(uint64_t x) {  // splitmix64 finaliser
+  x += 0x9e3779b97f4a7c15ull;
+  x = (x ^ (x >> 30)) * 0xbf58476d1ce4e5b9ull;
+  x = (x ^ (x >> 27)) * 0x94d049bb133111ebull;
+  return x ^ (x >> 31);
+}
+
+// out = x * inv_temp + G with G ~ Gumbel(0, 1) drawn from (seed, counter, row, column); entries at or below half
+// the float minimum (what the search uses for "impossible") become -inf.  The k largest of a perturbed row are k
+// draws without replacement from softmax(x * inv_temp) (the Gumbel-top-k property), which is how
+// torch.multinomial(probabilities, k) of the reference's samplers (olmo/beam_search.py:135-146, 171-203, 238-289) is
+// realised here; k launches with different counters and k = 1 give draws with replacement.
+__global__ __launch_bounds__(256) void gumbel_perturb_kernel(const float* __restrict__ x, float* __restrict__ out,
+                                                             int64_t total, int n, float inv_temp, uint64_t seed,
+                                                             uint64_t counter) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const float v = x[i];
+  if (!(v > -1.7e38f)) {
+    out[i] = -INFINITY;
+    return;
+  }
+  const uint64_t r = mix64(mix64(seed ^ (counter * 0xd1342543de82ef95ull)) + (uint64_t)i);
+  const float u = ((float)(uint32_t)(r >> 40) + 0.5f) * (1.f / 16777216.f);  // (0, 1), 24 bits
+  out[i] = v * inv_temp - logf(-logf(u));
+}
+
 }  // namespace
+
+extern "C" int olmo355_gumbel_perturb(const float* x, float* out, int rows, int n, float inv_temp, uint64_t seed,
+                                      uint64_t counter, void* stream) {
+  if (!x || !out || rows <= 0 || n <= 0 || !(inv_temp > 0.f)) return O355_EINVAL;
+  const int64_t total = (int64_t)rows * n;
+  hipLaunchKernelGGL(gumbel_perturb_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, as_stream(stream), x, out,
+                     total, n, inv_temp, seed, counter);
+  O355_CHECK_LAUNCH();
+}
 
 extern "C" int olmo355_log_softmax(const void* logits, float* out, int rows, int n, int dtype, void* stream) {
   if (!logits || !out || rows <= 0 || n <= 0) return O355_EINVAL;

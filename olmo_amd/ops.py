@@ -400,6 +400,21 @@ def topk(x: torch.Tensor, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
     return vals, idx
 
 
+def gumbel_perturb(x: torch.Tensor, inv_temp: float = 1.0, seed: int = 0, counter: int = 0) -> torch.Tensor:
+    """``x * inv_temp`` plus Gumbel(0, 1) noise per element (float32 rows); ``topk`` of the result draws without
+    replacement from ``softmax(x * inv_temp)``."""
+    _dev(x)
+    if x.dtype != torch.float32:
+        raise TypeError("gumbel_perturb: float32 expected")
+    x = x.contiguous()
+    n = x.shape[-1]
+    out = torch.empty_like(x)
+    check("olmo355_gumbel_perturb",
+          lib().olmo355_gumbel_perturb(_p(x), _p(out), x.numel() // n, n, float(inv_temp), int(seed) & (2**64 - 1),
+                                       int(counter) & (2**64 - 1), _stream()))
+    return out
+
+
 def sample(logits: torch.Tensor, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0,
            counter: int = 0, counter_dev: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
            logprob: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:

@@ -119,8 +119,87 @@ def test_search_argument_checks_state_and_warnings(dev):
                 dict(min_steps=11, max_steps=10)):
         with pytest.raises(ValueError):
             BeamSearch(5, **bad)
+    from olmo_amd.beam_search import GumbelSampler
     with pytest.raises(NotImplementedError):
-        BeamSearch(5, beam_size=2, sampler=TopPSampler())
+        GumbelSampler()
+    with pytest.raises(ValueError):
+        TopPSampler(p=1.2)
+
+
+def test_gumbel_topk_draws_without_replacement(dev):
+    """The k largest of Gumbel-perturbed log-probabilities are k draws without replacement: first picks follow p,
+    ordered pairs follow p_i p_j / (1 - p_i) (chi-square over 120000 rows, 6 classes, 0.1 % level), a temperature
+    reshapes p, impossible entries are never drawn, and (seed, counter) reproduce."""
+    say("gumbel top-k")
+    from olmo_amd import ops
+    from scipy.stats import chi2
+
+    p = torch.tensor([0.35, 0.25, 0.2, 0.1, 0.07, 0.03], dtype=torch.float64)
+    rows = 120000
+    lp = torch.log(p).float().repeat(rows, 1).to(dev)
+    g = ops.gumbel_perturb(lp, 1.0, seed=5, counter=1)
+    assert torch.equal(g, ops.gumbel_perturb(lp, 1.0, seed=5, counter=1))
+    assert not torch.equal(g, ops.gumbel_perturb(lp, 1.0, seed=5, counter=2))
+    idx = ops.topk(g, 2)[1].cpu()
+    first = torch.bincount(idx[:, 0], minlength=6).double()
+    stat = ((first - rows * p) ** 2 / (rows * p)).sum().item()
+    assert stat < chi2.ppf(0.999, 5), stat
+    pair = torch.zeros(6, 6, dtype=torch.float64)
+    pair.index_put_((idx[:, 0], idx[:, 1]), torch.ones(rows, dtype=torch.float64), accumulate=True)
+    want = rows * p[:, None] * p[None, :] / (1 - p[:, None])
+    want.fill_diagonal_(0)
+    assert pair.diag().sum() == 0
+    off = want > 0
+    stat = ((pair[off] - want[off]) ** 2 / want[off]).sum().item()
+    assert stat < chi2.ppf(0.999, 29), stat
+    # temperature 2: weights p^(1/2)
+    q = p.sqrt() / p.sqrt().sum()
+    t = torch.bincount(ops.topk(ops.gumbel_perturb(lp, 0.5, seed=9, counter=3), 1)[1].cpu()[:, 0], minlength=6).double()
+    assert ((t - rows * q) ** 2 / (rows * q)).sum().item() < chi2.ppf(0.999, 5)
+    # impossible entries
+    lp2 = lp.clone()
+    lp2[:, 1] = torch.finfo(torch.float32).min
+    lp2[:, 4] = -float("inf")
+    i2 = ops.topk(ops.gumbel_perturb(lp2, 1.0, seed=1, counter=1), 4)[1].cpu()
+    assert not bool(((i2 == 1) | (i2 == 4)).any())
+
+
+def test_stochastic_samplers_in_search(dev):
+    """``tests/beam_search_test.py:320-384, 417-455``: searches with the multinomial, top-k and top-p samplers
+    (shapes, token range, an ended beam only repeats the end token), what each sampler may pick, the argument
+    checks, and that a seed reproduces."""
+    say("samplers in beam search")
+    from olmo_amd.beam_search import BeamSearch, MultinomialSampler, TopKSampler, TopPSampler
+
+    m = torch.tensor(KAT["matrices"]["T"], device=dev)
+    start = torch.zeros(5, dtype=torch.long, device=dev)
+    for make in (lambda: MultinomialSampler(temperature=0.9), lambda: TopKSampler(k=5, with_replacement=True),
+                 lambda: TopPSampler(p=0.8), lambda: TopKSampler(k=3, temperature=0.7), lambda: TopPSampler(p=0.5, with_replacement=True)):
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore", RuntimeWarning)
+            top, lp = BeamSearch(5, beam_size=3, max_steps=10, sampler=make()).search(start, {}, chain_step(m))
+            top2, lp2 = BeamSearch(5, beam_size=3, max_steps=10, sampler=make()).search(start, {}, chain_step(m))
+        assert list(top.shape[:2]) == [5, 3] and list(lp.shape) == [5, 3]
+        assert bool(((0 <= top) & (top <= 5)).all())
+        assert torch.equal(top, top2) and torch.equal(lp, lp2)  # same seed, same draws
+        ended = torch.cumsum((top == 5).long(), dim=2) > 0
+        assert bool((top[ended] == 5).all())
+    lps = torch.log(torch.tensor([[0.1, 0.3, 0.3, 0.3, 0.0, 0.0], [0.0, 0.0, 0.4, 0.3, 0.2, 0.1]])).to(dev)  # :66
+    for rep in range(20):
+        s = MultinomialSampler(temperature=0.9, seed=rep)
+        pr, cl, _ = s.sample_nodes(lps, 3, {})
+        assert pr.shape == cl.shape == (2, 3) and bool((cl[0] < 4).all()) and bool((cl[1] > 1).all())
+        assert torch.equal(pr, lps.gather(1, cl))
+        pr, cl, _ = TopKSampler(k=3, temperature=0.9, seed=rep).sample_nodes(lps, 3, {})
+        assert bool(((cl[0] > 0) & (cl[0] < 4)).all()) and bool(((cl[1] > 1) & (cl[1] < 5)).all())
+        pr, cl, _ = TopPSampler(p=0.8, temperature=0.9, seed=rep).sample_nodes(lps, 3, {})
+        assert bool(((cl[0] > 0) & (cl[0] < 4)).all()) and bool(((cl[1] > 1) & (cl[1] < 5)).all())
+        pr, cl, _ = TopPSampler(p=0.7, temperature=1.0, with_replacement=True, seed=rep).sample_nodes(lps, 3, {})
+        assert bool(((cl[0] >= 1) & (cl[0] <= 3)).all()) and bool(((cl[1] == 2) | (cl[1] == 3)).all())
+    for k in (-1, 0, 7):
+        with pytest.raises(ValueError):
+            BeamSearch(5, beam_size=3, max_steps=10, sampler=TopKSampler(k=k, with_replacement=True)).search(
+                start, {}, chain_step(m))
 
 
 @pytest.mark.parametrize("dtype,hd", [(torch.bfloat16, 128), (torch.float32, 32), (torch.bfloat16, 64)])
@@ -253,6 +332,13 @@ def test_generate_with_beams_bf16_consistency(dev):
         B, K, T = out.token_ids.shape
         assert (B, K) == (2, 4) and bool((out.scores[:, :-1] >= out.scores[:, 1:]).all())
         assert bool((out.scores[:, 0] >= one.scores[:, 0] - 1e-3).all())
+        from olmo_amd.beam_search import TopKSampler
+
+        drawn = model.generate(ids, max_steps=5, beam_size=3, sampler=TopKSampler(k=20, temperature=1.3, seed=3))
+        assert drawn.token_ids.shape[:2] == (2, 3)
+        for b in range(B):  # sampled candidates, true log-probabilities
+            for j in range(3):
+                assert abs(teacher_forced(b, drawn.token_ids[b, j]) - drawn.scores[b, j].item()) < 0.05 * T
         from olmo_amd.hf import OLMoConfig, OLMoForCausalLM
 
         hf = OLMoForCausalLM(OLMoConfig.from_model_config(cfg), model=model)
