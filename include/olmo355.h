@@ -244,6 +244,10 @@ int olmo355_topk(const float* x, int rows, int n, int k, float* out_vals, int64_
  * from softmax(x * inv_temp); the reference's random stream is not reproduced. */
 int olmo355_gumbel_perturb(const float* x, float* out, int rows, int n, float inv_temp, uint64_t seed,
                            uint64_t counter, void* stream);
+/* GumbelSampler.gumbel_with_max (olmo/beam_search.py:395-421): per row, Gumbel(phi) samples conditioned on their
+ * maximum being row_max[row]; fp32 [rows, n] in and out, noise from (seed, counter, element). */
+int olmo355_gumbel_with_max(const float* phi, const float* row_max, float* out, int rows, int n, uint64_t seed,
+                            uint64_t counter, void* stream);
 
 /* One sampled step (olmo/beam_search.py:117-277 with beam size 1): z = logits / temperature; top_k > 0 keeps the
  * k largest, then top_p < 1 keeps the most probable tokens up to and including the one at which the cumulative

@@ -57,6 +57,7 @@ EXPORTS = {
     "olmo355_log_softmax": (I, [P, P, I, I, I, P]),
     "olmo355_topk": (I, [P, I, I, I, P, P, P]),
     "olmo355_gumbel_perturb": (I, [P, P, I, I, F, c_uint64, c_uint64, P]),
+    "olmo355_gumbel_with_max": (I, [P, P, P, I, I, c_uint64, c_uint64, P]),
     "olmo355_gemm_splitk_plan": (I, [I, I, I]),
     "olmo355_w4_gemm_splitk": (I, [P, P, P, P, P, I, I, I, I, P, P]),
     "olmo355_b16_gemm_splitk": (I, [P, P, P, I, I, I, I, P, P]),

@@ -4,8 +4,7 @@
 Beam size 1: the samplers are parameter holders for the device-side sampling step (``olmo355_sample``);
 ``OLMo.generate(..., sampler=TopPSampler(p=0.9))`` draws one token per step on the GPU inside the captured
 decode step.  Beam sizes above 1: ``BeamSearch`` below; the samplers' ``sample_nodes`` draw per-node candidates
-on the device (Gumbel-perturbed log-weights + top-k).  The ``GumbelSampler`` (``olmo/beam_search.py:291-421``)
-is not implemented.
+on the device (Gumbel-perturbed log-weights + top-k), as does the ``GumbelSampler``'s stochastic beam search.
 """
 
 from __future__ import annotations
@@ -149,10 +148,43 @@ class TopPSampler(Sampler):
 
 
 class GumbelSampler(Sampler):
-    """Stochastic beam search (``olmo/beam_search.py:291-421``): not implemented."""
+    """Stochastic beam search (``olmo/beam_search.py:291-421``; Kool, van Hoof, Welling: the Gumbel-top-k trick):
+    the ``beam_size`` sequences kept are a sample without replacement from the sequence distribution.  Every
+    candidate carries a perturbed log-probability ``G`` drawn conditionally on its parent's (``gumbel_with_max``,
+    one device launch per step); beams are cut by ``G``, then ordered by true log-probability."""
 
-    def __init__(self, temperature: float = 1.0):
-        raise NotImplementedError("the GumbelSampler (stochastic beam search) is not implemented")
+    def __init__(self, temperature: float = 1.0, seed: int = 0):
+        self.temperature = temperature
+        self.seed = seed
+
+    def _gumbel_with_max(self, phi: torch.Tensor, t: torch.Tensor) -> torch.Tensor:
+        from . import ops
+
+        self._draws += 1
+        return ops.gumbel_with_max(phi, t.reshape(-1).to(torch.float32), self.seed, self._draws)
+
+    def init_state(self, start_class_log_probabilities, batch_size, num_classes):
+        self._draws = 0
+        zeros = torch.zeros(batch_size, dtype=torch.float32, device=start_class_log_probabilities.device)
+        return {"G_phi_S": self._gumbel_with_max(start_class_log_probabilities, zeros)}
+
+    def sample_nodes(self, log_probs, per_node_beam_size, state):
+        from . import ops
+
+        lp = log_probs if self.temperature == 1.0 else ops.log_softmax(log_probs * (1.0 / float(self.temperature)))
+        phi_new = state["phi_S"].unsqueeze(-1) + lp
+        g_new = self._gumbel_with_max(phi_new, state["G_phi_S"])
+        top_g, idx = ops.topk(g_new, per_node_beam_size)
+        return log_probs.gather(1, idx), idx, {"G_phi_S": top_g}
+
+    def sample_beams(self, log_probs, beam_size, state):
+        from . import ops
+
+        batch = log_probs.size(0)
+        g, sel = ops.topk(state["G_phi_S"].reshape(log_probs.shape).contiguous(), beam_size)
+        sel_lp, order = log_probs.gather(1, sel).sort(dim=-1, descending=True, stable=True)
+        sel, g = sel.gather(1, order), g.gather(1, order)
+        return sel_lp, sel, {"G_phi_S": g.reshape(batch * beam_size), "phi_S": sel_lp.reshape(batch * beam_size)}
 
 
 # ---------------------------------------------------------------------------------------------------
@@ -258,9 +290,7 @@ class BeamSearch:
     ``[batch, beam]``-sized tensors with torch.  State values are either tensors ``[group, ...]``, gathered along
     the group axis as in the reference (``:1047-1078``), or objects with ``expand_beams(batch, beam)`` and
     ``reorder_beams(backpointer)`` that keep their own books (the KV cache of ``OLMo.generate`` does: it
-    updates a table of row numbers instead of moving cache rows).  A finished beam's candidates are the end token
-    at no cost and others at the float minimum, whatever the sampler (the reference feeds the sampler a one-hot
-    row, ``:948-957``).  The ``GumbelSampler`` is not implemented."""
+    updates a table of row numbers instead of moving cache rows)."""
 
     def __init__(self, end_index: int, *, max_steps: int = 50, beam_size: int = 10,
                  per_node_beam_size: Optional[int] = None, sampler: Optional[Sampler] = None,
@@ -329,11 +359,11 @@ class BeamSearch:
                              f"Please decrease beam_size or per_node_beam_size.")
         if K > V:
             raise ValueError(f"Vocab size ({V:d}) too small relative to beam_size ({K:d}).")
+        sstate = self.sampler.init_state(lp, B, V)  # before the constraints, as in the reference (:851)
         for c, cs in zip(self.constraints, cstates):
             lp = c.apply(cs, lp.unsqueeze(1)).squeeze(1)
         if self.min_steps >= 1:
             lp[:, end] = fmin
-        sstate = self.sampler.init_state(lp, B, V)
         last_lp, cls, sstate = self.sampler.sample_beams(lp, K, sstate)
         if K == 1 and bool((cls == end).all()):
             warnings.warn("Empty sequences predicted. You may want to increase the beam size or ensure "
@@ -361,9 +391,14 @@ class BeamSearch:
                 lp = c.apply(cs, lp.view(B, K, -1)).view(B * K, -1)
             if timestep + 2 <= self.min_steps:
                 lp[:, end] = fmin
-            node_lp, node_cls, sstate = self.sampler.sample_nodes(lp, PN, sstate)
-            node_lp = torch.where(finished.unsqueeze(1), after_v, node_lp)
-            node_cls = torch.where(finished.unsqueeze(1), after_i, node_cls)
+            if getattr(self.sampler, "greedy", False):
+                # the top of a finished beam's one-hot row is known: patch the rows instead of building it
+                node_lp, node_cls, sstate = self.sampler.sample_nodes(lp, PN, sstate)
+                node_lp = torch.where(finished.unsqueeze(1), after_v, node_lp)
+                node_cls = torch.where(finished.unsqueeze(1), after_i, node_cls)
+            else:  # a sampler may keep state per candidate: give it the rows the reference gives it (:948-957)
+                node_lp, node_cls, sstate = self.sampler.sample_nodes(torch.where(finished.unsqueeze(1), after_end, lp),
+                                                                      PN, sstate)
             summed = (node_lp.view(B, K, PN) + last_lp.unsqueeze(2)).reshape(B, K * PN)
             last_lp, pick, sstate = self.sampler.sample_beams(summed, K, sstate)
             predictions.append(node_cls.reshape(B, K * PN).gather(1, pick))

@@ -91,7 +91,7 @@ __global__ __launch_bounds__(kThreads) void topk_kernel(const float* __restrict_
   }
 }
 
-__device__ __forceinline__ uint64_t mix64(uint64_t x) {  // splitmix64 finaliser
+__host__ __device__ __forceinline__ uint64_t mix64(uint64_t x) {  // splitmix64 finaliser
   x += 0x9e3779b97f4a7c15ull;
   x = (x ^ (x >> 30)) * 0xbf58476d1ce4e5b9ull;
   x = (x ^ (x >> 27)) * 0x94d049bb133111ebull;
@@ -118,7 +118,42 @@ __global__ __launch_bounds__(256) void gumbel_perturb_kernel(const float* __rest
   out[i] = v * inv_temp - logf(-logf(u));
 }
 
+__device__ __forceinline__ float gumbel_at(float phi, uint64_t key, int64_t i) {
+  if (!(phi > -1.7e38f)) return -INFINITY;
+  const uint64_t r = mix64(key + (uint64_t)i);
+  const float u = ((float)(uint32_t)(r >> 40) + 0.5f) * (1.f / 16777216.f);
+  return phi - logf(-logf(u));
+}
+
+// Gumbel(phi) per element conditioned on the row maximum being T[row] (GumbelSampler.gumbel_with_max,
+// olmo/beam_search.py:403-421): G = phi + noise, Z = max G, v = T - G + log1p(-exp(G - Z)),
+// out = T - max(v, 0) - log1p(exp(-|v|)).  One workgroup per row; the noise is regenerated for the second pass
+// instead of being stored.
+__global__ __launch_bounds__(kThreads) void gumbel_with_max_kernel(const float* __restrict__ phi,
+                                                                   const float* __restrict__ t_row,
+                                                                   float* __restrict__ out, int n, uint64_t key) {
+  __shared__ float red[kWaves];
+  const int64_t base = (int64_t)blockIdx.x * n;
+  float z = -INFINITY;
+  for (int i = threadIdx.x; i < n; i += kThreads) z = fmaxf(z, gumbel_at(phi[base + i], key, base + i));
+  z = block_max_f(z, red);
+  const float t = t_row[blockIdx.x];
+  for (int i = threadIdx.x; i < n; i += kThreads) {
+    const float g = gumbel_at(phi[base + i], key, base + i);
+    const float v = t - g + log1pf(-expf(g - z));
+    out[base + i] = t - fmaxf(v, 0.f) - log1pf(expf(-fabsf(v)));
+  }
+}
+
 }  // namespace
+
+extern "C" int olmo355_gumbel_with_max(const float* phi, const float* row_max, float* out, int rows, int n, uint64_t seed,
+                                       uint64_t counter, void* stream) {
+  if (!phi || !row_max || !out || rows <= 0 || n <= 0) return O355_EINVAL;
+  hipLaunchKernelGGL(gumbel_with_max_kernel, dim3(rows), dim3(kThreads), 0, as_stream(stream), phi, row_max, out, n,
+                     mix64(seed ^ (counter * 0xd1342543de82ef95ull)));
+  O355_CHECK_LAUNCH();
+}
 
 extern "C" int olmo355_gumbel_perturb(const float* x, float* out, int rows, int n, float inv_temp, uint64_t seed,
                                       uint64_t counter, void* stream) {

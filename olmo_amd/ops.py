@@ -415,6 +415,24 @@ def gumbel_perturb(x: torch.Tensor, inv_temp: float = 1.0, seed: int = 0, counte
     return out
 
 
+def gumbel_with_max(phi: torch.Tensor, row_max: torch.Tensor, seed: int = 0, counter: int = 0) -> torch.Tensor:
+    """Gumbel(``phi``) samples per row ``[rows, n]`` conditioned on their maximum being ``row_max[row]``
+    (``GumbelSampler.gumbel_with_max``)."""
+    _dev(phi, row_max)
+    if phi.dtype != torch.float32 or row_max.dtype != torch.float32:
+        raise TypeError("gumbel_with_max: float32 expected")
+    phi = phi.contiguous()
+    n = phi.shape[-1]
+    rows = phi.numel() // n
+    if row_max.numel() != rows:
+        raise ValueError("one maximum per row expected")
+    out = torch.empty_like(phi)
+    check("olmo355_gumbel_with_max",
+          lib().olmo355_gumbel_with_max(_p(phi), _p(row_max.contiguous()), _p(out), rows, n, int(seed) & (2**64 - 1),
+                                        int(counter) & (2**64 - 1), _stream()))
+    return out
+
+
 def sample(logits: torch.Tensor, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0,
            counter: int = 0, counter_dev: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
            logprob: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:

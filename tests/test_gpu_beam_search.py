@@ -119,9 +119,6 @@ def test_search_argument_checks_state_and_warnings(dev):
                 dict(min_steps=11, max_steps=10)):
         with pytest.raises(ValueError):
             BeamSearch(5, **bad)
-    from olmo_amd.beam_search import GumbelSampler
-    with pytest.raises(NotImplementedError):
-        GumbelSampler()
     with pytest.raises(ValueError):
         TopPSampler(p=1.2)
 
@@ -200,6 +197,58 @@ def test_stochastic_samplers_in_search(dev):
         with pytest.raises(ValueError):
             BeamSearch(5, beam_size=3, max_steps=10, sampler=TopKSampler(k=k, with_replacement=True)).search(
                 start, {}, chain_step(m))
+
+
+def test_gumbel_sampler_stochastic_beam_search(dev):
+    """``GumbelSampler``: (a) ``gumbel_with_max`` puts each row's maximum exactly at the given value and leaves the
+    arg-max distributed as the softmax; (b) the reference's own checks (``tests/beam_search_test.py:386-415, 457-472``:
+    shapes, ranges, beams ordered by log-probability, ended beams repeat the end token); (c) what the algorithm is
+    for: the two sequences a two-step search keeps are a sample without replacement from the joint sequence
+    distribution, so a sequence s is kept with probability q_s + sum_r q_r q_s / (1 - q_r) -- checked on 40000
+    independent batch rows against the exact figures for all nine sequences of a three-token chain."""
+    say("gumbel sampler")
+    from olmo_amd import ops
+    from olmo_amd.beam_search import BeamSearch, GumbelSampler
+    from scipy.stats import chi2
+
+    p = torch.tensor([0.4, 0.3, 0.15, 0.1, 0.05], dtype=torch.float64)
+    rows = 60000
+    phi = torch.log(p).float().repeat(rows, 1).to(dev)
+    t = torch.linspace(-3, 2, rows).to(dev)
+    g = ops.gumbel_with_max(phi, t, seed=2, counter=1)
+    assert (g.max(dim=1).values - t).abs().max().item() < 1e-5
+    am = torch.bincount(g.argmax(dim=1).cpu(), minlength=5).double()
+    assert ((am - rows * p) ** 2 / (rows * p)).sum().item() < chi2.ppf(0.999, 4)
+
+    m = torch.tensor(KAT["matrices"]["T"], device=dev)
+    top, lp = BeamSearch(5, beam_size=3, max_steps=10, sampler=GumbelSampler()).search(
+        torch.zeros(5, dtype=torch.long, device=dev), {}, chain_step(m))
+    assert list(top.shape[:2]) == [5, 3] and list(lp.shape) == [5, 3] and bool(((0 <= top) & (top <= 5)).all())
+    ended = torch.cumsum((top == 5).long(), dim=2) > 0
+    assert bool((top[ended] == 5).all())
+    lps = torch.log(torch.tensor([[0.1, 0.3, 0.3, 0.3, 0.0, 0.0], [0.0, 0.0, 0.4, 0.3, 0.2, 0.1]])).to(dev)
+    smp = GumbelSampler(seed=4)
+    st = smp.init_state(lps, 2, 6)
+    lp_b, idx, st = smp.sample_beams(lps, 3, st)
+    assert lp_b.shape == idx.shape == (2, 3) and bool((lp_b[:, :-1] >= lp_b[:, 1:]).all())
+    assert bool((idx[0] < 4).all()) and bool((idx[1] > 1).all())
+    assert st["G_phi_S"].shape == (6,) and st["phi_S"].shape == (6,)
+
+    tr = torch.tensor([[0.5, 0.3, 0.2, 0.0], [0.2, 0.2, 0.6, 0.0], [0.1, 0.7, 0.2, 0.0], [0.3, 0.3, 0.4, 0.0]],
+                      dtype=torch.float64)  # rows: last token 0..2 (and an unused end row); the end token never occurs
+    q = {(a, b): (tr[0, a] * tr[a, b]).item() for a in range(3) for b in range(3)}
+    batch = 40000
+    top, _ = BeamSearch(3, beam_size=2, max_steps=2, sampler=GumbelSampler(seed=11)).search(
+        torch.zeros(batch, dtype=torch.long, device=dev), {}, chain_step(tr.float().to(dev)))
+    codes = (top[:, :, 0] * 3 + top[:, :, 1]).cpu()
+    assert bool((codes[:, 0] != codes[:, 1]).all())  # without replacement
+    worst = 0.0
+    for (a, b), qs in q.items():
+        want = qs + sum(qr * qs / (1 - qr) for r, qr in q.items() if r != (a, b))
+        got = (codes == a * 3 + b).any(dim=1).double().mean().item()
+        sigma = (want * (1 - want) / batch) ** 0.5
+        worst = max(worst, abs(got - want) / sigma)
+    assert worst < 4.5, worst
 
 
 @pytest.mark.parametrize("dtype,hd", [(torch.bfloat16, 128), (torch.float32, 32), (torch.bfloat16, 64)])
