@@ -56,6 +56,9 @@ def main() -> int:
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: one plain copy of known size, then the four "
                          "int4 linears of a layer at one row; nothing is timed or printed")
+    ap.add_argument("--gemm-probe", action="store_true",
+                    help="for rocprofv3 --pmc matrix-core counters: the four int4 block linears of a layer at 2048 "
+                         "rows, three times each over distinct weights; nothing is timed or printed")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this build runs the whole model on ONE GPU; --gpus N with N > 1 is not supported.")
@@ -76,6 +79,8 @@ def main() -> int:
     cfg = PRESETS["olmo2-7b"]
     if args.traffic_probe:
         return traffic_probe(cfg, dev)
+    if args.gemm_probe:
+        return traffic_probe(cfg, dev, rows=2048)
     if args.sweep:
         return linear_sweep(dev)
     if args.config4:
@@ -361,10 +366,10 @@ def config4(dev, steps: int) -> int:
     return 0
 
 
-def traffic_probe(cfg, dev) -> int:
-    """Launches whose HBM traffic the hardware counters are read for: a 256 MiB device copy (the
-    yardstick: 256 MiB read, 256 MiB written) and the four int4 block linears at one row, three
-    times each over distinct weights."""
+def traffic_probe(cfg, dev, rows: int = 1) -> int:
+    """Launches whose hardware counters are read: a 256 MiB device copy (the yardstick for HBM traffic: 256 MiB
+    read, 256 MiB written) and the four int4 block linears at ``rows`` rows, three times each over distinct
+    weights."""
     import torch
 
     from olmo_amd import ops
@@ -378,7 +383,7 @@ def traffic_probe(cfg, dev) -> int:
     dst.copy_(src)
     torch.cuda.synchronize()
     for n, k in linear_shapes(cfg):
-        x = torch.randn(1, k, device=dev).to(torch.bfloat16)
+        x = torch.randn(rows, k, device=dev).to(torch.bfloat16)
         for _ in range(3):
             q = QuantLinear(4, 128, k, n, True, device=dev)
             fill_random_int4(q, gen)
