@@ -93,10 +93,13 @@ def _prefill(model, input_ids, attention_mask, sampling: Optional[dict] = None):
 @torch.no_grad()
 def greedy_generate(model, input_ids: torch.Tensor, attention_mask: Optional[torch.Tensor], max_new_tokens: int,
                     use_graph: bool = True, eos_token_id: Optional[int] = None, pad_token_id: Optional[int] = None,
-                    return_scores: bool = False, return_logits: bool = False, sampling: Optional[dict] = None):
+                    return_scores: bool = False, return_logits: bool = False, sampling: Optional[dict] = None,
+                    stop_when_all_ended: bool = False):
     """Returns ``tokens [B, max_new_tokens]`` (and, on request, the summed log-probabilities of the
-    chosen tokens and / or the per-step logits).  Always runs ``max_new_tokens`` steps; with
-    ``eos_token_id`` the tokens after a sequence's first EOS are replaced by ``pad_token_id``.
+    chosen tokens and / or the per-step logits).  Runs ``max_new_tokens`` steps; with
+    ``eos_token_id`` the tokens after a sequence's first EOS are replaced by ``pad_token_id`` and add nothing to
+    the score, and with ``stop_when_all_ended`` the loop also ends (and the result is cut) once every sequence has
+    emitted it, as the reference's search does.
     ``sampling`` (``temperature``, ``top_k``, ``top_p``, ``seed``) draws the tokens instead of taking the
     arg-max; the same seed and prompt give the same tokens."""
     if max_new_tokens < 1:
@@ -110,25 +113,41 @@ def greedy_generate(model, input_ids: torch.Tensor, attention_mask: Optional[tor
     tokens = torch.empty(B, max_new_tokens, dtype=torch.int64, device=model.device)
     tokens[:, 0] = sess.ids.view(B)
     all_logits = [out.logits[:, -1].clone()] if (return_scores or return_logits) else None
+    steps = max_new_tokens
     for i in range(1, max_new_tokens):
+        if stop_when_all_ended and eos_token_id is not None and i % 16 == 0:
+            # the search ends once every sequence has emitted the end token (olmo/beam_search.py:918-923); looked at
+            # every 16 steps only: the check is a host synchronisation
+            if bool((tokens[:, :i] == eos_token_id).any(dim=1).all()):
+                steps = i
+                break
         if use_graph and sess.graph is None and i == 3:
             sess.capture()
         sess.step()
         tokens[:, i] = sess.ids.view(B)
         if all_logits is not None:
             all_logits.append(sess.logits.view(B, -1).clone())
+    tokens = tokens[:, :steps]
     result = [tokens]
+    after = None
     if eos_token_id is not None:
         pad = eos_token_id if pad_token_id is None else pad_token_id
         seen = (tokens == eos_token_id).cumsum(dim=1)
         after = (seen - (tokens == eos_token_id).to(seen.dtype)) > 0
         tokens = torch.where(after, torch.full_like(tokens, pad), tokens)
+        if stop_when_all_ended:  # as long as the longest sequence, its end token included
+            keep = int((~after).sum(dim=1).max().item())
+            tokens, after = tokens[:, :keep], after[:, :keep]
         result[0] = tokens
     if return_scores:
         # log-probability bookkeeping of the search (olmo/model.py:1705, beam_search.py:1003-1019);
-        # not on the timed path, so plain torch on the saved logits
-        lp = torch.stack([torch.log_softmax(l.float(), dim=-1) for l in all_logits], dim=1)
-        result.append(lp.gather(-1, tokens.clamp_min(0).unsqueeze(-1)).squeeze(-1).sum(dim=1))
+        # not on the timed path, so plain torch on the saved logits.  An ended sequence adds nothing
+        # (beam_search.py:948-957: the forced end token has log-probability 0).
+        lp = torch.stack([torch.log_softmax(l.float(), dim=-1) for l in all_logits[: tokens.shape[1]]], dim=1)
+        tok_lp = lp.gather(-1, tokens.clamp_min(0).unsqueeze(-1)).squeeze(-1)
+        if after is not None:
+            tok_lp = tok_lp.masked_fill(after, 0.0)
+        result.append(tok_lp.sum(dim=1))
     if return_logits:
-        result.append(torch.stack(all_logits, dim=1))
+        result.append(torch.stack(all_logits[: tokens.shape[1]], dim=1))
     return result[0] if len(result) == 1 else tuple(result)

@@ -582,15 +582,17 @@ class OLMo(nn.Module):
     def generate(self, input_ids: torch.LongTensor, attention_mask: Optional[torch.Tensor] = None,
                  max_steps: int = 10, beam_size: int = 1, per_node_beam_size: Optional[int] = None,
                  sampler=None, min_steps: Optional[int] = None, final_sequence_scorer=None,
-                 constraints: Optional[list] = None, use_graph: bool = True, stop_at_eos: bool = False,
+                 constraints: Optional[list] = None, use_graph: bool = True, stop_at_eos: bool = True,
                  seed: int = 0) -> OLMoGenerateOutput:
         """``OLMo.generate`` (``olmo/model.py:1603-1728``).
 
         Beam size 1 without constraints, ``min_steps`` or a scorer is the captured greedy loop
         (``DeterministicSampler``), or one draw per step on the device with the ``MultinomialSampler`` /
-        ``TopKSampler`` / ``TopPSampler`` of ``olmo_amd.beam_search``; it always runs ``max_steps`` steps
-        (``stop_at_eos`` pads after the first end token).  Anything else is ``olmo_amd.beam_search.BeamSearch``
-        over a :class:`BeamKVCache`: it stops when every beam has ended, as the reference does.  ``scores`` is the
+        ``TopKSampler`` / ``TopPSampler`` of ``olmo_amd.beam_search``.  As in the reference's search a sequence
+        that has emitted the end token only repeats it at no cost and the result is as long as the longest
+        sequence (the captured loop looks for "all ended" every 16 steps; ``stop_at_eos=False`` runs all
+        ``max_steps`` and leaves the tokens as generated).  Anything else is ``olmo_amd.beam_search.BeamSearch``
+        over a :class:`BeamKVCache`.  ``scores`` is the
         summed log-probability of the chosen tokens under the unfiltered distribution (passed through
         ``final_sequence_scorer`` in a beam search)."""
         plain = beam_size == 1 and not constraints and not min_steps and final_sequence_scorer is None
@@ -606,7 +608,7 @@ class OLMo(nn.Module):
             sampling = dict(sampler.params(), seed=seed)
         toks, scores = greedy_generate(self, input_ids, attention_mask, max_steps, use_graph=use_graph,
                                        eos_token_id=self.config.eos_token_id if stop_at_eos else None,
-                                       return_scores=True, sampling=sampling)
+                                       return_scores=True, sampling=sampling, stop_when_all_ended=stop_at_eos)
         return OLMoGenerateOutput(token_ids=toks.unsqueeze(1), scores=scores.unsqueeze(1))
 
     def _generate_beam(self, input_ids, attention_mask, max_steps, beam_size, per_node_beam_size, sampler, min_steps,

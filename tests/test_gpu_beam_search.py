@@ -350,6 +350,31 @@ def test_generate_with_beams_against_oracle_fp32(dev, kind, masked):
         assert (out.scores.cpu() - want_s).abs().max().item() < 2e-3, kw
 
 
+def test_greedy_generate_end_token_semantics_fp32(dev):
+    """The captured greedy loop follows the search's rules for the end token (``olmo/beam_search.py:918-957``): a
+    sequence that emitted it only repeats it at no cost, and the result is as long as the longest sequence.  An end
+    token is chosen that the model does emit early in one sequence; result against the oracle's search with beam 1
+    and against this build's own search."""
+    say("greedy end-token semantics")
+    cfg = small_cfg("ln")
+    model, oracle = build_pair(cfg, torch.float32, dev, seed=5)
+    ids = torch.randint(8, cfg.vocab_size, (3, 11), generator=torch.Generator().manual_seed(2))
+    free = model.generate(ids.to(dev), max_steps=20, stop_at_eos=False).token_ids[:, 0].cpu()
+    assert free.shape == (3, 20)
+    for eos in (int(free[0, 2]), int(free[1, 0])):
+        cfg.eos_token_id = eos
+        out = model.generate(ids.to(dev), max_steps=20)
+        want_t, want_s = oracle_generate(oracle, ids, None, eos, beam_size=1, max_steps=20)
+        assert torch.equal(out.token_ids.cpu(), want_t), (eos, out.token_ids.cpu(), want_t)
+        assert (out.scores.cpu() - want_s).abs().max().item() < 2e-3
+        via = model._generate_beam(ids.to(dev), None, 20, 1, None, None, None, None, None)
+        assert torch.equal(via.token_ids, out.token_ids) and (via.scores - out.scores).abs().max().item() < 2e-3
+    # every sequence ends at once: the loop stops at its 16-step check and the result is cut to the end token
+    cfg.eos_token_id = int(free[0, 0])
+    one = model.generate(ids[:1].to(dev), max_steps=40)
+    assert one.token_ids.shape == (1, 1, 1) and int(one.token_ids[0, 0, 0]) == cfg.eos_token_id
+
+
 def test_generate_with_beams_bf16_consistency(dev):
     """bf16 OLMo-2 wiring (QK-norm, GQA off / on).  Every returned sequence's score equals its teacher-forced
     log-probability from a plain forward pass of the same model (so the row table handed each beam its own
