@@ -156,10 +156,18 @@ class OLMoForCausalLM(nn.Module):
             # OLMo's own search (olmo/beam_search.py via OLMo.generate), not transformers' BeamSearchScorer:
             # summed log-probabilities, no length penalty; the best beam of each sequence, padded with the
             # end token once it has ended
-            if do_sample:
-                raise NotImplementedError("sampling inside a beam search is not implemented")
+            sampler = None
+            if do_sample:  # per-node candidates drawn instead of taken from the top (olmo/beam_search.py samplers)
+                from .beam_search import MultinomialSampler, TopKSampler, TopPSampler
+
+                if top_p < 1.0:
+                    sampler = TopPSampler(p=top_p, temperature=temperature, seed=seed)
+                elif top_k:
+                    sampler = TopKSampler(k=top_k, temperature=temperature, seed=seed)
+                else:
+                    sampler = MultinomialSampler(temperature=temperature, seed=seed)
             out = self.model.generate(input_ids, attention_mask=attention_mask, max_steps=max_new_tokens,
-                                      beam_size=num_beams)
+                                      beam_size=num_beams, sampler=sampler)
             return torch.cat((input_ids.to(out.token_ids.device), out.token_ids[:, 0]), dim=1)
         sampling = dict(temperature=temperature, top_k=top_k or 0, top_p=top_p, seed=seed) if do_sample else None
         new = greedy_generate(self.model, input_ids, attention_mask, max_new_tokens, use_graph=use_graph,
