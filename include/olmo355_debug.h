@@ -1,27 +1,35 @@
-/* Test hooks of libolmo355.so: force one of the kernel variants the dispatchers choose between, so that tests
- * and tuning runs can reach every variant on any shape.  They set process-wide state, are not thread-safe and are
- * not part of the drop-in interface (include/olmo355.h has no state); 0 / -1 restores the dispatcher's choice.
- * No counterpart in the reference. */
+/* Variant entry points of libolmo355.so: each is one of the declared entry points of include/olmo355.h with one
+ * more argument that names the kernel variant the dispatcher would otherwise choose by shape, so that tests and
+ * tuning runs can reach every variant on any shape.  Like the rest of the library they keep no state: the choice
+ * is an argument of the call.  Not part of the drop-in interface; no counterpart in the reference. */
 #ifndef OLMO355_DEBUG_H
 #define OLMO355_DEBUG_H
+#include <stdint.h>
 #ifdef __cplusplus
 extern "C" {
 #endif
 
-/* GEMM tile: 0 = choose; 256 / 192 / 128 = 256 rows by that many columns; 128128 / 128064 = 128-row tiles. */
-void olmo355_debug_set_gemm_tile(int shape);
-/* Older small-M int4 kernel (w4_gemv_kernel / w4_gemv_rot_kernel): waves per workgroup (-1 = choose) and
- * whether the activations are staged in LDS (-1 = choose). */
-void olmo355_debug_set_gemv_plan(int waves, int xlds);
-/* 1 = the dispatcher's choice (default); 0 = never the lean / staged-activation kernels; 2 = the
- * staged-activation kernel (w4_mid_kernel) for every plain call. */
-void olmo355_debug_set_gemv_small(int mode);
-/* w4_mid_kernel: column-tile pairs per workgroup, 0 = choose, 1 or 2. */
-void olmo355_debug_set_mid_pairs(int pairs);
-/* Fused decode attention, how the key chunks of a head are merged: -1 = choose (default), 0 = always in the
- * kernel (last workgroup of a head, ticket), 1 = one workgroup per (batch, head) and no chunks, 2 = always the
- * separate combine kernel. */
-void olmo355_debug_set_attn_mode(int mode);
+/* olmo355_w4_gemm / olmo355_b16_gemm with the tile shape given: 0 = choose; 256 / 192 / 128 = 256 rows by that
+ * many columns; 128128 / 128064 = 128-row tiles. */
+int olmo355_w4_gemm_tile(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
+                         int M, int N, int K, int tile, void* stream);
+int olmo355_b16_gemm_tile(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, int tile,
+                          void* stream);
+
+/* olmo355_w4_gemv with the kernel family given: 0 = choose; 1 = the kernels that keep all rows of x in LDS per
+ * workgroup (the lean M <= 16 kernel where it applies), never the staged-activation kernel; 2 = the
+ * staged-activation kernel (w4_mid_kernel), 3 / 4 = the same with one / two column-tile pairs per workgroup;
+ * 5 = the older kernels only (w4_gemv_rot_kernel / w4_gemv_kernel). */
+int olmo355_w4_gemv_form(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
+                         int M, int N, int K, int form, void* stream);
+
+/* olmo355_attn_decode_fused with the merge of a head's key chunks given: -1 = choose, 0 = in the kernel (the last
+ * workgroup of a (batch, head) to finish, found by a ticket), 2 = the separate combine kernel. */
+int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
+                                    const float* cos_tab, void* kcache, void* vcache, const float* key_bias, void* out,
+                                    void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos, int past_len,
+                                    const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps,
+                                    const float* qk_ssq, const float* rope_now, int dtype, int merge, void* stream);
 
 #ifdef __cplusplus
 }

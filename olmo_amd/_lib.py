@@ -74,6 +74,14 @@ EXPORTS = {
     "olmo355_incr_i32": (I, [P, P]),
 }
 
+# variant entry points of include/olmo355_debug.h (the dispatcher's choice as an explicit argument; tests and tuning)
+VARIANT_EXPORTS = {
+    "olmo355_w4_gemm_tile": (I, [P, P, P, P, P, I, I, I, I, P]),
+    "olmo355_b16_gemm_tile": (I, [P, P, P, I, I, I, I, P]),
+    "olmo355_w4_gemv_form": (I, [P, P, P, P, P, I, I, I, I, P]),
+    "olmo355_attn_decode_fused_merge": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, P, I, I, P]),
+}
+
 _lib: Optional[ctypes.CDLL] = None
 
 
@@ -90,7 +98,7 @@ def lib() -> ctypes.CDLL:
             h = ctypes.CDLL(LIB_PATH)
         except OSError as e:  # pragma: no cover
             raise Olmo355Unavailable(f"cannot load {LIB_PATH}: {e}") from e
-        for name, (res, args) in EXPORTS.items():
+        for name, (res, args) in {**EXPORTS, **VARIANT_EXPORTS}.items():
             fn = getattr(h, name)
             fn.restype = res
             fn.argtypes = args

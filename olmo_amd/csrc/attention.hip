@@ -956,246 +956,15 @@ extern "C" int olmo355_attn_decode_beam(const void* q, const void* kcache, const
                          bias_stride, beam_src, src_stride, prompt_len, beam, dtype, stream);
 }
 
-
-namespace {
-// ---- decode, one workgroup per (batch, head): no partials, no second kernel ---------------------------
-// 16 waves; wave w takes the 16-key pieces w, w+16, w+32, ... of the cache (balanced for any length
-// without knowing it when the first loads go out), keeps two pieces in flight, carries a running
-// (max, sum, o) and the 16 waves merge once in LDS.  Same front end as attn_decode_fused_kernel.
-// With few (batch, head) pairs only that many CUs pull data (about 150 GB/s each), so this form is
-// chosen when batch * heads is large or the cache is short.
-template <int HD>
-__global__ __launch_bounds__(1024) void attn_decode_onepass_kernel(
-    const uint16_t* __restrict__ qkv, const uint16_t* __restrict__ qw, const uint16_t* __restrict__ kw,
-    const float* __restrict__ sin_t, const float* __restrict__ cos_t, uint16_t* __restrict__ kc,
-    uint16_t* __restrict__ vc, const float* __restrict__ key_bias, uint16_t* __restrict__ out, int H, int Hkv,
-    int Lmax, int n_pos, int past_len, const int32_t* __restrict__ past_dev, int n_keys_max, int bias_stride,
-    float eps) {
-  constexpr int WAVES = 16;
-  constexpr int LPK = HD / 8, KPI = 64 / LPK;  // lanes per key, keys per load instruction
-  constexpr int PIECE = 16, ITERS = PIECE / KPI;  // keys per piece, load instructions per piece
-  constexpr int HALF = HD / 2, CPH = HD / 16;
-  constexpr int QV = 1;  // 16-byte pieces of the q (k) row per thread: (H*HD/8) <= 1024
-  __shared__ float red_o[WAVES][HD];
-  __shared__ float red_ml[WAVES][2];
-  __shared__ float red2[2][WAVES];
-  __shared__ __align__(16) float qs[HD];
-  __shared__ __align__(16) u32x4 knew[HD / 8], vnew[HD / 8];
-  const int h = blockIdx.x, b = blockIdx.y, gsz = H / Hkv, hk = h / gsz;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int sub = lane % LPK, kslot = lane / LPK;
-  const float scale = 1.f / sqrtf((float)HD);
-  const float lowest = -3.3895313892515355e38f;
-  const int64_t cbase = ((int64_t)b * Hkv + hk) * Lmax * HD;
-  const int kmax = min(n_keys_max, Lmax) - 1;
-  const int dq = H * HD, dk = Hkv * HD;
-  const uint16_t* row = qkv + (int64_t)b * (dq + 2 * dk);
-  const bool norm = (qw != nullptr);
-
-  // ---- front end loads first (they return in order and the scores wait on them) ------------------------
-  u32x4 qrow, krow;
-  if (norm) {
-    if (tid < (dq >> 3)) qrow = reinterpret_cast<const u32x4*>(row)[tid];
-    if (tid < (dk >> 3)) krow = reinterpret_cast<const u32x4*>(row + dq)[tid];
-  }
-  const int pos = past_dev ? *past_dev : past_len;
-  const bool role_q = tid < CPH, role_k = tid >= 64 && tid < 64 + CPH, role_v = tid >= 128 && tid < 128 + HD / 8;
-  const int c = role_q ? tid : tid - 64, j = c * 8;
-  u32x4 x1, x2, w1, w2, vrow;
-  if (role_q || role_k) {
-    const uint16_t* src = role_q ? row + h * HD : row + dq + hk * HD;
-    const uint16_t* wsrc = role_q ? qw + h * HD : kw + hk * HD;
-    x1 = reinterpret_cast<const u32x4*>(src + j)[0];
-    x2 = reinterpret_cast<const u32x4*>(src + j + HALF)[0];
-    if (norm) {
-      w1 = reinterpret_cast<const u32x4*>(wsrc + j)[0];
-      w2 = reinterpret_cast<const u32x4*>(wsrc + j + HALF)[0];
-    }
-  }
-  if (role_v) vrow = reinterpret_cast<const u32x4*>(row + dq + dk + hk * HD)[tid - 128];
-
-  // ---- cache pieces: two in flight --------------------------------------------------------------------------
-  u32x4 kreg[2][ITERS], vreg[2][ITERS];
-  float bias[2][ITERS];
-  auto issue = [&](int slot, int piece) {
-#pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-      const int keyc = min(piece * PIECE + it * KPI + kslot, kmax);
-      const int64_t e = (cbase + (int64_t)keyc * HD + sub * 8) >> 3;
-      kreg[slot][it] = reinterpret_cast<const u32x4*>(kc)[e];
-      vreg[slot][it] = reinterpret_cast<const u32x4*>(vc)[e];
-      bias[slot][it] = key_bias ? key_bias[(int64_t)b * bias_stride + keyc] : 0.f;
-    }
-  };
-  const int npieces_max = (kmax + PIECE) / PIECE;
-  if (wave < npieces_max) issue(0, wave);
-  if (wave + WAVES < npieces_max) issue(1, wave + WAVES);
-
-  const int L = pos + 1;
-  if (pos >= Lmax || pos >= n_pos || pos > kmax) return;  // uniform
-  f32x4 cs1[2], cs2[2], sn1[2], sn2[2];
-  if (role_q || role_k) {
-    const float* cp = cos_t + (int64_t)pos * HD;
-    const float* sp = sin_t + (int64_t)pos * HD;
-#pragma unroll
-    for (int v4 = 0; v4 < 2; ++v4) {
-      cs1[v4] = reinterpret_cast<const f32x4*>(cp + j)[v4], cs2[v4] = reinterpret_cast<const f32x4*>(cp + j + HALF)[v4];
-      sn1[v4] = reinterpret_cast<const f32x4*>(sp + j)[v4], sn2[v4] = reinterpret_cast<const f32x4*>(sp + j + HALF)[v4];
-    }
-  }
-  float rq = 1.f, rk = 1.f;
-  if (norm) {
-    float sq = 0.f, sk = 0.f, f[8];
-    if (tid < (dq >> 3)) {
-      Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(qrow), f);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) sq += f[e] * f[e];
-    }
-    if (tid < (dk >> 3)) {
-      Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(krow), f);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) sk += f[e] * f[e];
-    }
-    sq = wave_sum(sq), sk = wave_sum(sk);
-    if (lane == 0) red2[0][wave] = sq, red2[1][wave] = sk;
-    lds_barrier();
-    float tq = 0.f, tk = 0.f;
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) tq += red2[0][w], tk += red2[1][w];
-    rq = 1.f / sqrtf(tq / (float)dq + eps);
-    rk = 1.f / sqrtf(tk / (float)dk + eps);
-  }
-  if (role_q || role_k) {
-    float a1[8], a2[8], ww1[8], ww2[8];
-    Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(x1), a1);
-    Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(x2), a2);
-    if (norm) {
-      Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(w1), ww1);
-      Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(w2), ww2);
-    }
-    const float r = role_q ? rq : rk;
-    float o1[8], o2[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float u1 = a1[e], u2 = a2[e];
-      if (norm) {
-        u1 = round_bf16(ww1[e] * round_bf16(u1 * r));
-        u2 = round_bf16(ww2[e] * round_bf16(u2 * r));
-      }
-      o1[e] = round_bf16(__fadd_rn(__fmul_rn(u1, cs1[e >> 2][e & 3]), __fmul_rn(-u2, sn1[e >> 2][e & 3])));
-      o2[e] = round_bf16(__fadd_rn(__fmul_rn(u2, cs2[e >> 2][e & 3]), __fmul_rn(u1, sn2[e >> 2][e & 3])));
-    }
-    if (role_q) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) qs[j + e] = o1[e], qs[j + HALF + e] = o2[e];
-    } else {
-      u32x4 p1, p2;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) p1[e] = pack_bf16x2(o1[2 * e], o1[2 * e + 1]), p2[e] = pack_bf16x2(o2[2 * e], o2[2 * e + 1]);
-      knew[c] = p1, knew[c + CPH] = p2;
-      if (h % gsz == 0) {
-        const int64_t o = cbase + (int64_t)pos * HD + j;
-        reinterpret_cast<u32x4*>(kc)[o >> 3] = p1;
-        reinterpret_cast<u32x4*>(kc)[(o + HALF) >> 3] = p2;
-      }
-    }
-  }
-  if (role_v) {
-    vnew[tid - 128] = vrow;
-    if (h % gsz == 0) reinterpret_cast<u32x4*>(vc)[(cbase + (int64_t)pos * HD + (tid - 128) * 8) >> 3] = vrow;
-  }
-  lds_barrier();
-  float qr[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) qr[i] = qs[sub * 8 + i];
-
-  // ---- stream the pieces ----------------------------------------------------------------------------------
-  const int npieces = (L + PIECE - 1) / PIECE;
-  float m_run = -INFINITY, l_run = 0.f;  // wave-uniform running max, per-lane partial sum
-  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  auto consume = [&](int slot, int piece) {
-    float sc[ITERS];
-    float pmax = -INFINITY;
-#pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-      const int key = piece * PIECE + it * KPI + kslot;
-      if (key == pos) kreg[slot][it] = knew[sub], vreg[slot][it] = vnew[sub];
-      if (key >= L) vreg[slot][it] = u32x4{0u, 0u, 0u, 0u};  // unwritten rows: 0 * NaN
-      float kf[8];
-      Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(kreg[slot][it]), kf);
-      float d = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) d = __builtin_fmaf(qr[i], kf[i], d);
-      d = group_sum<LPK>(d);
-      float v = bias[slot][it] <= kMaskThreshold ? lowest : d * scale + bias[slot][it];
-      v = key < L ? v : -INFINITY;
-      sc[it] = v;
-      pmax = fmaxf(pmax, v);
-    }
-#pragma unroll
-    for (int o = LPK; o < 64; o <<= 1) pmax = fmaxf(pmax, __shfl_xor(pmax, o, 64));
-    const float mn = fmaxf(m_run, pmax);  // finite: a piece below npieces has at least one key
-    const float alpha = __expf(m_run - mn);
-    l_run *= alpha;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] *= alpha;
-#pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-      const float p = __expf(sc[it] - mn);
-      l_run += p;
-      float vf[8];
-      Vec8<O355_BF16>::unpack(reinterpret_cast<const u32x4(&)[1]>(vreg[slot][it]), vf);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, vf[i], acc[i]);
-    }
-    m_run = mn;
-  };
-  for (int piece = wave; piece < npieces; piece += 2 * WAVES) {
-    consume(0, piece);
-    if (piece + 2 * WAVES < npieces) issue(0, piece + 2 * WAVES);
-    if (piece + WAVES < npieces) {
-      consume(1, piece + WAVES);
-      if (piece + 3 * WAVES < npieces) issue(1, piece + 3 * WAVES);
-    }
-  }
-  // sum over the key slots of the wave (lanes with equal `sub`), then over the waves
-#pragma unroll
-  for (int o = LPK; o < 64; o <<= 1) {
-    l_run += __shfl_xor(l_run, o, 64);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] += __shfl_xor(acc[i], o, 64);
-  }
-  if (lane < LPK) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) red_o[wave][sub * 8 + i] = acc[i];
-  }
-  if (lane == 0) red_ml[wave][0] = m_run, red_ml[wave][1] = l_run;
-  __syncthreads();
-  if (tid < HD) {
-    float mm = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) mm = fmaxf(mm, red_ml[w][0]);
-    float ov = 0.f, lv = 0.f;
-#pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
-      const float f = __expf(red_ml[w][0] - mm);  // waves without a piece: exp(-inf) = 0
-      ov += red_o[w][tid] * f, lv += red_ml[w][1] * f;
-    }
-    out[((int64_t)b * H + h) * HD + tid] = f32_to_bf16_bits(ov / lv);
-  }
-}
-
-int g_dbg_attn_mode = -1;  // test hook (include/olmo355_debug.h); -1 = choose
-}  // namespace
-
-extern "C" void olmo355_debug_set_attn_mode(int mode) { g_dbg_attn_mode = mode; }
-
-extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
-                                         const float* cos_tab, void* kcache, void* vcache, const float* key_bias,
-                                         void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
-                                         int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride,
-                                         float eps, const float* qk_ssq, const float* rope_now, int dtype,
-                                         void* stream) {
+// merge: how the key chunks of a (batch, head) are merged: -1 = choose, 0 = in the kernel (last workgroup of the
+// head, ticket), 2 = the separate combine kernel
+extern "C" int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
+                                               const float* cos_tab, void* kcache, void* vcache, const float* key_bias,
+                                               void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
+                                               int past_len, const int32_t* past_len_dev, int n_keys_max,
+                                               int bias_stride, float eps, const float* qk_ssq, const float* rope_now,
+                                               int dtype, int merge, void* stream) {
+  if (merge != -1 && merge != 0 && merge != 2) return O355_EINVAL;
   if (!qkv || !sin_tab || !cos_tab || !kcache || !vcache || !out || !ws) return O355_EINVAL;
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || past_len < 0 || n_keys_max <= 0 || n_keys_max > Lmax)
     return O355_EINVAL;
@@ -1205,22 +974,6 @@ extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const 
   if (dtype != O355_BF16 || (hd != 128 && hd != 64) || H * hd > 8 * 4 * 256) return O355_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
   const int nch = (n_keys_max + kDecodeChunk - 1) / kDecodeChunk;
-  // one workgroup per (batch, head) is kept as an experiment only: never faster than the chunked form
-  bool onepass = false;
-  if (g_dbg_attn_mode >= 0) onepass = g_dbg_attn_mode == 1 && H * hd <= 8 * 1024;
-  if (onepass) {
-#define ONEPASS(HDv)                                                                                                  \
-  hipLaunchKernelGGL(attn_decode_onepass_kernel<HDv>, dim3(H, B), dim3(1024), 0, s, (const uint16_t*)qkv,            \
-                     (const uint16_t*)qw, (const uint16_t*)kw, sin_tab, cos_tab, (uint16_t*)kcache, (uint16_t*)vcache, \
-                     key_bias, (uint16_t*)out, H, Hkv, Lmax, n_pos, past_len, past_len_dev, n_keys_max, bias_stride, eps)
-    if (hd == 128) {
-      ONEPASS(128);
-    } else {
-      ONEPASS(64);
-    }
-#undef ONEPASS
-    O355_CHECK_LAUNCH();
-  }
 #define FUSED(HDv, QVv)                                                                                                 \
   hipLaunchKernelGGL((attn_decode_fused_kernel<HDv, QVv>), dim3(nch, H, B), dim3(256), 0, s, (const uint16_t*)qkv,   \
                      (const uint16_t*)qw, (const uint16_t*)kw, sin_tab, cos_tab, (uint16_t*)kcache, (uint16_t*)vcache, \
@@ -1234,7 +987,7 @@ extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const 
   // (measured at the 7B shapes, context 2048: the in-kernel merge wins while the launch is a single round of
   // workgroups -- 17.0 against 20.4 us at batch 1 -- and loses once workgroups queue up -- 69.7 against 61.6 us
   // at batch 8, where one workgroup per (batch, head) takes 66.9)
-  const bool merge_in_kernel = g_dbg_attn_mode == 0 || (g_dbg_attn_mode < 0 && (int64_t)B * H * nch <= 1536);
+  const bool merge_in_kernel = merge == 0 || (merge < 0 && (int64_t)B * H * nch <= 1536);
   int* tickets = merge_in_kernel ? reinterpret_cast<int*>(ws) : nullptr;
   ws = reinterpret_cast<float*>(ws) + (int64_t)B * H;
   const int qv = (H * hd / 8 + 255) / 256;
@@ -1245,4 +998,15 @@ extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const 
   }
 #undef FUSED
   O355_CHECK_LAUNCH();
+}
+
+extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
+                                         const float* cos_tab, void* kcache, void* vcache, const float* key_bias,
+                                         void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
+                                         int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride,
+                                         float eps, const float* qk_ssq, const float* rope_now, int dtype,
+                                         void* stream) {
+  return olmo355_attn_decode_fused_merge(qkv, qw, kw, sin_tab, cos_tab, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd,
+                                         Lmax, n_pos, past_len, past_len_dev, n_keys_max, bias_stride, eps, qk_ssq,
+                                         rope_now, dtype, -1, stream);
 }

@@ -24,9 +24,10 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 static inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
-// int4 linear for 17..64 rows (gemv_mid.hip); arguments as olmo355_w4_gemv, already validated
+// int4 linear for 17..64 rows (gemv_mid.hip); arguments as olmo355_w4_gemv, already validated;
+// pairs = column-tile pairs per workgroup (0 = choose)
 int o355_w4_mid_dispatch(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
-                         int M, int N, int K, void* stream);
+                         int M, int N, int K, int pairs, void* stream);
 
 // ---- scalar conversions -------------------------------------------------------------------
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }

@@ -1,18 +1,17 @@
 // Large-M linear layers (prefill): y[M,N] = x[M,K] . W[K,N] on the matrix cores
 // (v_mfma_f32_32x32x16_bf16), fp32 accumulation, bf16 output.
 //
-// Workgroup = 4 waves in a 2x2 arrangement over a BM x BN output tile (up to 256 x 256, one wave
-// per SIMD: a single wave sustains the 8-pass 32x32x16 MFMA back to back, which it does not for
-// the 4-pass 16x16x32), K advanced 64 at a time.  Both operands are staged in LDS in
-// *fragment-major* order -- [32-row tile][k-step of 16][64 lanes][16 bytes] -- so every MFMA operand
-// is one conflict-free ds_read_b128 and each 16-byte piece fetched from memory lands in exactly one
-// LDS slot.  The activation pieces are written with an XOR swizzle of the slot (the 16 lanes of one
-// LDS write cycle hold 2 rows x 8 column chunks, which would otherwise share two bank groups).
-// LDS is double-buffered: while the matrix cores work on stage s the same waves write stage s+1
-// (for int4 weights: unpack the tiled words, apply scale and zero in fp32, round to bf16) and fetch
-// stage s+2 from memory into registers; the staging work is spread between the k-steps of the MFMA
-// loop so that the VALU / LDS / memory instructions issue in the shadow of the matrix pipeline; one
-// barrier per stage.
+// Workgroup = 8 waves (two per SIMD) in a 2x4 or 4x2 arrangement over a BM x BN output tile: 256 rows by
+// 256, 192 or 128 columns, or 128 rows by 128 or 64 columns; each wave owns WMT x WNT MFMA tiles of
+// 32 x 32.  K advances 64 per stage.  Activations go memory -> LDS directly (8 rows x 128 bytes per
+// instruction, the 16-byte chunks of a row XOR-swizzled so the operand reads are conflict-free), ring of
+// three stages requested two stages ahead.  Weights are staged in LDS in *fragment-major* order
+// -- [32-column tile][k-step of 16][64 lanes][16 bytes] -- so every MFMA operand is one conflict-free
+// ds_read_b128; int4 words come into registers two stages ahead and are dequantised (scale and zero
+// in fp32, one rounding to bf16) into LDS one stage ahead, double-buffered; dense weights are copied
+// memory -> LDS as they are tiled.  The staging work is spread between the k-steps of the MFMA loop so
+// that the VALU / LDS / memory instructions issue in the shadow of the matrix pipeline; one barrier per
+// stage.
 //
 // The int4 operand is W = bf16(scale * (q - zero)) (fp32 product, one rounding).
 #include "common.h"
@@ -419,8 +418,6 @@ int launch_splitk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, con
   return launch_splitk_shape<4, 2, W4>(x, wt, st, zt, y, M, N, K, splits, part, stream);
 }
 
-int g_force_tile = 0;  // debug: 0 = choose, else 1000 * rows + columns of the tile (rows 0 = 256)
-
 // Tiles are 256 rows by 256, 192 or 128 columns, or 128 rows by 128 or 64 columns.  A launch runs in
 // rounds of one tile per CU (two for the smallest tile, whose LDS fits twice), and the time of a round
 // is far from proportional to the tile's area: a K-stage costs about 0.5 us of latency however small
@@ -428,7 +425,7 @@ int g_force_tile = 0;  // debug: 0 = choose, else 1000 * rows + columns of the t
 // are what matters); the shape with the smallest rounds x time wins.
 template <bool W4>
 int dispatch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M,
-                  int N, int K, hipStream_t stream) {
+                  int N, int K, hipStream_t stream, int force_tile = 0) {  // force_tile: 1000 * rows + columns, 0 = choose
   const int cus = 256;
   struct Shape { int bm, bn, per_cu; double round_us; };
   static const Shape shapes[] = {{256, 256, 1, 95.}, {256, 192, 1, 80.}, {256, 128, 1, 55.}, {128, 128, 1, 37.}, {128, 64, 2, 47.}};
@@ -441,7 +438,7 @@ int dispatch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, con
     if (sh.per_cu == 2 && tiles <= cus) ci = 32.;  // one tile per CU: no sharing of the CU
     if (ci < c) c = ci, best = 1000 * sh.bm + sh.bn;
   }
-  if (g_force_tile) best = g_force_tile < 1000 ? 256000 + g_force_tile : g_force_tile;
+  if (force_tile) best = force_tile < 1000 ? 256000 + force_tile : force_tile;
   switch (best) {
     case 256256: return launch_gemm<2, 4, 4, 2, W4>(x, wt, st, zt, y, M, N, K, stream);
     case 256192: return launch_gemm<4, 2, 2, 3, W4>(x, wt, st, zt, y, M, N, K, stream);
@@ -454,7 +451,20 @@ int dispatch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, con
 
 }  // namespace
 
-extern "C" void olmo355_debug_set_gemm_tile(int width) { g_force_tile = width; }
+extern "C" int olmo355_w4_gemm_tile(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
+                                    uint16_t* y, int M, int N, int K, int tile, void* stream) {
+  if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0 || tile < 0) return O355_EINVAL;
+  if ((K & 127) || (N & 15)) return O355_EUNSUPPORTED;
+  return dispatch_gemm<true>(x, wt, st, zt, y, M, N, K, as_stream(stream), tile);
+}
+
+extern "C" int olmo355_b16_gemm_tile(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, int tile,
+                                     void* stream) {
+  if (!x || !wt || !y || M <= 0 || N <= 0 || K <= 0 || tile < 0) return O355_EINVAL;
+  if ((K & 63) || (N & 15)) return O355_EUNSUPPORTED;
+  return dispatch_gemm<false>(x, reinterpret_cast<const uint32_t*>(wt), nullptr, nullptr, y, M, N, K, as_stream(stream),
+                              tile);
+}
 
 extern "C" int olmo355_w4_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
                                uint16_t* y, int M, int N, int K, void* stream) {

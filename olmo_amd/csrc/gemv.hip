@@ -929,8 +929,8 @@ struct GemvPlan {
   int pro, epi;
 };
 
-// Experiment hook (not part of the public interface): overrides waves / xlds when >= 0.
-int g_dbg_waves = -1, g_dbg_xlds = -1, g_dbg_small = 1;
+// Which kernel family a plain product goes to (olmo355_w4_gemv_form; 0 for every other entry point)
+enum GemvForm { kFormChoose = 0, kFormLean = 1, kFormMid = 2, kFormMid1 = 3, kFormMid2 = 4, kFormOlder = 5 };
 
 constexpr int kXldsMaxBytes = 64 * 1024;     // activations (+ zero row) in LDS, kernels for M <= 16
 constexpr int kSmallMaxBytes = 128 * 1024;   // the same for the lean M <= 4 kernel (160 KiB of LDS per CU)
@@ -956,8 +956,6 @@ inline GemvPlan plan_gemv(int M, int N, int K, bool w4, bool pro, bool epi) {
   }
   p.waves = waves;
   p.xlds = p.mt == 1 && (int64_t)(M + 1) * K * 2 <= kXldsMaxBytes;
-  if (g_dbg_waves >= 0 && !pro && !epi) p.waves = g_dbg_waves;
-  if (g_dbg_xlds >= 0 && !pro && !epi) p.xlds = g_dbg_xlds && p.xlds;
   return p;
 }
 
@@ -1038,18 +1036,20 @@ int launch_small(Kern kern, const GemvPlan& p, const GemvArgs& a, hipStream_t st
   ROT_WAVES(GPAv, 2, 1, 1) ROT_WAVES(GPAv, 2, 4, 1)
 
 int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, bool pro, bool epi,
-                     void* stream) {
+                     void* stream, int form = kFormChoose) {
   GemvPlan p = plan_gemv(a.M, a.N, a.K, true, pro, epi);
   const u32x4* w = (const u32x4*)wt;
   const int sgpa = a.M <= 4 ? 4 : (a.M <= 8 ? 2 : 1);
-  const bool small_ok = a.M <= 16 && (a.M <= 4 || p.pro == 0) && (int64_t)(a.M + 1) * a.K * 2 <= kSmallMaxBytes && (int64_t)(a.N >> 4) * (a.K >> 7) * 1024 < (1ll << 31) && g_dbg_small;
+  const bool small_ok = a.M <= 16 && (a.M <= 4 || p.pro == 0) && (int64_t)(a.M + 1) * a.K * 2 <= kSmallMaxBytes && (int64_t)(a.N >> 4) * (a.K >> 7) * 1024 < (1ll << 31) && form != kFormOlder;
   // Plain products with many columns: from 9 rows (5 for wide outputs) the staged-activation kernel
   // wins over the kernels below, which keep all rows of x in LDS per workgroup (measured).
   const bool plain = !pro && !epi && !a.ssq_in && !a.ssq_out;
   const bool mid_wins = a.M > 16 || (a.M > 8 && a.N >= 8192) || (a.M > 4 && a.N >= 12288);
-  if (plain && g_dbg_small && (mid_wins || g_dbg_small == 2)) {
-    const int st_mid = o355_w4_mid_dispatch(a.x, wt, st, zt, a.y, a.M, a.N, a.K, stream);
-    if (st_mid != O355_EUNSUPPORTED) return st_mid;  // else: sizes beyond its 32-bit offsets
+  const bool force_mid = form == kFormMid || form == kFormMid1 || form == kFormMid2;
+  if (plain && ((mid_wins && form == kFormChoose) || force_mid)) {
+    const int pairs = form == kFormMid1 ? 1 : (form == kFormMid2 ? 2 : 0);
+    const int st_mid = o355_w4_mid_dispatch(a.x, wt, st, zt, a.y, a.M, a.N, a.K, pairs, stream);
+    if (st_mid != O355_EUNSUPPORTED || force_mid) return st_mid;  // else: sizes beyond its 32-bit offsets
   }
   if (a.ssq_in || a.ssq_out) {  // chained norms: only the lean kernel speaks that protocol
     if (!small_ok || a.M > 4 || (a.ssq_out && epi)) return O355_EUNSUPPORTED;
@@ -1096,8 +1096,13 @@ int b16_gemv_dispatch(const GemvArgs& a, const uint16_t* wt, bool pro, bool epi,
 
 }  // namespace
 
-extern "C" void olmo355_debug_set_gemv_plan(int waves, int xlds) { g_dbg_waves = waves, g_dbg_xlds = xlds; }
-extern "C" void olmo355_debug_set_gemv_small(int on) { g_dbg_small = on; }
+extern "C" int olmo355_w4_gemv_form(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
+                                    uint16_t* y, int M, int N, int K, int form, void* stream) {
+  if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0 || form < kFormChoose || form > kFormOlder) return O355_EINVAL;
+  if (M > 64 || (K & 127) || (N & 15)) return O355_EUNSUPPORTED;
+  const GemvArgs a{x, nullptr, nullptr, nullptr, y, 0.f, M, N, K};
+  return w4_gemv_dispatch(a, wt, st, zt, false, false, stream, form);
+}
 
 extern "C" int olmo355_w4_gemv(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
                                uint16_t* y, int M, int N, int K, void* stream) {

@@ -213,22 +213,19 @@ int launch_mid(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const 
   O355_CHECK_LAUNCH();
 }
 
-int g_dbg_np = 0;  // test hook (include/olmo355_debug.h): 0 = choose, 1 / 2 = column-tile pairs per workgroup
-
 }  // namespace
 
-extern "C" void olmo355_debug_set_mid_pairs(int np) { g_dbg_np = np; }
-
 // 1..64 rows; the caller has checked pointers and that K is a multiple of 128 and N of 16.
+// pairs: column-tile pairs per workgroup, 0 = choose, 1 or 2.
 int o355_w4_mid_dispatch(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
-                         int M, int N, int K, void* stream) {
+                         int M, int N, int K, int pairs, void* stream) {
   if (M < 1 || M > 64 || (int64_t)M * K * 2 >= (1ll << 31) || (int64_t)(N >> 4) * (K >> 7) * 1024 >= (1ll << 31))
     return O355_EUNSUPPORTED;  // 32-bit buffer offsets
   hipStream_t s = as_stream(stream);
   const int quads = ((N >> 4) + 3) / 4;  // workgroups with four column tiles each
   const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
   int np = quads >= (mt == 1 ? 512 : 128) ? 2 : 1;
-  if (g_dbg_np) np = g_dbg_np;
+  if (pairs == 1 || pairs == 2) np = pairs;
   if (mt == 1) return np == 2 ? launch_mid<1, 2, 4>(x, wt, st, zt, y, M, N, K, s) : launch_mid<1, 1, 4>(x, wt, st, zt, y, M, N, K, s);
   if (mt == 2) return np == 2 ? launch_mid<2, 2, 4>(x, wt, st, zt, y, M, N, K, s) : launch_mid<2, 1, 4>(x, wt, st, zt, y, M, N, K, s);
   return np == 2 ? launch_mid<4, 2, 4>(x, wt, st, zt, y, M, N, K, s) : launch_mid<4, 1, 4>(x, wt, st, zt, y, M, N, K, s);

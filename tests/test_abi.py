@@ -22,17 +22,29 @@ def test_header_symbols_are_exported_and_bound():
     assert b"unsupported" in h.olmo355_status_string(2)
 
 
-def test_debug_header_symbols_are_exported():
-    import ctypes
-
+def test_variant_header_symbols_are_exported_and_bound():
     from olmo_amd import _lib
 
     hdr = open(os.path.join(ROOT, "include", "olmo355_debug.h")).read()
-    declared = set(re.findall(r"\b(olmo355_debug_\w+)\s*\(", hdr))
-    assert len(declared) == 5
-    h = ctypes.CDLL(_lib.LIB_PATH)
+    declared = set(re.findall(r"\b(olmo355_\w+)\s*\(", hdr))
+    assert declared == set(_lib.VARIANT_EXPORTS), (declared ^ set(_lib.VARIANT_EXPORTS))
+    h = _lib.lib()
     for name in declared:
         assert getattr(h, name) is not None
+    # the choice is an argument, not state: a bad value is refused before anything is launched
+    assert h.olmo355_w4_gemv_form(None, None, None, None, None, 1, 16, 128, 9, None) == 1
+
+
+def test_library_exports_no_state_setters():
+    """The drop-in library promises no process-global state: nothing named *_set_* or *debug* is exported."""
+    import subprocess
+
+    from olmo_amd import _lib
+
+    out = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    names = [ln.split()[-1] for ln in out.splitlines() if " T " in ln and "olmo355_" in ln]
+    assert names and not [n for n in names if "_set_" in n or "debug" in n]
+    assert set(names) == set(_lib.EXPORTS) | set(_lib.VARIANT_EXPORTS)
 
 
 def test_argument_checks_return_status_without_launching():

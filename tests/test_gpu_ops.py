@@ -174,12 +174,6 @@ def test_b16_linear(dev, M, N, K):
     assert torch.allclose(y, ref, rtol=2 ** -8, atol=2 ** -8 * ref.abs().max().item())
 
 
-def _force_gemm_tile(width):
-    # test-only hook of the library (not part of the declared interface): 0 = choose by shape
-    from olmo_amd import _lib
-    _lib.lib().olmo355_debug_set_gemm_tile(int(width))
-
-
 @pytest.mark.parametrize("width", [256, 192, 128, 128128, 128064])
 @pytest.mark.parametrize("M,N,K", [(65, 208, 128), (300, 1008, 384), (513, 400, 1408), (256, 768, 256), (1, 16, 640)])
 def test_w4_gemm_every_tile_width(dev, width, M, N, K):
@@ -194,13 +188,9 @@ def test_w4_gemm_every_tile_width(dev, width, M, N, K):
     y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     xd = x.to(dev)
     from olmo_amd import _lib
-    _force_gemm_tile(width)
-    try:
-        st = _lib.lib().olmo355_w4_gemm(xd.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y.data_ptr(),
-                                        M, N, K, torch.cuda.current_stream().cuda_stream)
-        torch.cuda.synchronize()
-    finally:
-        _force_gemm_tile(0)
+    st = _lib.lib().olmo355_w4_gemm_tile(xd.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y.data_ptr(),
+                                         M, N, K, width, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
     assert st == 0
     scale = ref.abs().max().item()
     assert (y.float().cpu() - ref).abs().max().item() <= 2 ** -7 * scale
@@ -220,13 +210,9 @@ def test_b16_gemm_every_tile_width(dev, width, M, N, K):
     y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     xd = x.to(dev)
     from olmo_amd import _lib
-    _force_gemm_tile(width)
-    try:
-        st = _lib.lib().olmo355_b16_gemm(xd.data_ptr(), t.wt.data_ptr(), y.data_ptr(), M, N, K,
-                                         torch.cuda.current_stream().cuda_stream)
-        torch.cuda.synchronize()
-    finally:
-        _force_gemm_tile(0)
+    st = _lib.lib().olmo355_b16_gemm_tile(xd.data_ptr(), t.wt.data_ptr(), y.data_ptr(), M, N, K, width,
+                                          torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
     assert st == 0
     assert torch.allclose(y.float().cpu(), ref, rtol=2 ** -8, atol=2 ** -8 * ref.abs().max().item())
 
