@@ -22,7 +22,13 @@ Pinned by (tests/test_oracle_model.py): ``F.layer_norm`` for LayerNorm, an fp64 
 with explicit rounding for RMSNorm, closed-form and relative-position invariants for RoPE,
 ``F.scaled_dot_product_attention(is_causal=True)`` and a brute-force softmax for attention,
 and the reference's own forward invariants (cache == no cache, padded batch == single:
-``tests/model_test.py:188-199``).  No stored golden logits exist in the reference.
+``tests/model_test.py:188-199``).  No stored golden logits exist in the reference, so the *composition*
+(``_block`` / ``_attention`` / ``forward``: norm placement, full-width QK-norm, q | k | v and up | gate split
+orders, cache path, padding bias) is pinned by tests/test_oracle_composition.py against logits of
+``transformers``' own ``Olmo2ForCausalLM`` (MHA, GQA) and ``OlmoForCausalLM`` (with and without ``clip_qkv``)
+on seeded weights mapped the way ``scripts/convert_olmo2_to_hf.py:110-163`` maps them (fixture
+tests/golden/hf_olmo2_kat.npz), with negative cases for swapped up / gate, swapped block norms and per-head
+QK-norm.
 """
 
 from __future__ import annotations

@@ -420,6 +420,49 @@ def test_unsharded_checkpoint_and_hf_layout(dev, tmp_path):
     assert torch.equal(m3.post_init()(ids).logits, ref)
 
 
+@pytest.mark.parametrize("name", ["olmo2_mha", "olmo2_gqa", "olmo1", "olmo1_clip"])
+def test_hf_transformers_fixture(dev, name):
+    """Logits of ``transformers``' own Olmo2ForCausalLM / OlmoForCausalLM (stored by
+    tests/golden/make_hf_olmo2_kat.py; an implementation independent of this repository) against the HIP path on
+    the same seeded weights, loaded through ``hf_olmo2_to_olmo_state_dict`` -> ``load_reference_state_dict``:
+    fp32, logits within 2e-4; plain, left-padded, and prefill 16 + 8 cached single-token steps.  The layout
+    conversion (scripts/convert_olmo2_to_hf.py:110-163) is thereby checked against that model, not against its
+    own inverse."""
+    say("hf fixture", name)
+    import os
+
+    import numpy as np
+
+    from olmo_amd.model import OLMo
+    from tests.golden import hf_kat_recipe as R
+
+    kat = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "hf_olmo2_kat.npz"), allow_pickle=False)
+    case, seed = R.CASES[name], R.seed_of(name)
+    cfg = R.model_config(case)
+    w = R.to_olmo_state_dict(case, R.hf_state_dict(case, seed))
+    ids, mask = R.inputs(case, seed)
+    model = OLMo(cfg, device=dev, dtype=torch.float32)
+    model.load_reference_state_dict(w)
+    model.post_init()
+    ref = torch.from_numpy(kat[name + ".logits"])
+    got = model(ids.to(dev)).logits.cpu()
+    err = (got - ref).abs().max().item()
+    say("  plain max-abs logit error", err)
+    assert err <= 2e-4
+    refp = torch.from_numpy(kat[name + ".logits_left_padded"])
+    gotp = model(ids.to(dev), attention_mask=mask.to(dev)).logits.cpu()
+    errp = (gotp - refp).abs()[mask.bool()].max().item()
+    say("  left-padded max-abs logit error (real tokens)", errp)
+    assert errp <= 2e-4
+    out = model(ids[:, :16].to(dev), use_cache=True)
+    assert (out.logits.cpu() - ref[:, :16]).abs().max().item() <= 2e-4
+    kv = out.attn_key_values
+    for t in range(16, R.SEQ):
+        out = model(ids[:, t:t + 1].to(dev), past_key_values=kv, use_cache=True)
+        kv = out.attn_key_values
+        assert (out.logits[:, 0].cpu() - ref[:, t]).abs().max().item() <= 2e-4
+
+
 def test_sampled_generation(dev):
     """Sampling inside the decode step: the captured graph draws the same tokens as eager launches (the random
     number is a function of seed and device-side position), a seed reproduces, and top_k=1 is greedy."""
