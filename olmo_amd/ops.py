@@ -545,9 +545,10 @@ def attn_decode(q, kcache, vcache, ws, B: int, H: int, Hkv: int, hd: int, past_l
 def attn_decode_fused(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, ws, B: int, H: int, Hkv: int, hd: int,
                       past_len: int, n_keys_max: int, eps: float, key_bias: Optional[torch.Tensor] = None,
                       past_len_dev: Optional[torch.Tensor] = None, qk_ssq: Optional[torch.Tensor] = None,
-                      rope_now: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+                      rope_now: Optional[torch.Tensor] = None, merge: int = -1) -> Optional[torch.Tensor]:
     """One new token per sequence: QK-norm, rotary, cache append and attention in one pass.  Returns
-    ``None`` when the fused kernel does not cover the shape (use the separate calls then)."""
+    ``None`` when the fused kernel does not cover the shape (use the separate calls then).  ``merge`` other than
+    -1 names how a head's key chunks are merged (the variant entry point: 0 in the kernel, 2 separate kernel)."""
     _dev(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, ws, key_bias, past_len_dev, qk_ssq, rope_now)
     if rope_now is not None and (rope_now.dtype != torch.float32 or rope_now.numel() != 2 * hd):
         raise ValueError("rope_now: float32 [2 * hd] expected")
@@ -562,10 +563,13 @@ def attn_decode_fused(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache,
     if ws.numel() * ws.element_size() < need:
         raise ValueError("attention workspace too small")
     out = torch.empty(B, 1, H * hd, dtype=qkv.dtype, device=qkv.device)
-    st = lib().olmo355_attn_decode_fused(_p(qkv), _p(q_weight), _p(k_weight), _p(sin_tab), _p(cos_tab), _p(kcache),
-                                         _p(vcache), _p(key_bias), _p(out), _p(ws), B, H, Hkv, hd, Lmax, n_pos, past_len,
-                                         _p(past_len_dev), n_keys_max, key_bias.shape[1] if key_bias is not None else 0,
-                                         float(eps), _p(qk_ssq), _p(rope_now), _dt(qkv), _stream())
+    args = (_p(qkv), _p(q_weight), _p(k_weight), _p(sin_tab), _p(cos_tab), _p(kcache), _p(vcache), _p(key_bias), _p(out),
+            _p(ws), B, H, Hkv, hd, Lmax, n_pos, past_len, _p(past_len_dev), n_keys_max,
+            key_bias.shape[1] if key_bias is not None else 0, float(eps), _p(qk_ssq), _p(rope_now), _dt(qkv))
+    if merge == -1:
+        st = lib().olmo355_attn_decode_fused(*args, _stream())
+    else:
+        st = lib().olmo355_attn_decode_fused_merge(*args, int(merge), _stream())
     if st == 2:
         return None
     check("olmo355_attn_decode_fused", st)

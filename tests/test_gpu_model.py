@@ -463,6 +463,65 @@ def test_hf_transformers_fixture(dev, name):
         assert (out.logits[:, 0].cpu() - ref[:, t]).abs().max().item() <= 2e-4
 
 
+def test_13b_decode_at_its_workload_shape(dev):
+    """BASELINE's fourth configuration at its real shape: OLMo-2 13B int4-g128 at full depth (40 layers), 16
+    sequences, KV context 4090 (random weights; the prompt is prefilled in four batches of 4 x 4090 rows, the
+    4 x 4096 prefill shape).  Size-independent properties, no oracle at this size: (1) a decode step over the
+    cache gives the last row of a full causal forward of the same tokens (reference tests/model_test.py:196-199)
+    -- different kernels on the two sides: the staged-activation / lean int4 kernels and the chunked decode
+    attention with its separate combine kernel (16 x 40 x 33 workgroups) against the MFMA GEMM and the prefill
+    attention; (2) the captured-graph loop reproduces the eager loop bit for bit."""
+    say("13b decode at batch 16, context 4090")
+    from olmo_amd.generate import DecodeSession
+    from olmo_amd import ops
+    from olmo_amd.synthetic import build_random_model
+
+    cfg = PRESETS["olmo2-13b"]
+    B, ctx, steps = 16, 4090, 3
+    model = build_random_model(cfg, torch.bfloat16, quantized=True, seed=3, device=dev, max_cache_len=ctx + 8,
+                               free_checkpoint_buffers=True)
+    gen = torch.Generator().manual_seed(11)
+    ids = torch.randint(0, cfg.vocab_size, (B, ctx), generator=gen).to(dev)
+    cache = model.new_cache(B, ctx + 8)
+    first = torch.empty(B, dtype=torch.int64, device=dev)
+    for b0 in range(0, B, 4):  # prefill 4 x 4090 at a time into rows b0 .. b0+3 of the shared cache
+        out = model(ids[b0:b0 + 4], use_cache=True, last_logits_only=True)
+        sub = out.attn_key_values[0].cache
+        for i in range(cfg.n_layers):
+            cache.k[i][b0:b0 + 4, :, :ctx] = sub.k[i][:, :, :ctx]
+            cache.v[i][b0:b0 + 4, :, :ctx] = sub.v[i][:, :, :ctx]
+        first[b0:b0 + 4] = ops.argmax(out.logits.view(4, -1))
+        del out, sub
+    cache.set_length(ctx)
+
+    def run(use_graph):
+        cache.set_length(ctx)
+        sess = DecodeSession(model, cache, first.clone(), None)
+        toks, logits = [first.clone()], []
+        for i in range(steps):
+            if use_graph and i == 2:
+                sess.capture()
+            sess.step()
+            toks.append(sess.ids.view(B).clone())
+            logits.append(sess.logits.view(B, -1).clone())
+        return torch.stack(toks, 1), logits
+
+    toks_e, logits_e = run(False)
+    toks_g, logits_g = run(True)
+    assert torch.equal(toks_e, toks_g)
+    for a, b in zip(logits_e, logits_g):
+        assert torch.equal(a, b), "graph replay differs from eager decode"
+    # (1) step k fed token k-1 at position ctx+k-1: its logits are the last row of a full forward over ctx+k tokens
+    for k in (1, 2):
+        full = torch.cat((ids, toks_e[:, :k]), dim=1)
+        worst = 0.0
+        for b0 in range(0, B, 4):
+            ref = model(full[b0:b0 + 4], last_logits_only=True).logits.view(4, -1)
+            worst = max(worst, softmax_err(logits_e[k - 1][b0:b0 + 4], ref))
+        say(f"  step {k}: softmax max-abs difference cache vs full forward {worst:.2e}")
+        assert worst <= 2e-2
+
+
 def test_sampled_generation(dev):
     """Sampling inside the decode step: the captured graph draws the same tokens as eager launches (the random
     number is a function of seed and device-side position), a seed reproduces, and top_k=1 is greedy."""

@@ -159,6 +159,73 @@ def test_w4_gemm(dev, M, N, K):
     assert err <= 2 ** -7 * scale, (err, scale)
 
 
+def _w4_big_case(dev, N, K, Ms, seed):
+    """The int4 linear at full layer sizes.  The oracle product is evaluated on column bands (all columns unless N is
+    the vocabulary-sized one: first, middle and last 4096) and, above 64 rows, on a sample of rows (first and last
+    tile rows and 24 random ones); at the largest M the whole output is additionally checked through a property
+    that needs no oracle: permuting the rows of x permutes the rows of y bit for bit."""
+    ops = _ops()
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=seed)
+    t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    bands = [(0, N)] if N <= 30000 else [(0, 4096), (N // 2 - 2048, N // 2 + 2048), (N - 4096, N)]
+    Wb = [ow4.dequantize(qw[:, lo:hi].contiguous(), qz[:, lo // 8: hi // 8].contiguous(), sc[:, lo:hi].contiguous(), 128).float()
+          for lo, hi in bands]
+    for M in Ms:
+        say("  M", M)
+        g = torch.Generator().manual_seed(seed + M)
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        y = ops.w4_linear(x.to(dev), t)
+        rows = torch.arange(M) if M <= 64 else torch.unique(torch.cat([
+            torch.arange(0, 8), torch.arange(M - 8, M), torch.randint(0, M, (24,), generator=g)]))
+        ysel = y[rows.to(dev)].float().cpu()
+        for (lo, hi), W in zip(bands, Wb):
+            ref = x[rows].float() @ W
+            scale = ref.abs().max().item()
+            err = (ysel[:, lo:hi] - ref).abs().max().item()
+            assert err <= 2 ** -7 * scale, (M, lo, hi, err, scale)
+        if M == max(Ms) and M > 64:
+            perm = torch.randperm(M, generator=g)
+            y2 = ops.w4_linear(x[perm].contiguous().to(dev), t)
+            assert torch.equal(y2, y[perm.to(dev)])
+
+
+@pytest.mark.parametrize("N,K", [(4096, 4096), (11008, 4096), (4096, 11008), (13824, 5120), (100352, 4096)])
+def test_w4_linear_isolated_sweep_shapes(dev, N, K):
+    """Every cell of the isolated sweep (`bench.py --sweep`): M in {1, 8, 64, 512, 4096} on its five (N, K)."""
+    say("w4_linear sweep shape", N, K)
+    _w4_big_case(dev, N, K, (1, 8, 64, 512, 4096), seed=N + K)
+
+
+@pytest.mark.parametrize("N,K", [(15360, 5120), (5120, 5120), (27648, 5120), (5120, 13824)])
+def test_w4_linear_13b_decode_rows(dev, N, K):
+    """The four block Linears of the 13B shape at the 16 rows of its decode batch (and at 4 prefill-sized rows
+    counts of the same shapes)."""
+    say("w4_linear 13b", N, K)
+    _w4_big_case(dev, N, K, (16, 4096), seed=N + K + 1)
+
+
+@pytest.mark.parametrize("form", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("M,N,K", [(1, 1024, 512), (4, 4096, 4096), (9, 8208, 640), (16, 272, 1408), (40, 2064, 896), (64, 4096, 1024)])
+def test_w4_gemv_every_kernel_family(dev, form, M, N, K):
+    """Each kernel family the small-M dispatcher chooses between (lean / staged-activation with one or two
+    column-tile pairs / the older kernels), forced on shapes it would not have been given, against the oracle."""
+    say("w4_gemv form", form, M, N, K)
+    ops = _ops()
+    from olmo_amd import _lib
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=M + N + K)
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16)
+    ref = ow4.linear_fp32(x, ow4.dequantize(qw, qz, sc, 128))
+    t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    xd = x.to(dev)
+    y = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    st = _lib.lib().olmo355_w4_gemv_form(xd.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y.data_ptr(),
+                                         M, N, K, form, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert st == 0
+    scale = ref.abs().max().item()
+    assert (y.float().cpu() - ref).abs().max().item() <= 2 ** -7 * scale
+
+
 @pytest.mark.parametrize("M", [1, 8, 40, 64, 65, 300, 1024])
 @pytest.mark.parametrize("N,K", [(256, 256), (2048, 2048), (1008, 1408)])
 def test_b16_linear(dev, M, N, K):
@@ -532,7 +599,10 @@ def test_linear_fused(dev, quant, M, N, K, pro, epi):
 
 @pytest.mark.parametrize("qknorm,B,past,H,Hkv,hd", [(True, 1, 2048, 32, 32, 128), (True, 3, 700, 4, 2, 128),
                                                      (False, 2, 0, 2, 2, 64), (True, 2, 127, 8, 8, 64),
-                                                     (True, 2, 128, 4, 4, 128)])
+                                                     (True, 2, 128, 4, 4, 128),
+                                                     # more than 1536 workgroups: partials + the separate combine
+                                                     # kernel (batch 8 at context 2048 of the 7B shape; 13B heads at 4090)
+                                                     (True, 8, 2048, 32, 32, 128), (True, 3, 4090, 40, 40, 128)])
 def test_attn_decode_fused(dev, qknorm, B, past, H, Hkv, hd):
     """QK-norm + rotary + cache append + attention in one pass == the two separate kernels == the oracle."""
     say("attn_decode_fused", qknorm, B, past, H, Hkv, hd)
@@ -595,6 +665,43 @@ def test_attn_decode_fused(dev, qknorm, B, past, H, Hkv, hd):
                                      qk_ssq=ssq.to(dev))
         assert torch.allclose(out4.float(), out.float(), rtol=2 ** -7, atol=2 ** -7)
         assert torch.allclose(kc4[:, :, past].float(), kc[:, :, past].float(), rtol=2 ** -7, atol=2 ** -7)
+
+
+@pytest.mark.parametrize("merge", [0, 2])
+@pytest.mark.parametrize("B,past,H,Hkv,hd", [(2, 300, 4, 2, 128), (8, 2048, 32, 32, 128), (1, 1000, 8, 8, 64)])
+def test_attn_decode_fused_both_merges(dev, merge, B, past, H, Hkv, hd):
+    """Both ways of merging a head's key chunks (in the kernel by the last workgroup; partials + combine kernel),
+    each forced on a launch the dispatcher would give to the other, against the oracle."""
+    say("attn_decode_fused merge", merge, B, past, H, Hkv, hd)
+    ops = _ops()
+    dtype, theta, eps = torch.bfloat16, 500000.0, 1e-6
+    Lmax = past + 120
+    gen = torch.Generator().manual_seed(past + hd + H + merge)
+    qkv = torch.randn(B, (H + 2 * Hkv) * hd, generator=gen).to(dtype)
+    qw = (1 + 0.1 * torch.randn(H * hd, generator=gen)).to(dtype)
+    kw = (1 + 0.1 * torch.randn(Hkv * hd, generator=gen)).to(dtype)
+    k_old = torch.randn(B, Hkv, past, hd, generator=gen).to(dtype)
+    v_old = torch.randn(B, Hkv, past, hd, generator=gen).to(dtype)
+    qr, kr, vr = _rope_ref(qkv, qw, kw, B, 1, H, Hkv, hd, past, theta, eps, Lmax)
+    ref = om.attention(qr, torch.cat((k_old, kr), 2), torch.cat((v_old, vr), 2), None, dtype)
+    ref = ref.transpose(1, 2).reshape(B, 1, H * hd)
+    sin, cos = ops.rope_tables(hd, theta, Lmax, dev)
+    kc = torch.full((B, Hkv, Lmax, hd), float("nan"), dtype=dtype)
+    vc = torch.full((B, Hkv, Lmax, hd), float("nan"), dtype=dtype)
+    kc[:, :, :past], vc[:, :, :past] = k_old, v_old
+    kc, vc = kc.to(dev), vc.to(dev)
+    ws = ops.attn_decode_workspace(B, H, hd, Lmax, dev)
+    pl = torch.tensor([past], dtype=torch.int32, device=dev)
+    # twice on the same workspace: the ticket counters must be back at zero after a launch
+    for rep in range(2):
+        out = ops.attn_decode_fused(qkv.to(dev), qw.to(dev), kw.to(dev), sin, cos, kc, vc, ws, B, H, Hkv, hd, 0, Lmax, eps,
+                                    past_len_dev=pl, merge=merge)
+        assert out is not None
+        assert torch.allclose(out.cpu().float(), ref.float(), rtol=2 ** -7, atol=2 ** -7), rep
+    # and the dispatcher's own choice agrees with the forced one up to the order of the fp32 merge
+    out_auto = ops.attn_decode_fused(qkv.to(dev), qw.to(dev), kw.to(dev), sin, cos, kc, vc, ws, B, H, Hkv, hd, 0, Lmax, eps,
+                                     past_len_dev=pl)
+    assert torch.allclose(out_auto.float(), out.float(), rtol=2 ** -8, atol=2 ** -10)
 
 
 @pytest.mark.parametrize("M", [1, 2, 4])
