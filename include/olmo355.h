@@ -8,7 +8,8 @@
  *     launched on it asynchronously and the call returns without synchronising;
  *   - returns 0 on success, else an O355_E* code; olmo355_status_string() names it.  No
  *     kernel is launched when an argument check fails;
- *   - no process-global state: safe from any host thread that has made its device current;
+ *   - no process-global state: safe from any host thread that has made its device current
+ *     (one stated exception: olmo355_attn_decode_static, which owns a fixed device scratch array);
  *   - `dtype` is O355_F32 or O355_BF16 (the activation dtype); fp16 appears only as the
  *     scale / dequant-table type of the int4 format.
  *
@@ -28,6 +29,7 @@ extern "C" {
 #define O355_EINVAL 1       /* null pointer, non-positive or misaligned size */
 #define O355_EUNSUPPORTED 2 /* shape / dtype / group size outside what the kernel handles */
 #define O355_ELAUNCH 3      /* hipGetLastError() != hipSuccess after the launch */
+#define O355_ETOOBIG 4      /* sizes beyond the fixed scratch of an entry point that allocates nothing */
 
 #define O355_F32 0
 #define O355_BF16 1
@@ -179,6 +181,19 @@ int64_t olmo355_attn_decode_workspace_bytes(int B, int H, int hd, int n_keys_max
 int olmo355_attn_decode(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out,
                         void* ws, int B, int H, int Hkv, int hd, int Lmax, int past_len,
                         const int32_t* past_len_dev, int n_keys_max, int bias_stride, int dtype, void* stream);
+
+/* olmo355_attn_decode for callers that cannot allocate device memory or pass a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments without `ws`: the per-chunk partial results live in a device array of the library itself,
+ * olmo355_attn_decode_static_max_bytes() = 16 MiB per GPU, held from the first call on that GPU until the
+ * process ends.  Returns O355_ETOOBIG (nothing launched) when
+ * olmo355_attn_decode_workspace_bytes(B, H, hd, n_keys_max) exceeds that.  Calls no hipMalloc / hipFree / allocating
+ * library routine.  All calls on one GPU share the array and it keeps the last call's contents: calls that
+ * overlap on one GPU (different streams or host threads) race; calls on one stream are ordered. */
+int64_t olmo355_attn_decode_static_max_bytes(void);
+int olmo355_attn_decode_static(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out,
+                               int B, int H, int Hkv, int hd, int Lmax, int past_len, const int32_t* past_len_dev,
+                               int n_keys_max, int bias_stride, int dtype, void* stream);
 
 /* olmo355_attn_decode for beam search: the B rows are beam b % beam of sequence b / beam.  Where the
  * reference keeps the beams' caches consistent by gathering every cache tensor along the batch axis after each

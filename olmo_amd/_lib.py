@@ -52,6 +52,8 @@ EXPORTS = {
     "olmo355_attn_prefill": (I, [P, P, P, P, P, I, I, I, I, I, I, I, I, I, P]),
     "olmo355_attn_decode_workspace_bytes": (L, [I, I, I, I]),
     "olmo355_attn_decode": (I, [P, P, P, P, P, P, I, I, I, I, I, I, P, I, I, I, P]),
+    "olmo355_attn_decode_static_max_bytes": (L, []),
+    "olmo355_attn_decode_static": (I, [P, P, P, P, P, I, I, I, I, I, I, P, I, I, I, P]),
     "olmo355_attn_decode_fused": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, P, I, P]),
     "olmo355_attn_decode_beam": (I, [P, P, P, P, P, P, I, I, I, I, I, I, P, I, I, P, I, I, I, I, P]),
     "olmo355_log_softmax": (I, [P, P, I, I, I, P]),

@@ -15,6 +15,8 @@
 // plain average of the values it sees instead of NaN.
 #include "common.h"
 
+#include <mutex>
+
 namespace {
 
 constexpr float kMaskThreshold = -1e30f;
@@ -954,6 +956,51 @@ extern "C" int olmo355_attn_decode_beam(const void* q, const void* kcache, const
   if (!beam_src) return O355_EINVAL;
   return attn_decode_any(q, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd, Lmax, past_len, past_len_dev, n_keys_max,
                          bias_stride, beam_src, src_stride, prompt_len, beam, dtype, stream);
+}
+
+// ---- olmo355_attn_decode without a workspace argument and without any allocation ------------------------------
+// For callers that cannot allocate (HIP graph capture, tight serving loops): the per-chunk partial results
+// (o, max, sum) live in a file-scope device array instead of a caller-provided workspace.  Each GPU holds its own
+// copy of the array at its own address, found once per device with hipGetSymbolAddress (the array's name is not a
+// device address in host code).  Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two
+// streams, two host threads) race.  Nothing in it has to start at zero: every partial a launch's combine kernel
+// reads was written by the same launch's first kernel.
+namespace {
+constexpr int64_t kStaticScratchBytes = 16ll << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+void* g_scratch_ptr[kMaxDevices];      // per device, set once under the mutex
+bool g_scratch_known[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+int scratch_of_current_device(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return O355_ELAUNCH;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_known[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return O355_ELAUNCH;
+    g_scratch_ptr[dev] = p;
+    g_scratch_known[dev] = true;
+  }
+  *out = g_scratch_ptr[dev];
+  return O355_OK;
+}
+}  // namespace
+
+extern "C" int64_t olmo355_attn_decode_static_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int olmo355_attn_decode_static(const void* q, const void* kcache, const void* vcache, const float* key_bias,
+                                          void* out, int B, int H, int Hkv, int hd, int Lmax, int past_len,
+                                          const int32_t* past_len_dev, int n_keys_max, int bias_stride, int dtype,
+                                          void* stream) {
+  if (B <= 0 || H <= 0 || hd <= 0 || n_keys_max <= 0) return O355_EINVAL;
+  if (olmo355_attn_decode_workspace_bytes(B, H, hd, n_keys_max) > kStaticScratchBytes) return O355_ETOOBIG;
+  void* ws = nullptr;
+  const int st = scratch_of_current_device(&ws);
+  if (st != O355_OK) return st;
+  return attn_decode_any(q, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd, Lmax, past_len, past_len_dev, n_keys_max,
+                         bias_stride, nullptr, 0, 0, 1, dtype, stream);
 }
 
 // merge: how the key chunks of a (batch, head) are merged: -1 = choose, 0 = in the kernel (last workgroup of the

@@ -583,6 +583,7 @@ extern "C" const char* olmo355_status_string(int status) {
     case O355_EINVAL: return "invalid argument (null pointer or bad size)";
     case O355_EUNSUPPORTED: return "unsupported shape, dtype or group size";
     case O355_ELAUNCH: return "kernel launch failed";
+    case O355_ETOOBIG: return "sizes exceed the fixed scratch of this entry point";
     default: return "unknown status";
   }
 }
