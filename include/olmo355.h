@@ -128,6 +128,40 @@ int olmo355_w4_gemm_swiglu(const uint16_t* x, const uint32_t* wt, const uint16_t
  * (lane l: row n = 16*nt + (l&15), columns 32*ks + 8*(l>>4) .. +7); K % 32 == 0, N % 16 == 0.
  * fp32: weight in torch layout [N,K]. */
 int olmo355_b16_repack(const uint16_t* w_nk, uint16_t* wt, int N, int K, void* stream);
+/* Up to four decode-step int4 linears (at most 4 rows) in ONE launch: phase p computes y_p = x_p . W_p where x_p
+ * is phase p-1's output, directly or as resid + rmsnorm(y_{p-1}) -- e.g. attn_out -> ff_proj (+ SwiGLU) -> ff_out ->
+ * the next block's att_proj, the calls OLMoSequentialBlock.forward makes one after the other (olmo/model.py:786-821,
+ * then :746-757 of the following block), each a QuantLinear.forward (AGQ/auto_gptq/nn_modules/qlinear/
+ * qlinear_cuda_old.py:192-290).  A persistent grid of olmo355_w4_chain_grid() workgroups (one per CU) with a
+ * grid-wide barrier between phases; the weight requests of phase p+1 go out before the wait for phase p.
+ * Per phase (all device pointers; argument meaning as olmo355_w4_gemv_chain):
+ *   x [M,K]; resid / norm_w / ssq_in / x_out all NULL, or all given: then the phase multiplies
+ *   x_out = resid + rmsnorm(x; norm_w, eps) with the mean square from ssq_in [M][K/16];
+ *   y [M,N], or [M,N/2] with swiglu; ssq_out NULL or [M][N/16] (not with swiglu);
+ *   rot in [0, grid): workgroup b owns the column tiles (b + rot) mod grid, + grid, ... (vary it between phases and
+ *   layers so that the workgroups with one tile more are not always the same).
+ * sync: n_phases + 1 int32, zero on entry; the launch leaves them zero.  status: one int32, set to 1 if a
+ * barrier wait gave up after spin_limit polls (the results are then undefined; the launch still ends).
+ * Needs every workgroup resident: nothing else may occupy the device's CUs while it runs. */
+#define O355_CHAIN_MAX_PHASES 4
+typedef struct {
+  const uint16_t* x;
+  const uint16_t* resid;
+  const uint16_t* norm_w;
+  const float* ssq_in;
+  uint16_t* x_out;
+  const uint32_t* wt;
+  const uint16_t* st;
+  const uint8_t* zt;
+  uint16_t* y;
+  float* ssq_out;
+  int N, K, swiglu, rot;
+  float eps;
+} olmo355_chain_phase;
+int olmo355_w4_chain_grid(void);
+int olmo355_w4_chain(const olmo355_chain_phase* phases, int n_phases, int M, int32_t* sync, int32_t* status,
+                     int spin_limit, void* stream);
+
 /* small-M (<= 64) path */
 int olmo355_b16_gemv(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, void* stream);
 int olmo355_b16_gemv_fused(const uint16_t* x, const uint16_t* resid, const uint16_t* norm_w, float eps,

@@ -14,7 +14,7 @@ from typing import Optional
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "lib", "libolmo355.so")
 
-__all__ = ["lib", "LIB_PATH", "Olmo355Unavailable", "Olmo355Error", "check", "EXPORTS"]
+__all__ = ["lib", "LIB_PATH", "Olmo355Unavailable", "Olmo355Error", "check", "EXPORTS", "ChainPhase"]
 
 
 class Olmo355Unavailable(RuntimeError):
@@ -29,6 +29,14 @@ class Olmo355Error(RuntimeError):
 
 P, I, L, F = c_void_p, c_int, c_int64, c_float
 
+
+class ChainPhase(ctypes.Structure):
+    """``olmo355_chain_phase`` of include/olmo355.h."""
+
+    _fields_ = [(n, c_void_p) for n in ("x", "resid", "norm_w", "ssq_in", "x_out", "wt", "st", "zt", "y", "ssq_out")] + \
+               [(n, c_int) for n in ("N", "K", "swiglu", "rot")] + [("eps", c_float)]
+
+
 # name -> (restype, argtypes); must list every symbol include/olmo355.h declares
 EXPORTS = {
     "olmo355_version": (I, []),
@@ -39,6 +47,8 @@ EXPORTS = {
     "olmo355_w4_gemv": (I, [P, P, P, P, P, I, I, I, P]),
     "olmo355_w4_gemv_fused": (I, [P, P, P, F, P, P, P, P, P, I, I, I, I, P]),
     "olmo355_w4_gemv_chain": (I, [P, P, P, F, P, P, P, P, P, P, P, I, I, I, I, P]),
+    "olmo355_w4_chain_grid": (I, []),
+    "olmo355_w4_chain": (I, [ctypes.POINTER(ChainPhase), I, I, P, P, I, P]),
     "olmo355_b16_gemv_fused": (I, [P, P, P, F, P, P, P, I, I, I, I, P]),
     "olmo355_w4_gemm": (I, [P, P, P, P, P, I, I, I, P]),
     "olmo355_w4_gemm_swiglu": (I, [P, P, P, P, P, I, I, I, P]),

@@ -96,6 +96,35 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// sum over an aligned row of 16 lanes; every lane gets it
+__device__ __forceinline__ float row16_sum(float v) {
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 16);
+  return v;
+}
+// wave sum whose first four steps are DPP adds within rows of 16 lanes (fixed order: the same on every wave)
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+// eight bf16 (one 16-byte piece) widened to fp32
+__device__ __forceinline__ void unpack8(const u32x4& v, float (&f)[8]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f[2 * i] = bf16lo_to_f32(v[i]), f[2 * i + 1] = bf16hi_to_f32(v[i]);
+}
+
+// MFMA operand of eight ones: its product with the activations is their sum over k
+__device__ __forceinline__ bf16x8 ones_bf16x8() {
+  u32x4 r = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  return __builtin_bit_cast(bf16x8, r);
+}
+
 // Sum over the whole workgroup (blockDim.x a multiple of 64, at most 1024). `red` holds 16 floats.
 __device__ __forceinline__ float block_sum(float v, float* red) {
   v = wave_sum(v);

@@ -44,20 +44,10 @@ struct GemvArgs {
   float* ssq_out = nullptr;
 };
 
-__device__ __forceinline__ bf16x8 ones_bf16x8() {
-  u32x4 r = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
-  return __builtin_bit_cast(bf16x8, r);
-}
-
 __device__ __forceinline__ bf16x8 load_x_frag(const uint16_t* __restrict__ x, int row, int M, int K, int k) {
   if (row < M) return *reinterpret_cast<const bf16x8*>(x + (int64_t)row * K + k);
   u32x4 z = {0u, 0u, 0u, 0u};
   return __builtin_bit_cast(bf16x8, z);
-}
-
-__device__ __forceinline__ void unpack8(const u32x4& v, float (&f)[8]) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) f[2 * i] = bf16lo_to_f32(v[i]), f[2 * i + 1] = bf16hi_to_f32(v[i]);
 }
 
 // ---- activation staging --------------------------------------------------------------------------
@@ -66,13 +56,6 @@ __device__ __forceinline__ void unpack8(const u32x4& v, float (&f)[8]) {
 // The global loads are issued in begin() -- before the weight prologue -- and consumed in
 // finish(), after the weight loads have been issued; the barrier orders LDS only.
 constexpr int kXStageRegs = 4;  // plain copy: 16-byte pieces per thread held across the weight prologue
-
-// sum over an aligned row of 16 lanes; every lane gets it
-__device__ __forceinline__ float row16_sum(float v) {
-#pragma unroll
-  for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 16);
-  return v;
-}
 
 // Per-group sums of the staged activations, xs[g][rp] (rp rows per group, row m of group g): 16
 // consecutive 16-byte pieces are one group of 128, i.e. one row of 16 lanes.  `v` is the piece as
@@ -508,16 +491,6 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_rot_kernel(GemvArgs args, 
 // Same arithmetic and rounding points as NormStage, written for few instructions: buffer loads
 // with the thread index as offset, rows found by comparison instead of division (M <= 4 and a wave's
 // 64 pieces lie in one row, K % 512 == 0), sums over a wave with DPP.
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
-  v += __shfl_xor(v, 16, 64);
-  v += __shfl_xor(v, 32, 64);
-  return v;
-}
-
 template <int WAVES, int VPT>
 struct SmallNorm {
   u32x4 av[VPT], rv[VPT], wv[VPT];
