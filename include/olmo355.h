@@ -140,8 +140,10 @@ int olmo355_b16_repack(const uint16_t* w_nk, uint16_t* wt, int N, int K, void* s
  *   y [M,N], or [M,N/2] with swiglu; ssq_out NULL or [M][N/16] (not with swiglu);
  *   rot in [0, grid): workgroup b owns the column tiles (b + rot) mod grid, + grid, ... (vary it between phases and
  *   layers so that the workgroups with one tile more are not always the same).
- * sync: n_phases + 1 int32, zero on entry; the launch leaves them zero.  status: one int32, set to 1 if a
- * barrier wait gave up after spin_limit polls (the results are then undefined; the launch still ends).
+ * sync: olmo355_w4_chain_sync_ints() int32 (an epoch counter, then one arrival flag per workgroup), zeroed once
+ * when allocated and then owned by the launches that use it, one at a time: every launch leaves it ready for the
+ * next.  status: one int32, set to 1 if a barrier wait gave up after spin_limit polls (the results are then
+ * undefined; the launch still ends and sync stays usable).
  * Needs every workgroup resident: nothing else may occupy the device's CUs while it runs. */
 #define O355_CHAIN_MAX_PHASES 4
 typedef struct {
@@ -159,6 +161,7 @@ typedef struct {
   float eps;
 } olmo355_chain_phase;
 int olmo355_w4_chain_grid(void);
+int olmo355_w4_chain_sync_ints(void);
 int olmo355_w4_chain(const olmo355_chain_phase* phases, int n_phases, int M, int32_t* sync, int32_t* status,
                      int spin_limit, void* stream);
 

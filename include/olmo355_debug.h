@@ -31,6 +31,13 @@ int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, const void*
                                     const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps,
                                     const float* qk_ssq, const float* rope_now, int dtype, int merge, void* stream);
 
+/* olmo355_w4_chain that also records when each wave passed the stations of each phase: trace is
+ * int64 [grid][8 waves][4 phases][8 stations], ticks of the 100 MHz constant clock (phase entered, activations staged,
+ * staging barrier passed, first weights landed, items done, rows published, all workgroups arrived, phase left). */
+#include "olmo355.h"
+int olmo355_w4_chain_trace(const olmo355_chain_phase* phases, int n_phases, int M, int32_t* sync, int32_t* status,
+                           int spin_limit, int64_t* trace, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

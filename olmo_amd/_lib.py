@@ -48,6 +48,7 @@ EXPORTS = {
     "olmo355_w4_gemv_fused": (I, [P, P, P, F, P, P, P, P, P, I, I, I, I, P]),
     "olmo355_w4_gemv_chain": (I, [P, P, P, F, P, P, P, P, P, P, P, I, I, I, I, P]),
     "olmo355_w4_chain_grid": (I, []),
+    "olmo355_w4_chain_sync_ints": (I, []),
     "olmo355_w4_chain": (I, [ctypes.POINTER(ChainPhase), I, I, P, P, I, P]),
     "olmo355_b16_gemv_fused": (I, [P, P, P, F, P, P, P, I, I, I, I, P]),
     "olmo355_w4_gemm": (I, [P, P, P, P, P, I, I, I, P]),
@@ -91,6 +92,7 @@ VARIANT_EXPORTS = {
     "olmo355_w4_gemm_tile": (I, [P, P, P, P, P, I, I, I, I, P]),
     "olmo355_b16_gemm_tile": (I, [P, P, P, I, I, I, I, P]),
     "olmo355_w4_gemv_form": (I, [P, P, P, P, P, I, I, I, I, P]),
+    "olmo355_w4_chain_trace": (I, [ctypes.POINTER(ChainPhase), I, I, P, P, I, P, P]),
     "olmo355_attn_decode_fused_merge": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, P, I, I, P]),
 }
 

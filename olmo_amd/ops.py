@@ -290,10 +290,17 @@ def chain_grid() -> int:
     return int(lib().olmo355_w4_chain_grid())
 
 
-def w4_chain(steps, sync: torch.Tensor, status: torch.Tensor, spin_limit: int = CHAIN_SPIN_LIMIT) -> bool:
+def chain_sync(device) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Barrier state and status word of :func:`w4_chain`: zeroed once, then reused by one launch at a time."""
+    n = int(lib().olmo355_w4_chain_sync_ints())
+    return torch.zeros(n, dtype=torch.int32, device=device), torch.zeros(1, dtype=torch.int32, device=device)
+
+
+def w4_chain(steps, sync: torch.Tensor, status: torch.Tensor, spin_limit: int = CHAIN_SPIN_LIMIT,
+             trace: Optional[torch.Tensor] = None) -> bool:
     """Up to four decode-step int4 linears (at most 4 rows) in one launch of a persistent grid; every tensor is
-    given by the caller (outputs included: nothing is allocated here).  ``sync``: int32 ``[>= len(steps) + 1]``,
-    zero; ``status``: int32 ``[1]``, becomes 1 if a barrier wait gave up.  Returns ``False`` when the kernel does
+    given by the caller (outputs included: nothing is allocated here).  ``sync``, ``status``: from
+    :func:`chain_sync`; ``status`` becomes 1 if a barrier wait gave up.  Returns ``False`` when the kernel does
     not cover the shapes (nothing launched)."""
     from ._lib import ChainPhase
 
@@ -316,10 +323,13 @@ def w4_chain(steps, sync: torch.Tensor, status: torch.Tensor, spin_limit: int = 
         p.x, p.resid, p.norm_w, p.ssq_in, p.x_out = _p(s.x), _p(s.resid), _p(s.norm_w), _p(s.ssq_in), _p(s.x_out)
         p.wt, p.st, p.zt, p.y, p.ssq_out = _p(s.w.wt), _p(s.w.st), _p(s.w.zt), _p(s.y), _p(s.ssq_out)
         p.N, p.K, p.swiglu, p.rot, p.eps = s.w.N, s.w.K, int(s.swiglu), int(s.rot), float(s.eps)
-    if sync.dtype != torch.int32 or sync.numel() < n + 1 or status.dtype != torch.int32:
-        raise ValueError("w4_chain: sync int32 [n + 1] and status int32 [1] expected")
+    if sync.dtype != torch.int32 or sync.numel() < int(lib().olmo355_w4_chain_sync_ints()) or status.dtype != torch.int32:
+        raise ValueError("w4_chain: sync and status as made by chain_sync expected")
     _dev(sync, status)
-    st = lib().olmo355_w4_chain(arr, n, M, _p(sync), _p(status), int(spin_limit), _stream())
+    if trace is None:
+        st = lib().olmo355_w4_chain(arr, n, M, _p(sync), _p(status), int(spin_limit), _stream())
+    else:  # tuning runs: int64 [grid, 8, 4, 8] time stamps
+        st = lib().olmo355_w4_chain_trace(arr, n, M, _p(sync), _p(status), int(spin_limit), _p(trace), _stream())
     if st == 2:
         return False
     check("olmo355_w4_chain", st)

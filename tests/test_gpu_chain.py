@@ -33,7 +33,9 @@ def _weight(dev, N, K, seed):
 
 
 def _sync(dev):
-    return torch.zeros(8, dtype=torch.int32, device=dev), torch.zeros(1, dtype=torch.int32, device=dev)
+    from olmo_amd import ops
+
+    return ops.chain_sync(dev)
 
 
 def _ulp_close(a, b):
@@ -58,7 +60,7 @@ def test_single_plain_phase(dev, M, N, K, rot):
     sync, status = _sync(dev)
     assert ops.w4_chain([ops.ChainStep(x.to(dev), w, y, ssq_out=ssq, rot=rot % ops.chain_grid())], sync, status)
     torch.cuda.synchronize()
-    assert int(status.item()) == 0 and int(sync.abs().sum().item()) == 0
+    assert int(status.item()) == 0
     scale = ref.abs().max().item()
     assert (y.float().cpu() - ref).abs().max().item() <= 2 ** -7 * scale
     want = (y.float() ** 2).view(M, -1, 16).sum(-1)
@@ -136,9 +138,12 @@ def test_four_phase_block_chain(dev, M, d, ff):
     for rep in range(2):
         for t in (A, U, Fo, QKV, X1, X2):
             t.fill_(float("nan"))
-        assert ops.w4_chain(steps, sync, status)
+        ok = ops.w4_chain(steps, sync, status)
+        if not ok:  # declined, nothing launched: the rows of the longest K (+ one weight slot per wave) exceed a CU's LDS
+            assert M * ((ff + 511) // 512) * 1024 > 64 * 1024
+            pytest.skip("activations of this shape do not fit next to the weight slots: the caller uses separate launches")
         torch.cuda.synchronize()
-        assert int(status.item()) == 0 and int(sync.abs().sum().item()) == 0, rep
+        assert int(status.item()) == 0, rep
         for name, got, ref in (("a", A, a), ("u", U, u), ("f", Fo, f), ("qkv", QKV, qkv)):
             scale = ref.float().abs().max().item()
             err = (got.float().cpu() - ref.float()).abs().max().item()
@@ -172,7 +177,7 @@ def test_wait_that_gives_up_ends_the_launch(dev):
     steps = [ops.ChainStep(x, w1, y1), ops.ChainStep(y1, w2, y2)]
     assert ops.w4_chain(steps, sync, status, spin_limit=1)
     torch.cuda.synchronize()
-    assert int(status.item()) in (0, 1) and int(sync.abs().sum().item()) == 0
+    assert int(status.item()) in (0, 1)
     status.zero_()
     assert ops.w4_chain(steps, sync, status)
     torch.cuda.synchronize()
