@@ -124,38 +124,77 @@ def main() -> int:
     extra = {"prefill_tokens_per_s": ctx / t_prefill, "prefill_ms": t_prefill * 1e3}
 
     # ---- roofline of the dominant kernel: the int4 small-M linear --------------------------------
+    # Timed: exactly the launches a decode step issues for its block Linears (olmo_amd.model.OLMo._block_decode_chain
+    # without the attention launch): att_proj with the chained-norm prologue and the per-tile sums of squares,
+    # attn_out, ff_proj with the chained-norm prologue and the SwiGLU epilogue, ff_out -- 128 launches over the 32
+    # layers' distinct weights (3.36 GB, so neither L2 nor the 256 MB Infinity Cache can serve them), captured into
+    # one graph, HIP events around its replays on the stream that replays it.
     shapes = linear_shapes(cfg)
     qls = [m for m in model.modules() if isinstance(m, QuantLinear)]
-    xs = {k: torch.randn(1, k, device=dev).to(torch.bfloat16) for k in {s[1] for s in shapes}}
+    blocks = list(model.transformer["blocks"])
+    eps = cfg.layer_norm_eps
+    x_res = torch.randn(1, 1, cfg.d_model, device=dev).to(torch.bfloat16)
+    att_in = torch.randn(1, 1, cfg.d_model, device=dev).to(torch.bfloat16)
 
     def one_step_of_linears():
+        x, pend = x_res, None
+        for blk in blocks:
+            if pend is None:
+                ops.w4_linear_chain(x, blk.att_proj.tiled, want_ssq=True)
+            else:
+                _, x, _ = ops.w4_linear_chain(pend[0], blk.att_proj.tiled, resid=x, norm_w=pend[1], eps=eps, ssq_in=pend[2],
+                                              want_ssq=True)
+            a, _, ssq_a = ops.w4_linear_chain(att_in, blk.attn_out.tiled, want_ssq=True)
+            u, x, _ = ops.w4_linear_chain(a, blk.ff_proj.tiled, resid=x, norm_w=blk.attn_norm.weight.data, eps=eps,
+                                          ssq_in=ssq_a, swiglu_out=True)
+            f, _, ssq_f = ops.w4_linear_chain(u, blk.ff_out.tiled, want_ssq=True)
+            pend = (f, blk.ff_norm.weight.data, ssq_f)
+
+    def timed_graph(fn, reps=20):
+        fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / reps
+
+    reps = 20
+    n_launch = len(qls)
+    avg_s = timed_graph(one_step_of_linears, reps) / n_launch
+    bytes_per_launch = sum(n * k * W4_BYTES_PER_WEIGHT + 2 * k + 2 * n for n, k in shapes) * cfg.n_layers / n_launch
+    achieved = bytes_per_launch / avg_s / 1e9
+    roofline = {"bound": "hbm", "kernel": "w4_gemv_small_kernel (M=1): the decode step's own 4 block-Linear launches x 32 layers "
+                                          "(chained-norm prologues, SwiGLU epilogue, per-tile sums of squares)",
+                "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                "traffic": GEMV_TRAFFIC_BYTES_7B,
+                "traffic_source": "profiles/w4_gemv_small_kernel_7b_m1_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE "
+                                  "of `bench.py --traffic-probe`, scaled by a 256 MiB copy)",
+                "avg_launch_us": avg_s * 1e6, "bytes_per_launch": bytes_per_launch}
+    log(f"[bench] int4 decode linears (the step's own launches): {avg_s * 1e6:.2f} us/launch avg, {achieved:.0f} GB/s = "
+        f"{achieved / HBM_PEAK_GBS:.1%} of HBM peak")
+
+    # the same weights through plain launches (no prologue / epilogue): what the isolated kernel does
+    xs = {k: torch.randn(1, k, device=dev).to(torch.bfloat16) for k in {s[1] for s in shapes}}
+
+    def plain_linears():
         for q in qls:
             ops.w4_linear(xs[q.infeatures], q.tiled)
 
-    one_step_of_linears()
-    torch.cuda.synchronize()
-    g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
-        one_step_of_linears()
-    reps = 20
-    g.replay()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(reps):
-        g.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    n_launch = len(qls)
-    avg_s = e0.elapsed_time(e1) * 1e-3 / (reps * n_launch)
-    bytes_per_launch = sum(n * k * W4_BYTES_PER_WEIGHT + 2 * k + 2 * n for n, k in shapes) * cfg.n_layers / n_launch
-    achieved = bytes_per_launch / avg_s / 1e9
-    roofline = {"bound": "hbm", "kernel": "w4_gemv_small_kernel (M=1, the 4 block Linears x 32 layers)",
-                "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                "traffic": GEMV_TRAFFIC_BYTES_7B, "avg_launch_us": avg_s * 1e6, "bytes_per_launch": bytes_per_launch}
-    log(f"[bench] int4 GEMV: {avg_s * 1e6:.2f} us/launch avg, {achieved:.0f} GB/s = {achieved / HBM_PEAK_GBS:.1%} of HBM peak")
+    plain_s = timed_graph(plain_linears, reps) / n_launch
+    extra["plain_linear_launches"] = {"avg_launch_us": plain_s * 1e6, "achieved": bytes_per_launch / plain_s / 1e9, "unit": "GB/s",
+                                      "frac": bytes_per_launch / plain_s / 1e9 / HBM_PEAK_GBS}
+    log(f"[bench] int4 linears, plain launches: {plain_s * 1e6:.2f} us/launch = {bytes_per_launch / plain_s / 1e9:.0f} GB/s")
 
     # ---- prefill GEMMs (M = context): TFLOP/s against the bf16 MFMA peak ---------------------------
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     xp = {k: torch.randn(ctx, k, device=dev).to(torch.bfloat16) for k in {s[1] for s in shapes}}
     layer = qls[:4]
     for q in layer:
@@ -209,6 +248,29 @@ def main() -> int:
     }
     log(f"[bench] ceiling on this box: streaming the same weights {s_avg * 1e6:.2f} us/launch = {wt_bytes / s_avg / 1e9:.0f} GB/s "
         f"(linear / stream = {avg_s / s_avg:.2f})")
+    # ... and all 128 weight buffers streamed by ONE launch of a persistent grid: no launch boundary, no ramp
+    import ctypes as _ct
+
+    ptrs = (_ct.c_void_p * n_launch)(*[q.tiled.wt.data_ptr() for q in qls])
+    sizes = (_ct.c_int64 * n_launch)(*[q.tiled.wt.numel() * q.tiled.wt.element_size() for q in qls])
+
+    def stream_many():
+        _check("olmo355_probe_stream_read_many",
+               _lib().olmo355_probe_stream_read_many(ptrs, sizes, n_launch, sink.data_ptr(), torch.cuda.current_stream().cuda_stream))
+
+    stream_many()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(5):
+        stream_many()
+    e1.record()
+    torch.cuda.synchronize()
+    m_s = e0.elapsed_time(e1) * 1e-3 / 5
+    assert int(sink.abs().sum().item()) == 0
+    extra["ceilings"]["stream_read_one_persistent_launch"] = {
+        "what": "the same 128 weight buffers (3.3 GB) read by one launch of a persistent grid (2 workgroups per CU)",
+        "ms": m_s * 1e3, "achieved": sum(sizes) / m_s / 1e9, "unit": "GB/s", "frac_of_peak": sum(sizes) / m_s / 1e9 / HBM_PEAK_GBS}
+    log(f"[bench] ceiling on this box: one persistent launch streaming all weights: {m_s * 1e3:.3f} ms = {sum(sizes) / m_s / 1e9:.0f} GB/s")
 
     # matrix cores alone, after the GEMM timing (a sustained MFMA burst lowers the clocks of what follows)
     import ctypes

@@ -320,6 +320,9 @@ int olmo355_incr_i32(int32_t* p, void* stream);
  * (256 workgroups x 8 waves x iters x 8 v_mfma_f32_32x32x16_bf16; *flops = total floating-point operations).
  * `sink` is a device buffer of at least 2 KiB that stays unwritten. */
 int olmo355_probe_stream_read(const void* src, int64_t bytes, void* sink, void* stream);
+/* The same over n buffers (host arrays of device pointers and byte counts, n <= 160) in ONE launch of a persistent
+ * grid of two workgroups per CU: no launch boundary and no ramp per buffer. */
+int olmo355_probe_stream_read_many(const void* const* srcs, const int64_t* bytes, int n, void* sink, void* stream);
 int olmo355_probe_mfma_bf16(int iters, void* sink, double* flops, void* stream);
 
 #ifdef __cplusplus

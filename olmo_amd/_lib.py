@@ -81,6 +81,7 @@ EXPORTS = {
     "olmo355_clamp": (I, [P, L, F, I, P]),
     "olmo355_sample": (I, [P, I, I, F, I, F, c_uint64, P, I, P, P, I, P]),
     "olmo355_probe_stream_read": (I, [P, L, P, P]),
+    "olmo355_probe_stream_read_many": (I, [P, P, I, P, P]),
     "olmo355_probe_mfma_bf16": (I, [I, P, P, P]),
     "olmo355_add": (I, [P, P, P, L, I, P]),
     "olmo355_argmax": (I, [P, P, I, I, I, P]),

@@ -27,6 +27,40 @@ __global__ __launch_bounds__(512) void stream_read_kernel(const u32x4* __restric
   if (acc == 0x9e3779b9u) sink[threadIdx.x] = acc;
 }
 
+// The same for many buffers in ONE launch of a grid that stays (two workgroups per CU): the pieces of all buffers
+// form one sequence dealt round-robin to the waves, 8 requests in flight per wave.  No launch boundary, no ramp
+// per buffer: what the memory system sustains when nothing but streaming happens.
+constexpr int kManyMax = 160;
+struct ManyArgs {
+  const u32x4* src[kManyMax];
+  int32_t first_piece[kManyMax + 1];  // prefix sums of the buffers' piece counts
+  int n;
+};
+__global__ __launch_bounds__(512) void stream_read_many_kernel(ManyArgs a, uint32_t* __restrict__ sink) {
+  constexpr int U = 8;
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 6), nw = (int64_t)gridDim.x * 8;
+  const int64_t pieces = a.first_piece[a.n];
+  uint32_t acc = 0;
+  int b = 0;
+  // a wave's 8 requests are 8 consecutive KiB (a workgroup's: 64 KiB in a row), so a CU touches few pages at a time
+  for (int64_t p = wave * U; p < pieces; p += nw * U) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t q = p + u;
+      v[u] = u32x4{0u, 0u, 0u, 0u};
+      if (q < pieces) {
+        while (q >= a.first_piece[b + 1]) ++b;  // wave-uniform; q grows monotonically
+        v[u] = __builtin_nontemporal_load(&a.src[b][(q - a.first_piece[b]) * 64 + lane]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  if (acc == 0x9e3779b9u) sink[threadIdx.x] = acc;
+}
+
 // 8 waves per workgroup, 8 independent 32x32 accumulators per wave, operands drawn once from a generator
 // (random mantissas and signs, exponents near 1: constant operands run faster than a real product does).
 __global__ __launch_bounds__(512) void mfma_bf16_kernel(float* __restrict__ sink, int iters, uint32_t seed) {
@@ -78,6 +112,27 @@ extern "C" int olmo355_probe_stream_read(const void* src, int64_t bytes, void* s
     hipLaunchKernelGGL(stream_read_kernel<2>, dim3(grid), dim3(512), 0, as_stream(stream), (const u32x4*)src, pieces,
                        (uint32_t*)sink);
   }
+  O355_CHECK_LAUNCH();
+}
+
+extern "C" int olmo355_probe_stream_read_many(const void* const* srcs, const int64_t* bytes, int n, void* sink,
+                                              void* stream) {
+  if (!srcs || !bytes || !sink || n < 1 || n > kManyMax) return O355_EINVAL;
+  ManyArgs a;
+  int64_t total = 0;
+  for (int i = 0; i < n; ++i) {
+    if (!srcs[i] || bytes[i] < 1024) return O355_EINVAL;
+    a.src[i] = (const u32x4*)srcs[i];
+    a.first_piece[i] = (int32_t)total;
+    total += bytes[i] >> 10;
+    if (total >= (1ll << 31)) return O355_EUNSUPPORTED;
+  }
+  a.first_piece[n] = (int32_t)total;
+  a.n = n;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    return O355_ELAUNCH;
+  hipLaunchKernelGGL(stream_read_many_kernel, dim3((unsigned)(2 * cus)), dim3(512), 0, as_stream(stream), a, (uint32_t*)sink);
   O355_CHECK_LAUNCH();
 }
 
