@@ -59,6 +59,9 @@ def main() -> int:
     ap.add_argument("--gemm-probe", action="store_true",
                     help="for rocprofv3 --pmc matrix-core counters: the four int4 block linears of a layer at 2048 "
                          "rows, three times each over distinct weights; nothing is timed or printed")
+    ap.add_argument("--counters-probe", action="store_true",
+                    help="for rocprofv3 --pmc over every kernel of the path: a 256 MiB device copy (the yardstick), one "
+                         "prefill 1 x context and four eager batch-1 decode steps of the 7B int4 model; nothing is timed")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this build runs the whole model on ONE GPU; --gpus N with N > 1 is not supported.")
@@ -93,6 +96,20 @@ def main() -> int:
     torch.cuda.synchronize()
     log(f"[bench] model built in {time.time() - t0:.1f}s")
     gen = torch.Generator().manual_seed(0)
+    if args.counters_probe:
+        src = torch.randint(0, 255, (256 << 20,), dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        ids = torch.randint(0, cfg.vocab_size, (1, ctx), generator=gen).to(dev)
+        out, cache, first, kb = _prefill(model, ids, None)
+        sess = DecodeSession(model, cache, first, kb)
+        for _ in range(4):
+            sess.step()
+        torch.cuda.synchronize()
+        return 0
 
     def run_decode(B: int):
         ids = torch.randint(0, cfg.vocab_size, (B, ctx), generator=gen).to(dev)
