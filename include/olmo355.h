@@ -279,6 +279,10 @@ int olmo355_gather_columns(const uint16_t* x, const int32_t* perm, uint16_t* out
 int olmo355_clamp(void* x, int64_t n, float c, int dtype, void* stream);
 /* out = a + b (residual add of the pre-norm block, olmo/model.py:794,821). */
 int olmo355_add(const void* a, const void* b, void* out, int64_t n, int dtype, void* stream);
+/* out[m][n] = x[m][n] + bias[n]: the bias of a quantised Linear
+ * (AGQ/auto_gptq/nn_modules/qlinear/qlinear_cuda_old.py:288-290); x, out bf16 [M, N], bias fp16 [N] as the
+ * checkpoint stores it, sum in fp32, one rounding. */
+int olmo355_add_bias_bf16(const uint16_t* x, const uint16_t* bias_f16, uint16_t* out, int M, int N, void* stream);
 /* Greedy step (olmo/beam_search.py:102-113 with beam 1): first index of the row maximum,
  * written as int64 to out[r], and the same value appended at ids_next when non-NULL. */
 int olmo355_argmax(const void* logits, int64_t* out, int rows, int n, int dtype, void* stream);

@@ -84,6 +84,7 @@ EXPORTS = {
     "olmo355_probe_stream_read_many": (I, [P, P, I, P, P]),
     "olmo355_probe_mfma_bf16": (I, [I, P, P, P]),
     "olmo355_add": (I, [P, P, P, L, I, P]),
+    "olmo355_add_bias_bf16": (I, [P, P, P, I, I, P]),
     "olmo355_argmax": (I, [P, P, I, I, I, P]),
     "olmo355_incr_i32": (I, [P, P]),
 }

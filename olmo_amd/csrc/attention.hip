@@ -11,8 +11,10 @@
 //
 // Masking: keys after the query position are skipped.  A key whose key_bias entry is <= -1e30
 // (padding) keeps a *finite* score, the dtype's most negative value, as in the reference
-// (olmo/model.py:1337-1376, olmo/torch_util.py:81-90): a query that sees only padding gets the
-// plain average of the values it sees instead of NaN.
+// (olmo/model.py:1337-1376, olmo/torch_util.py:81-90): a query that sees only padding gets a
+// plain average of values instead of NaN -- in the reference over every key of the call, which
+// attn_masked_rows_kernel reproduces after a prefill launch; a decode step's single query (a real
+// token, never masked itself) needs no such pass.
 #include "common.h"
 
 #include <mutex>
@@ -849,13 +851,72 @@ int launch_generic(const void* q, const void* kc, const void* vc, const float* k
 
 }  // namespace
 
+namespace {
+// Query rows that see only masked keys.  The reference gives a masked score the dtype's most negative
+// *finite* value -- padding keys and keys after the query alike (olmo/model.py:375-381,1337-1376,
+// olmo/torch_util.py:81-90) -- so for such a row every key of the call, later ones included, has the
+// same score and the softmax is uniform over all of them: the row's output is the plain mean of the
+// values of all past_len + T keys.  The attention kernels skip later keys, so this pass rewrites those rows
+// (positions before a sequence's first unmasked key: the padding positions of a left-padded batch).
+// One workgroup per (kv head, sequence); sums in a fixed order.
+template <int DT>
+__global__ __launch_bounds__(256) void attn_masked_rows_kernel(const void* __restrict__ vc, const float* __restrict__ key_bias,
+                                                               void* __restrict__ out, int T, int H, int Hkv, int hd,
+                                                               int Lmax, int past_len, int bias_stride) {
+  __shared__ int first;
+  __shared__ float part[256];
+  const int hk = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const int L = past_len + T;
+  if (tid == 0) first = L;
+  __syncthreads();
+  for (int k = tid; k < L; k += 256)
+    if (key_bias[(int64_t)b * bias_stride + k] > kMaskThreshold) atomicMin(&first, k);
+  __syncthreads();
+  const int nrows = min(first, L) - past_len;  // query rows t < nrows sit before the first unmasked key
+  if (nrows <= 0) return;                      // workgroup-uniform
+  const int nsl = 256 / hd, c = tid % hd, sl = tid / hd;
+  const int64_t vbase = ((int64_t)b * Hkv + hk) * Lmax * hd;
+  float acc = 0.f;
+  if (sl < nsl)
+    for (int k = sl; k < L; k += nsl) acc += Act<DT>::ld(vc, vbase + (int64_t)k * hd + c);
+  part[tid] = acc;
+  __syncthreads();
+  if (sl == 0) {
+    float sum = 0.f;
+    for (int j = 0; j < nsl; ++j) sum += part[j * hd + c];
+    const float mean = sum / (float)L;
+    const int rep = H / Hkv;
+    for (int t = 0; t < nrows; ++t)
+      for (int h = hk * rep; h < (hk + 1) * rep; ++h) Act<DT>::st(out, ((int64_t)(b * T + t) * H + h) * hd + c, mean);
+  }
+}
+
+int attn_prefill_main(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out, int B, int T,
+                      int H, int Hkv, int hd, int Lmax, int past_len, int bias_stride, int dtype, hipStream_t s);
+}  // namespace
+
 extern "C" int olmo355_attn_prefill(const void* q, const void* kcache, const void* vcache, const float* key_bias,
                                     void* out, int B, int T, int H, int Hkv, int hd, int Lmax, int past_len,
                                     int bias_stride, int dtype, void* stream) {
   if (!q || !kcache || !vcache || !out) return O355_EINVAL;
+  if (hd <= 0 || hd > 256) return O355_EUNSUPPORTED;
+  hipStream_t s = as_stream(stream);
+  const int rc = attn_prefill_main(q, kcache, vcache, key_bias, out, B, T, H, Hkv, hd, Lmax, past_len, bias_stride, dtype, s);
+  if (rc != O355_OK || !key_bias) return rc;
+  if (dtype == O355_BF16)
+    hipLaunchKernelGGL(attn_masked_rows_kernel<O355_BF16>, dim3(Hkv, B), dim3(256), 0, s, vcache, key_bias, out, T, H, Hkv,
+                       hd, Lmax, past_len, bias_stride);
+  else
+    hipLaunchKernelGGL(attn_masked_rows_kernel<O355_F32>, dim3(Hkv, B), dim3(256), 0, s, vcache, key_bias, out, T, H, Hkv,
+                       hd, Lmax, past_len, bias_stride);
+  O355_CHECK_LAUNCH();
+}
+
+namespace {
+int attn_prefill_main(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out, int B, int T,
+                      int H, int Hkv, int hd, int Lmax, int past_len, int bias_stride, int dtype, hipStream_t s) {
   if (B <= 0 || T <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || past_len < 0 || past_len + T > Lmax) return O355_EINVAL;
   if (key_bias && bias_stride < past_len + T) return O355_EINVAL;
-  hipStream_t s = as_stream(stream);
   if (dtype == O355_BF16 && (hd == 128 || hd == 64) && (int64_t)Lmax * hd < (1ll << 31)) {  // 32-bit offsets within a head
     const dim3 grid(H, (T + 127) / 128, B);  // heads fastest, then query blocks by rank (see the kernel)
     if (hd == 128)
@@ -880,6 +941,7 @@ extern "C" int olmo355_attn_prefill(const void* q, const void* kcache, const voi
 #undef GENERIC
   return O355_EUNSUPPORTED;
 }
+}  // namespace
 
 namespace {
 // *pos += delta, then rope_now = [sin_tab[*pos] | cos_tab[*pos]] (the last table row when *pos runs past it)

@@ -366,6 +366,16 @@ __global__ __launch_bounds__(256) void add_kernel(const void* __restrict__ a, co
   if (i < n) Act<DT>::st(out, i, Act<DT>::ld(a, i) + Act<DT>::ld(b, i));
 }
 
+// out[m][n] = x[m][n] + bias[n], bias fp16 (the QuantLinear bias buffer), sum in fp32, one rounding
+__global__ __launch_bounds__(256) void add_bias_bf16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ bias,
+                                                            uint16_t* __restrict__ out, int64_t total, int N) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < total) {
+    const float b = (float)__builtin_bit_cast(_Float16, bias[i % N]);
+    out[i] = (uint16_t)f32_to_bf16_bits(bf16_bits_to_f32(x[i]) + b);
+  }
+}
+
 // first index of the maximum of each row (torch.argmax tie rule); all loads of a thread issued
 // up front when the row is 16-byte divisible
 template <int DT>
@@ -559,6 +569,14 @@ extern "C" int olmo355_add(const void* a, const void* b, void* out, int64_t n, i
   if (!a || !b || !out || n <= 0) return O355_EINVAL;
   DT_SWITCH(dtype, hipLaunchKernelGGL(add_kernel<DT>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
                                       as_stream(stream), a, b, out, n));
+  O355_CHECK_LAUNCH();
+}
+
+extern "C" int olmo355_add_bias_bf16(const uint16_t* x, const uint16_t* bias_f16, uint16_t* out, int M, int N, void* stream) {
+  if (!x || !bias_f16 || !out || M <= 0 || N <= 0) return O355_EINVAL;
+  const int64_t total = (int64_t)M * N;
+  hipLaunchKernelGGL(add_bias_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, as_stream(stream), x,
+                     bias_f16, out, total, N);
   O355_CHECK_LAUNCH();
 }
 

@@ -74,8 +74,12 @@ class DecodeSession:
         self.graph = g
 
 
-def _prefill(model, input_ids, attention_mask, sampling: Optional[dict] = None):
-    out = model(input_ids, attention_mask=attention_mask, use_cache=True, last_logits_only=True)
+def _prefill(model, input_ids, attention_mask, sampling: Optional[dict] = None,
+             attention_bias: Optional[torch.Tensor] = None, key_bias_extra: Optional[torch.Tensor] = None):
+    """``key_bias_extra``: ``attention_bias`` as a per-key bias over prompt + new tokens (see
+    ``OLMo.key_bias_from_attention_bias``), for the decode steps that follow."""
+    out = model(input_ids, attention_mask=attention_mask, attention_bias=attention_bias, use_cache=True,
+                last_logits_only=True)
     cache = out.attn_key_values[0].cache
     B = input_ids.shape[0]
     if sampling is None:
@@ -87,6 +91,10 @@ def _prefill(model, input_ids, attention_mask, sampling: Optional[dict] = None):
         am = attention_mask.to(model.device, torch.float32).view(B, -1)
         key_bias_full = torch.zeros(B, cache.capacity, dtype=torch.float32, device=model.device)
         key_bias_full[:, : am.shape[1]] = (1.0 - am) * torch.finfo(torch.float32).min
+    if key_bias_extra is not None:
+        if key_bias_full is None:
+            key_bias_full = torch.zeros(B, cache.capacity, dtype=torch.float32, device=model.device)
+        key_bias_full[:, : key_bias_extra.shape[1]] += key_bias_extra
     return out, cache, first, key_bias_full
 
 
@@ -94,7 +102,7 @@ def _prefill(model, input_ids, attention_mask, sampling: Optional[dict] = None):
 def greedy_generate(model, input_ids: torch.Tensor, attention_mask: Optional[torch.Tensor], max_new_tokens: int,
                     use_graph: bool = True, eos_token_id: Optional[int] = None, pad_token_id: Optional[int] = None,
                     return_scores: bool = False, return_logits: bool = False, sampling: Optional[dict] = None,
-                    stop_when_all_ended: bool = False):
+                    stop_when_all_ended: bool = False, attention_bias: Optional[torch.Tensor] = None):
     """Returns ``tokens [B, max_new_tokens]`` (and, on request, the summed log-probabilities of the
     chosen tokens and / or the per-step logits).  Runs ``max_new_tokens`` steps; with
     ``eos_token_id`` the tokens after a sequence's first EOS are replaced by ``pad_token_id`` and add nothing to
@@ -108,7 +116,10 @@ def greedy_generate(model, input_ids: torch.Tensor, attention_mask: Optional[tor
     B, T0 = input_ids.shape
     if T0 + max_new_tokens - 1 > model.max_cache_len:
         raise ValueError(f"prompt {T0} + {max_new_tokens} new tokens exceeds max_cache_len {model.max_cache_len}")
-    out, cache, first, key_bias_full = _prefill(model, input_ids, attention_mask, sampling)
+    key_bias_extra = None
+    if attention_bias is not None:  # olmo/model.py:1607,1645-1651: one bias over prompt + generated tokens
+        key_bias_extra = model.key_bias_from_attention_bias(attention_bias, B, 0, T0 + max_new_tokens - 1)
+    out, cache, first, key_bias_full = _prefill(model, input_ids, attention_mask, sampling, attention_bias, key_bias_extra)
     sess = DecodeSession(model, cache, first, key_bias_full, sampling)
     tokens = torch.empty(B, max_new_tokens, dtype=torch.int64, device=model.device)
     tokens[:, 0] = sess.ids.view(B)

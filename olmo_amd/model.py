@@ -256,9 +256,10 @@ class OLMo(nn.Module):
             self._tied_head = ops.b16_repack(self.transformer["wte"].weight.data.contiguous())
         n_pos = max(self.max_cache_len, c.max_sequence_length)
         self._rope = ops.rope_tables(c.head_dim, float(c.rope_theta), n_pos, self.device)
-        # act-order int4 layers gather their activation columns in QuantLinear.forward: the fused decode forms
-        # (which hand the tiled weights to the kernels directly) are not used for such models
-        self._act_order = any(isinstance(m, QuantLinear) and m._perm is not None for m in self.modules())
+        # act-order int4 layers gather their activation columns in QuantLinear.forward, which also adds a
+        # non-zero bias: the fused decode forms (which hand the tiled weights to the kernels directly) are
+        # not used for such models
+        self._act_order = any(isinstance(m, QuantLinear) and (m._perm is not None or m._has_bias) for m in self.modules())
         self._chain_ok = {}  # rows -> whether the chained decode block covers this model
         self._rope_now = None  # rotary rows of the current position during a captured decode step
         self._beam = None  # the beam cache while a beam-search step runs
@@ -476,8 +477,6 @@ class OLMo(nn.Module):
         max_doc_lens: Optional[Sequence[int]] = None,
     ) -> OLMoOutput:
         c = self.config
-        if attention_bias is not None:
-            raise NotImplementedError("an explicit attention_bias is not implemented; causal + attention_mask only")
         if doc_lens is not None or max_doc_lens is not None:
             raise NotImplementedError("intra-document masking is a training feature and is not implemented")
         if not self._prepared:
@@ -520,6 +519,9 @@ class OLMo(nn.Module):
             if am.shape[1] != past_len + T:
                 raise ValueError(f"attention_mask covers {am.shape[1]} positions, expected {past_len + T}")
             key_bias = ((1.0 - am) * torch.finfo(torch.float32).min).contiguous()
+        if attention_bias is not None:
+            kb = self.key_bias_from_attention_bias(attention_bias, B, past_len, past_len + T)
+            key_bias = kb if key_bias is None else (key_bias + kb).contiguous()
 
         logits, hidden = self._forward_tokens(x, cache, B, T, past_len, key_bias, None, last_logits_only,
                                               bool(output_hidden_states))
@@ -527,6 +529,34 @@ class OLMo(nn.Module):
             cache.set_length(past_len + T)
         kvs = cache.views() if (use_cache and cache is not None) else None
         return OLMoOutput(logits=logits, attn_key_values=kvs, hidden_states=hidden)
+
+    def key_bias_from_attention_bias(self, attention_bias: torch.Tensor, B: int, q0: int, q1: int) -> torch.Tensor:
+        """An explicit ``attention_bias`` (``olmo/model.py:1343-1376``: ``[1 or B, 1, L, L]``, additive, or bool /
+        int8 with 0 = masked) as the per-key bias ``[B, q1]`` the attention kernels take, for the query rows
+        ``q0 .. q1-1``.  The kernels mask causally themselves and add one number per key, so the bias must be
+        causal (every key after the query masked) and, below the diagonal, the same for every query row of the
+        call: causal + padding, per-key penalties, anything for a single query row.  Other biases (ALiBi-like
+        ones over several rows) raise ``NotImplementedError``.  Values are rounded to the activation dtype as the
+        reference does (``olmo/model.py:516-531``)."""
+        ab = attention_bias
+        if ab.dim() != 4 or ab.shape[1] != 1 or ab.shape[0] not in (1, B) or ab.shape[2] < q1 or ab.shape[3] < q1:
+            raise ValueError(f"attention_bias of shape {tuple(ab.shape)} does not cover {q1} positions of batch {B}")
+        ab = ab.to(self.device)
+        if ab.dtype in (torch.int8, torch.bool):
+            ab = ab.to(torch.float32)
+            ab = ab.masked_fill(ab == 0.0, torch.finfo(torch.float32).min)
+        rows = ab[:, 0, q0:q1, :q1].to(torch.float32)  # [b, T, q1]
+        kb = rows[:, -1, :]                            # the last row sees every key of the call
+        qpos = torch.arange(q0, q1, device=self.device).view(1, -1, 1)
+        future = torch.arange(q1, device=self.device).view(1, 1, -1) > qpos
+        masked = rows <= -1e30
+        same = (rows == kb.unsqueeze(1)) | (masked & (kb.unsqueeze(1) <= -1e30))
+        if not bool((torch.where(future, masked, same)).all()):
+            raise NotImplementedError("attention_bias must be causal and the same for every query row below the "
+                                      "diagonal (causal + per-key terms); general biases are not implemented")
+        if self.dtype != torch.float32:
+            kb = kb.to(self.dtype).to(torch.float32)  # -inf where the dtype cannot hold the value: still masked
+        return kb.expand(B, q1).contiguous()
 
     def _forward_tokens(self, x, cache: Optional[KVCache], B: int, T: int, past_len: int, key_bias, graph_pos,
                         last_logits_only: bool, collect_hidden: bool = False):
@@ -580,7 +610,7 @@ class OLMo(nn.Module):
     # ------------------------------------------------------------------------------------------
     @torch.no_grad()
     def generate(self, input_ids: torch.LongTensor, attention_mask: Optional[torch.Tensor] = None,
-                 max_steps: int = 10, beam_size: int = 1, per_node_beam_size: Optional[int] = None,
+                 attention_bias: Optional[torch.Tensor] = None, max_steps: int = 10, beam_size: int = 1, per_node_beam_size: Optional[int] = None,
                  sampler=None, min_steps: Optional[int] = None, final_sequence_scorer=None,
                  constraints: Optional[list] = None, use_graph: bool = True, stop_at_eos: bool = True,
                  seed: int = 0) -> OLMoGenerateOutput:
@@ -595,10 +625,14 @@ class OLMo(nn.Module):
         over a :class:`BeamKVCache`.  ``scores`` is the
         summed log-probability of the chosen tokens under the unfiltered distribution (passed through
         ``final_sequence_scorer`` in a beam search)."""
+        if attention_bias is not None:  # olmo/model.py:1645-1657
+            B, P = input_ids.shape
+            assert attention_bias.dim() == 4 and tuple(attention_bias.shape[:2]) == (B, 1)
+            assert P + max_steps <= attention_bias.shape[2] == attention_bias.shape[3]
         plain = beam_size == 1 and not constraints and not min_steps and final_sequence_scorer is None
         if not plain:
             return self._generate_beam(input_ids, attention_mask, max_steps, beam_size, per_node_beam_size, sampler,
-                                       min_steps, final_sequence_scorer, constraints, use_graph)
+                                       min_steps, final_sequence_scorer, constraints, use_graph, attention_bias)
         from .generate import greedy_generate
 
         sampling = None
@@ -608,11 +642,13 @@ class OLMo(nn.Module):
             sampling = dict(sampler.params(), seed=seed)
         toks, scores = greedy_generate(self, input_ids, attention_mask, max_steps, use_graph=use_graph,
                                        eos_token_id=self.config.eos_token_id if stop_at_eos else None,
-                                       return_scores=True, sampling=sampling, stop_when_all_ended=stop_at_eos)
+                                       return_scores=True, sampling=sampling, stop_when_all_ended=stop_at_eos,
+                                       attention_bias=attention_bias)
         return OLMoGenerateOutput(token_ids=toks.unsqueeze(1), scores=scores.unsqueeze(1))
 
     def _generate_beam(self, input_ids, attention_mask, max_steps, beam_size, per_node_beam_size, sampler, min_steps,
-                       final_sequence_scorer, constraints, use_graph: bool = True) -> OLMoGenerateOutput:
+                       final_sequence_scorer, constraints, use_graph: bool = True,
+                       attention_bias: Optional[torch.Tensor] = None) -> OLMoGenerateOutput:
         """The step function of ``olmo/model.py:1677-1714`` for ``BeamSearch``: prefill once with the batch, then
         one token per beam and step against a :class:`BeamKVCache`; log-softmax of the last position on the
         device.  The model's part of a step (embedding to log-probabilities) is captured into a HIP graph after
@@ -629,6 +665,9 @@ class OLMo(nn.Module):
         if P + max_steps - 1 > self.max_cache_len:
             raise ValueError(f"prompt {P} + {max_steps} new tokens exceeds max_cache_len {self.max_cache_len}")
         model, c = self, self.config
+        ab_keys = None  # attention_bias as a per-key bias over prompt + generated tokens
+        if attention_bias is not None:
+            ab_keys = self.key_bias_from_attention_bias(attention_bias, B, 0, P + max_steps - 1)
 
         class _Beams:  # the search's state: BeamSearch calls expand_beams once, reorder_beams after every step
             cache = None
@@ -646,10 +685,13 @@ class OLMo(nn.Module):
                     bc.k[i].view(batch, beam, *bc.k[i].shape[1:])[:, 0, :, :P] = pre.k[i][:, :, :P]
                     bc.v[i].view(batch, beam, *bc.v[i].shape[1:])[:, 0, :, :P] = pre.v[i][:, :, :P]
                 bc.set_length(P)
-                if attention_mask is not None:
-                    am = attention_mask.to(model.device, torch.float32).view(batch, P)
+                if attention_mask is not None or ab_keys is not None:
                     kb = torch.zeros(batch, beam, bc.capacity, dtype=torch.float32, device=model.device)
-                    kb[:, :, :P] = ((1.0 - am) * torch.finfo(torch.float32).min).unsqueeze(1)
+                    if attention_mask is not None:
+                        am = attention_mask.to(model.device, torch.float32).view(batch, P)
+                        kb[:, :, :P] = ((1.0 - am) * torch.finfo(torch.float32).min).unsqueeze(1)
+                    if ab_keys is not None:
+                        kb[:, :, : ab_keys.shape[1]] += ab_keys.unsqueeze(1)
                     st.key_bias = kb.view(batch * beam, bc.capacity)
                 st.cache = bc
 
@@ -659,7 +701,8 @@ class OLMo(nn.Module):
         def step(last_predictions: torch.Tensor, state: dict, timestep: int):
             st = state["beams"]
             if timestep == 0:
-                out = model(input_ids, attention_mask=attention_mask, use_cache=True, last_logits_only=True)
+                out = model(input_ids, attention_mask=attention_mask, attention_bias=attention_bias, use_cache=True,
+                            last_logits_only=True)
                 st.cache = out.attn_key_values[0].cache
                 logits = out.logits[:, -1]
             else:

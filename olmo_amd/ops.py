@@ -436,6 +436,20 @@ def add(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def add_bias(x: torch.Tensor, bias_f16: torch.Tensor) -> torch.Tensor:
+    """``x + bias`` over the last axis: bf16 rows, the fp16 bias buffer of a quantised Linear."""
+    _dev(x, bias_f16)
+    N = x.shape[-1]
+    if x.dtype != torch.bfloat16 or bias_f16.dtype != torch.float16 or bias_f16.shape != (N,):
+        raise ValueError("add_bias takes bf16 rows and an fp16 bias of the row length")
+    x = x.contiguous()
+    out = torch.empty_like(x)
+    if x.numel():
+        check("olmo355_add_bias_bf16",
+              lib().olmo355_add_bias_bf16(_p(x), _p(bias_f16.contiguous()), _p(out), x.numel() // N, N, _stream()))
+    return out
+
+
 def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     _dev(logits, out)
     n = logits.shape[-1]

@@ -64,6 +64,7 @@ class QuantLinear(nn.Module):
         self.trainable = trainable
         self._tiled: Optional[ops.W4Tiled] = None
         self._perm: Optional[torch.Tensor] = None  # act-order: row order of the tiled copy (int32 [K])
+        self._has_bias = False  # decided in post_init: whether forward() adds the bias buffer
 
     # -- one-time preparation ------------------------------------------------------------------
     def post_init(self, free_checkpoint_buffers: bool = False):
@@ -87,8 +88,8 @@ class QuantLinear(nn.Module):
             q = ((qweight.unsqueeze(1) >> sh) & 15).reshape(K, self.outfeatures)[perm]  # nibbles, rows sorted
             qweight = (q.view(K // 8, 8, self.outfeatures) << sh).sum(1, dtype=torch.int32)  # nibble 7 lands in the sign bit
             self._perm = perm.to(torch.int32).contiguous()
-        if self.bias is not None and bool(self.bias.any()):
-            raise NotImplementedError("a non-zero QuantLinear bias is not implemented")
+        # a bias that is all zero (what make_quant creates and OLMo checkpoints hold) costs nothing
+        self._has_bias = self.bias is not None and bool(self.bias.any())
         self._tiled = ops.w4_repack(qweight, self.qzeros, self.scales, self.group_size)
         if free_checkpoint_buffers:
             empty = torch.empty(0, dtype=torch.int32, device=self.qweight.device)
@@ -153,6 +154,8 @@ class QuantLinear(nn.Module):
         if self._perm is not None:
             x = ops.gather_columns(x, self._perm)
         y = ops.w4_linear(x, t)
+        if self._has_bias:  # qlinear_cuda_old.py:288-290
+            y = ops.add_bias(y, self.bias)
         return y if in_dtype == torch.bfloat16 else y.to(in_dtype)
 
     def extra_repr(self):

@@ -148,8 +148,13 @@ class OracleModel:
 
     def linear(self, prefix: str, x: torch.Tensor) -> torch.Tensor:
         """``nn.Linear`` without bias, or ``QuantLinear.forward``'s dequantise-then-matmul
-        (``AGQ:qlinear_cuda_old.py:284-290`` with the zero bias), result in the activation dtype."""
-        return (x.to(torch.float32) @ self._weight_kn_f32(prefix)).to(self.act)
+        (``AGQ:qlinear_cuda_old.py:284-290``: the product in the activation dtype, then ``+ bias`` when the
+        layer has a bias buffer), result in the activation dtype."""
+        y = (x.to(torch.float32) @ self._weight_kn_f32(prefix)).to(self.act)
+        b = self.w.get(prefix + ".bias")
+        if b is not None and prefix + ".qweight" in self.w:
+            y = (y.to(torch.float32) + b.to(torch.float32)).to(self.act)
+        return y
 
     def drop_cache(self):
         self._wf32.clear()
@@ -228,6 +233,7 @@ class OracleModel:
         past_key_values: Optional[Sequence[Tuple[torch.Tensor, torch.Tensor]]] = None,
         use_cache: bool = False,
         last_logits_only: bool = False,
+        attention_bias: Optional[torch.Tensor] = None,
     ) -> Tuple[torch.Tensor, Optional[List[Tuple[torch.Tensor, torch.Tensor]]]]:
         c = self.cfg
         B, T = input_ids.shape
@@ -240,12 +246,20 @@ class OracleModel:
             am = (1.0 - am) * _finfo_min(torch.float)
         else:
             am = None
-        if am is not None or past_key_values is not None:
-            # olmo/model.py:1343-1376 with causal_attention_bias (:375-381)
+        if am is not None or past_key_values is not None or attention_bias is not None:
+            # olmo/model.py:1343-1376 with causal_attention_bias (:375-381); an explicit bias replaces the
+            # causal one, and a bool / int8 one is turned into 1.0 / most-negative first (:1358-1360)
             L = past_len + T
-            bias = torch.triu(torch.ones(L, L, dtype=torch.float), diagonal=1)
-            bias = bias.masked_fill(bias == 1, _finfo_min(torch.float)).view(1, 1, L, L)
+            if attention_bias is None:
+                bias = torch.triu(torch.ones(L, L, dtype=torch.float), diagonal=1)
+                bias = bias.masked_fill(bias == 1, _finfo_min(torch.float)).view(1, 1, L, L)
+            elif attention_bias.dtype in (torch.int8, torch.bool):
+                bias = attention_bias.to(torch.float)
+                bias = bias.masked_fill(bias == 0.0, _finfo_min(torch.float))
+            else:
+                bias = attention_bias
             mask_len = am.shape[-1] if am is not None else L
+            bias = bias.to(torch.float)
             bias = bias[:, :, :mask_len, :mask_len]
             if am is not None:
                 bias = bias + am

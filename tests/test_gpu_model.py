@@ -148,6 +148,17 @@ def test_forward_parity_and_invariants(dev, kind, dtype, quantized):
     else:
         assert softmax_err(ll[1, 60:], rl[1, 60:]) <= 2e-2
     assert torch.isfinite(ll.float()).all()
+    # the rows of the padding tokens themselves: before the first real key a query sees masked keys only, and
+    # the reference then averages the values of *all* keys of the sequence (olmo/model.py:1371-1376)
+    if dtype == torch.float32:
+        assert torch.allclose(ll, rl, **tol) and torch.allclose(lb, rb, **tol)
+    else:  # no worse on the padding rows than on the real ones (a wrong average moves these logits by O(1))
+        def worst(a, b):
+            return (a.float() - b.float()).abs().max().item()
+
+        lreal, rreal = lmask.bool(), mask.bool()
+        assert softmax_err(ll, rl) <= 2e-2 and worst(ll[~lreal], rl[~lreal]) <= max(0.12, 2 * worst(ll[lreal], rl[lreal]))
+        assert softmax_err(lb, rb) <= 2e-2 and worst(lb[~rreal], rb[~rreal]) <= max(0.12, 2 * worst(lb[rreal], rb[rreal]))
 
     # (b) reference tests/model_test.py:196-199: cache == full forward, one token at a time
     o1 = model(ids[:, :140].to(dev), use_cache=True)
@@ -266,6 +277,129 @@ def test_quantlinear_module_surface(dev):
     assert ql3._perm is not None
     W3 = ow4.dequantize(qw, qz, sc, 128, (torch.arange(K) // 128).flip(0))
     assert torch.equal(ql3.dequantize().cpu().view(torch.int16), W3.view(torch.int16))
+
+
+@pytest.mark.parametrize("kind,dtype", [("olmo2", torch.bfloat16), ("ln", torch.float32)])
+def test_explicit_attention_bias(dev, kind, dtype):
+    """``attention_bias`` tensors (olmo/model.py:1343-1376): causal (float and bool), causal + padding, causal +
+    finite per-key penalties, against the oracle; rows of a cached step; ``OLMo.generate(attention_bias=...)``;
+    a bias that is not causal + per-key raises."""
+    say("explicit attention_bias", kind, dtype)
+    cfg = small_cfg(kind)
+    model, oracle = build_pair(cfg, dtype, dev, seed=41)
+    B, T, L = 2, 70, 96
+    ids = torch.randint(0, cfg.vocab_size, (B, T), generator=torch.Generator().manual_seed(42))
+    fmin = torch.finfo(torch.float32).min
+    causal = torch.triu(torch.full((L, L), fmin), diagonal=1).view(1, 1, L, L)
+
+    def close(a, b):
+        if dtype == torch.float32:
+            return torch.allclose(a, b, atol=2e-4, rtol=1e-4)
+        # logits of magnitude 2 in bf16: a wrong or missing bias moves them by more than 1 (asserted below)
+        return softmax_err(a, b) <= 2e-2 and (a.float() - b.float()).abs().max().item() <= 0.12
+
+    ref, _ = oracle.forward(ids)
+    assert close(model(ids.to(dev), attention_bias=causal.to(dev)).logits.cpu(), ref)
+    assert close(model(ids.to(dev), attention_bias=torch.tril(torch.ones(L, L, dtype=torch.bool)).view(1, 1, L, L)).logits.cpu(), ref)
+    # per-key penalties (finite) and one padded key per sequence, different per sequence
+    g = torch.Generator().manual_seed(43)
+    pen = torch.randn(B, L, generator=g) * 2.0
+    pen[0, 3], pen[1, 0] = fmin, fmin
+    full = causal + pen[:, None, None, :]
+    full = full.masked_fill(full == float("-inf"), fmin)
+    refb, _ = oracle.forward(ids, attention_bias=full)
+    assert (refb.float() - ref.float()).abs().max().item() > 1.0, "the penalties must matter"
+    got = model(ids.to(dev), attention_bias=full.to(dev), use_cache=True)
+    assert close(got.logits.cpu(), refb)
+    # with an attention_mask on top
+    mask = torch.ones(B, T)
+    mask[0, :5] = 0
+    refm, _ = oracle.forward(ids, attention_mask=mask, attention_bias=full)
+    gm = model(ids.to(dev), attention_mask=mask.to(dev), attention_bias=full.to(dev)).logits.cpu()
+    assert close(gm[:, 5:], refm[:, 5:])
+    # a cached step takes its own row; for one row any bias is per-key
+    nxt = torch.randint(0, cfg.vocab_size, (B, 1), generator=g)
+    _, okv = oracle.forward(ids, use_cache=True, attention_bias=full)
+    row = full.clone()
+    row[:, :, T, : T + 1] += torch.randn(B, 1, T + 1, generator=g)
+    ref1, _ = oracle.forward(nxt, past_key_values=okv, attention_bias=row)
+    got1 = model(nxt.to(dev), past_key_values=got.attn_key_values, attention_bias=row.to(dev)).logits.cpu()
+    assert close(got1, ref1)
+    # generate: the bias covers prompt + new tokens (olmo/model.py:1645-1657)
+    steps = 8
+    toks = model.generate(ids.to(dev), attention_bias=full[:, :, : T + steps, : T + steps].to(dev), max_steps=steps,
+                          stop_at_eos=False).token_ids[:, 0].cpu()
+    cur, kv, n_ok = ids, None, 0
+    seq = torch.cat([ids, toks], dim=1)
+    lg, _ = oracle.forward(seq[:, :-1], attention_bias=full)  # teacher-forced on the device's tokens
+    strict, loose = agreement(toks, lg[:, T - 1:])
+    assert loose >= 0.99, (strict, loose)
+    # not causal + per-key: ALiBi-like
+    alibi = causal + (torch.arange(L).view(1, L) - torch.arange(L).view(L, 1)).float().clamp(max=0).view(1, 1, L, L) * 0.1
+    with pytest.raises(NotImplementedError, match="causal"):
+        model(ids.to(dev), attention_bias=alibi.to(dev))
+    with pytest.raises(NotImplementedError, match="causal"):
+        model(ids.to(dev), attention_bias=torch.zeros(1, 1, L, L, device=dev))
+
+
+def test_quantlinear_bias(dev):
+    """A non-zero bias buffer is added after the product (qlinear_cuda_old.py:288-290): the module against the
+    oracle, and an int4 model whose four block Linears all carry one -- prefill and cached decode steps against the
+    oracle (such a model takes the plain per-layer launches; the fused decode forms hand over no bias)."""
+    from olmo_amd.qlinear import QuantLinear
+    from oracle import w4 as ow4
+
+    say("QuantLinear bias")
+    K, N = 256, 192
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=5)
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(6)) * 0.5).half()
+    ql = QuantLinear(4, 128, K, N, True).to(dev)
+    ql.load_state_dict({"qweight": qw, "qzeros": qz, "scales": sc, "g_idx": torch.arange(K, dtype=torch.int32) // 128,
+                        "bias": bias})
+    ql.post_init()
+    assert ql._has_bias
+    for M in (1, 7, 80):
+        x = torch.randn(M, K, generator=torch.Generator().manual_seed(M)).bfloat16()
+        prod = ow4.linear_fp32(x, ow4.dequantize(qw, qz, sc, 128)).bfloat16()
+        ref = (prod.float() + bias.float()).bfloat16()
+        y = ql(x.to(dev)).cpu()
+        assert (y.float() - ref.float()).abs().max().item() <= 2 ** -7 * ref.float().abs().max().item()
+        assert (y.float() - prod.float() - bias.float()).abs().max().item() <= 2 ** -6 * ref.float().abs().max().item()
+
+    cfg = small_cfg("olmo2")
+    w = om.random_weights(cfg, torch.bfloat16, seed=31, quantized=True, norm_weight_std=0.1)
+    g = torch.Generator().manual_seed(32)
+    for k in [k for k in w if k.endswith(".qweight")]:
+        w[k[:-8] + ".bias"] = (torch.randn(w[k].shape[1], generator=g) * 0.02).half()
+    oracle = om.OracleModel(cfg, w, torch.bfloat16)
+    from olmo_amd.model import OLMo
+    from olmo_amd.qlinear import OLMoGPTQForCausalLM, make_quant
+
+    model = OLMo(cfg, device=dev, dtype=torch.bfloat16, block_weight_device="meta")
+    make_quant(model, [f"transformer.blocks.{i}.{n}" for i in range(cfg.n_layers)
+                       for (n,) in OLMoGPTQForCausalLM.inside_layer_modules], 4, 128)
+    for m in model.modules():
+        if isinstance(m, QuantLinear):
+            m.to(dev)
+    model.load_reference_state_dict(w)
+    model.post_init()
+    assert model._act_order  # plain launches
+    ids = torch.randint(0, cfg.vocab_size, (2, 24), generator=torch.Generator().manual_seed(33))
+    ref, _ = oracle.forward(ids)
+    nobias = om.OracleModel(cfg, {k: v for k, v in w.items() if not k.endswith(".bias")}, torch.bfloat16).forward(ids)[0]
+    effect = (ref.float() - nobias.float()).abs().max().item()
+    assert effect > 1.0, "the bias must matter for this test to mean anything"
+
+    def close(a, b):  # a dropped bias moves the logits by `effect`
+        return softmax_err(a, b) <= 2e-2 and (a.float() - b.float()).abs().max().item() <= 0.2 * effect
+
+    out = model(ids.to(dev)[:, :20], use_cache=True)
+    assert close(out.logits.cpu(), ref[:, :20])
+    past = out.attn_key_values
+    for t in range(20, 24):
+        o = model(ids.to(dev)[:, t:t + 1], past_key_values=past, use_cache=True)
+        past = o.attn_key_values
+        assert close(o.logits.cpu(), ref[:, t:t + 1])
 
 
 def test_config1_fp32_20m_full(dev):

@@ -68,6 +68,46 @@ def test_oracle_cache_continuation_matches_transformers(kat, name):
         assert (logits[:, 0] - ref[:, t]).abs().max().item() <= TOL
 
 
+def _causal_bias(L, dtype):
+    """``causal_attention_bias`` of the reference (``olmo/model.py:375-381``) written out as data."""
+    if dtype == torch.bool:
+        return torch.tril(torch.ones(L, L, dtype=torch.bool)).view(1, 1, L, L)
+    return torch.triu(torch.full((L, L), torch.finfo(torch.float32).min), diagonal=1).view(1, 1, L, L)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bool])
+def test_explicit_attention_bias_against_transformers_logits(kat, dtype):
+    """The explicit-``attention_bias`` branch of the oracle's forward (``olmo/model.py:1343-1376``): the causal bias
+    passed as a tensor (float, and bool with 0 = masked -- allowed keys then carry +1.0, which a softmax does not
+    see) must give the stored logits of the independent model; with the padding mask folded into the tensor, the
+    stored left-padded logits; a transposed (anti-causal) tensor must not."""
+    name = "olmo2_gqa"
+    case, seed = R.CASES[name], R.seed_of(name)
+    w = R.to_olmo_state_dict(case, R.hf_state_dict(case, seed))
+    ids, mask = R.inputs(case, seed)
+    o = om.OracleModel(R.model_config(case), w, torch.float32)
+    L = R.SEQ + 4  # larger than needed: forward slices it (olmo/model.py:1367)
+    ref = torch.from_numpy(kat[name + ".logits"])
+    got, _ = o.forward(ids, attention_bias=_causal_bias(L, dtype))
+    assert (got - ref).abs().max().item() <= TOL
+    bad, _ = o.forward(ids, attention_bias=_causal_bias(L, dtype).transpose(-1, -2))
+    assert (bad - ref).abs().max().item() > 1000 * TOL
+    # padding folded into the bias tensor, per sequence
+    if dtype == torch.bool:
+        full = _causal_bias(R.SEQ, dtype) & mask.bool()[:, None, None, :]
+    else:
+        full = _causal_bias(R.SEQ, dtype) + ((1.0 - mask.float()) * torch.finfo(torch.float32).min)[:, None, None, :]
+        full = full.masked_fill(full == float("-inf"), torch.finfo(torch.float32).min)
+    got, _ = o.forward(ids, attention_bias=full)
+    refp = torch.from_numpy(kat[name + ".logits_left_padded"])
+    assert (got - refp).abs()[mask.bool()].max().item() <= TOL
+    # cached continuation: the rows of the new tokens are taken (olmo/model.py:627-635)
+    logits, kv = o.forward(ids[:, :16], use_cache=True, attention_bias=_causal_bias(L, dtype))
+    for t in range(16, 20):
+        logits, kv = o.forward(ids[:, t:t + 1], past_key_values=kv, use_cache=True, attention_bias=_causal_bias(L, dtype))
+        assert (logits[:, 0] - ref[:, t]).abs().max().item() <= TOL
+
+
 @pytest.mark.parametrize("name,wrong", [("olmo2_mha", "swap_up_gate"), ("olmo1", "swap_up_gate"),
                                         ("olmo2_gqa", "swap_norms")])
 def test_wrong_wiring_is_detected(kat, name, wrong):
