@@ -412,7 +412,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const void* __restrict
     const int64_t e = kb[it];
 #pragma unroll
     for (int v = 0; v < VW; ++v) vreg[it][v] = reinterpret_cast<const u32x4*>(vc)[e * VW / 8 + v];
-    bias[it] = key_bias ? key_bias[(int64_t)b * bias_stride + keyc] : 0.f;
+    // a row of key_bias holds bias_stride entries, which may be fewer than the rows the launch may touch
+    // (eager steps pass exactly past_len + 1): keys past the end of the row are past L and discarded below
+    bias[it] = key_bias ? key_bias[(int64_t)b * bias_stride + min(keyc, bias_stride - 1)] : 0.f;
   }
   float qr[8];
   Vec8<DT>::ld(q, ((int64_t)b * H + h) * HD + sub * 8, qr);
@@ -636,7 +638,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     vreg[it] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rv, lane * 16, min(kbase + it * KPI, rowcap) * HD * 2, 2));
-    bias[it] = key_bias ? key_bias[(int64_t)b * bias_stride + min(kbase + it * KPI + kslot, kmax)] : 0.f;
+    bias[it] = key_bias ? key_bias[(int64_t)b * bias_stride + min(min(kbase + it * KPI + kslot, kmax), bias_stride - 1)] : 0.f;  // keys past the row's end are past L
   }
 
   // ---- 2. QK-norm scale factors, rotary, the new cache row --------------------------------------------------
