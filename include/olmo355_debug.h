@@ -24,7 +24,9 @@ int olmo355_w4_gemv_form(const uint16_t* x, const uint32_t* wt, const uint16_t* 
                          int M, int N, int K, int form, void* stream);
 
 /* olmo355_attn_decode_fused with the merge of a head's key chunks given: -1 = choose, 0 = in the kernel (the last
- * workgroup of a (batch, head) to finish, found by a ticket), 2 = the separate combine kernel. */
+ * workgroup of a (batch, head) to finish, found by a ticket drawn after its stores have landed), 1 = in the kernel by
+ * the workgroup of the head's last chunk, which polls flag words stored together with the numbers (the writers
+ * wait for nothing), 2 = the separate combine kernel. */
 int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
                                     const float* cos_tab, void* kcache, void* vcache, const float* key_bias, void* out,
                                     void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos, int past_len,

@@ -337,6 +337,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
 // a wave covers 64/LPK keys per load instruction.  All K and V loads of the wave's 32 keys are
 // issued before the first use (the kernel is latency-bound at batch 1); the dot product is reduced
 // over the LPK lanes with DPP adds.
+constexpr int kFlagMergeFromChunks = 24;  // chunks per head from which "choose" takes the flag form of the in-kernel merge
+constexpr int kLLSpinLimit = 1 << 21;  // polls of the merging workgroup before it gives up (seconds)
 constexpr int kDecodeChunk = 128;
 constexpr int kDecodeKeysPerWave = 32;
 
@@ -546,7 +548,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     uint16_t* __restrict__ vc, const float* __restrict__ key_bias, float* __restrict__ ws, int H, int Hkv, int Lmax,
     int n_pos, int past_len, const int32_t* __restrict__ past_dev, int nchunks_max, int bias_stride, float eps,
     const float* __restrict__ qk_ssq, const float* __restrict__ rope_now, uint16_t* __restrict__ out,
-    int* __restrict__ tickets) {
+    int* __restrict__ tickets, int ll) {
   constexpr int LPK = HD / 8, KPI = 64 / LPK, ITERS = kDecodeKeysPerWave / KPI;
   constexpr int HALF = HD / 2, CPH = HD / 16;  // pair chunks per head
   constexpr int ROWS = 4 * KPI;                 // partial results of the workgroup: one per (wave, key slot)
@@ -556,8 +558,18 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   __shared__ __align__(16) float qs[HD];
   __shared__ __align__(16) u32x4 knew[HD / 8], vnew[HD / 8];
   __shared__ int s_last;
+  __shared__ uint32_t s_flag;
   const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z, gsz = H / Hkv, hk = h / gsz;
   const int tid = threadIdx.x, lane = tid & 63;
+  // ll (flags in the data): the workgroup of the head's last chunk merges.  Workgroups start in the order of their
+  // index (chunks of a head are consecutive), so when it runs all the others of its head have started, and since
+  // none of them ever waits they will finish; should that order ever not hold, its polling is bounded.  Every
+  // workgroup reads the launch counter of the head first, before any other request, so that waiting for it later
+  // waits for nothing else.  (Drawing a number per workgroup instead was measured: 17 device-scope read-modify-writes
+  // on one address take 6 us to drain.)
+  int my_epoch = 0;
+  if (ll && tid == 0)
+    my_epoch = __hip_atomic_load(tickets + 2 * (b * H + h) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int sub = lane % LPK, kslot = lane / LPK;
   const float scale = 1.f / sqrtf((float)HD);
@@ -706,7 +718,17 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   if (role_v) vnew[tid - 64] = vrow;
   // ---- the position is needed from here on ----------------------------------------------------------------
   const int L = pos + 1;
-  if (chunk * kDecodeChunk >= L || pos >= Lmax || pos >= n_pos || pos > kmax) return;  // whole workgroup
+  const bool bad_pos = pos >= Lmax || pos >= n_pos || pos > kmax;
+  bool merger = false, active = chunk * kDecodeChunk < L;
+  uint32_t flag = 0;  // what this launch writes next to every number of a partial: a NaN pattern no partial holds
+  if (ll) {
+    if (tid == 0) s_flag = 0x7FC00000u | ((uint32_t)(my_epoch + 1) & 0x3FFFFFu);
+    __syncthreads();
+    merger = chunk == nchunks_max - 1, flag = s_flag;
+    if (bad_pos || (!active && !merger)) return;  // an unusable position: nothing is computed, nothing to tidy up
+  } else if (!active || bad_pos) {
+    return;  // whole workgroup
+  }
   if (pos / kDecodeChunk == chunk && h % gsz == 0) {  // the chunk that holds the new position appends it
     if (role_k) {
       const int64_t o = cbase + (int64_t)pos * HD + j;
@@ -778,6 +800,75 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   if (!tickets) {  // partials merged by attn_decode_combine_kernel
     if (tid < HD) dst[tid] = ov;
     if (tid == 0) dst[HD] = mm, dst[HD + 1] = lv;
+    return;
+  }
+  if (ll) {
+    // ---- 4'. flags in the data.  A partial is (HD + 2) pairs (number, flag) written with 8-byte device-scope
+    // stores, so a reader that sees this launch's flag sees the number too: the writers do not wait for their
+    // stores, draw no second ticket and leave; the merging workgroup polls the pairs of the other chunks.
+    const int nact = min((L + kDecodeChunk - 1) / kDecodeChunk, nchunks_max);
+    uint64_t* w64 = reinterpret_cast<uint64_t*>(ws) + ((int64_t)b * H + h) * nchunks_max * (HD + 2);
+    auto pair_of = [&](float v) { return (uint64_t)__float_as_uint(v) | ((uint64_t)flag << 32); };
+    if (!merger) {
+      uint64_t* d64 = w64 + (int64_t)chunk * (HD + 2);
+      if (tid < HD) __hip_atomic_store(d64 + tid, pair_of(ov), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (tid == 0) {
+        __hip_atomic_store(d64 + HD, pair_of(mm), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(d64 + HD + 1, pair_of(lv), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      return;
+    }
+    if (tid == 0) red2[0][0] = mm, red2[0][1] = lv;  // this workgroup's own share stays on chip
+    __syncthreads();
+    if (tid >= HD) return;
+    float gm = active ? red2[0][0] : -INFINITY, go = active ? ov : 0.f, gl = active ? red2[0][1] : 0.f;
+    constexpr int UN = 8;
+    bool gave_up = false;
+    for (int c0 = 0; c0 < nact; c0 += UN) {
+      uint64_t po[UN], pm[UN], pl[UN];
+      for (int spins = 0;; ++spins) {
+        bool ok = true;
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+          const int c = c0 + u;
+          if (c < nact && !(active && c == chunk)) {
+            const uint64_t* pp = w64 + (int64_t)c * (HD + 2);
+            po[u] = __hip_atomic_load(pp + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            pm[u] = __hip_atomic_load(pp + HD, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            pl[u] = __hip_atomic_load(pp + HD + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+          const int c = c0 + u;
+          if (c < nact && !(active && c == chunk))
+            ok = ok && (uint32_t)(po[u] >> 32) == flag && (uint32_t)(pm[u] >> 32) == flag && (uint32_t)(pl[u] >> 32) == flag;
+        }
+        if (ok) break;
+        if (spins > kLLSpinLimit) { gave_up = true; break; }  // never seen: a writer that died; the result is marked
+        __builtin_amdgcn_s_sleep(1);
+      }
+      float rm = gm;
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int c = c0 + u;
+        if (c < nact && !(active && c == chunk)) rm = fmaxf(rm, __uint_as_float((uint32_t)pm[u]));
+      }
+      const float a = __expf(gm - rm);  // exp(-inf) = 0 while nothing has been merged yet
+      go *= a, gl *= a;
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int c = c0 + u;
+        if (c < nact && !(active && c == chunk)) {
+          const float wgt = __expf(__uint_as_float((uint32_t)pm[u]) - rm);
+          go += __uint_as_float((uint32_t)po[u]) * wgt, gl += __uint_as_float((uint32_t)pl[u]) * wgt;
+        }
+      }
+      gm = rm;
+    }
+    out[((int64_t)b * H + h) * HD + tid] = gave_up ? (uint16_t)0x7FC0 : f32_to_bf16_bits(go / gl);
+    if (tid == 0)  // the next launch's flag
+      __hip_atomic_store(tickets + 2 * (b * H + h) + 1, (int)(flag & 0x3FFFFFu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
   }
   // ---- 4. the last workgroup of a (batch, head) to finish merges the partials itself ---------------------
@@ -971,7 +1062,8 @@ extern "C" int olmo355_rope_advance(int32_t* pos, int delta, const float* sin_ta
 extern "C" int64_t olmo355_attn_decode_workspace_bytes(int B, int H, int hd, int n_keys_max) {
   if (B <= 0 || H <= 0 || hd <= 0 || n_keys_max <= 0) return 0;
   const int64_t nch = (n_keys_max + kDecodeChunk - 1) / kDecodeChunk;
-  return (int64_t)B * H * 4 + (int64_t)B * H * nch * (hd + 2) * 4;  // ticket counters, then the partials
+  // two counters per (batch, head), then the partials: (hd + 2) numbers per chunk, each with room for a flag word
+  return (int64_t)B * H * 8 + (int64_t)B * H * nch * (hd + 2) * 8;
 }
 
 namespace {
@@ -988,7 +1080,7 @@ int attn_decode_any(const void* q, const void* kcache, const void* vcache, const
     return O355_EINVAL;
   hipStream_t s = as_stream(stream);
 #define DECODE(DTv, HDv)                                                                                          \
-  return launch_decode<DTv, HDv>(q, kcache, vcache, key_bias, out, (float*)ws + (int64_t)B * H, B, H, Hkv, Lmax, past_len, \
+  return launch_decode<DTv, HDv>(q, kcache, vcache, key_bias, out, (float*)ws + (int64_t)2 * B * H, B, H, Hkv, Lmax, past_len, \
                                  past_len_dev, n_keys_max, bias_stride, beam_src, src_stride, prompt_len, beam, s)
   if (dtype == O355_BF16) {
     if (hd == 128) DECODE(O355_BF16, 128);
@@ -1067,15 +1159,16 @@ extern "C" int olmo355_attn_decode_static(const void* q, const void* kcache, con
                          bias_stride, nullptr, 0, 0, 1, dtype, stream);
 }
 
-// merge: how the key chunks of a (batch, head) are merged: -1 = choose, 0 = in the kernel (last workgroup of the
-// head, ticket), 2 = the separate combine kernel
+// merge: how the key chunks of a (batch, head) are merged: -1 = choose, 0 = in the kernel by the workgroup that
+// finishes last (a ticket drawn after its stores have landed), 1 = in the kernel by the workgroup of the head's last
+// chunk, which polls flags stored with the numbers, 2 = the separate combine kernel
 extern "C" int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
                                                const float* cos_tab, void* kcache, void* vcache, const float* key_bias,
                                                void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
                                                int past_len, const int32_t* past_len_dev, int n_keys_max,
                                                int bias_stride, float eps, const float* qk_ssq, const float* rope_now,
                                                int dtype, int merge, void* stream) {
-  if (merge != -1 && merge != 0 && merge != 2) return O355_EINVAL;
+  if (merge < -1 || merge > 2) return O355_EINVAL;
   if (!qkv || !sin_tab || !cos_tab || !kcache || !vcache || !out || !ws) return O355_EINVAL;
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || past_len < 0 || n_keys_max <= 0 || n_keys_max > Lmax)
     return O355_EINVAL;
@@ -1089,7 +1182,7 @@ extern "C" int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, 
   hipLaunchKernelGGL((attn_decode_fused_kernel<HDv, QVv>), dim3(nch, H, B), dim3(256), 0, s, (const uint16_t*)qkv,   \
                      (const uint16_t*)qw, (const uint16_t*)kw, sin_tab, cos_tab, (uint16_t*)kcache, (uint16_t*)vcache, \
                      key_bias, (float*)ws, H, Hkv, Lmax, n_pos, past_len, past_len_dev, nch, bias_stride, eps, qk_ssq, \
-                     rope_now, (uint16_t*)out, tickets);                                                                         \
+                     rope_now, (uint16_t*)out, tickets, ll);                                                                     \
   if (!tickets)                                                                                                        \
   hipLaunchKernelGGL((attn_decode_combine_kernel<O355_BF16, HDv>), dim3(H, B), dim3(HDv), 0, s, (const float*)ws, out, \
                      H, past_len, past_len_dev, nch)
@@ -1098,9 +1191,12 @@ extern "C" int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, 
   // (measured at the 7B shapes, context 2048: the in-kernel merge wins while the launch is a single round of
   // workgroups -- 17.0 against 20.4 us at batch 1 -- and loses once workgroups queue up -- 69.7 against 61.6 us
   // at batch 8, where one workgroup per (batch, head) takes 66.9)
-  const bool merge_in_kernel = merge == 0 || (merge < 0 && (int64_t)B * H * nch <= 1536);
+  const bool merge_in_kernel = merge == 0 || merge == 1 || (merge < 0 && (int64_t)B * H * nch <= 1536);
+  // (measured, batch 1: the flag form is level with the ticket form at 17 chunks per head -- 17.2 against 16.4 us,
+  // 7B at context 2048 -- and ahead from about two dozen -- 34.4 against 36.5 us, 13B at context 4090)
+  const int ll = merge_in_kernel && (merge == 1 || (merge < 0 && nch >= kFlagMergeFromChunks)) ? 1 : 0;  // needs the counters
   int* tickets = merge_in_kernel ? reinterpret_cast<int*>(ws) : nullptr;
-  ws = reinterpret_cast<float*>(ws) + (int64_t)B * H;
+  ws = reinterpret_cast<float*>(ws) + (int64_t)2 * B * H;
   const int qv = (H * hd / 8 + 255) / 256;
   if (hd == 128) {
     if (qv <= 1) { FUSED(128, 1); } else if (qv <= 2) { FUSED(128, 2); } else { FUSED(128, 4); }

@@ -667,7 +667,7 @@ def test_attn_decode_fused(dev, qknorm, B, past, H, Hkv, hd):
         assert torch.allclose(kc4[:, :, past].float(), kc[:, :, past].float(), rtol=2 ** -7, atol=2 ** -7)
 
 
-@pytest.mark.parametrize("merge", [0, 2])
+@pytest.mark.parametrize("merge", [0, 1, 2])
 @pytest.mark.parametrize("B,past,H,Hkv,hd", [(2, 300, 4, 2, 128), (8, 2048, 32, 32, 128), (1, 1000, 8, 8, 64)])
 def test_attn_decode_fused_both_merges(dev, merge, B, past, H, Hkv, hd):
     """Both ways of merging a head's key chunks (in the kernel by the last workgroup; partials + combine kernel),
