@@ -285,7 +285,7 @@ def main() -> int:
     m_s = e0.elapsed_time(e1) * 1e-3 / 5
     assert int(sink.abs().sum().item()) == 0
     extra["ceilings"]["stream_read_one_persistent_launch"] = {
-        "what": "the same 128 weight buffers (3.3 GB) read by one launch of a persistent grid (2 workgroups per CU)",
+        "what": "the same 128 weight buffers (3.3 GB) read by one launch of a grid that stays (2 workgroups per CU, 8 KiB in flight per wave at all times)",
         "ms": m_s * 1e3, "achieved": sum(sizes) / m_s / 1e9, "unit": "GB/s", "frac_of_peak": sum(sizes) / m_s / 1e9 / HBM_PEAK_GBS}
     log(f"[bench] ceiling on this box: one persistent launch streaming all weights: {m_s * 1e3:.3f} ms = {sum(sizes) / m_s / 1e9:.0f} GB/s")
 
@@ -509,10 +509,23 @@ def cpu_baseline(cfg, ctx: int):
     t_head = time.perf_counter() - ts
     t_token = per_layer * cfg.n_layers + t_head
     log(f"[bench] cpu baseline: {per_layer:.2f} s/layer, head {t_head:.2f} s -> {1.0 / t_token:.4f} tok/s")
+    # BASELINE configs[0] in full (the reference's own CPU-runnable case): 20M-style fp32 model, batch 4 x 512
+    from olmo_amd.config import PRESETS
+
+    c1 = PRESETS["olmo-20m"]
+    o1 = om.OracleModel(c1, om.random_weights(c1, torch.float32, seed=2), torch.float32)
+    ids1 = torch.randint(0, 50280, (4, 512), generator=torch.Generator().manual_seed(3))
+    t_c1 = []
+    for _ in range(2):
+        ts = time.perf_counter()
+        o1.forward(ids1)
+        t_c1.append(time.perf_counter() - ts)
+    log(f"[bench] cpu baseline: 20M fp32 model, forward on 4 x 512 tokens: {min(t_c1):.2f} s = {2048 / min(t_c1):.0f} tok/s")
     return {"value": 1.0 / t_token, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"{n_sample} of {cfg.n_layers} layers x 2 decode steps (best) at KV context {ctx}, batch 1, "
                       f"dequantise per call; scaled to {cfg.n_layers} layers + the bf16 head",
-            "os_cpu_count": os.cpu_count()}
+            "os_cpu_count": os.cpu_count(),
+            "config1_20m_fp32_forward_4x512": {"seconds": min(t_c1), "tokens_per_s": 2048 / min(t_c1), "sample": "in full, best of 2"}}
 
 
 if __name__ == "__main__":

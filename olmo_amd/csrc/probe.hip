@@ -28,8 +28,8 @@ __global__ __launch_bounds__(512) void stream_read_kernel(const u32x4* __restric
 }
 
 // The same for many buffers in ONE launch of a grid that stays (two workgroups per CU): the pieces of all buffers
-// form one sequence dealt round-robin to the waves, 8 requests in flight per wave.  No launch boundary, no ramp
-// per buffer: what the memory system sustains when nothing but streaming happens.
+// form one sequence dealt round-robin to the waves, 8 requests in flight per wave at all times.  No launch
+// boundary, no ramp per buffer: what the memory system sustains when nothing but streaming happens.
 constexpr int kManyMax = 160;
 struct ManyArgs {
   const u32x4* src[kManyMax];
@@ -43,20 +43,34 @@ __global__ __launch_bounds__(512) void stream_read_many_kernel(ManyArgs a, uint3
   const int64_t pieces = a.first_piece[a.n];
   uint32_t acc = 0;
   int b = 0;
-  // a wave's 8 requests are 8 consecutive KiB (a workgroup's: 64 KiB in a row), so a CU touches few pages at a time
-  for (int64_t p = wave * U; p < pieces; p += nw * U) {
-    u32x4 v[U];
+  // Piece q of the sequence belongs to wave q % nw: at any moment the grid reads one contiguous window.  A wave
+  // keeps U requests in flight all the time: the oldest is folded and its slot asked for the next piece at once
+  // (a loop that issues U and then waits for all of them has nothing in flight half of the time).
+  // the buffer of the current piece is kept in registers and looked up again only when q leaves it (q grows
+  // monotonically and is wave-uniform): the table is a kernel argument indexed at run time, not something to
+  // touch per request
+  int64_t cur_first = 0, cur_end = a.first_piece[1];
+  const u32x4* cur = a.src[0];
+  auto request = [&](int64_t q) {
+    u32x4 v = u32x4{0u, 0u, 0u, 0u};
+    if (q < pieces) {
+      while (q >= cur_end) {
+        ++b;
+        cur_first = a.first_piece[b], cur_end = a.first_piece[b + 1], cur = a.src[b];
+      }
+      v = __builtin_nontemporal_load(&cur[(q - cur_first) * 64 + lane]);
+    }
+    return v;
+  };
+  u32x4 v[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) v[u] = request(wave + u * nw);
+  for (int64_t p = wave; p < pieces; p += nw * U) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t q = p + u;
-      v[u] = u32x4{0u, 0u, 0u, 0u};
-      if (q < pieces) {
-        while (q >= a.first_piece[b + 1]) ++b;  // wave-uniform; q grows monotonically
-        v[u] = __builtin_nontemporal_load(&a.src[b][(q - a.first_piece[b]) * 64 + lane]);
-      }
+      acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+      v[u] = request(p + (U + u) * nw);
     }
-#pragma unroll
-    for (int u = 0; u < U; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
   }
   if (acc == 0x9e3779b9u) sink[threadIdx.x] = acc;
 }

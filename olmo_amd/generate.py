@@ -123,7 +123,20 @@ def greedy_generate(model, input_ids: torch.Tensor, attention_mask: Optional[tor
     sess = DecodeSession(model, cache, first, key_bias_full, sampling)
     tokens = torch.empty(B, max_new_tokens, dtype=torch.int64, device=model.device)
     tokens[:, 0] = sess.ids.view(B)
-    all_logits = [out.logits[:, -1].clone()] if (return_scores or return_logits) else None
+    all_logits = [out.logits[:, -1].clone()] if return_logits else None
+    # scores: the chosen token's log-probability per step.  The logits of a step are kept only until a batch of
+    # steps has been turned into those numbers (a [B, 64, V] block at a time, not steps x V for the whole run)
+    tok_lp = torch.zeros(B, max_new_tokens, dtype=torch.float32, device=model.device) if return_scores else None
+    pending = [(0, out.logits[:, -1].clone())] if return_scores else []
+
+    def settle():
+        if not pending:
+            return
+        idx = torch.tensor([i for i, _ in pending], device=model.device)
+        lp = torch.log_softmax(torch.stack([l for _, l in pending], dim=1).float(), dim=-1)
+        tok_lp[:, idx] = lp.gather(-1, tokens[:, idx].unsqueeze(-1)).squeeze(-1)
+        pending.clear()
+
     steps = max_new_tokens
     for i in range(1, max_new_tokens):
         if stop_when_all_ended and eos_token_id is not None and i % 16 == 0:
@@ -138,6 +151,11 @@ def greedy_generate(model, input_ids: torch.Tensor, attention_mask: Optional[tor
         tokens[:, i] = sess.ids.view(B)
         if all_logits is not None:
             all_logits.append(sess.logits.view(B, -1).clone())
+        if return_scores:
+            pending.append((i, sess.logits.view(B, -1).clone()))
+            if len(pending) >= 64:
+                settle()
+    settle()
     tokens = tokens[:, :steps]
     result = [tokens]
     after = None
@@ -154,8 +172,7 @@ def greedy_generate(model, input_ids: torch.Tensor, attention_mask: Optional[tor
         # log-probability bookkeeping of the search (olmo/model.py:1705, beam_search.py:1003-1019);
         # not on the timed path, so plain torch on the saved logits.  An ended sequence adds nothing
         # (beam_search.py:948-957: the forced end token has log-probability 0).
-        lp = torch.stack([torch.log_softmax(l.float(), dim=-1) for l in all_logits[: tokens.shape[1]]], dim=1)
-        tok_lp = lp.gather(-1, tokens.clamp_min(0).unsqueeze(-1)).squeeze(-1)
+        tok_lp = tok_lp[:, : tokens.shape[1]]  # of the tokens as generated (the padding written over them adds nothing)
         if after is not None:
             tok_lp = tok_lp.masked_fill(after, 0.0)
         result.append(tok_lp.sum(dim=1))
