@@ -55,7 +55,7 @@ def test_argument_checks_return_status_without_launching():
     assert h.olmo355_w4_dequant_fp16(None, None, None, None, None, 8, 8, 8, None) == 1
     assert h.olmo355_rmsnorm(None, None, None, None, 1, 8, 1e-6, 1, None) == 1
     # workspace sizing is pure host arithmetic
-    assert h.olmo355_attn_decode_workspace_bytes(1, 32, 128, 2048) == 32 * 16 * 130 * 4 + 32 * 4
+    assert h.olmo355_attn_decode_workspace_bytes(1, 32, 128, 2048) == 32 * 16 * 130 * 8 + 32 * 8
 
 
 def test_ops_refuse_cpu_tensors():
