@@ -228,6 +228,25 @@ def main() -> int:
     extra["prefill_gemm"] = {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
                              "frac": tf / MFMA_BF16_PEAK_TF, "M": ctx}
     log(f"[bench] int4 prefill GEMMs (M={ctx}): {tf:.0f} TFLOP/s = {tf / MFMA_BF16_PEAK_TF:.1%} of bf16 MFMA peak")
+    # yardstick: the vendor library's *dense* bf16 GEMM (torch.matmul -> hipBLASLt) on the same four shapes at the
+    # same M, nothing to dequantise: what a tuned library reaches at this size on this box
+    wd = [torch.randn(n, k, device=dev).to(torch.bfloat16) * 0.02 for n, k in shapes]
+    for wmat in wd:
+        torch.matmul(xp[wmat.shape[1]], wmat.t())
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(3):
+        for wmat in wd:
+            torch.matmul(xp[wmat.shape[1]], wmat.t())
+    e1.record()
+    torch.cuda.synchronize()
+    tf_lib = flops * 3 / (e0.elapsed_time(e1) * 1e-3) / 1e12
+    del wd
+    extra["prefill_gemm"]["vendor_library_dense_bf16_same_shapes"] = {
+        "what": "torch.matmul (hipBLASLt) on dense bf16 weights of the same four shapes at the same M", "achieved": tf_lib,
+        "unit": "TFLOP/s", "frac": tf_lib / MFMA_BF16_PEAK_TF}
+    log(f"[bench] yardstick: vendor library, dense bf16 GEMMs of the same shapes (M={ctx}): {tf_lib:.0f} TFLOP/s = "
+        f"{tf_lib / MFMA_BF16_PEAK_TF:.1%} of bf16 MFMA peak")
     # ---- what this box gives a kernel that only streams the same weights / only issues MFMAs ----------
     # Same launches as above (one per block Linear, distinct buffers, one captured graph), but the kernel reads
     # the tiled weight bytes and does nothing else: the distance from here to the published 8 TB/s is not the
