@@ -407,6 +407,38 @@ def linear_sweep(dev) -> int:
             rows.append(row)
             log(f"[sweep] M={m:5d} N={n:6d} K={k:5d}: {us:9.2f} us  {row['achieved']:8.1f} {row['unit']:8s} {row['frac']:6.1%}")
         del tiles
+        # yardstick beside each cell: the vendor library's dense bf16 product of the same shape (torch.matmul ->
+        # hipBLASLt; four times the weight bytes, nothing to dequantise), same rotation over >= 2 GB of copies
+        nd = int(min(64, max(3, -(-2e9 // (2.0 * n * k)))))
+        dense = [torch.randn(n, k, device=dev).to(torch.bfloat16) * 0.02 for _ in range(nd)]
+        for m in (1, 8, 64, 512, 4096):
+            x = torch.randn(m, k, device=dev).to(torch.bfloat16)
+
+            def run_lib():
+                for wmat in dense:
+                    torch.matmul(x, wmat.t())
+
+            run_lib()
+            run_lib()
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                run_lib()
+            g.replay()
+            torch.cuda.synchronize()
+            reps = 5 if m <= 64 else 2
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            us_lib = e0.elapsed_time(e1) * 1e3 / (reps * nd)
+            for row in rows:
+                if (row["M"], row["N"], row["K"]) == (m, n, k):
+                    row["vendor_dense_bf16_us"] = us_lib
+            log(f"[sweep] M={m:5d} N={n:6d} K={k:5d}: vendor library, dense bf16: {us_lib:9.2f} us")
+        del dense
     print(json.dumps(rows))
     return 0
 
