@@ -238,17 +238,22 @@ class OLMoForCausalLM(*_ModelBase):
     supports_gradient_checkpointing = False  # inference only
 
     def __init__(self, config: OLMoConfig, model: Optional[OLMo] = None, init_params: bool = False, device="cuda",
-                 dtype: torch.dtype = torch.bfloat16, **model_kwargs):
+                 dtype: Optional[torch.dtype] = None, **model_kwargs):
         if HAVE_TRANSFORMERS:
             super().__init__(config)
         else:
             super().__init__()
             self.config = config
         if model is None:
+            if dtype is None:  # what the directory being loaded says (``from_pretrained``), else bfloat16
+                dtype = getattr(config, "dtype", None)
+                dtype = dtype if dtype in (torch.bfloat16, torch.float32) else torch.bfloat16
             model = OLMo(config.to_model_config(), device=device, dtype=dtype, **model_kwargs)
             if init_params:
                 model.reset_parameters()
         self.model = model
+        if HAVE_TRANSFORMERS:
+            self.post_init()  # transformers' own bookkeeping (tied-weight keys, parallel plans); initialises nothing here
 
     # ------------------------------------------------------------------------------------------
     def forward(

@@ -246,6 +246,10 @@ class OLMo(nn.Module):
 
     def post_init(self) -> "OLMo":
         """Build the kernel-side weight layouts, rotary tables (idempotent)."""
+        # a loader that swaps parameters in (transformers' ``from_pretrained`` without a device map leaves them in
+        # host memory) is followed here: everything the kernels read lives on this model's GPU
+        if any(t.device.type not in (self.device.type, "meta") for t in list(self.parameters()) + list(self.buffers())):
+            self.to(self.device)
         for m in self.modules():
             if isinstance(m, (DenseLinear, QuantLinear)) and m is not self:
                 if isinstance(m, DenseLinear) and m.weight.device.type == "meta":

@@ -82,6 +82,25 @@ def test_is_a_transformers_model_and_registered():
     assert H.OLMoForCausalLM.can_generate() and H.OLMoForCausalLM._no_split_modules == ["OLMoBlock"]
 
 
+def test_config_save_and_load(tmp_path):
+    """``tests/hf_olmo/configuration_olmo_test.py:6-19``: ``save_pretrained`` / ``from_pretrained`` keep every
+    ``ModelConfig`` field, a non-default one included."""
+    from dataclasses import asdict
+
+    from olmo_amd.config import ModelConfig
+
+    mc = ModelConfig(d_model=128, n_heads=4, rope=True, rope_theta=500000, clip_qkv=8.0)
+    d = asdict(mc)
+    d.pop("extra", None)
+    cfg = H.OLMoConfig(**d)
+    cfg.save_pretrained(tmp_path)
+    loaded = H.OLMoConfig.from_pretrained(tmp_path)
+    assert cfg.to_dict() == loaded.to_dict()
+    for k, v in d.items():
+        assert getattr(loaded, k) == v, k
+    assert loaded.to_model_config() == mc and loaded.model_type == "hf_olmo"
+
+
 @pytest.mark.parametrize("name", ["olmo2_gqa", "olmo1_clip"])
 def test_transformers_greedy_loop_matches_independent_model(name):
     case, seed, ours, theirs, core = wrapped(name)
@@ -219,3 +238,27 @@ def test_gpu_foreign_dynamic_cache_is_taken_over():
     c.reorder_cache(torch.tensor([1, 2, 0], device="cuda"))
     out3 = ours(ids[[1, 2, 0], 8:12], past_key_values=c, use_cache=True)
     assert (out3.logits - full[[1, 2, 0], 8:12]).abs().max() < 2e-4
+
+
+@pytest.mark.gpu
+def test_gpu_save_pretrained_from_pretrained(tmp_path):
+    """A directory written by ``save_pretrained`` loads back through ``OLMoForCausalLM.from_pretrained`` and through
+    ``AutoModelForCausalLM`` (the registration of ``modeling_olmo.py:261``) with identical logits -- what
+    ``tests/hf_olmo/modeling_olmo_test.py:9-26`` does with the reference's fixture checkpoint (whose weight file does
+    not ship)."""
+    from olmo_amd.model import OLMo
+
+    case, seed = R.CASES["olmo2_gqa"], R.seed_of("olmo2_gqa")
+    cfg = R.model_config(case)
+    model = OLMo(cfg, device="cuda", dtype=torch.float32, max_cache_len=64)
+    model.load_reference_state_dict(R.to_olmo_state_dict(case, R.hf_state_dict(case, seed)))
+    hf = H.OLMoForCausalLM(H.OLMoConfig.from_model_config(cfg, use_cache=True), model=model)
+    ids, _ = R.inputs(case, seed)
+    ids = ids.cuda()
+    want = hf(ids).logits
+    hf.save_pretrained(tmp_path)
+    for cls in (H.OLMoForCausalLM, transformers.AutoModelForCausalLM):
+        back = cls.from_pretrained(tmp_path, dtype=torch.float32)
+        assert isinstance(back, H.OLMoForCausalLM)
+        got = back(ids).logits
+        assert torch.equal(got, want)
