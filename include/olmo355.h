@@ -101,7 +101,9 @@ int olmo355_w4_gemv_chain(const uint16_t* x, const uint16_t* resid, const uint16
 
 /* Large-M path: dequantise tiles into LDS as bf16 and multiply on the matrix cores.  Stands
  * in for the reference's dequantise-then-matmul branch (AGQ qlinear_cuda_old.py:236-287) and
- * exllama's reconstruct + cublasHgemm (exllama/cuda_func/q4_matmul.cu:222-260). */
+ * exllama's reconstruct + cublasHgemm (exllama/cuda_func/q4_matmul.cu:222-260).
+ * The matrix-core entries (this one, olmo355_b16_gemm, the split-K and SwiGLU forms) write 16 bytes at a time:
+ * y (and the split-K workspace) must be 16-byte aligned, O355_EINVAL otherwise; N % 16 == 0 keeps every row so. */
 int olmo355_w4_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
                     int M, int N, int K, void* stream);
 /* Split-K forms of olmo355_w4_gemm / olmo355_b16_gemm for launches with fewer output tiles than CUs (prompts of

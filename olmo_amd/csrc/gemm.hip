@@ -8,10 +8,13 @@
 // three stages requested two stages ahead.  Weights are staged in LDS in *fragment-major* order
 // -- [32-column tile][k-step of 16][64 lanes][16 bytes] -- so every MFMA operand is one conflict-free
 // ds_read_b128; int4 words come into registers two stages ahead and are dequantised (scale and zero
-// in fp32, one rounding to bf16) into LDS one stage ahead, double-buffered; dense weights are copied
+// in fp32, one rounding to bf16) into LDS ahead of their stage, double-buffered; dense weights are copied
 // memory -> LDS as they are tiled.  The staging work is spread between the k-steps of the MFMA loop so
-// that the VALU / LDS / memory instructions issue in the shadow of the matrix pipeline; one barrier per
-// stage.
+// that the VALU / LDS / memory instructions issue in the shadow of the matrix pipeline; operand fragments are
+// read one k-step ahead of the matrix instructions that use them; one barrier per stage, after its third
+// k-step.  The matrix instructions take the weight fragment as their first operand, so the accumulators hold
+// the output tile transposed (a lane owns runs of neighbouring columns of one row) and the epilogue writes 16
+// bytes per lane and store.
 //
 // The int4 operand is W = bf16(scale * (q - zero)) (fp32 product, one rounding).
 #include "common.h"
@@ -25,17 +28,34 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 constexpr int BK = 64;      // K per stage
 constexpr int KSTEPS = 4;   // MFMA k-steps of 16 per stage
 
-// dequantise one tiled word (8 weights of one column) to 8 bf16 in MFMA operand order
-__device__ __forceinline__ u32x4 dequant_word_bf16(uint32_t w, float s, float c) {
-  // c = -(128 + zero) * s ; value = (128+q)*s + c = s*(q - zero), single fp32 rounding of the fma
+// dequantise one tiled word (8 weights of one column) to 8 bf16 in MFMA operand order.
+// The nibbles are turned into fp16 numbers where they stand: (w & 0x000f000f) | 0x64006400 is the pair
+// (1024 + q_lo, 1024 + q_hi), and the same with the mask one nibble up the pair (1024 + 16 q); a mixed-precision
+// fma takes either half as it is.  s * (1024 + q) + c0 with c0 = -(1024 + zero) * s, and (s / 16) * (1024 + 16 q)
+// + c1 with c1 = -(64 + zero) * s: every product and sum is exact in fp32 (11 x 11 bits), so the value is
+// s * (q - zero) with the single rounding to bf16 at the end.
+struct DequantConsts { float s, c0, s16, c1; };
+__device__ __forceinline__ DequantConsts dequant_consts(float s, int zero) {
+  return {s, -(float)(1024 + zero) * s, s * 0.0625f, -(float)(64 + zero) * s};
+}
+__device__ __forceinline__ u32x4 dequant_word_bf16(uint32_t w, const DequantConsts& d) {
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  auto pair = [](uint32_t p, float sm, float cm) {
+    const f16x2 h = __builtin_bit_cast(f16x2, p);
+    return pack_bf16x2(__builtin_fmaf((float)h[0], sm, cm), __builtin_fmaf((float)h[1], sm, cm));
+  };
+  // (w & mask) | magic in one instruction: it takes one scalar operand only, so the magic sits in a vector register
+  auto and_or = [](uint32_t v, uint32_t mask, uint32_t magic) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "s"(mask), "v"(magic));
+    return r;
+  };
+  const uint32_t w8 = w >> 8, magic = 0x64006400u;
   u32x4 o;
-#pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const uint32_t p = ((w >> (4 * t)) & 0x000f000fu) | 0x43004300u;
-    const float lo = __builtin_fmaf(bf16lo_to_f32(p), s, c);
-    const float hi = __builtin_fmaf(bf16hi_to_f32(p), s, c);
-    o[t] = pack_bf16x2(lo, hi);
-  }
+  o[0] = pair(and_or(w, 0x000f000fu, magic), d.s, d.c0);
+  o[1] = pair(and_or(w, 0x00f000f0u, magic), d.s16, d.c1);
+  o[2] = pair(and_or(w8, 0x000f000fu, magic), d.s, d.c0);
+  o[3] = pair(and_or(w8, 0x00f000f0u, magic), d.s16, d.c1);
   return o;
 }
 
@@ -173,8 +193,8 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     const int slot = (kq & 1) * 32 + (ntl & 1) * 16 + (lane & 15);
     const int f = (ntl >> 1) * KSTEPS + 2 * (j & 1) + (kq >> 1);
     const float sc = (float)__builtin_bit_cast(_Float16, (uint16_t)rsb[set][i]);
-    const float cc = -(float)(129 + (int)((rzb[set][i] >> (4 * (lane & 1))) & 15u)) * sc;
-    lds_b[(buf * B_BLK + f) * 64 + slot] = dequant_word_bf16(rbw[set][i][j], sc, cc);
+    const DequantConsts dc = dequant_consts(sc, 1 + (int)((rzb[set][i] >> (4 * (lane & 1))) & 15u));  // stored zero points are one less
+    lds_b[(buf * B_BLK + f) * 64 + slot] = dequant_word_bf16(rbw[set][i][j], dc);
   };
   // dense: the tiled pieces [16-column tile][32-row step][64][16 B] are copied as they are
   int bd_voff[W4 ? 1 : B_PW];
@@ -196,6 +216,10 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   const int b_rd = W4 ? lane : (row32 >> 4) * 128 + (row32 & 15) + 16 * kh;
   auto b_slot = [&](int ct, int ks) { return W4 ? (ct * KSTEPS + ks) * 64 : ct * 256 + (ks >> 1) * 64 + (ks & 1) * 32; };
 
+  // requests of a stage issued in its first three k-steps (those after them are the next stage's business)
+  constexpr int keep_a = [] { int n = 0; for (int i = 0; i < A_PW; ++i) n += (i * KSTEPS / A_PW <= KSTEPS - 2); return n; }();
+  constexpr int keep_b = [] { int n = 0; for (int i = 0; i < NBI; ++i) n += ((2 * i + 1) * KSTEPS / (2 * NBI) <= KSTEPS - 2); return n; }();
+
   f32x16 acc[WMT][WNT];
 #pragma unroll
   for (int i = 0; i < WMT; ++i)
@@ -204,57 +228,92 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  bf16x8 fa[WMT], fb[WNT];
-  auto load_frags = [&](int abuf, int bbuf, int ks) {
-    const u32x4* a = lds_a + abuf * A_BLK * 64;
-    const u32x4* b = lds_b + bbuf * B_BLK * 64;
-#pragma unroll
-    for (int i = 0; i < WMT; ++i) fa[i] = __builtin_bit_cast(bf16x8, a[(wm * WMT + i) * 256 + a_rd[ks]]);
-#pragma unroll
-    for (int j = 0; j < WNT; ++j) fb[j] = __builtin_bit_cast(bf16x8, b[b_slot(wn * WNT + j, ks) + b_rd]);
+  // Operand fragments are read one k-step ahead.  The operand with fewer fragments per wave is double-buffered
+  // in registers; a fragment of the other one is asked for again as soon as the matrix instructions that read
+  // its registers have been issued.
+  constexpr bool OUTER_A = WNT <= WMT;
+  bf16x8 fa[OUTER_A ? 1 : 2][WMT], fb[OUTER_A ? 2 : 1][WNT];
+  auto read_a = [&](int abuf, int i, int ks) {
+    return __builtin_bit_cast(bf16x8, lds_a[abuf * A_BLK * 64 + (wm * WMT + i) * 256 + a_rd[ks]]);
   };
-  auto mfmas = [&]() {
-#pragma unroll
-    for (int i = 0; i < WMT; ++i)
-#pragma unroll
-      for (int j = 0; j < WNT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+  auto read_b = [&](int bbuf, int j, int ks) {
+    return __builtin_bit_cast(bf16x8, lds_b[bbuf * B_BLK * 64 + b_slot(wn * WNT + j, ks) + b_rd]);
   };
   auto ring_next = [](int ab) { return ab == 2 ? 0 : ab + 1; };
+  // int4: a thread's 2 * B_ITEMS words of a stage are dequantised in the four k-steps before the barrier that
+  // publishes the stage: slot 0 = the last k-step of the stage before the previous one's barrier ... see do_stage
+  auto word_slot = [](int i) { return i * KSTEPS / (2 * B_ITEMS); };
 
   // One stage.  Activations sit in a ring of three LDS buffers and are requested two stages ahead;
   // the weights are double-buffered in LDS (int4: requested two stages ahead into registers, set
-  // = parity of the 128-row group, and dequantised into LDS one stage ahead; dense: copied one stage
-  // ahead).  Memory operations complete in order, so waiting until only this stage's own requests
-  // (KEEP of them) are outstanding means everything the next stage reads has landed.
+  // = parity of the 128-row group, and dequantised into LDS ahead of their stage; dense: copied one stage
+  // ahead).  The stage's one barrier stands after its third k-step: by then every wave has read the stage's last
+  // fragments, so the buffers of this stage may be written again, and everything of the next stage is in LDS, so
+  // the last k-step reads the next stage's first fragments.  Memory operations complete in order, so waiting until
+  // only the requests of this stage's first three k-steps (KEEP of them) are outstanding means that everything the
+  // next stage reads has landed.
   //   h = parity of the stage = weight LDS buffer (and, int4, the half of the group)
   //   p = parity of the group (int4 register set)
   auto do_stage = [&](int s, int ab, auto hc, auto pc) {
     constexpr int h = decltype(hc)::value, p = decltype(pc)::value;
     const int s2 = min(s + 2, stages - 1);  // past the end: re-fetch the last stage into a buffer nobody reads
-    const int ab2 = ring_next(ring_next(ab));
+    const int ab1 = ring_next(ab), ab2 = ring_next(ab1);
     if constexpr (!W4) {
       load_b_dense(min(s + 1, stages - 1), h ^ 1);
       __builtin_amdgcn_sched_barrier(0);  // keep the order: the weights' requests are the older ones
     }
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
-      load_frags(ab, h, ks);
+      const int cur = ks & 1, nxt = cur ^ 1, nks = (ks + 1) & (KSTEPS - 1);
+      const int nab = ks == KSTEPS - 1 ? ab1 : ab, nh = ks == KSTEPS - 1 ? (h ^ 1) : h;
+      if constexpr (OUTER_A) {
+#pragma unroll
+        for (int j = 0; j < WNT; ++j) fb[nxt][j] = read_b(nh, j, nks);
+      } else {
+#pragma unroll
+        for (int i = 0; i < WMT; ++i) fa[nxt][i] = read_a(nab, i, nks);
+      }
       // requests are spread over the stage: a burst of them stalls the wave at issue
       load_a(s2, ab2, ks);
       if constexpr (W4 && h == 1) fetch_b(min((s >> 1) + 2, Gn - 1), p, ks);
       __builtin_amdgcn_sched_barrier(0);
-      mfmas();
-      if constexpr (W4) {
-        // next stage's words: second half of this group (h == 0) or first half of the next (h == 1)
+      if constexpr (OUTER_A) {
 #pragma unroll
-        for (int i = 0; i < 2 * B_ITEMS; ++i)
-          if (i * KSTEPS / (2 * B_ITEMS) == ks) stash_b_word(h ^ 1, p ^ h, i >> 1, 2 * (h ^ 1) + (i & 1));
+        for (int i = 0; i < WMT; ++i) {
+#pragma unroll
+          for (int j = 0; j < WNT; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[0][i], acc[i][j], 0, 0, 0);
+          fa[0][i] = read_a(nab, i, nks);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < WNT; ++j) {
+#pragma unroll
+          for (int i = 0; i < WMT; ++i)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[0][j], fa[cur][i], acc[i][j], 0, 0, 0);
+          fb[0][j] = read_b(nh, j, nks);
+        }
+      }
+      if constexpr (W4) {
+#pragma unroll
+        for (int i = 0; i < 2 * B_ITEMS; ++i) {
+          if (ks < KSTEPS - 1) {
+            // next stage's words: second half of this group (h == 0) or first half of the next (h == 1)
+            if (word_slot(i) == ks + 1) stash_b_word(h ^ 1, p ^ h, i >> 1, 2 * (h ^ 1) + (i & 1));
+          } else {
+            // after the barrier: first words of the stage after the next (same half, next group) into this stage's buffer
+            if (word_slot(i) == 0) stash_b_word(h, p ^ 1, i >> 1, 2 * h + (i & 1));
+          }
+        }
+      }
+      if (ks == KSTEPS - 2) {
+        constexpr int KEEP = keep_a + ((W4 && h == 1) ? 3 * keep_b : 0);
+        static_assert(KEEP < 64, "vmcnt range");
+        __builtin_amdgcn_s_waitcnt((KEEP & 15) | ((KEEP >> 4) << 14) | 0x0070);  // vmcnt(KEEP) lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
-    constexpr int KEEP = A_PW + ((W4 && h == 1) ? 3 * NBI : 0);
-    static_assert(KEEP < 64, "vmcnt range");
-    __builtin_amdgcn_s_waitcnt((KEEP & 15) | ((KEEP >> 4) << 14) | 0x0070);  // vmcnt(KEEP) lgkmcnt(0)
-    __builtin_amdgcn_s_barrier();
   };
 
   // ---- prologue: stages 0 and 1 of the activations, stage 0 of the weights -----------------------
@@ -264,12 +323,19 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     fetch_b(0, 0);
 #pragma unroll
     for (int i = 0; i < 2 * B_ITEMS; ++i) stash_b_word(0, 0, i >> 1, i & 1);
+#pragma unroll
+    for (int i = 0; i < 2 * B_ITEMS; ++i)
+      if (word_slot(i) == 0) stash_b_word(1, 0, i >> 1, 2 + (i & 1));  // what the k-step before stage 0 would have done
     fetch_b(min(1, Gn - 1), 1);
   } else {
     load_b_dense(0, 0);
   }
   __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
   __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int i = 0; i < WMT; ++i) fa[0][i] = read_a(0, i, 0);
+#pragma unroll
+  for (int j = 0; j < WNT; ++j) fb[0][j] = read_b(0, j, 0);
 
   using H0 = std::integral_constant<int, 0>;
   using H1 = std::integral_constant<int, 1>;
@@ -294,35 +360,75 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     }
   }
 
-  // ---- epilogue: D[m = 8*(r/4) + 4*(lane>>5) + r%4][n = lane&31] of each 32x32 tile ---------------------
+  // ---- epilogue ------------------------------------------------------------------------------------------
+  // The products were formed as W^T-tile x X^T-tile, so a lane holds one output row m = lane & 31 of its 32 x 32
+  // block and the columns n = 8 q + 4 (lane >> 5) + (r & 3) in register r = 4 q + (r & 3): four neighbours in a
+  // row per register quad.  As bf16 pairs, the quads q = 0, 1 (and 2, 3) of the two half-waves are exchanged so that
+  // every lane ends up with 8 neighbouring columns: two 16-byte stores per block and lane instead of sixteen
+  // 2-byte ones.
+  const int half = lane >> 5, mrow = lane & 31;
+  auto store_block = [&](const uint32_t (&pk)[4][2], uint16_t* __restrict__ dst, int m, int nb, int ncols, int ld) {
+    uint32_t o[4][2];
+#pragma unroll
+    for (int qq = 0; qq < 4; qq += 2)
+#pragma unroll
+      for (int x = 0; x < 2; ++x) {
+        const auto sw = __builtin_amdgcn_permlane32_swap(pk[qq][x], pk[qq + 1][x], false, false);
+        o[qq][x] = sw[0], o[qq + 1][x] = sw[1];
+      }
+#pragma unroll
+    for (int qq = 0; qq < 4; qq += 2) {
+      const int n = nb + 8 * qq + 8 * half;
+      if (m < M && n < ncols)
+        *reinterpret_cast<u32x4*>(dst + (int64_t)m * ld + n) = u32x4{o[qq][0], o[qq][1], o[qq + 1][0], o[qq + 1][1]};
+    }
+  };
   if constexpr (SWIGLU) {
     const int half_n = N >> 1;
-    const int n = tile_n * (BN / 2) + wn * 32 + (lane & 31);  // no ragged columns: N/2 is a multiple of BN/2
+    const int nb = tile_n * (BN / 2) + wn * 32;  // no ragged columns: N/2 is a multiple of BN/2
 #pragma unroll
-    for (int i = 0; i < WMT; ++i)
+    for (int i = 0; i < WMT; ++i) {
+      uint32_t pk[4][2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + (wm * WMT + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        const float up = round_bf16(acc[i][0][r]), gate = round_bf16(acc[i][1][r]);  // the Linear's bf16 output
-        const float sg = round_bf16(gate / (1.f + expf(-gate)));
-        if (m < M) y[(int64_t)m * half_n + n] = f32_to_bf16_bits(sg * up);
-      }
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+          float v[2];
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            const int r = 4 * q + 2 * x + e;
+            const float up = round_bf16(acc[i][0][r]), gate = round_bf16(acc[i][1][r]);  // the Linear's bf16 output
+            const float sg = round_bf16(gate / (1.f + expf(-gate)));
+            v[e] = sg * up;
+          }
+          pk[q][x] = pack_bf16x2(v[0], v[1]);
+        }
+      store_block(pk, y, m0 + (wm * WMT + i) * 32 + mrow, nb, half_n, half_n);
+    }
     return;
   }
 #pragma unroll
   for (int i = 0; i < WMT; ++i)
 #pragma unroll
     for (int j = 0; j < WNT; ++j) {
-      const int n = (nt0 >> 1) * 32 + (wn * WNT + j) * 32 + (lane & 31);
-      if (n >= N) continue;
+      const int nb = (nt0 >> 1) * 32 + (wn * WNT + j) * 32;  // wave-uniform
+      if (nb >= N) continue;
+      const int m = m0 + (wm * WMT + i) * 32 + mrow;
+      if constexpr (SPLIT) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + (wm * WMT + i) * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if constexpr (SPLIT) {
-          if (m < M) part[((int64_t)blockIdx.y * M + m) * N + n] = acc[i][j][r];
-        } else {
-          if (m < M) y[(int64_t)m * N + n] = f32_to_bf16_bits(acc[i][j][r]);
+        for (int q = 0; q < 4; ++q) {
+          const int n = nb + 8 * q + 4 * half;
+          if (m < M && n < N)
+            *reinterpret_cast<f32x4*>(part + ((int64_t)blockIdx.y * M + m) * N + n) =
+                f32x4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
         }
+      } else {
+        uint32_t pk[4][2];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int x = 0; x < 2; ++x) pk[q][x] = pack_bf16x2(acc[i][j][4 * q + 2 * x], acc[i][j][4 * q + 2 * x + 1]);
+        store_block(pk, y, m, nb, N, N);
       }
     }
 }
@@ -451,9 +557,13 @@ int dispatch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, con
 
 }  // namespace
 
+// the epilogues store 16 bytes at a time
+static inline bool misaligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; }
+
 extern "C" int olmo355_w4_gemm_tile(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
                                     uint16_t* y, int M, int N, int K, int tile, void* stream) {
   if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0 || tile < 0) return O355_EINVAL;
+  if (misaligned16(y)) return O355_EINVAL;
   if ((K & 127) || (N & 15)) return O355_EUNSUPPORTED;
   return dispatch_gemm<true>(x, wt, st, zt, y, M, N, K, as_stream(stream), tile);
 }
@@ -461,6 +571,7 @@ extern "C" int olmo355_w4_gemm_tile(const uint16_t* x, const uint32_t* wt, const
 extern "C" int olmo355_b16_gemm_tile(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, int tile,
                                      void* stream) {
   if (!x || !wt || !y || M <= 0 || N <= 0 || K <= 0 || tile < 0) return O355_EINVAL;
+  if (misaligned16(y)) return O355_EINVAL;
   if ((K & 63) || (N & 15)) return O355_EUNSUPPORTED;
   return dispatch_gemm<false>(x, reinterpret_cast<const uint32_t*>(wt), nullptr, nullptr, y, M, N, K, as_stream(stream),
                               tile);
@@ -469,6 +580,7 @@ extern "C" int olmo355_b16_gemm_tile(const uint16_t* x, const uint16_t* wt, uint
 extern "C" int olmo355_w4_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
                                uint16_t* y, int M, int N, int K, void* stream) {
   if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
+  if (misaligned16(y)) return O355_EINVAL;
   if ((K & 127) || (N & 15)) return O355_EUNSUPPORTED;
   return dispatch_gemm<true>(x, wt, st, zt, y, M, N, K, as_stream(stream));
 }
@@ -478,6 +590,7 @@ extern "C" int olmo355_gemm_splitk_plan(int M, int N, int K) { return splitk_pla
 extern "C" int olmo355_w4_gemm_splitk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
                                       uint16_t* y, int M, int N, int K, int splits, float* workspace, void* stream) {
   if (!x || !wt || !st || !zt || !y || !workspace || M <= 0 || N <= 0 || K <= 0 || splits < 2) return O355_EINVAL;
+  if (misaligned16(workspace)) return O355_EINVAL;
   if ((K & 255) || (N & 63) || ((int64_t)M * N & 3) || splits > (K >> 8)) return O355_EUNSUPPORTED;
   return launch_splitk<true>(x, wt, st, zt, y, M, N, K, splits, workspace, as_stream(stream));
 }
@@ -485,6 +598,7 @@ extern "C" int olmo355_w4_gemm_splitk(const uint16_t* x, const uint32_t* wt, con
 extern "C" int olmo355_b16_gemm_splitk(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K,
                                        int splits, float* workspace, void* stream) {
   if (!x || !wt || !y || !workspace || M <= 0 || N <= 0 || K <= 0 || splits < 2) return O355_EINVAL;
+  if (misaligned16(workspace)) return O355_EINVAL;
   if ((K & 255) || (N & 63) || ((int64_t)M * N & 3) || splits > (K >> 8)) return O355_EUNSUPPORTED;
   return launch_splitk<false>(x, reinterpret_cast<const uint32_t*>(wt), nullptr, nullptr, y, M, N, K, splits, workspace,
                               as_stream(stream));
@@ -493,6 +607,7 @@ extern "C" int olmo355_b16_gemm_splitk(const uint16_t* x, const uint16_t* wt, ui
 extern "C" int olmo355_w4_gemm_swiglu(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
                                       uint16_t* y, int M, int N, int K, void* stream) {
   if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
+  if (misaligned16(y)) return O355_EINVAL;
   if ((K & 127) || (N & 255) || (int64_t)(N >> 4) * (K >> 7) * 1024 >= (1ll << 32)) return O355_EUNSUPPORTED;
   // rounds of one tile per CU, as in dispatch_gemm: 256 or 128 virtual columns (half up, half gate) per tile
   const int64_t tm = (M + 255) / 256;
@@ -504,6 +619,7 @@ extern "C" int olmo355_w4_gemm_swiglu(const uint16_t* x, const uint32_t* wt, con
 extern "C" int olmo355_b16_gemm(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K,
                                 void* stream) {
   if (!x || !wt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
+  if (misaligned16(y)) return O355_EINVAL;
   if ((K & 63) || (N & 15)) return O355_EUNSUPPORTED;
   return dispatch_gemm<false>(x, reinterpret_cast<const uint32_t*>(wt), nullptr, nullptr, y, M, N, K,
                               as_stream(stream));

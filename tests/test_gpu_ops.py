@@ -263,6 +263,26 @@ def test_w4_gemm_every_tile_width(dev, width, M, N, K):
     assert (y.float().cpu() - ref).abs().max().item() <= 2 ** -7 * scale
 
 
+def test_gemm_rejects_misaligned_output(dev):
+    """The matrix-core epilogue stores 16 bytes per lane: an output that does not start on a 16-byte boundary is
+    refused (status 1, nothing launched); the same call on the aligned buffer runs."""
+    from olmo_amd import _lib
+    ops = _ops()
+    M, N, K = 65, 64, 128
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=3)
+    t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    x = torch.randn(M, K, device=dev).to(torch.bfloat16)
+    buf = torch.zeros(M * N + 8, dtype=torch.bfloat16, device=dev)
+    s = torch.cuda.current_stream().cuda_stream
+    st = _lib.lib().olmo355_w4_gemm(x.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), buf.data_ptr() + 2,
+                                    M, N, K, s)
+    torch.cuda.synchronize()
+    assert st == 1 and not buf.any()
+    st = _lib.lib().olmo355_w4_gemm(x.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), buf.data_ptr(), M, N, K, s)
+    torch.cuda.synchronize()
+    assert st == 0 and buf.any()
+
+
 @pytest.mark.parametrize("width", [256, 192, 128, 128128, 128064])
 @pytest.mark.parametrize("M,N,K", [(65, 208, 64), (300, 1008, 192), (513, 400, 320), (256, 768, 448), (40, 48, 1024)])
 def test_b16_gemm_every_tile_width(dev, width, M, N, K):
