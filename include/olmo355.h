@@ -119,6 +119,27 @@ int olmo355_w4_gemm_splitk(const uint16_t* x, const uint32_t* wt, const uint16_t
 int olmo355_b16_gemm_splitk(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, int splits,
                             float* workspace, void* stream);
 
+/* Stream-K forms of the same products for row counts whose 256 x 256 tiles do not fill a whole number of rounds of
+ * the CUs (one prompt of 2048 tokens: 384 tiles for att_proj, 128 for attn_out and ff_out): one workgroup per CU,
+ * the tiles' K runs (units of 256) dealt out evenly, so a tile's K may be shared by two or three workgroups; the one
+ * that ends it adds the others' fp32 partials (in a fixed order: results are reproducible, and differ from the
+ * tiled entry only in the order of fp32 additions) and writes the output.  Same product as QuantLinear.forward's
+ * matmul (qlinear_cuda_old.py:287-290) / F.linear (olmo/model.py:746-823).
+ * `workspace`: olmo355_gemm_streamk_workspace_bytes() bytes, 16-byte aligned, zero before its first use; a launch
+ * leaves its first 4096 bytes (the hand-over flags) zero again.  Launches that share a workspace must be ordered on
+ * one stream.  A finishing workgroup that does not see a partial announced within about two seconds writes NaN
+ * into its tile instead of waiting on (then zero the workspace before the next use).
+ * Needs K % 256 == 0, N % 16 == 0 (SwiGLU form: N % 256 == 0) and at least one unit of 256 per CU; otherwise
+ * O355_EUNSUPPORTED.  olmo355_gemm_streamk_plan: 1 when this form is expected to beat the tiled launch. */
+int64_t olmo355_gemm_streamk_workspace_bytes(void);
+int olmo355_gemm_streamk_plan(int M, int N, int K);
+int olmo355_w4_gemm_streamk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
+                            int M, int N, int K, void* workspace, void* stream);
+int olmo355_w4_gemm_swiglu_streamk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
+                                   uint16_t* y, int M, int N, int K, void* workspace, void* stream);
+int olmo355_b16_gemm_streamk(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, void* workspace,
+                             void* stream);
+
 /* The same product for an ff_proj weight ([up | gate] column halves) with SwiGLU (olmo/model.py:365-368,813-819)
  * in the epilogue: y [M, N/2] = silu(gate) * up, each factor rounded to bf16 first as the separate Linear and
  * activation would.  N a multiple of 256; O355_EUNSUPPORTED otherwise: olmo355_w4_gemm + olmo355_swiglu. */

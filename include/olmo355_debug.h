@@ -16,6 +16,12 @@ int olmo355_w4_gemm_tile(const uint16_t* x, const uint32_t* wt, const uint16_t* 
 int olmo355_b16_gemm_tile(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, int tile,
                           void* stream);
 
+/* olmo355_w4_gemm_streamk with the finishing workgroups' patience (polls of a hand-over flag before the tile is
+ * given up as NaN) and with publish = 0, which makes the partials' owners leave their flags down: the give-up path
+ * forced from the host, every workgroup still exits. */
+int olmo355_w4_gemm_streamk_patience(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
+                                  int M, int N, int K, void* workspace, int spin_limit, int publish, void* stream);
+
 /* olmo355_w4_gemv with the kernel family given: 0 = choose; 1 = the kernels that keep all rows of x in LDS per
  * workgroup (the lean M <= 16 kernel where it applies), never the staged-activation kernel; 2 = the
  * staged-activation kernel (w4_mid_kernel), 3 / 4 = the same with one / two column-tile pairs per workgroup;

@@ -74,6 +74,11 @@ EXPORTS = {
     "olmo355_gemm_splitk_plan": (I, [I, I, I]),
     "olmo355_w4_gemm_splitk": (I, [P, P, P, P, P, I, I, I, I, P, P]),
     "olmo355_b16_gemm_splitk": (I, [P, P, P, I, I, I, I, P, P]),
+    "olmo355_gemm_streamk_workspace_bytes": (L, []),
+    "olmo355_gemm_streamk_plan": (I, [I, I, I]),
+    "olmo355_w4_gemm_streamk": (I, [P, P, P, P, P, I, I, I, P, P]),
+    "olmo355_w4_gemm_swiglu_streamk": (I, [P, P, P, P, P, I, I, I, P, P]),
+    "olmo355_b16_gemm_streamk": (I, [P, P, P, I, I, I, P, P]),
     "olmo355_rope_advance": (I, [P, I, P, P, P, I, I, P]),
     "olmo355_swiglu": (I, [P, P, I, I, I, P]),
     "olmo355_embedding": (I, [P, P, P, I, I, I, I, P]),
@@ -93,6 +98,7 @@ EXPORTS = {
 VARIANT_EXPORTS = {
     "olmo355_w4_gemm_tile": (I, [P, P, P, P, P, I, I, I, I, P]),
     "olmo355_b16_gemm_tile": (I, [P, P, P, I, I, I, I, P]),
+    "olmo355_w4_gemm_streamk_patience": (I, [P, P, P, P, P, I, I, I, P, I, I, P]),
     "olmo355_w4_gemv_form": (I, [P, P, P, P, P, I, I, I, I, P]),
     "olmo355_w4_chain_trace": (I, [ctypes.POINTER(ChainPhase), I, I, P, P, I, P, P]),
     "olmo355_attn_decode_fused_merge": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, P, I, I, P]),

@@ -81,11 +81,40 @@ __device__ __forceinline__ void tile_of(int pid, int tiles_m, int tiles_n, int& 
 // evenly), writing fp32 partial tiles to part[split][M][N]; splitk_reduce_kernel adds them in split order and
 // rounds once.  For launches with fewer tiles than CUs: the K loop is a serial chain of stages of about half a
 // microsecond each, so a tile count of 64 leaves three quarters of the chip idle for K / 64 such stages.
-template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false, bool SPLIT = false>  // wave grid, 32x32 MFMA tiles per wave
+// STREAMK: a workgroup of a grid that stays (one per CU) is handed segments -- a tile and a run of K -- one after
+// the other.  sk_mode says what becomes of the accumulators: 0: the run is the tile's whole K, write the output;
+// 1: leave the fp32 partial in this workgroup's slot and raise its flag; 2: add the partials of workgroups
+// sk_first .. sk_self - 1, then write the output.  What the hand-over needs beyond that is read from the kernel's
+// argument block when it is needed (StreamKArgs is the kernel's only parameter), so that none of it occupies
+// registers during the K loop.
+struct StreamKArgs {
+  const uint16_t* x;
+  const uint32_t* wt;
+  const uint16_t* st;
+  const uint8_t* zt;
+  uint16_t* y;
+  float* slots;    // [grid][8 waves][128 registers / 4][64 lanes] float4: a wave's accumulators as they stand
+  int* flags;      // [grid], zero between launches
+  int M, N, K, tiles_n, tiles;
+  int spin_limit;  // polls of a flag before a finishing workgroup gives up and writes NaN
+  int publish;     // 0 (tests of the give-up path only): leave the flag down
+};
+typedef const __attribute__((address_space(4))) StreamKArgs* StreamKArgsPtr;
+__device__ __forceinline__ StreamKArgsPtr streamk_args() {
+  StreamKArgsPtr p = (StreamKArgsPtr)__builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(p));  // read again wherever it is used
+  return p;
+}
+enum { GEMM_PLAIN = 0, GEMM_SPLIT = 1, GEMM_STREAMK = 2 };
+
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false, int KIND = GEMM_PLAIN>  // wave grid, 32x32 MFMA tiles per wave
 __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wt,
                                           const uint16_t* __restrict__ st, const uint8_t* __restrict__ zt,
-                                          uint16_t* __restrict__ y, int M, int N, int K, int tiles_m, int tiles_n,
-                                          float* __restrict__ part = nullptr) {
+                                          uint16_t* __restrict__ y, int M, int N, int K, int tile_m, int tile_n,
+                                          int k0, int Kn,  // this workgroup's run of K (whole units of 256 unless all of K)
+                                          float* __restrict__ part = nullptr, int sk_mode = 0, int sk_self = 0,
+                                          int sk_first = 0) {
+  constexpr bool SPLIT = KIND == GEMM_SPLIT;
   constexpr int NW = WAVES_M * WAVES_N, NT = 64 * NW;
   constexpr int BM = 32 * WMT * WAVES_M, BN = 32 * WNT * WAVES_N;
   constexpr int A_BLK = BM / 8;        // 1 KiB blocks per stage: activations, 8 rows x 128 bytes each
@@ -100,11 +129,13 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   u32x4* lds_a = reinterpret_cast<u32x4*>(smem);  // [3][A_BLK][64]: ring of three stages
   u32x4* lds_b = lds_a + 3 * A_BLK * 64;          // [2][B_BLK][64]
 
-  const int tid = threadIdx.x, lane = tid & 63;
+  int tid_ = threadIdx.x;
+  // stream-K calls this once per segment inside a loop: what depends on the thread id only must be worked out again
+  // per segment, or it is all kept in registers across the K loops (and accumulators are spilled to make room)
+  if constexpr (KIND == GEMM_STREAMK) asm volatile("" : "+v"(tid_));
+  const int tid = tid_, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-  int tile_m, tile_n;
-  tile_of(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
   static_assert(!SWIGLU || (W4 && WNT == 2), "fused SwiGLU: int4 weights, two column blocks per wave");
   const int m0 = tile_m * BM, nt0 = SWIGLU ? 0 : tile_n * (BN / 16);  // fused: absolute tile indices, see tile_abs
   const int ntiles = N >> 4;
@@ -115,12 +146,6 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     return (j ? (ntiles >> 1) : 0) + tile_n * (BN / 32) + wn_ * 2 + (ntl & 1);
   };
   const int G = K >> 7, KS = K >> 5;  // strides of the tiled weight: always of the whole K
-  int k0 = 0, Kn = K;                 // this workgroup's run of K
-  if constexpr (SPLIT) {
-    const int units = K >> 8, z = blockIdx.y, nz = gridDim.y;
-    const int u0 = units * z / nz, u1 = units * (z + 1) / nz;
-    k0 = u0 << 8, Kn = (u1 - u0) << 8;
-  }
   const int Gn = Kn >> 7;             // groups of 128 rows in the run
   const int stages = Kn / BK;
   const int row32 = lane & 31, kh = lane >> 5;
@@ -360,12 +385,81 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     }
   }
 
+  // ---- stream-K: partial tiles travel between workgroups as the accumulators stand ------------------------
+  constexpr int QUADS = WMT * WNT * 4;  // float4 per lane
+  constexpr int SLOT_BYTES = NW * QUADS * 64 * 16;
+  auto quad_off = [&](int i, int j, int q) { return ((wave * QUADS + (i * WNT + j) * 4 + q) * 64 + lane) * 16; };
+  if constexpr (KIND == GEMM_STREAMK) {
+    // (a partial is left behind -- sk_mode 1 -- from inside the ordinary epilogue's loops below: as a block of
+    // its own before them it drives the register allocation of the whole function into spilling accumulators)
+    if (sk_mode == 2) {
+      const StreamKArgsPtr ka = streamk_args();
+      float* const slots = ka->slots;
+      int* const flags = ka->flags;
+      const int spin_limit = ka->spin_limit;
+      // the workgroups first .. self - 1 hold the earlier runs of this tile's K and finished them before anything
+      // else they had to do; their partials are added in a fixed order.  The wait is bounded: a flag that does
+      // not come up in spin_limit polls turns the tile into NaN instead of hanging the grid.
+      int* s_ok = reinterpret_cast<int*>(smem);  // the operand buffers are done with once every wave is past the K loop
+      for (int pc = sk_self - 1; pc >= sk_first; --pc) {
+        __syncthreads();
+        if (tid == 0) {
+          int ok = 0;
+          for (int spin = 0; spin <= spin_limit; ++spin) {
+            if (__hip_atomic_load(flags + pc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+              ok = 1;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(8);
+          }
+          if (ok) __hip_atomic_store(flags + pc, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+          *s_ok = ok;
+        }
+        __syncthreads();
+        const int ok = *s_ok;
+        const __amdgpu_buffer_rsrc_t rs = make_rsrc(reinterpret_cast<const char*>(slots) + (int64_t)pc * SLOT_BYTES, SLOT_BYTES);
+#pragma unroll
+        for (int i = 0; i < WMT; ++i)
+#pragma unroll
+          for (int j = 0; j < WNT; ++j) {
+            f32x4 v[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              v[q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, quad_off(i, j, q), 0, 16 /* sc1 */));
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = ok ? acc[i][j][4 * q + e] + v[q][e] : __builtin_nanf("");
+          }
+      }
+    }
+  }
+
   // ---- epilogue ------------------------------------------------------------------------------------------
   // The products were formed as W^T-tile x X^T-tile, so a lane holds one output row m = lane & 31 of its 32 x 32
   // block and the columns n = 8 q + 4 (lane >> 5) + (r & 3) in register r = 4 q + (r & 3): four neighbours in a
   // row per register quad.  As bf16 pairs, the quads q = 0, 1 (and 2, 3) of the two half-waves are exchanged so that
   // every lane ends up with 8 neighbouring columns: two 16-byte stores per block and lane instead of sixteen
   // 2-byte ones.
+  // sk_mode 1: device-scope stores (they do not stay in this XCD's L2) of one block's accumulators into this
+  // workgroup's slot; once all are out every wave waits for its own to be acknowledged, then one thread raises the flag
+  auto leave_partial_block = [&](int i, int j) {
+    const StreamKArgsPtr ka = streamk_args();
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(reinterpret_cast<const char*>(ka->slots) + (int64_t)sk_self * SLOT_BYTES, SLOT_BYTES);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      __builtin_amdgcn_raw_buffer_store_b128(
+          __builtin_bit_cast(u32x4, f32x4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]}),
+          rs, quad_off(i, j, q), 0, 16 /* sc1 */);
+  };
+  auto announce_partial = [&]() {
+    const StreamKArgsPtr ka = streamk_args();
+    int* const flags = ka->flags;
+    const int publish = ka->publish;
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, false));
+    __syncthreads();
+    if (tid == 0 && publish) __hip_atomic_store(flags + sk_self, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
   const int half = lane >> 5, mrow = lane & 31;
   auto store_block = [&](const uint32_t (&pk)[4][2], uint16_t* __restrict__ dst, int m, int nb, int ncols, int ld) {
     uint32_t o[4][2];
@@ -388,6 +482,11 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     const int nb = tile_n * (BN / 2) + wn * 32;  // no ragged columns: N/2 is a multiple of BN/2
 #pragma unroll
     for (int i = 0; i < WMT; ++i) {
+      if (KIND == GEMM_STREAMK && sk_mode == 1) {
+        leave_partial_block(i, 0);
+        leave_partial_block(i, 1);
+        continue;
+      }
       uint32_t pk[4][2];
 #pragma unroll
       for (int q = 0; q < 4; ++q)
@@ -405,12 +504,17 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
         }
       store_block(pk, y, m0 + (wm * WMT + i) * 32 + mrow, nb, half_n, half_n);
     }
+    if (KIND == GEMM_STREAMK && sk_mode == 1) announce_partial();
     return;
   }
 #pragma unroll
   for (int i = 0; i < WMT; ++i)
 #pragma unroll
     for (int j = 0; j < WNT; ++j) {
+      if (KIND == GEMM_STREAMK && sk_mode == 1) {
+        leave_partial_block(i, j);
+        continue;
+      }
       const int nb = (nt0 >> 1) * 32 + (wn * WNT + j) * 32;  // wave-uniform
       if (nb >= N) continue;
       const int m = m0 + (wm * WMT + i) * 32 + mrow;
@@ -431,6 +535,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
         store_block(pk, y, m, nb, N, N);
       }
     }
+  if (KIND == GEMM_STREAMK && sk_mode == 1) announce_partial();
 }
 
 template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4>
@@ -440,7 +545,13 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_splitk_kernel(con
                                                                             const uint8_t* __restrict__ zt,
                                                                             float* __restrict__ part, int M, int N, int K,
                                                                             int tiles_m, int tiles_n) {
-  gemm_body<WAVES_M, WAVES_N, WMT, WNT, W4, false, true>(x, wt, st, zt, nullptr, M, N, K, tiles_m, tiles_n, part);
+  int tile_m, tile_n;
+  tile_of(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+  // this workgroup's run of K: whole units of 256, dealt evenly over gridDim.y
+  const int units = K >> 8, z = blockIdx.y, nz = gridDim.y;
+  const int u0 = units * z / nz, u1 = units * (z + 1) / nz;
+  gemm_body<WAVES_M, WAVES_N, WMT, WNT, W4, false, GEMM_SPLIT>(x, wt, st, zt, nullptr, M, N, K, tile_m, tile_n, u0 << 8,
+                                                              (u1 - u0) << 8, part);
 }
 
 // y = bf16(part[0] + part[1] + ... ) in that order, four outputs per thread
@@ -463,7 +574,87 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const uint
                                                                      const uint8_t* __restrict__ zt,
                                                                      uint16_t* __restrict__ y, int M, int N, int K,
                                                                      int tiles_m, int tiles_n) {
-  gemm_body<WAVES_M, WAVES_N, WMT, WNT, W4, SWIGLU>(x, wt, st, zt, y, M, N, K, tiles_m, tiles_n);
+  int tile_m, tile_n;
+  tile_of(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
+  gemm_body<WAVES_M, WAVES_N, WMT, WNT, W4, SWIGLU>(x, wt, st, zt, y, M, N, K, tile_m, tile_n, 0, K);
+}
+
+// Stream-K: a grid that stays, one workgroup per CU.  The tiles' K runs, in units of 256, form one sequence (tile
+// after tile, consecutive tiles share their row panel); it is cut into gridDim.x equal pieces, so every CU does the
+// same amount of matrix work whatever the tile count.  A piece is a run of segments: at most one tile whose K it
+// only begins (or only continues: the piece lies inside one tile) -- done first, left as an fp32 partial in the
+// workgroup's slot --, whole tiles, and at most one tile whose K it ends -- done last: it adds the partials of
+// the workgroups before it, which were the first thing those did.  No workgroup waits for one that waits.
+// Consecutive pieces go to the CUs of one XCD (workgroup ids go round-robin over the XCDs), so an XCD works on a
+// band of consecutive tiles and their row panels stay in its L2.
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_streamk_kernel(StreamKArgs) {
+  for (int i = 0;; ++i) {
+    // everything about the piece is worked out again per segment from the argument block and the workgroup id
+    // (a few scalar instructions) instead of being carried through the K loop
+    const StreamKArgsPtr ka = streamk_args();
+    const int tiles = ka->tiles, tiles_n = ka->tiles_n, K = ka->K;
+    int bid = blockIdx.x;
+    asm volatile("" : "+s"(bid));
+    const int G = gridDim.x;
+    const int c = (G & 7) == 0 ? (bid & 7) * (G >> 3) + (bid >> 3) : bid;
+    const int KU = K >> 8;
+    const int W = tiles * KU;  // the host keeps W * G below 2^31
+    const int u0 = W * c / G, u1 = W * (c + 1) / G;
+    if (u0 >= u1) break;
+    const int t_first = u0 / KU, t_last = (u1 - 1) / KU;
+    const bool tail_partial = (u1 % KU) != 0;                          // the last tile's K is only begun or continued
+    const bool head_finish = (u0 % KU) != 0 && (t_first + 1) * KU <= u1;  // the first tile's K is ended here
+    const int nseg = t_last - t_first + 1, nrest = nseg - (tail_partial ? 1 : 0);
+    if (i >= nseg) break;
+    int t;
+    if (tail_partial && i == 0) {
+      t = t_last;
+    } else {
+      const int j = i - (tail_partial ? 1 : 0);
+      t = head_finish ? (j < nrest - 1 ? t_first + j + 1 : t_first) : t_first + j;
+    }
+    const int tb = t * KU;
+    const int k_a = max(u0, tb) - tb, k_b = min(u1, tb + KU) - tb;
+    const int mode = (k_a == 0 && k_b == KU) ? 0 : (k_b < KU ? 1 : 2);
+    int first = c;
+    if (mode == 2) {  // the workgroup whose piece holds the tile's first unit
+      first = (int)((int64_t)tb * G / W);
+      while (W * (first + 1) / G <= tb) ++first;
+      while (W * first / G > tb) --first;
+    }
+    __syncthreads();  // every wave is done with the LDS buffers of the segment before
+    gemm_body<WAVES_M, WAVES_N, WMT, WNT, W4, SWIGLU, GEMM_STREAMK>(ka->x, ka->wt, ka->st, ka->zt, ka->y, ka->M, ka->N, K,
+                                                                    t / tiles_n, t % tiles_n, k_a << 8, (k_b - k_a) << 8,
+                                                                    nullptr, mode, c, first);
+  }
+}
+
+constexpr int kStreamKMaxGrid = 256;
+constexpr int64_t kStreamKSlotBytes = 8 * 128 * 64 * 4;  // 256 x 256 fp32
+constexpr int64_t kStreamKFlagBytes = 4096;
+constexpr int kStreamKSpinLimit = 1 << 21;
+
+template <bool W4, bool SWIGLU>
+int launch_streamk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M, int N,
+                   int K, void* ws, int spin_limit, int publish, hipStream_t stream) {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+    return O355_ELAUNCH;
+  const int grid = std::min(cus >= 8 ? (cus & ~7) : cus, kStreamKMaxGrid);
+  if (grid <= 0) return O355_ELAUNCH;
+  const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;  // fused SwiGLU: 128 up + 128 gate columns per tile
+  if ((int64_t)tiles_m * tiles_n * (K >> 8) < grid) return O355_EUNSUPPORTED;  // every workgroup must own at least one unit
+  auto kern = gemm_streamk_kernel<2, 4, 4, 2, W4, SWIGLU>;
+  const size_t lds = (size_t)(3 * 32 + 2 * 32) * 1024;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return O355_ELAUNCH;
+  int* flags = reinterpret_cast<int*>(ws);
+  float* slots = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + kStreamKFlagBytes);
+  if ((int64_t)tiles_m * tiles_n * (K >> 8) * grid >= (1ll << 31)) return O355_EUNSUPPORTED;
+  const StreamKArgs args{x, wt, st, zt, y, slots, flags, M, N, K, tiles_n, tiles_m * tiles_n, spin_limit, publish};
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, stream, args);
+  O355_CHECK_LAUNCH();
 }
 
 template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false>
@@ -586,6 +777,60 @@ extern "C" int olmo355_w4_gemm(const uint16_t* x, const uint32_t* wt, const uint
 }
 
 extern "C" int olmo355_gemm_splitk_plan(int M, int N, int K) { return splitk_plan(M, N, K); }
+
+// ---- stream-K entries ------------------------------------------------------------------------------------
+extern "C" int64_t olmo355_gemm_streamk_workspace_bytes(void) { return kStreamKFlagBytes + kStreamKMaxGrid * kStreamKSlotBytes; }
+
+// 1 when the stream-K form is expected to beat the tiled launch.  Measured on the 7B shapes at 2048 rows: where the
+// 256 x 256 tiles make a whole number of rounds the two are level; with 1.5 or 2.7 tiles per CU stream-K gains
+// 4-15 %; with fewer tiles than CUs every tile is shared and the hand-over (about 15 us of partials written, read
+// and waited for) must be earned by the better rate of the large tile: yes at K = 11008, no at K = 4096.
+extern "C" int olmo355_gemm_streamk_plan(int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K <= 0 || (K & 255) || (N & 15)) return 0;
+  const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+  if (tiles < 128) return 0;
+  if (tiles < 256) return 2.0 * M * N * K >= 150e9 ? 1 : 0;
+  const int64_t rounds = (tiles + 255) / 256;
+  return tiles * 100 < rounds * 256 * 92 ? 1 : 0;  // the last round less than 92 % full
+}
+
+static int streamk_args_ok(const void* x, const void* wt, const void* y, const void* ws, int M, int N, int K) {
+  if (!x || !wt || !y || !ws || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
+  if (misaligned16(y) || misaligned16(ws)) return O355_EINVAL;
+  if ((K & 255) || (N & 15)) return O355_EUNSUPPORTED;
+  return O355_OK;
+}
+
+extern "C" int olmo355_w4_gemm_streamk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
+                                       uint16_t* y, int M, int N, int K, void* workspace, void* stream) {
+  if (!st || !zt) return O355_EINVAL;
+  if (const int rc = streamk_args_ok(x, wt, y, workspace, M, N, K)) return rc;
+  return launch_streamk<true, false>(x, wt, st, zt, y, M, N, K, workspace, kStreamKSpinLimit, 1, as_stream(stream));
+}
+
+extern "C" int olmo355_w4_gemm_swiglu_streamk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
+                                              uint16_t* y, int M, int N, int K, void* workspace, void* stream) {
+  if (!st || !zt) return O355_EINVAL;
+  if (const int rc = streamk_args_ok(x, wt, y, workspace, M, N, K)) return rc;
+  if ((N & 255) || (int64_t)(N >> 4) * (K >> 7) * 1024 >= (1ll << 32)) return O355_EUNSUPPORTED;
+  return launch_streamk<true, true>(x, wt, st, zt, y, M, N, K, workspace, kStreamKSpinLimit, 1, as_stream(stream));
+}
+
+extern "C" int olmo355_b16_gemm_streamk(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K,
+                                        void* workspace, void* stream) {
+  if (const int rc = streamk_args_ok(x, wt, y, workspace, M, N, K)) return rc;
+  return launch_streamk<false, false>(x, reinterpret_cast<const uint32_t*>(wt), nullptr, nullptr, y, M, N, K, workspace,
+                                      kStreamKSpinLimit, 1, as_stream(stream));
+}
+
+// test hook: the finishing workgroups' patience and whether partials are announced at all
+extern "C" int olmo355_w4_gemm_streamk_patience(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
+                                             uint16_t* y, int M, int N, int K, void* workspace, int spin_limit, int publish,
+                                             void* stream) {
+  if (!st || !zt || spin_limit < 0) return O355_EINVAL;
+  if (const int rc = streamk_args_ok(x, wt, y, workspace, M, N, K)) return rc;
+  return launch_streamk<true, false>(x, wt, st, zt, y, M, N, K, workspace, spin_limit, publish, as_stream(stream));
+}
 
 extern "C" int olmo355_w4_gemm_splitk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
                                       uint16_t* y, int M, int N, int K, int splits, float* workspace, void* stream) {

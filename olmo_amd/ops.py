@@ -143,16 +143,41 @@ def w4_linear(x: torch.Tensor, w: W4Tiled) -> torch.Tensor:
         check("olmo355_w4_gemv",
               lib().olmo355_w4_gemv(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream()))
     else:
-        check("olmo355_w4_gemm",
-              lib().olmo355_w4_gemm(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream()))
+        ws = _streamk(M, w.N, w.K, x.device)
+        st = 2
+        if ws is not None:
+            st = lib().olmo355_w4_gemm_streamk(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _p(ws), _stream())
+            if st != 2:
+                check("olmo355_w4_gemm_streamk", st)
+        if st == 2:
+            check("olmo355_w4_gemm",
+                  lib().olmo355_w4_gemm(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream()))
     return y
 
 
 SPLITK = True  # tests switch it off to compare the two forms
+STREAMK = True  # likewise
 
 
 def _splitk(M: int, N: int, K: int) -> int:
     return int(lib().olmo355_gemm_splitk_plan(M, N, K)) if SPLITK else 1
+
+
+_streamk_ws = {}
+
+
+def _streamk(M: int, N: int, K: int, device: torch.device):
+    """The stream-K workspace to use for this shape on the current stream, or None when the tiled launch is the better
+    one.  One zeroed buffer per (device, stream), kept for the life of the process: launches that share it are
+    ordered on their stream, and every launch leaves its flags zero again."""
+    if not STREAMK or not lib().olmo355_gemm_streamk_plan(M, N, K):
+        return None
+    key = (device.index if device.index is not None else torch.cuda.current_device(), _stream())
+    ws = _streamk_ws.get(key)
+    if ws is None:
+        ws = torch.zeros(int(lib().olmo355_gemm_streamk_workspace_bytes()), dtype=torch.uint8, device=device)
+        _streamk_ws[key] = ws
+    return ws
 
 
 # ---------------------------------------------------------------------------------------------
@@ -196,7 +221,14 @@ def b16_linear(x: torch.Tensor, w: B16Tiled) -> torch.Tensor:
             check("olmo355_b16_gemm_splitk",
                   lib().olmo355_b16_gemm_splitk(_p(x), _p(w.wt), _p(y), M, w.N, w.K, splits, _p(part), _stream()))
         else:
-            check("olmo355_b16_gemm", lib().olmo355_b16_gemm(_p(x), _p(w.wt), _p(y), M, w.N, w.K, _stream()))
+            ws = _streamk(M, w.N, w.K, x.device)
+            st = 2
+            if ws is not None:
+                st = lib().olmo355_b16_gemm_streamk(_p(x), _p(w.wt), _p(y), M, w.N, w.K, _p(ws), _stream())
+                if st != 2:
+                    check("olmo355_b16_gemm_streamk", st)
+            if st == 2:
+                check("olmo355_b16_gemm", lib().olmo355_b16_gemm(_p(x), _p(w.wt), _p(y), M, w.N, w.K, _stream()))
     return y
 
 
@@ -230,7 +262,15 @@ def linear_fused(x: torch.Tensor, w, resid: Optional[torch.Tensor] = None, norm_
     x_new = rmsnorm(x, norm_w, eps, residual=resid) if resid is not None else x
     if swiglu_out and isinstance(w, W4Tiled) and M > GEMV_MAX_M:  # many rows: SwiGLU in the GEMM's epilogue
         y = torch.empty(*x.shape[:-1], n_out, dtype=torch.bfloat16, device=x.device)
-        st = lib().olmo355_w4_gemm_swiglu(_p(x_new), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream())
+        ws = _streamk(M, w.N, w.K, x.device)
+        st = 2
+        if ws is not None:
+            st = lib().olmo355_w4_gemm_swiglu_streamk(_p(x_new), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _p(ws),
+                                                     _stream())
+            if st not in (0, 2):
+                check("olmo355_w4_gemm_swiglu_streamk", st)
+        if st == 2:
+            st = lib().olmo355_w4_gemm_swiglu(_p(x_new), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream())
         if st == 0:
             return y, x_new
         if st != 2:

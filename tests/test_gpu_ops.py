@@ -163,7 +163,9 @@ def _w4_big_case(dev, N, K, Ms, seed):
     """The int4 linear at full layer sizes.  The oracle product is evaluated on column bands (all columns unless N is
     the vocabulary-sized one: first, middle and last 4096) and, above 64 rows, on a sample of rows (first and last
     tile rows and 24 random ones); at the largest M the whole output is additionally checked through a property
-    that needs no oracle: permuting the rows of x permutes the rows of y bit for bit."""
+    that needs no oracle: permuting the rows of x permutes the rows of y -- bit for bit on the tiled launches; where
+    the stream-K form runs, a row's fp32 partial sums are cut at a K that depends on its tile, so there the two agree
+    to one rounding of the output and are bit-equal with stream-K switched off."""
     ops = _ops()
     qw, qz, sc = ow4.random_quantized(K, N, 128, seed=seed)
     t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
@@ -185,8 +187,19 @@ def _w4_big_case(dev, N, K, Ms, seed):
             assert err <= 2 ** -7 * scale, (M, lo, hi, err, scale)
         if M == max(Ms) and M > 64:
             perm = torch.randperm(M, generator=g)
-            y2 = ops.w4_linear(x[perm].contiguous().to(dev), t)
-            assert torch.equal(y2, y[perm.to(dev)])
+            xp = x[perm].contiguous().to(dev)
+            y2 = ops.w4_linear(xp, t)
+            from olmo_amd import _lib
+            if _lib.lib().olmo355_gemm_streamk_plan(M, N, K):
+                a, b = y2.float(), y[perm.to(dev)].float()
+                assert ((a - b).abs() <= 2 ** -7 * torch.maximum(a.abs(), b.abs()) + 2 ** -16 * b.abs().max()).all()
+                ops.STREAMK = False
+                try:
+                    assert torch.equal(ops.w4_linear(xp, t), ops.w4_linear(x.to(dev), t)[perm.to(dev)])
+                finally:
+                    ops.STREAMK = True
+            else:
+                assert torch.equal(y2, y[perm.to(dev)])
 
 
 @pytest.mark.parametrize("N,K", [(4096, 4096), (11008, 4096), (4096, 11008), (13824, 5120), (100352, 4096)])
@@ -261,6 +274,115 @@ def test_w4_gemm_every_tile_width(dev, width, M, N, K):
     assert st == 0
     scale = ref.abs().max().item()
     assert (y.float().cpu() - ref).abs().max().item() <= 2 ** -7 * scale
+
+
+def _streamk_ws(dev):
+    from olmo_amd import _lib
+    return torch.zeros(_lib.lib().olmo355_gemm_streamk_workspace_bytes(), dtype=torch.uint8, device=dev)
+
+
+@pytest.mark.parametrize("M,N,K", [(1024, 4096, 1024), (1000, 4080, 1280), (2048, 8192, 512), (700, 6160, 2048),
+                                   (2048, 12288, 1024)])
+def test_w4_gemm_streamk(dev, M, N, K):
+    """The stream-K form against the oracle on shapes where a tile's K is shared by four workgroups (one unit of 256
+    per CU), by two with uneven pieces, by none (256 tiles of two units: one whole tile per CU), with ragged M and N,
+    and with 1.5 tiles per CU; the flags are zero again afterwards and a second launch on the same
+    workspace gives the same bits."""
+    say("w4_gemm_streamk", M, N, K)
+    from olmo_amd import _lib
+    ops = _ops()
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=M + N + K)
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(11)).to(torch.bfloat16)
+    ref = ow4.linear_fp32(x, ow4.dequantize(qw, qz, sc, 128))
+    t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    xd = x.to(dev)
+    ws = _streamk_ws(dev)
+    s = torch.cuda.current_stream().cuda_stream
+    ys = []
+    for _ in range(2):
+        y = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+        st = _lib.lib().olmo355_w4_gemm_streamk(xd.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y.data_ptr(),
+                                                M, N, K, ws.data_ptr(), s)
+        torch.cuda.synchronize()
+        assert st == 0
+        assert not ws[:4096].any()
+        ys.append(y)
+    assert torch.equal(ys[0], ys[1])
+    scale = ref.abs().max().item()
+    assert (ys[0].float().cpu() - ref).abs().max().item() <= 2 ** -7 * scale
+    # against the tiled launch: the same fp32 products added in another order
+    y0 = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    assert _lib.lib().olmo355_w4_gemm(xd.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y0.data_ptr(), M, N, K, s) == 0
+    torch.cuda.synchronize()
+    a, b = ys[0].float(), y0.float()  # one rounding step of the element, or what fp32 sums of this size differ by near zero
+    assert ((a - b).abs() <= 2 ** -7 * torch.maximum(a.abs(), b.abs()) + 2 ** -16 * scale).all()
+
+
+def test_w4_gemm_swiglu_streamk_and_dense_streamk(dev):
+    """The SwiGLU-epilogue and dense forms of the stream-K launch against their tiled counterparts."""
+    say("w4_gemm_swiglu_streamk / b16_gemm_streamk")
+    from olmo_amd import _lib
+    ops = _ops()
+    L = _lib.lib()
+    M, N, K = 1100, 8192, 1024
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=77)
+    t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(12)).to(torch.bfloat16).to(dev)
+    ws = _streamk_ws(dev)
+    s = torch.cuda.current_stream().cuda_stream
+    y0 = torch.empty(M, N // 2, dtype=torch.bfloat16, device=dev)
+    y1 = torch.full_like(y0, float("nan"))
+    assert L.olmo355_w4_gemm_swiglu(x.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y0.data_ptr(), M, N, K, s) == 0
+    assert L.olmo355_w4_gemm_swiglu_streamk(x.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y1.data_ptr(), M, N, K,
+                                            ws.data_ptr(), s) == 0
+    torch.cuda.synchronize()
+    a, b = y1.float(), y0.float()
+    # silu(gate) * up of two bf16-rounded factors: one rounding step of either factor moves the product by 2^-7
+    assert ((a - b).abs() <= 2 ** -6 * torch.maximum(a.abs(), b.abs()) + 2 ** -14 * b.abs().max()).all()
+    assert not ws[:4096].any()
+    w = (torch.randn(N, K, generator=torch.Generator().manual_seed(13)) * 0.02).to(torch.bfloat16).to(dev)
+    tw = ops.b16_repack(w)
+    z0 = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    z1 = torch.full_like(z0, float("nan"))
+    assert L.olmo355_b16_gemm(x.data_ptr(), tw.wt.data_ptr(), z0.data_ptr(), M, N, K, s) == 0
+    assert L.olmo355_b16_gemm_streamk(x.data_ptr(), tw.wt.data_ptr(), z1.data_ptr(), M, N, K, ws.data_ptr(), s) == 0
+    torch.cuda.synchronize()
+    a, b = z1.float(), z0.float()
+    assert ((a - b).abs() <= 2 ** -7 * torch.maximum(a.abs(), b.abs()) + 2 ** -16 * b.abs().max()).all()
+    ref = x.float() @ w.float().t()
+    assert torch.allclose(z1.float(), ref, rtol=2 ** -8, atol=2 ** -8 * ref.abs().max().item())
+
+
+def test_w4_gemm_streamk_gives_up_instead_of_hanging(dev):
+    """With the partials' owners told not to raise their flags (a host-side switch of the variant entry) and a
+    patience of four polls, every finishing workgroup gives its tile up as NaN, the tiles that were never shared are
+    right, the launch ends, and the workspace needs no cleaning (no flag was raised)."""
+    say("w4_gemm_streamk give-up")
+    from olmo_amd import _lib
+    ops = _ops()
+    L = _lib.lib()
+    M, N, K = 2048, 12288, 1024  # 384 tiles on 256 CUs: every second tile is shared by two workgroups
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=5)
+    t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(14)).to(torch.bfloat16).to(dev)
+    ws = _streamk_ws(dev)
+    s = torch.cuda.current_stream().cuda_stream
+    y = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
+    st = L.olmo355_w4_gemm_streamk_patience(x.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y.data_ptr(),
+                                            M, N, K, ws.data_ptr(), 4, 0, s)
+    torch.cuda.synchronize()
+    assert st == 0
+    assert not ws[:4096].any()
+    y0 = torch.empty_like(y)
+    assert L.olmo355_w4_gemm(x.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y0.data_ptr(), M, N, K, s) == 0
+    torch.cuda.synchronize()
+    tiles = y.float().view(M // 256, 256, N // 256, 256).permute(0, 2, 1, 3).reshape(-1, 256 * 256)
+    ref_tiles = y0.float().view(M // 256, 256, N // 256, 256).permute(0, 2, 1, 3).reshape(-1, 256 * 256)
+    nan_tiles = torch.isnan(tiles).all(dim=1)
+    clean = ~torch.isnan(tiles).any(dim=1)
+    assert (nan_tiles | clean).all()                     # a tile is given up whole or not at all
+    assert nan_tiles.sum().item() == 128 and clean.sum().item() == 256
+    assert torch.equal(tiles[clean], ref_tiles[clean])   # whole tiles: the same additions in the same order as the tiled launch
 
 
 def test_gemm_rejects_misaligned_output(dev):
