@@ -109,8 +109,14 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const void* __restrict
 // =====================================================================================================
 // Workgroup: 4 waves x 32 queries = 128 queries of one (batch, head); KV tile: 64 keys.
 // LDS  K  : [key-tile 4][hd-step HD/32][64 lanes][8 bf16]   A operand of S^T = K . Q^T
-//      V^T: [hd-tile HD/16][key-step 2][64 lanes][8 bf16]   A operand of O^T = V^T . P^T
-//      (plus pad slots, see the declarations)
+//      V  : [key 64][hd] row-major as it comes from the cache, rows 32 bytes longer than the data so that four
+//           neighbouring keys start 8 banks apart.  The A operand of O^T = V^T . P^T is read with the LDS
+//           transposing load (ds_read_b64_tr_b16): per group of 16 lanes, lane r supplies the address of four
+//           consecutive bf16 and lane j receives element j % 4 of the four rows supplied by lanes j / 4 + 4 e
+//           (e = 0 .. 3).  With lane r pointing at key 4 kq + r / 4, channels 4 (r % 4) .. + 3 of the hd tile, lane j
+//           receives channel j of keys 4 kq .. 4 kq + 3: one load per half of an operand fragment, no shuffling
+//           of V on the way into LDS.
+//      (K: plus pad slots, see the declaration)
 // In the second product the 8 key slots of lane group kq in key-step s are
 //   e<4 : key 32s + 4kq + e        e>=4 : key 32s + 16 + 4kq + (e-4)
 // which is exactly how the S^T accumulators of the two 16-key tiles 2s, 2s+1 sit in a lane, so
@@ -128,7 +134,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
   constexpr int QT = 2;              // 16-query tiles per wave
   // 16-byte slots; a pad slot after every 16 (K) / every 128 (V) spreads the staging writes over the banks
   __shared__ __align__(16) u32x4 lds_k[4 * STEPS * 4 * 17];
-  __shared__ __align__(16) u32x4 lds_v[HT * 129];
+  constexpr int VROW = HD * 2 + 32;  // bytes per key row of V in LDS
+  __shared__ __align__(16) unsigned char lds_v[KT * VROW];
   __shared__ float lds_bias[KT];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -173,8 +180,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
   // after tile k0 has been written to LDS, so the requests are in flight while tile k0 is multiplied.
   constexpr int CPR = HD / 8;                     // 16-byte chunks per key row
   constexpr int KPT = KT * CPR / 256;             // K chunks per thread per tile
-  constexpr int VPT = (KT / 2) * CPR / 256;       // V chunk pairs (two consecutive keys) per thread per tile
-  u32x4 rkk[KPT], rv0[VPT], rv1[VPT];
+  u32x4 rkk[KPT], rvv[KPT];
   float rbias = 0.f;
   const uint16_t* kbase = kc + cbase;
   const uint16_t* vbase = vc + cbase;
@@ -185,13 +191,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
       const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
       const uint32_t row = tail ? min(k0 + kk, last_pos) : k0 + kk;
       rkk[i] = *reinterpret_cast<const u32x4*>(kbase + (row * HD + 8 * c));
-    }
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-      const int e = tid + i * 256, kk = 2 * (e / CPR), c = e % CPR;
-      const uint32_t r0 = tail ? min(k0 + kk, last_pos) : k0 + kk, r1 = tail ? min(k0 + kk + 1, last_pos) : k0 + kk + 1;
-      rv0[i] = *reinterpret_cast<const u32x4*>(vbase + (r0 * HD + 8 * c));
-      rv1[i] = *reinterpret_cast<const u32x4*>(vbase + (r1 * HD + 8 * c));
+      rvv[i] = *reinterpret_cast<const u32x4*>(vbase + (row * HD + 8 * c));
     }
     if (key_bias && tid < KT) rbias = key_bias[(int64_t)b * bias_stride + min(k0 + tid, last_pos)];
   };
@@ -201,24 +201,14 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
       const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
       lds_k[(((kk >> 4) * STEPS + (c >> 2)) * 4 + (c & 3)) * 17 + (kk & 15)] = rkk[i];
     }
-    // V^T: key pairs (kk, kk+1) x 8 hd values -> 8 dword writes
 #pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-      const int e = tid + i * 256, kk = 2 * (e / CPR), c = e % CPR;
-      const int kt = kk >> 4, s2 = kt >> 1, hf = kt & 1, k16 = kk & 15;
-      const int kq_ = k16 >> 2, e0 = (k16 & 3) + 4 * hf;  // e0 even
-      uint32_t* dst = reinterpret_cast<uint32_t*>(lds_v);
-#pragma unroll
-      for (int x = 0; x < 8; ++x) {
-        const int hd_ = 8 * c + x;
-        const int ht = hd_ >> 4, lo = hd_ & 15;
-        const uint32_t a = (x & 1) ? (rv0[i][x >> 1] >> 16) : (rv0[i][x >> 1] & 0xffffu);
-        const uint32_t bb = (x & 1) ? (rv1[i][x >> 1] >> 16) : (rv1[i][x >> 1] & 0xffffu);
-        dst[((ht * 129 + s2 * 64 + kq_ * 16 + lo) * 8 + e0) >> 1] = a | (bb << 16);
-      }
+    for (int i = 0; i < KPT; ++i) {
+      const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
+      *reinterpret_cast<u32x4*>(lds_v + kk * VROW + c * 16) = rvv[i];
     }
     if (tid < KT) lds_bias[tid] = rbias;
   };
+  const int v_rd = (4 * kq + (col >> 2)) * VROW + 8 * (col & 3);  // this lane's row of the transposing loads
   fetch(0);
   for (int k0 = 0; k0 <= last_pos; k0 += KT) {
     __syncthreads();  // the previous tile has been read
@@ -307,7 +297,13 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
     for (int ht = 0; ht < HT; ++ht)
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
-        const bf16x8 vf = __builtin_bit_cast(bf16x8, lds_v[ht * 129 + s2 * 64 + lane]);
+        typedef short s16x4 __attribute__((ext_vector_type(4)));
+        typedef s16x4 __attribute__((address_space(3))) * tr_ptr;
+        const unsigned char* vp = lds_v + v_rd + (32 * s2) * VROW + 32 * ht;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr)vp);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr)(vp + 16 * VROW));
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        const bf16x8 vf = __builtin_bit_cast(bf16x8, s16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
 #pragma unroll
         for (int qt = 0; qt < QT; ++qt) o[qt][ht] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[qt][s2], o[qt][ht], 0, 0, 0);
       }
