@@ -226,7 +226,10 @@ def main() -> int:
     flops = sum(2.0 * ctx * n * k for n, k in shapes)
     tf = flops * 3 / (e0.elapsed_time(e1) * 1e-3) / 1e12
     extra["prefill_gemm"] = {"bound": "mfma", "achieved": tf, "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
-                             "frac": tf / MFMA_BF16_PEAK_TF, "M": ctx}
+                             "frac": tf / MFMA_BF16_PEAK_TF, "M": ctx,
+                             "what": "the four block Linears of one layer at M rows through olmo_amd.ops.w4_linear, three "
+                                     "times each, HIP events around the twelve launches: gemm_streamk_kernel for att_proj, "
+                                     "ff_proj and ff_out, gemm_kernel (256 x 128 tiles) for attn_out"}
     log(f"[bench] int4 prefill GEMMs (M={ctx}): {tf:.0f} TFLOP/s = {tf / MFMA_BF16_PEAK_TF:.1%} of bf16 MFMA peak")
     # yardstick: the vendor library's *dense* bf16 GEMM (torch.matmul -> hipBLASLt) on the same four shapes at the
     # same M, nothing to dequantise: what a tuned library reaches at this size on this box
