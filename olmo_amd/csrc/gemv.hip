@@ -1014,10 +1014,11 @@ int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, 
   const u32x4* w = (const u32x4*)wt;
   const int sgpa = a.M <= 4 ? 4 : (a.M <= 8 ? 2 : 1);
   const bool small_ok = a.M <= 16 && (a.M <= 4 || p.pro == 0) && (int64_t)(a.M + 1) * a.K * 2 <= kSmallMaxBytes && (int64_t)(a.N >> 4) * (a.K >> 7) * 1024 < (1ll << 31) && form != kFormOlder;
-  // Plain products with many columns: from 9 rows (5 for wide outputs) the staged-activation kernel
+  // Plain products with many columns: from 9 rows (8 for wide outputs; measured at N = 12288, K = 4096: 5 rows 8.7
+  // against 11.3 us, 8 rows 11.2 against 10.8) the staged-activation kernel
   // wins over the kernels below, which keep all rows of x in LDS per workgroup (measured).
   const bool plain = !pro && !epi && !a.ssq_in && !a.ssq_out;
-  const bool mid_wins = a.M > 16 || (a.M > 8 && a.N >= 8192) || (a.M > 4 && a.N >= 12288);
+  const bool mid_wins = a.M > 16 || (a.M > 8 && a.N >= 8192) || (a.M > 7 && a.N >= 12288);
   const bool force_mid = form == kFormMid || form == kFormMid1 || form == kFormMid2;
   if (plain && ((mid_wins && form == kFormChoose) || force_mid)) {
     const int pairs = form == kFormMid1 ? 1 : (form == kFormMid2 ? 2 : 0);

@@ -140,10 +140,10 @@ def test_w4_gemv(dev, M, N, K):
     assert err <= 2 ** -7 * scale, (err, scale)
 
 
-@pytest.mark.parametrize("M", [5, 9, 16, 17, 32, 48, 64])
+@pytest.mark.parametrize("M", [5, 8, 9, 16, 17, 32, 48, 64])
 @pytest.mark.parametrize("N,K", [(8208, 640), (11008, 4096), (4112, 128), (16, 1024), (16400, 256), (32784, 384)])
 def test_w4_gemv_mid_rows(dev, M, N, K):
-    """The kernel that stages the activations through LDS (every M > 16; from 9 rows at N >= 8192, from 5 at
+    """The kernel that stages the activations through LDS (every M > 16; from 9 rows at N >= 8192, from 8 at
     N >= 12288): one, two and four row tiles, both workgroup widths, an odd number of column tiles, and K
     that ends in the middle of a 512-wide stage or is shorter than one."""
     say("w4_gemv_mid", M, N, K)
