@@ -113,7 +113,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
                                           uint16_t* __restrict__ y, int M, int N, int K, int tile_m, int tile_n,
                                           int k0, int Kn,  // this workgroup's run of K (whole units of 256 unless all of K)
                                           float* __restrict__ part = nullptr, int sk_mode = 0, int sk_self = 0,
-                                          int sk_first = 0) {
+                                          int sk_first = 0, bool sk_raise = false, bool sk_defer = false) {
   constexpr bool SPLIT = KIND == GEMM_SPLIT;
   constexpr int NW = WAVES_M * WAVES_N, NT = 64 * NW;
   constexpr int BM = 32 * WMT * WAVES_M, BN = 32 * WNT * WAVES_N;
@@ -357,6 +357,14 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   }
   __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
   __builtin_amdgcn_s_barrier();
+  if constexpr (KIND == GEMM_STREAMK) {
+    // the partial this workgroup left in the segment before: every wave has just waited for all its memory
+    // operations, those stores among them, so the flag can go up without a wait of its own
+    if (sk_raise && tid == 0) {
+      const StreamKArgsPtr ka = streamk_args();
+      if (ka->publish) __hip_atomic_store(ka->flags + sk_self, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
 #pragma unroll
   for (int i = 0; i < WMT; ++i) fa[0][i] = read_a(0, i, 0);
 #pragma unroll
@@ -504,7 +512,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
         }
       store_block(pk, y, m0 + (wm * WMT + i) * 32 + mrow, nb, half_n, half_n);
     }
-    if (KIND == GEMM_STREAMK && sk_mode == 1) announce_partial();
+    if (KIND == GEMM_STREAMK && sk_mode == 1 && !sk_defer) announce_partial();
     return;
   }
 #pragma unroll
@@ -535,7 +543,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
         store_block(pk, y, m, nb, N, N);
       }
     }
-  if (KIND == GEMM_STREAMK && sk_mode == 1) announce_partial();
+  if (KIND == GEMM_STREAMK && sk_mode == 1 && !sk_defer) announce_partial();
 }
 
 template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4>
@@ -623,10 +631,13 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_streamk_kernel(St
       while (W * (first + 1) / G <= tb) ++first;
       while (W * first / G > tb) --first;
     }
+    // A partial is always the first segment of a piece.  When more segments follow, its flag goes up after the next
+    // segment's first barrier (which waits for all memory operations anyway) instead of after a wait of its own.
+    const bool defer = mode == 1 && nseg > 1, raise = i == 1 && tail_partial;
     __syncthreads();  // every wave is done with the LDS buffers of the segment before
     gemm_body<WAVES_M, WAVES_N, WMT, WNT, W4, SWIGLU, GEMM_STREAMK>(ka->x, ka->wt, ka->st, ka->zt, ka->y, ka->M, ka->N, K,
                                                                     t / tiles_n, t % tiles_n, k_a << 8, (k_b - k_a) << 8,
-                                                                    nullptr, mode, c, first);
+                                                                    nullptr, mode, c, first, raise, defer);
   }
 }
 
