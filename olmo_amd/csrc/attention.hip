@@ -22,6 +22,7 @@
 namespace {
 
 constexpr float kMaskThreshold = -1e30f;
+constexpr float kLazyMax = 8.f;
 
 // 8 consecutive channels as floats: one 16-byte vector of bf16 or two of fp32
 template <int DT> struct Vec8;
@@ -121,6 +122,19 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const void* __restrict
 //   e<4 : key 32s + 4kq + e        e>=4 : key 32s + 16 + 4kq + (e-4)
 // which is exactly how the S^T accumulators of the two 16-key tiles 2s, 2s+1 sit in a lane, so
 // P goes from accumulator registers to the B operand without leaving the lane.
+// v[l] op v[l ^ 16], then op over l ^ 32, in every lane: the reductions over the four lane groups that share a query
+// column.  Two register swaps between half-rows / half-waves (v_permlane16_swap, v_permlane32_swap) instead of two
+// trips through the LDS crossbar (what a shuffle by 16 or 32 lanes compiles to), each of which the wave waits out.
+template <typename Op>
+__device__ __forceinline__ float reduce_lane_groups(float v, Op op) {
+  uint32_t u = __builtin_bit_cast(uint32_t, v);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);  // rows (0, 1) and (2, 3) of 16 lanes trade places
+  v = op(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+  u = __builtin_bit_cast(uint32_t, v);
+  r = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // the two halves of the wave
+  return op(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+}
+
 template <int HD>
 __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_t* __restrict__ q,
                                                                 const uint16_t* __restrict__ kc,
@@ -182,16 +196,26 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
   constexpr int KPT = KT * CPR / 256;             // K chunks per thread per tile
   u32x4 rkk[KPT], rvv[KPT];
   float rbias = 0.f;
-  const uint16_t* kbase = kc + cbase;
-  const uint16_t* vbase = vc + cbase;
+  // range-checked loads: the tile's base as the scalar offset, a lane's place in the tile worked out once
+  const __amdgpu_buffer_rsrc_t rk_ = make_rsrc(kc + cbase, (int64_t)Lmax * HD * 2);
+  const __amdgpu_buffer_rsrc_t rv_ = make_rsrc(vc + cbase, (int64_t)Lmax * HD * 2);
+  int kv_off[KPT];
+#pragma unroll
+  for (int i = 0; i < KPT; ++i) {
+    const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
+    kv_off[i] = (kk * HD + 8 * c) * 2;
+  }
   auto fetch = [&](int k0) {
     const bool tail = k0 + KT - 1 > last_pos;  // only the last tile can reach past the last visible key
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
-      const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
-      const uint32_t row = tail ? min(k0 + kk, last_pos) : k0 + kk;
-      rkk[i] = *reinterpret_cast<const u32x4*>(kbase + (row * HD + 8 * c));
-      rvv[i] = *reinterpret_cast<const u32x4*>(vbase + (row * HD + 8 * c));
+      int off = kv_off[i], base = k0 * HD * 2;
+      if (tail) {  // rows past the last visible key may hold anything: read the last visible row instead
+        const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
+        off = (min(k0 + kk, last_pos) * HD + 8 * c) * 2, base = 0;
+      }
+      rkk[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rk_, off, base, 0));
+      rvv[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rv_, off, base, 0));
     }
     if (key_bias && tid < KT) rbias = key_bias[(int64_t)b * bias_stride + min(k0 + tid, last_pos)];
   };
@@ -258,9 +282,12 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
           for (int r = 0; r < 4; ++r) tmax = fmaxf(tmax, s[qt][kt][r]);
         tmax *= c2;  // c2 > 0: the maximum commutes with the scaling
       }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      const float mn = fmaxf(m[qt], tmax);  // finite: key 0 of the first tile is visible to every query
+      tmax = reduce_lane_groups(tmax, [](float a, float b) { return fmaxf(a, b); });
+      // The reference maximum follows the running maximum lazily: it moves only when the tile's maximum is more than
+      // kLazyMax (log2 units) above it, so probabilities stay below 2^kLazyMax and the accumulators are rescaled
+      // on a few tiles instead of nearly all (the same ratio o / l comes out; finite: key 0 of the first tile is
+      // visible to every query, and -inf + kLazyMax is -inf)
+      const float mn = tmax > m[qt] + kLazyMax ? tmax : m[qt];
       float psum = 0.f;
       float p[4][4];
 #pragma unroll
@@ -270,8 +297,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
           p[kt][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qt][kt][r], cs, -mn));
           psum += p[kt][r];
         }
-      psum += __shfl_xor(psum, 16, 64);
-      psum += __shfl_xor(psum, 32, 64);
+      psum = reduce_lane_groups(psum, [](float a, float b) { return a + b; });
       if (__builtin_amdgcn_ballot_w64(mn != m[qt]) != 0) {  // the running maximum moved for some query of the wave
         const float alpha = __builtin_amdgcn_exp2f(m[qt] - mn);
         l[qt] *= alpha;
