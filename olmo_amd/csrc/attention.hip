@@ -122,17 +122,11 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const void* __restrict
 //   e<4 : key 32s + 4kq + e        e>=4 : key 32s + 16 + 4kq + (e-4)
 // which is exactly how the S^T accumulators of the two 16-key tiles 2s, 2s+1 sit in a lane, so
 // P goes from accumulator registers to the B operand without leaving the lane.
-// v[l] op v[l ^ 16], then op over l ^ 32, in every lane: the reductions over the four lane groups that share a query
-// column.  Two register swaps between half-rows / half-waves (v_permlane16_swap, v_permlane32_swap) instead of two
-// trips through the LDS crossbar (what a shuffle by 16 or 32 lanes compiles to), each of which the wave waits out.
+// The prefill kernel's reductions over the four lane groups that share a query column: op over l ^ 16, then over
+// l ^ 32 (register swaps, see combine_xor16 / combine_xor32).
 template <typename Op>
 __device__ __forceinline__ float reduce_lane_groups(float v, Op op) {
-  uint32_t u = __builtin_bit_cast(uint32_t, v);
-  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);  // rows (0, 1) and (2, 3) of 16 lanes trade places
-  v = op(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
-  u = __builtin_bit_cast(uint32_t, v);
-  r = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // the two halves of the wave
-  return op(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+  return combine_xor32(combine_xor16(v, op), op);
 }
 
 template <int HD>
@@ -467,8 +461,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const void* __restrict
     s[it] = v;
     wmax = fmaxf(wmax, v);
   }
-#pragma unroll
-  for (int o = LPK; o < 64; o <<= 1) wmax = fmaxf(wmax, __shfl_xor(wmax, o, 64));
+  if constexpr (LPK <= 4) wmax = combine_xor<4>(wmax, MaxOp{});
+  if constexpr (LPK <= 8) wmax = combine_xor<8>(wmax, MaxOp{});
+  wmax = combine_xor<32>(combine_xor<16>(wmax, MaxOp{}), MaxOp{});
   // a wave whose keys all lie beyond L contributes nothing
   const bool empty = (kbase >= L);
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -484,12 +479,14 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const void* __restrict
       for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(p, vf[i], acc[i]);
     }
     // sum over the key slots of the wave (lanes with equal `sub`)
+    auto over_slots = [](float v) {
+      if constexpr (LPK <= 4) v = combine_xor<4>(v, AddOp{});
+      if constexpr (LPK <= 8) v = combine_xor<8>(v, AddOp{});
+      return combine_xor<32>(combine_xor<16>(v, AddOp{}), AddOp{});
+    };
+    lsum = over_slots(lsum);
 #pragma unroll
-    for (int o = LPK; o < 64; o <<= 1) {
-      lsum += __shfl_xor(lsum, o, 64);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] += __shfl_xor(acc[i], o, 64);
-    }
+    for (int i = 0; i < 8; ++i) acc[i] = over_slots(acc[i]);
   }
   if (lane < LPK) {
 #pragma unroll

@@ -291,8 +291,8 @@ __global__ __launch_bounds__(kCW * 64) void w4_chain_kernel(ChainArgs a) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         float v = acc[r];
-        v += __shfl_xor(v, 16, 64);
-        v += __shfl_xor(v, 32, 64);
+        v = combine_xor16(v, AddOp{});
+        v = combine_xor32(v, AddOp{});
         if (kq == 0) myred[tl * 64 + r * 16 + col] = v;
       }
     };

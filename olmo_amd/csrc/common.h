@@ -85,33 +85,63 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, in
 constexpr int waitcnt_imm(int vm, bool lds) { return (vm & 15) | ((vm >> 4) << 14) | 0x0070 | (lds ? 0 : 0x0f00); }
 
 // ---- wave64 reductions ------------------------------------------------------------------------
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+// A shuffle (`__shfl_xor`) compiles to a trip through the LDS crossbar that the wave waits out (ds_bpermute +
+// s_waitcnt), six in a row for a butterfly over 64 lanes.  The same butterflies from register-to-register moves:
+// DPP within rows of 16 lanes, v_permlane16_swap / v_permlane32_swap between half-rows and half-waves.  Operands and
+// order of every step are those of the xor butterfly (after the xor-1 and xor-2 steps the lanes of a quad agree, so
+// the mirrored partner of the next steps holds what the xor partner holds); the butterfly runs from distance 1 up
+// to distance 32.
+template <int CTRL>
+__device__ __forceinline__ float dpp_lane(float v) {  // the value of the lane that DPP control CTRL names
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+// op(v[l], v[l ^ 16]) in every lane (op commutative)
+template <typename Op>
+__device__ __forceinline__ float combine_xor16(float v, Op op) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);  // rows (0, 1) and (2, 3) trade places
+  return op(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+}
+// op(v[l], v[l ^ 32]) in every lane (op commutative)
+template <typename Op>
+__device__ __forceinline__ float combine_xor32(float v, Op op) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // the two halves of the wave
+  return op(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+}
+// reduction over an aligned row of 16 lanes; every lane gets it
+template <typename Op>
+__device__ __forceinline__ float row16_reduce(float v, Op op) {
+  v = op(v, dpp_lane<0xB1>(v));   // quad_perm [1,0,3,2]
+  v = op(v, dpp_lane<0x4E>(v));   // quad_perm [2,3,0,1]
+  v = op(v, dpp_lane<0x141>(v));  // row_half_mirror
+  v = op(v, dpp_lane<0x140>(v));  // row_mirror
   return v;
 }
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+template <typename Op>
+__device__ __forceinline__ float wave_reduce(float v, Op op) {
+  return combine_xor32(combine_xor16(row16_reduce(v, op), op), op);
 }
+// one step of an xor butterfly, op(v[l], v[l ^ O]): register moves for the distances that have one (8: rotation of
+// the row of 16 by 8; 16 and 32: the swaps above), a shuffle otherwise
+template <int O, typename Op>
+__device__ __forceinline__ float combine_xor(float v, Op op) {
+  if constexpr (O == 32) return combine_xor32(v, op);
+  else if constexpr (O == 16) return combine_xor16(v, op);
+  else if constexpr (O == 8) return op(v, dpp_lane<0x128>(v));  // row_ror:8
+  else if constexpr (O == 2) return op(v, dpp_lane<0x4E>(v));
+  else if constexpr (O == 1) return op(v, dpp_lane<0xB1>(v));
+  else return op(v, __shfl_xor(v, O, 64));
+}
+struct AddOp { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
+struct MaxOp { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 
+__device__ __forceinline__ float wave_sum(float v) { return wave_reduce(v, AddOp{}); }
+__device__ __forceinline__ float wave_max(float v) { return wave_reduce(v, MaxOp{}); }
 // sum over an aligned row of 16 lanes; every lane gets it
-__device__ __forceinline__ float row16_sum(float v) {
-#pragma unroll
-  for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 16);
-  return v;
-}
-// wave sum whose first four steps are DPP adds within rows of 16 lanes (fixed order: the same on every wave)
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
-  v += __shfl_xor(v, 16, 64);
-  v += __shfl_xor(v, 32, 64);
-  return v;
-}
+__device__ __forceinline__ float row16_sum(float v) { return row16_reduce(v, AddOp{}); }
+// (kept under its older name: the wave sum has this form everywhere now)
+__device__ __forceinline__ float wave_sum_dpp(float v) { return wave_sum(v); }
 
 // eight bf16 (one 16-byte piece) widened to fp32
 __device__ __forceinline__ void unpack8(const u32x4& v, float (&f)[8]) {

@@ -792,8 +792,8 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
     for (int r = 0; r < 4; ++r) {
       if (GPA == 4 && r >= M) continue;  // rows past M hold nothing (uniform: with GPA = 4 a lane's rows are r)
       float v = acc[nt][r];
-      if constexpr (GPA == 4) v += __shfl_xor(v, 16, 64);
-      if constexpr (GPA >= 2) v += __shfl_xor(v, 32, 64);
+      if constexpr (GPA == 4) v = combine_xor16(v, AddOp{});
+      if constexpr (GPA >= 2) v = combine_xor32(v, AddOp{});
       if (kq < KQS) red[((wave * NT + nt) * RP + 4 * kq + r) * 16 + col] = v;
     }
   __syncthreads();

@@ -840,10 +840,11 @@ def test_attn_decode_fused_both_merges(dev, merge, B, past, H, Hkv, hd):
                                     past_len_dev=pl, merge=merge)
         assert out is not None
         assert torch.allclose(out.cpu().float(), ref.float(), rtol=2 ** -7, atol=2 ** -7), rep
-    # and the dispatcher's own choice agrees with the forced one up to the order of the fp32 merge
+    # and the dispatcher's own choice agrees with the forced one up to the order of the fp32 merge: one rounding
+    # step of a bf16 output (2^-7 relative at most)
     out_auto = ops.attn_decode_fused(qkv.to(dev), qw.to(dev), kw.to(dev), sin, cos, kc, vc, ws, B, H, Hkv, hd, 0, Lmax, eps,
                                      past_len_dev=pl)
-    assert torch.allclose(out_auto.float(), out.float(), rtol=2 ** -8, atol=2 ** -10)
+    assert torch.allclose(out_auto.float(), out.float(), rtol=2 ** -7, atol=2 ** -10)
 
 
 @pytest.mark.parametrize("M", [1, 2, 4])
