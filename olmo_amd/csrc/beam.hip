@@ -71,12 +71,7 @@ __global__ __launch_bounds__(kThreads) void topk_kernel(const float* __restrict_
       // still to be emitted: strictly after the previous pick in the output order
       if (before(prev_v, prev_i, v, i) && before(v, i, best, bi)) best = v, bi = i;
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(best, o, 64);
-      const int oi = __shfl_xor(bi, o, 64);
-      if (before(ov, oi, best, bi)) best = ov, bi = oi;
-    }
+    wave_first_pair(best, bi, [](float ov, int oi, float v, int i) { return before(ov, oi, v, i); });
     if ((threadIdx.x & 63) == 0) sv[threadIdx.x >> 6] = best, si[threadIdx.x >> 6] = bi;
     __syncthreads();
     if (threadIdx.x == 0) {

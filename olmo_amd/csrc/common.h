@@ -133,6 +133,34 @@ __device__ __forceinline__ float combine_xor(float v, Op op) {
   else if constexpr (O == 1) return op(v, dpp_lane<0xB1>(v));
   else return op(v, __shfl_xor(v, O, 64));
 }
+// The (value, index) pair that comes first under `before` (a strict total order: before(av, ai, bv, bi) = "a goes
+// ahead of b") over the wave, in every lane.  DPP inside the rows of 16 lanes (after the first two steps a quad agrees,
+// so the mirrored partner holds what the xor partner would), then the swaps between half-rows and half-waves, after
+// which both candidates of a pair are at hand in every lane.
+template <typename Before>
+__device__ __forceinline__ void wave_first_pair(float& v, int& i, Before before) {
+  auto take = [&](float ov, int oi) {
+    if (before(ov, oi, v, i)) v = ov, i = oi;
+  };
+#define O355_PAIR_DPP(C) take(dpp_lane<C>(v), __builtin_amdgcn_update_dpp(0, i, C, 0xF, 0xF, true));
+  O355_PAIR_DPP(0xB1)
+  O355_PAIR_DPP(0x4E)
+  O355_PAIR_DPP(0x141)
+  O355_PAIR_DPP(0x140)
+#undef O355_PAIR_DPP
+  {
+    const auto rv = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, v), __builtin_bit_cast(uint32_t, v), false, false);
+    const auto ri = __builtin_amdgcn_permlane16_swap((uint32_t)i, (uint32_t)i, false, false);
+    v = __builtin_bit_cast(float, (uint32_t)rv[0]), i = (int)ri[0];
+    take(__builtin_bit_cast(float, (uint32_t)rv[1]), (int)ri[1]);
+  }
+  {
+    const auto rv = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, v), __builtin_bit_cast(uint32_t, v), false, false);
+    const auto ri = __builtin_amdgcn_permlane32_swap((uint32_t)i, (uint32_t)i, false, false);
+    v = __builtin_bit_cast(float, (uint32_t)rv[0]), i = (int)ri[0];
+    take(__builtin_bit_cast(float, (uint32_t)rv[1]), (int)ri[1]);
+  }
+}
 struct AddOp { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
 struct MaxOp { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
 

@@ -411,34 +411,8 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const void* __restrict__ x
       if (v > best || (v == best && i < bi)) best = v, bi = i;
     }
   }
-  // the wave's winner (largest value, smallest index among equals) through register moves: DPP inside the rows of 16
-  // lanes (after the first two steps a quad agrees, so the mirrored partner holds what the xor partner would),
-  // then the swaps between half-rows and half-waves, where both candidates of a pair are at hand in every lane
-  auto take_better = [&](float ov, int oi) {
-    if (ov > best || (ov == best && oi < bi)) best = ov, bi = oi;
-  };
-  auto dpp_step = [&](auto ctrl) {
-    constexpr int C = decltype(ctrl)::value;
-    const float ov = dpp_lane<C>(best);
-    const int oi = __builtin_amdgcn_update_dpp(0, bi, C, 0xF, 0xF, true);
-    take_better(ov, oi);
-  };
-  dpp_step(std::integral_constant<int, 0xB1>{});
-  dpp_step(std::integral_constant<int, 0x4E>{});
-  dpp_step(std::integral_constant<int, 0x141>{});
-  dpp_step(std::integral_constant<int, 0x140>{});
-  {
-    const auto rv = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, best), __builtin_bit_cast(uint32_t, best), false, false);
-    const auto ri = __builtin_amdgcn_permlane16_swap((uint32_t)bi, (uint32_t)bi, false, false);
-    best = __builtin_bit_cast(float, (uint32_t)rv[0]), bi = (int)ri[0];
-    take_better(__builtin_bit_cast(float, (uint32_t)rv[1]), (int)ri[1]);
-  }
-  {
-    const auto rv = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(uint32_t, best), __builtin_bit_cast(uint32_t, best), false, false);
-    const auto ri = __builtin_amdgcn_permlane32_swap((uint32_t)bi, (uint32_t)bi, false, false);
-    best = __builtin_bit_cast(float, (uint32_t)rv[0]), bi = (int)ri[0];
-    take_better(__builtin_bit_cast(float, (uint32_t)rv[1]), (int)ri[1]);
-  }
+  // the wave's winner: largest value, smallest index among equals
+  wave_first_pair(best, bi, [](float ov, int oi, float v, int i) { return ov > v || (ov == v && oi < i); });
   const int w = threadIdx.x >> 6;
   if ((threadIdx.x & 63) == 0) sv[w] = best, si[w] = bi;
   __syncthreads();

@@ -17,6 +17,7 @@
 // The draw walks the kept tokens in a fixed order (thread by thread, each in its own visiting order) with one 64-bit uniform number from
 // splitmix64(seed, counter, row): the distribution is the reference's, its random stream is not.
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
@@ -29,18 +30,38 @@ __device__ __forceinline__ uint64_t splitmix64(uint64_t x) {
   return x ^ (x >> 31);
 }
 
-__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int o) {
-  const uint32_t lo = __shfl_xor((uint32_t)v, o, 64), hi = __shfl_xor((uint32_t)(v >> 32), o, 64);
-  return ((uint64_t)hi << 32) | lo;
+// sum over the wave of a 64-bit count per lane, in every lane: the butterfly of wave_sum on both halves (register
+// moves, no trips through the LDS crossbar; integer sums do not depend on the order)
+__device__ __forceinline__ uint64_t wave_sum_u64(uint64_t v) {
+  auto join = [](uint32_t lo, uint32_t hi) { return ((uint64_t)hi << 32) | lo; };
+  auto dpp_step = [&](auto ctrl) {
+    constexpr int C = decltype(ctrl)::value;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, C, 0xF, 0xF, true);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), C, 0xF, 0xF, true);
+    v += join(lo, hi);
+  };
+  dpp_step(std::integral_constant<int, 0xB1>{});   // quad_perm [1,0,3,2]
+  dpp_step(std::integral_constant<int, 0x4E>{});   // quad_perm [2,3,0,1]
+  dpp_step(std::integral_constant<int, 0x141>{});  // row_half_mirror (the quads agree by now)
+  dpp_step(std::integral_constant<int, 0x140>{});  // row_mirror
+  {
+    const auto lo = __builtin_amdgcn_permlane16_swap((uint32_t)v, (uint32_t)v, false, false);
+    const auto hi = __builtin_amdgcn_permlane16_swap((uint32_t)(v >> 32), (uint32_t)(v >> 32), false, false);
+    v = join(lo[0], hi[0]) + join(lo[1], hi[1]);
+  }
+  {
+    const auto lo = __builtin_amdgcn_permlane32_swap((uint32_t)v, (uint32_t)v, false, false);
+    const auto hi = __builtin_amdgcn_permlane32_swap((uint32_t)(v >> 32), (uint32_t)(v >> 32), false, false);
+    v = join(lo[0], hi[0]) + join(lo[1], hi[1]);
+  }
+  return v;
 }
 
 // sum of NV 64-bit values per thread over the workgroup; every thread gets the totals
 template <int NV>
 __device__ __forceinline__ void block_sum_u64(uint64_t (&v)[NV], uint64_t* lds /* [kWaves][NV] */) {
 #pragma unroll
-  for (int j = 0; j < NV; ++j)
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v[j] += shfl_xor_u64(v[j], o);
+  for (int j = 0; j < NV; ++j) v[j] = wave_sum_u64(v[j]);
   const int w = threadIdx.x >> 6;
   __syncthreads();  // the previous use of lds is over
   if ((threadIdx.x & 63) == 0) {
