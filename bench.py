@@ -253,7 +253,8 @@ def main() -> int:
     # ---- what this box gives a kernel that only streams the same weights / only issues MFMAs ----------
     # Same launches as above (one per block Linear, distinct buffers, one captured graph), but the kernel reads
     # the tiled weight bytes and does nothing else: the distance from here to the published 8 TB/s is not the
-    # linear kernel's to close.  The matrix-core probe runs v_mfma_f32_32x32x16_bf16 on random operands.
+    # linear kernel's to close.  The matrix-core probe runs v_mfma_f32_16x16x32_bf16 (the GEMM's instruction) on
+    # random operands.
     from olmo_amd._lib import check as _check, lib as _lib
 
     sink = torch.zeros(1024, dtype=torch.int32, device=dev)
@@ -326,7 +327,7 @@ def main() -> int:
     mfma_tf = fl.value / (e0.elapsed_time(e1) * 1e-3) / 1e12
     extra["ceilings"]["mfma_bf16_random_operands"] = {"achieved": mfma_tf, "unit": "TFLOP/s",
                                                       "frac_of_peak": mfma_tf / MFMA_BF16_PEAK_TF}
-    log(f"[bench] ceiling on this box: MFMA-only bf16 (32x32x16, random operands, all CUs): {mfma_tf:.0f} TFLOP/s")
+    log(f"[bench] ceiling on this box: MFMA-only bf16 (16x16x32, random operands, all CUs): {mfma_tf:.0f} TFLOP/s")
     del xp
 
     # ---- batch 8 ------------------------------------------------------------------------------------

@@ -346,7 +346,8 @@ int olmo355_incr_i32(int32_t* p, void* stream);
 /* ---- measuring probes (no counterpart in the reference; used by bench.py only) -------------------
  * What a kernel that only streams `bytes` from HBM takes (16-byte non-temporal loads per lane, launch shaped
  * like the small-M linears; nothing is written), and what the matrix cores sustain on random bf16 operands
- * (256 workgroups x 8 waves x iters x 8 v_mfma_f32_32x32x16_bf16; *flops = total floating-point operations).
+ * (256 workgroups x 8 waves x iters x 16 v_mfma_f32_16x16x32_bf16, the prefill GEMM's instruction; *flops = total
+ * floating-point operations).
  * `sink` is a device buffer of at least 2 KiB that stays unwritten. */
 int olmo355_probe_stream_read(const void* src, int64_t bytes, void* sink, void* stream);
 /* The same over n buffers (host arrays of device pointers and byte counts, n <= 160) in ONE launch of a persistent

@@ -1,20 +1,23 @@
 // Large-M linear layers (prefill): y[M,N] = x[M,K] . W[K,N] on the matrix cores
-// (v_mfma_f32_32x32x16_bf16), fp32 accumulation, bf16 output.
+// (v_mfma_f32_16x16x32_bf16: with random operands it sustains 2.09 PFLOP/s on this part where
+// v_mfma_f32_32x32x16_bf16 sustains 1.85 -- the chip is power-bound and the smaller tile moves fewer
+// accumulator registers per flop), fp32 accumulation, bf16 output.
 //
 // Workgroup = 8 waves (two per SIMD) in a 2x4 or 4x2 arrangement over a BM x BN output tile: 256 rows by
-// 256, 192 or 128 columns, or 128 rows by 128 or 64 columns; each wave owns WMT x WNT MFMA tiles of
-// 32 x 32.  K advances 64 per stage.  Activations go memory -> LDS directly (8 rows x 128 bytes per
-// instruction, the 16-byte chunks of a row XOR-swizzled so the operand reads are conflict-free), ring of
+// 256, 192 or 128 columns, or 128 rows by 128 or 64 columns; each wave owns 2 WMT x 2 WNT MFMA tiles of
+// 16 x 16.  K advances 64 per stage, two k-steps of 32.  Activations go memory -> LDS directly (8 rows x 128
+// bytes per instruction, the 16-byte chunks of a row XOR-swizzled so the operand reads are conflict-free), ring of
 // three stages requested two stages ahead.  Weights are staged in LDS in *fragment-major* order
-// -- [32-column tile][k-step of 16][64 lanes][16 bytes] -- so every MFMA operand is one conflict-free
-// ds_read_b128; int4 words come into registers two stages ahead and are dequantised (scale and zero
-// in fp32, one rounding to bf16) into LDS ahead of their stage, double-buffered; dense weights are copied
-// memory -> LDS as they are tiled.  The staging work is spread between the k-steps of the MFMA loop so
-// that the VALU / LDS / memory instructions issue in the shadow of the matrix pipeline; operand fragments are
-// read one k-step ahead of the matrix instructions that use them; one barrier per stage, after its third
-// k-step.  The matrix instructions take the weight fragment as their first operand, so the accumulators hold
-// the output tile transposed (a lane owns runs of neighbouring columns of one row) and the epilogue writes 16
-// bytes per lane and store.
+// -- [16-column tile][k-step of 32][64 lanes][16 bytes], which is the order of the tiled weight formats themselves --
+// so every MFMA operand is one conflict-free ds_read_b128; int4 words come into registers two stages ahead and are
+// dequantised (scale and zero in fp32, one rounding to bf16) into LDS ahead of their stage, double-buffered; dense
+// weights are copied memory -> LDS as they are tiled.  The staging work is spread between the k-steps of the
+// MFMA loop so that the VALU / LDS / memory instructions issue in the shadow of the matrix pipeline; operand
+// fragments are read ahead of the matrix instructions that use them into registers that have just been read for
+// the last time; one barrier per stage, where the stage's last fragments have been asked for.  The matrix
+// instructions take the weight fragment as their first operand, so the accumulators hold the output tile transposed
+// (a lane owns four neighbouring columns of one row per 16 x 16 block) and the epilogue, after one exchange of
+// half-rows between neighbouring blocks, writes 16 bytes per lane and store.
 //
 // The int4 operand is W = bf16(scale * (q - zero)) (fp32 product, one rounding).
 #include "common.h"
@@ -23,10 +26,8 @@
 
 namespace {
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-
 constexpr int BK = 64;      // K per stage
-constexpr int KSTEPS = 4;   // MFMA k-steps of 16 per stage
+constexpr int KSTEPS = 2;   // MFMA k-steps of 32 per stage
 
 // dequantise one tiled word (8 weights of one column) to 8 bf16 in MFMA operand order.
 // The nibbles are turned into fp16 numbers where they stand: (w & 0x000f000f) | 0x64006400 is the pair
@@ -107,7 +108,7 @@ __device__ __forceinline__ StreamKArgsPtr streamk_args() {
 }
 enum { GEMM_PLAIN = 0, GEMM_SPLIT = 1, GEMM_STREAMK = 2 };
 
-template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false, int KIND = GEMM_PLAIN>  // wave grid, 32x32 MFMA tiles per wave
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false, int KIND = GEMM_PLAIN>  // wave grid, 32 x 32 blocks (of four 16 x 16 MFMA tiles) per wave
 __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wt,
                                           const uint16_t* __restrict__ st, const uint8_t* __restrict__ zt,
                                           uint16_t* __restrict__ y, int M, int N, int K, int tile_m, int tile_n,
@@ -117,6 +118,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   constexpr bool SPLIT = KIND == GEMM_SPLIT;
   constexpr int NW = WAVES_M * WAVES_N, NT = 64 * NW;
   constexpr int BM = 32 * WMT * WAVES_M, BN = 32 * WNT * WAVES_N;
+  constexpr int MT = 2 * WMT, NT16 = 2 * WNT;  // 16 x 16 MFMA tiles per wave
   constexpr int A_BLK = BM / 8;        // 1 KiB blocks per stage: activations, 8 rows x 128 bytes each
   constexpr int B_BLK = BN / 8;        // weights: 32x16 bf16 pieces (either layout)
   constexpr int A_PW = A_BLK / NW, B_PW = B_BLK / NW;
@@ -148,7 +150,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   const int G = K >> 7, KS = K >> 5;  // strides of the tiled weight: always of the whole K
   const int Gn = Kn >> 7;             // groups of 128 rows in the run
   const int stages = Kn / BK;
-  const int row32 = lane & 31, kh = lane >> 5;
+  const int row16 = lane & 15, kq4 = lane >> 4;  // operand row (or column) of a 16 x 32 fragment, its 8-wide k block
 
   // ---- activations: memory -> LDS directly ------------------------------------------------------
   // One instruction moves 8 rows x 128 bytes (the 64 k of a stage): 8 consecutive lanes cover one
@@ -171,11 +173,11 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(smem + ((buf * A_BLK + wave * A_PW + i) << 10)), 16, a_voff[i],
                                                s * (BK * 2), 0, 0);
   };
-  // operand read: lane (row32, kh), row tile rt, k-step ks -> 16-byte slot
-  const int a_swz = (row32 >> 1) & 7;
+  // operand read: lane (row16, kq4), 16-row tile rt, k-step ks -> 16-byte slot
+  const int a_swz = (row16 >> 1) & 7;
   int a_rd[KSTEPS];
 #pragma unroll
-  for (int ks = 0; ks < KSTEPS; ++ks) a_rd[ks] = row32 * 8 + ((2 * ks + kh) ^ a_swz);
+  for (int ks = 0; ks < KSTEPS; ++ks) a_rd[ks] = row16 * 8 + ((4 * ks + kq4) ^ a_swz);
 
   // ---- weights ---------------------------------------------------------------------------------
   const int g0 = k0 >> 7, ks0 = k0 >> 5;  // first group / 32-row step of the run
@@ -214,12 +216,10 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   auto stash_b_word = [&](int buf, int set, int i, int j) {  // word j (32-row step j of the group) of item i
     const int ntl = wave + NW * i;
     if (B_RAGGED && ntl >= BN / 16) return;  // wave-uniform
-    const int kq = lane >> 4;
-    const int slot = (kq & 1) * 32 + (ntl & 1) * 16 + (lane & 15);
-    const int f = (ntl >> 1) * KSTEPS + 2 * (j & 1) + (kq >> 1);
     const float sc = (float)__builtin_bit_cast(_Float16, (uint16_t)rsb[set][i]);
     const DequantConsts dc = dequant_consts(sc, 1 + (int)((rzb[set][i] >> (4 * (lane & 1))) & 15u));  // stored zero points are one less
-    lds_b[(buf * B_BLK + f) * 64 + slot] = dequant_word_bf16(rbw[set][i][j], dc);
+    // a tiled word is already the lane's piece of a 16-column x 32-row operand fragment: it stays in its lane
+    lds_b[(buf * B_BLK + ntl * KSTEPS + (j & 1)) * 64 + lane] = dequant_word_bf16(rbw[set][i][j], dc);
   };
   // dense: the tiled pieces [16-column tile][32-row step][64][16 B] are copied as they are
   int bd_voff[W4 ? 1 : B_PW];
@@ -236,88 +236,96 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_ptr_t)(smem + ((3 * A_BLK + buf * B_BLK + wave * B_PW + i) << 10)), 16,
                                                bd_voff[i], s * 2048, 0, 0);
   };
-  // operand read of column tile ct, k-step ks: int4 fragment-major; dense: piece (2 ct + n32/16, ks/2),
-  // lane (n32 & 15) + 16 (2 (ks & 1) + kh)
-  const int b_rd = W4 ? lane : (row32 >> 4) * 128 + (row32 & 15) + 16 * kh;
-  auto b_slot = [&](int ct, int ks) { return W4 ? (ct * KSTEPS + ks) * 64 : ct * 256 + (ks >> 1) * 64 + (ks & 1) * 32; };
+  // operand read of 16-column tile ct, k-step ks: either kind of weight sits in LDS as [tile][k-step][64 lanes][16 B]
+  const int b_rd = lane;
+  auto b_slot = [&](int ct, int ks) { return (ct * KSTEPS + ks) * 64; };
 
-  // requests of a stage issued in its first three k-steps (those after them are the next stage's business)
-  constexpr int keep_a = [] { int n = 0; for (int i = 0; i < A_PW; ++i) n += (i * KSTEPS / A_PW <= KSTEPS - 2); return n; }();
-  constexpr int keep_b = [] { int n = 0; for (int i = 0; i < NBI; ++i) n += ((2 * i + 1) * KSTEPS / (2 * NBI) <= KSTEPS - 2); return n; }();
+  // The stage's one barrier stands where its last operand fragments have been asked for: at the end of the k-step
+  // before the last when a k-step's fragments all sit in registers at once (they are then asked for one k-step
+  // ahead), otherwise inside the last k-step, after the RB rounds whose registers are refilled from this stage.
+  constexpr int MT_ = 2 * WMT, NT16_ = 2 * WNT, OUT_ = NT16_ <= MT_ ? MT_ : NT16_;
+  constexpr int RB = OUT_ > 4 ? OUT_ - 4 : 0;
+  constexpr int LAST_PART = RB > 0 ? KSTEPS - 1 : KSTEPS - 2;  // requests of a stage issued up to this k-step precede its barrier
+  constexpr int keep_a = [] { int n = 0; for (int i = 0; i < A_PW; ++i) n += (i * KSTEPS / A_PW <= LAST_PART); return n; }();
+  constexpr int keep_b = [] { int n = 0; for (int i = 0; i < NBI; ++i) n += ((2 * i + 1) * KSTEPS / (2 * NBI) <= LAST_PART); return n; }();
 
-  f32x16 acc[WMT][WNT];
+  f32x4 acc[MT][NT16];
 #pragma unroll
-  for (int i = 0; i < WMT; ++i)
+  for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int j = 0; j < WNT; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    for (int j = 0; j < NT16; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // Operand fragments are read one k-step ahead.  The operand with fewer fragments per wave is double-buffered
-  // in registers; a fragment of the other one is asked for again as soon as the matrix instructions that read
-  // its registers have been issued.
-  constexpr bool OUTER_A = WNT <= WMT;
-  bf16x8 fa[OUTER_A ? 1 : 2][WMT], fb[OUTER_A ? 2 : 1][WNT];
+  // Operand fragments are read ahead of the matrix instructions that use them, into registers that have just
+  // been read for the last time.  The k-step is a loop of rounds over the fragments of one operand (the one with
+  // more of them), each round multiplying one of them with all fragments of the other.  The outer operand keeps at
+  // most four fragments in registers: after round r its registers are asked for the fragment of round r + 4
+  // (of this k-step or of the next); the inner operand's fragments are asked for again during the k-step's last
+  // round.
+  constexpr bool OUTER_A = NT16 <= MT;
+  constexpr int OUT = OUTER_A ? MT : NT16, INN = OUTER_A ? NT16 : MT, OS = OUT < 4 ? OUT : 4;
+  static_assert((KSTEPS * OUT) % OS == 0, "a stage's rounds must fill the slots a whole number of times");
+  bf16x8 fo[OS], fi[INN];
   auto read_a = [&](int abuf, int i, int ks) {
-    return __builtin_bit_cast(bf16x8, lds_a[abuf * A_BLK * 64 + (wm * WMT + i) * 256 + a_rd[ks]]);
+    return __builtin_bit_cast(bf16x8, lds_a[abuf * A_BLK * 64 + (wm * MT + i) * 128 + a_rd[ks]]);
   };
   auto read_b = [&](int bbuf, int j, int ks) {
-    return __builtin_bit_cast(bf16x8, lds_b[bbuf * B_BLK * 64 + b_slot(wn * WNT + j, ks) + b_rd]);
+    return __builtin_bit_cast(bf16x8, lds_b[bbuf * B_BLK * 64 + b_slot(wn * NT16 + j, ks) + b_rd]);
   };
+  auto read_outer = [&](int abuf, int bbuf, int t, int ks) { return OUTER_A ? read_a(abuf, t, ks) : read_b(bbuf, t, ks); };
+  auto read_inner = [&](int abuf, int bbuf, int t, int ks) { return OUTER_A ? read_b(bbuf, t, ks) : read_a(abuf, t, ks); };
   auto ring_next = [](int ab) { return ab == 2 ? 0 : ab + 1; };
-  // int4: a thread's 2 * B_ITEMS words of a stage are dequantised in the four k-steps before the barrier that
-  // publishes the stage: slot 0 = the last k-step of the stage before the previous one's barrier ... see do_stage
+  // int4: a thread's 2 * B_ITEMS words of a stage are dequantised in the k-steps before the barrier that
+  // publishes the stage, an equal share in each: see do_stage
   auto word_slot = [](int i) { return i * KSTEPS / (2 * B_ITEMS); };
 
   // One stage.  Activations sit in a ring of three LDS buffers and are requested two stages ahead;
   // the weights are double-buffered in LDS (int4: requested two stages ahead into registers, set
   // = parity of the 128-row group, and dequantised into LDS ahead of their stage; dense: copied one stage
-  // ahead).  The stage's one barrier stands after its third k-step: by then every wave has read the stage's last
-  // fragments, so the buffers of this stage may be written again, and everything of the next stage is in LDS, so
-  // the last k-step reads the next stage's first fragments.  Memory operations complete in order, so waiting until
-  // only the requests of this stage's first three k-steps (KEEP of them) are outstanding means that everything the
-  // next stage reads has landed.
+  // ahead).  The stage's one barrier stands where the wave has asked for the stage's last fragments (inside the
+  // last k-step when the outer operand has more fragments than register slots, else before it): from there on
+  // the buffers of this stage may be written again, and everything of the next stage is in LDS, so the reads after
+  // it fetch the next stage's first fragments.  A read of this stage placed after the barrier would race with the
+  // faster waves' writes of the stage after next.  Memory operations complete in order, so waiting until only the
+  // requests issued in this stage before the barrier's part (KEEP of them) are outstanding means that everything
+  // the next stage reads has landed.
   //   h = parity of the stage = weight LDS buffer (and, int4, the half of the group)
   //   p = parity of the group (int4 register set)
   auto do_stage = [&](int s, int ab, auto hc, auto pc) {
     constexpr int h = decltype(hc)::value, p = decltype(pc)::value;
     const int s2 = min(s + 2, stages - 1);  // past the end: re-fetch the last stage into a buffer nobody reads
     const int ab1 = ring_next(ab), ab2 = ring_next(ab1);
+    auto stage_barrier = [&]() {
+      constexpr int KEEP = keep_a + ((W4 && h == 1) ? 3 * keep_b : 0);
+      static_assert(KEEP < 64, "vmcnt range");
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt((KEEP & 15) | ((KEEP >> 4) << 14) | 0x0070);  // vmcnt(KEEP) lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    };
     if constexpr (!W4) {
       load_b_dense(min(s + 1, stages - 1), h ^ 1);
       __builtin_amdgcn_sched_barrier(0);  // keep the order: the weights' requests are the older ones
     }
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
-      const int cur = ks & 1, nxt = cur ^ 1, nks = (ks + 1) & (KSTEPS - 1);
+      const int nks = (ks + 1) & (KSTEPS - 1);
       const int nab = ks == KSTEPS - 1 ? ab1 : ab, nh = ks == KSTEPS - 1 ? (h ^ 1) : h;
-      if constexpr (OUTER_A) {
-#pragma unroll
-        for (int j = 0; j < WNT; ++j) fb[nxt][j] = read_b(nh, j, nks);
-      } else {
-#pragma unroll
-        for (int i = 0; i < WMT; ++i) fa[nxt][i] = read_a(nab, i, nks);
-      }
       // requests are spread over the stage: a burst of them stalls the wave at issue
       load_a(s2, ab2, ks);
       if constexpr (W4 && h == 1) fetch_b(min((s >> 1) + 2, Gn - 1), p, ks);
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (OUTER_A) {
 #pragma unroll
-        for (int i = 0; i < WMT; ++i) {
+      for (int r = 0; r < OUT; ++r) {
+        const int slot = (ks * OUT + r) % OS;  // rounds are numbered through the stage: slots rotate across its k-steps
 #pragma unroll
-          for (int j = 0; j < WNT; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[0][i], acc[i][j], 0, 0, 0);
-          fa[0][i] = read_a(nab, i, nks);
+        for (int q = 0; q < INN; ++q) {
+          if constexpr (OUTER_A) acc[r][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fi[q], fo[slot], acc[r][q], 0, 0, 0);
+          else acc[q][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fo[slot], fi[q], acc[q][r], 0, 0, 0);
+          if (r == OUT - 1) fi[q] = read_inner(nab, nh, q, nks);
         }
-      } else {
-#pragma unroll
-        for (int j = 0; j < WNT; ++j) {
-#pragma unroll
-          for (int i = 0; i < WMT; ++i)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[0][j], fa[cur][i], acc[i][j], 0, 0, 0);
-          fb[0][j] = read_b(nh, j, nks);
-        }
+        const int rn = r + OS;  // the round this slot serves next
+        fo[slot] = rn < OUT ? read_outer(ab, h, rn, ks) : read_outer(nab, nh, rn - OUT, nks);
+        if (RB > 0 && ks == KSTEPS - 1 && r == RB - 1) stage_barrier();  // the stage's last fragments have been asked for
       }
       if constexpr (W4) {
 #pragma unroll
@@ -331,13 +339,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
           }
         }
       }
-      if (ks == KSTEPS - 2) {
-        constexpr int KEEP = keep_a + ((W4 && h == 1) ? 3 * keep_b : 0);
-        static_assert(KEEP < 64, "vmcnt range");
-        __builtin_amdgcn_s_waitcnt((KEEP & 15) | ((KEEP >> 4) << 14) | 0x0070);  // vmcnt(KEEP) lgkmcnt(0)
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-      }
+      if (RB == 0 && ks == KSTEPS - 2) stage_barrier();
     }
   };
 
@@ -366,9 +368,9 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     }
   }
 #pragma unroll
-  for (int i = 0; i < WMT; ++i) fa[0][i] = read_a(0, i, 0);
+  for (int t = 0; t < OS; ++t) fo[t] = read_outer(0, 0, t, 0);
 #pragma unroll
-  for (int j = 0; j < WNT; ++j) fb[0][j] = read_b(0, j, 0);
+  for (int t = 0; t < INN; ++t) fi[t] = read_inner(0, 0, t, 0);
 
   using H0 = std::integral_constant<int, 0>;
   using H1 = std::integral_constant<int, 1>;
@@ -394,9 +396,9 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   }
 
   // ---- stream-K: partial tiles travel between workgroups as the accumulators stand ------------------------
-  constexpr int QUADS = WMT * WNT * 4;  // float4 per lane
+  constexpr int QUADS = MT * NT16;  // float4 per lane: one per 16 x 16 block
   constexpr int SLOT_BYTES = NW * QUADS * 64 * 16;
-  auto quad_off = [&](int i, int j, int q) { return ((wave * QUADS + (i * WNT + j) * 4 + q) * 64 + lane) * 16; };
+  auto quad_off = [&](int i, int j) { return ((wave * QUADS + i * NT16 + j) * 64 + lane) * 16; };
   if constexpr (KIND == GEMM_STREAMK) {
     // (a partial is left behind -- sk_mode 1 -- from inside the ordinary epilogue's loops below: as a block of
     // its own before them it drives the register allocation of the whole function into spilling accumulators)
@@ -427,38 +429,32 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
         const int ok = *s_ok;
         const __amdgpu_buffer_rsrc_t rs = make_rsrc(reinterpret_cast<const char*>(slots) + (int64_t)pc * SLOT_BYTES, SLOT_BYTES);
 #pragma unroll
-        for (int i = 0; i < WMT; ++i)
+        for (int i = 0; i < MT; ++i) {
+          f32x4 v[NT16];
 #pragma unroll
-          for (int j = 0; j < WNT; ++j) {
-            f32x4 v[4];
+          for (int j = 0; j < NT16; ++j)
+            v[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, quad_off(i, j), 0, 16 /* sc1 */));
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-              v[q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, quad_off(i, j, q), 0, 16 /* sc1 */));
+          for (int j = 0; j < NT16; ++j)
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-#pragma unroll
-              for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] = ok ? acc[i][j][4 * q + e] + v[q][e] : __builtin_nanf("");
-          }
+            for (int e = 0; e < 4; ++e) acc[i][j][e] = ok ? acc[i][j][e] + v[j][e] : __builtin_nanf("");
+        }
       }
     }
   }
 
   // ---- epilogue ------------------------------------------------------------------------------------------
-  // The products were formed as W^T-tile x X^T-tile, so a lane holds one output row m = lane & 31 of its 32 x 32
-  // block and the columns n = 8 q + 4 (lane >> 5) + (r & 3) in register r = 4 q + (r & 3): four neighbours in a
-  // row per register quad.  As bf16 pairs, the quads q = 0, 1 (and 2, 3) of the two half-waves are exchanged so that
-  // every lane ends up with 8 neighbouring columns: two 16-byte stores per block and lane instead of sixteen
-  // 2-byte ones.
+  // The products were formed as W^T-tile x X^T-tile, so a lane holds one output row m = lane & 15 of its 16 x 16
+  // block and the four neighbouring columns n = 4 (lane >> 4) + r.  As bf16 pairs, two blocks that are neighbours along
+  // n trade half-rows of the wave (v_permlane16_swap): the lanes of rows 0 and 2 end up with columns 0-7 and 8-15 of
+  // the first block, those of rows 1 and 3 with the same of the second -- one 16-byte store per lane and pair of
+  // blocks instead of eight 2-byte ones.
   // sk_mode 1: device-scope stores (they do not stay in this XCD's L2) of one block's accumulators into this
   // workgroup's slot; once all are out every wave waits for its own to be acknowledged, then one thread raises the flag
   auto leave_partial_block = [&](int i, int j) {
     const StreamKArgsPtr ka = streamk_args();
     const __amdgpu_buffer_rsrc_t rs = make_rsrc(reinterpret_cast<const char*>(ka->slots) + (int64_t)sk_self * SLOT_BYTES, SLOT_BYTES);
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-      __builtin_amdgcn_raw_buffer_store_b128(
-          __builtin_bit_cast(u32x4, f32x4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]}),
-          rs, quad_off(i, j, q), 0, 16 /* sc1 */);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), rs, quad_off(i, j), 0, 16 /* sc1 */);
   };
   auto announce_partial = [&]() {
     const StreamKArgsPtr ka = streamk_args();
@@ -468,79 +464,63 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     __syncthreads();
     if (tid == 0 && publish) __hip_atomic_store(flags + sk_self, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   };
-  const int half = lane >> 5, mrow = lane & 31;
-  auto store_block = [&](const uint32_t (&pk)[4][2], uint16_t* __restrict__ dst, int m, int nb, int ncols, int ld) {
-    uint32_t o[4][2];
+  // va, vb: this lane's four outputs (columns 4 kq4 .. + 3 of row m) of two blocks whose first columns are nb and nb + 16
+  auto store_pair = [&](const f32x4& va, const f32x4& vb, uint16_t* __restrict__ dst, int m, int nb, int ncols, int ld) {
+    uint32_t o[2][2];
 #pragma unroll
-    for (int qq = 0; qq < 4; qq += 2)
-#pragma unroll
-      for (int x = 0; x < 2; ++x) {
-        const auto sw = __builtin_amdgcn_permlane32_swap(pk[qq][x], pk[qq + 1][x], false, false);
-        o[qq][x] = sw[0], o[qq + 1][x] = sw[1];
-      }
-#pragma unroll
-    for (int qq = 0; qq < 4; qq += 2) {
-      const int n = nb + 8 * qq + 8 * half;
-      if (m < M && n < ncols)
-        *reinterpret_cast<u32x4*>(dst + (int64_t)m * ld + n) = u32x4{o[qq][0], o[qq][1], o[qq + 1][0], o[qq + 1][1]};
+    for (int x = 0; x < 2; ++x) {
+      const auto sw = __builtin_amdgcn_permlane16_swap(pack_bf16x2(va[2 * x], va[2 * x + 1]), pack_bf16x2(vb[2 * x], vb[2 * x + 1]),
+                                                       false, false);
+      o[0][x] = sw[0], o[1][x] = sw[1];
     }
+    const int n = nb + 16 * (kq4 & 1) + 8 * (kq4 >> 1);
+    if (m < M && n < ncols) *reinterpret_cast<u32x4*>(dst + (int64_t)m * ld + n) = u32x4{o[0][0], o[0][1], o[1][0], o[1][1]};
   };
   if constexpr (SWIGLU) {
+    // per wave: 16-column blocks 0, 1 come from the up half of the weight, 2, 3 from the matching gate columns
     const int half_n = N >> 1;
     const int nb = tile_n * (BN / 2) + wn * 32;  // no ragged columns: N/2 is a multiple of BN/2
 #pragma unroll
-    for (int i = 0; i < WMT; ++i) {
+    for (int i = 0; i < MT; ++i) {
       if (KIND == GEMM_STREAMK && sk_mode == 1) {
-        leave_partial_block(i, 0);
-        leave_partial_block(i, 1);
+#pragma unroll
+        for (int j = 0; j < NT16; ++j) leave_partial_block(i, j);
         continue;
       }
-      uint32_t pk[4][2];
+      f32x4 v[2];
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
+      for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
-        for (int x = 0; x < 2; ++x) {
-          float v[2];
-#pragma unroll
-          for (int e = 0; e < 2; ++e) {
-            const int r = 4 * q + 2 * x + e;
-            const float up = round_bf16(acc[i][0][r]), gate = round_bf16(acc[i][1][r]);  // the Linear's bf16 output
-            const float sg = round_bf16(gate / (1.f + expf(-gate)));
-            v[e] = sg * up;
-          }
-          pk[q][x] = pack_bf16x2(v[0], v[1]);
+        for (int e = 0; e < 4; ++e) {
+          const float up = round_bf16(acc[i][jj][e]), gate = round_bf16(acc[i][jj + 2][e]);  // the Linear's bf16 output
+          const float sg = round_bf16(gate / (1.f + expf(-gate)));
+          v[jj][e] = sg * up;
         }
-      store_block(pk, y, m0 + (wm * WMT + i) * 32 + mrow, nb, half_n, half_n);
+      store_pair(v[0], v[1], y, m0 + (wm * MT + i) * 16 + row16, nb, half_n, half_n);
     }
     if (KIND == GEMM_STREAMK && sk_mode == 1 && !sk_defer) announce_partial();
     return;
   }
 #pragma unroll
-  for (int i = 0; i < WMT; ++i)
+  for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int j = 0; j < WNT; ++j) {
+    for (int j = 0; j < NT16; j += 2) {
       if (KIND == GEMM_STREAMK && sk_mode == 1) {
         leave_partial_block(i, j);
+        leave_partial_block(i, j + 1);
         continue;
       }
-      const int nb = (nt0 >> 1) * 32 + (wn * WNT + j) * 32;  // wave-uniform
+      const int nb = (nt0 >> 1) * 32 + (wn * NT16 + j) * 16;  // wave-uniform; columns come in whole blocks of 16
       if (nb >= N) continue;
-      const int m = m0 + (wm * WMT + i) * 32 + mrow;
+      const int m = m0 + (wm * MT + i) * 16 + row16;
       if constexpr (SPLIT) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = nb + 8 * q + 4 * half;
-          if (m < M && n < N)
-            *reinterpret_cast<f32x4*>(part + ((int64_t)blockIdx.y * M + m) * N + n) =
-                f32x4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+        for (int jj = 0; jj < 2; ++jj) {
+          const int n = nb + 16 * jj + 4 * kq4;
+          if (m < M && n < N) *reinterpret_cast<f32x4*>(part + ((int64_t)blockIdx.y * M + m) * N + n) = acc[i][j + jj];
         }
       } else {
-        uint32_t pk[4][2];
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-#pragma unroll
-          for (int x = 0; x < 2; ++x) pk[q][x] = pack_bf16x2(acc[i][j][4 * q + 2 * x], acc[i][j][4 * q + 2 * x + 1]);
-        store_block(pk, y, m, nb, N, N);
+        store_pair(acc[i][j], acc[i][j + 1], y, m, nb, N, N);
       }
     }
   if (KIND == GEMM_STREAMK && sk_mode == 1 && !sk_defer) announce_partial();

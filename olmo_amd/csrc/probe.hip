@@ -75,15 +75,14 @@ __global__ __launch_bounds__(512) void stream_read_many_kernel(ManyArgs a, uint3
   if (acc == 0x9e3779b9u) sink[threadIdx.x] = acc;
 }
 
-// 8 waves per workgroup, 8 independent 32x32 accumulators per wave, operands drawn once from a generator
+// 8 waves per workgroup, 16 independent 16x16 accumulators per wave, operands drawn once from a generator
 // (random mantissas and signs, exponents near 1: constant operands run faster than a real product does).
+// v_mfma_f32_16x16x32_bf16 is the instruction the prefill GEMM uses; on random operands it sustains more than
+// the 32x32x16 form does (the part is power-bound and this shape moves fewer accumulator registers per flop).
 __global__ __launch_bounds__(512) void mfma_bf16_kernel(float* __restrict__ sink, int iters, uint32_t seed) {
-  typedef float f32x16 __attribute__((ext_vector_type(16)));
-  f32x16 acc[8];
+  f32x4 acc[16];
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
-#pragma unroll
-    for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+  for (int i = 0; i < 16; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   uint32_t r = seed + (blockIdx.x * 512 + threadIdx.x) * 2654435761u;
   auto draw = [&]() {
     u32x4 v;
@@ -94,20 +93,18 @@ __global__ __launch_bounds__(512) void mfma_bf16_kernel(float* __restrict__ sink
     }
     return __builtin_bit_cast(bf16x8, v);
   };
-  bf16x8 a[4], b[2];
+  bf16x8 a[4], b[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) a[i] = draw();
 #pragma unroll
-  for (int i = 0; i < 2; ++i) b[i] = draw();
+  for (int i = 0; i < 4; ++i) b[i] = draw();
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i * 2 + j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i * 2 + j], 0, 0, 0);
+    for (int i = 0; i < 16; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i & 3], b[i >> 2], acc[i], 0, 0, 0);
   }
   float s = 0.f;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) s += acc[i][0];
+  for (int i = 0; i < 16; ++i) s += acc[i][0];
   if (s == 12345.678f) sink[threadIdx.x] = s;
 }
 
@@ -150,10 +147,10 @@ extern "C" int olmo355_probe_stream_read_many(const void* const* srcs, const int
   O355_CHECK_LAUNCH();
 }
 
-// 256 workgroups x 8 waves x iters x 8 MFMAs of 32x32x16 (32768 flop each); *flops receives the total.
+// 256 workgroups x 8 waves x iters x 16 MFMAs of 16x16x32 (16384 flop each); *flops receives the total.
 extern "C" int olmo355_probe_mfma_bf16(int iters, void* sink, double* flops, void* stream) {
   if (iters <= 0 || !sink) return O355_EINVAL;
   hipLaunchKernelGGL(mfma_bf16_kernel, dim3(256), dim3(512), 0, as_stream(stream), (float*)sink, iters, 77u);
-  if (flops) *flops = 256.0 * 8.0 * (double)iters * 8.0 * 32768.0;
+  if (flops) *flops = 256.0 * 8.0 * (double)iters * 16.0 * 16384.0;
   O355_CHECK_LAUNCH();
 }
