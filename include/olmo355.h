@@ -354,6 +354,10 @@ int olmo355_probe_stream_read(const void* src, int64_t bytes, void* sink, void* 
  * grid of two workgroups per CU: no launch boundary and no ramp per buffer. */
 int olmo355_probe_stream_read_many(const void* const* srcs, const int64_t* bytes, int n, void* sink, void* stream);
 int olmo355_probe_mfma_bf16(int iters, void* sink, double* flops, void* stream);
+/* For tests: leaves `pattern` in every 32-bit word of the LDS of every CU (LDS keeps what the last workgroup left
+ * there, so a kernel that reads LDS it has not written gives results that depend on what ran before it; with a NaN
+ * pattern in place such a read shows in the output). */
+int olmo355_probe_fill_lds(uint32_t pattern, void* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -88,6 +88,7 @@ EXPORTS = {
     "olmo355_probe_stream_read": (I, [P, L, P, P]),
     "olmo355_probe_stream_read_many": (I, [P, P, I, P, P]),
     "olmo355_probe_mfma_bf16": (I, [I, P, P, P]),
+    "olmo355_probe_fill_lds": (I, [ctypes.c_uint32, P, P]),
     "olmo355_add": (I, [P, P, P, L, I, P]),
     "olmo355_add_bias_bf16": (I, [P, P, P, I, I, P]),
     "olmo355_argmax": (I, [P, P, I, I, I, P]),

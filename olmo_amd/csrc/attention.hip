@@ -108,16 +108,19 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(const void* __restrict
 // =====================================================================================================
 // prefill on the matrix cores (bf16)
 // =====================================================================================================
-// Workgroup: 4 waves x 32 queries = 128 queries of one (batch, head); KV tile: 64 keys.
-// LDS  K  : [key-tile 4][hd-step HD/32][64 lanes][8 bf16]   A operand of S^T = K . Q^T
-//      V  : [key 64][hd] row-major as it comes from the cache, rows 32 bytes longer than the data so that four
-//           neighbouring keys start 8 banks apart.  The A operand of O^T = V^T . P^T is read with the LDS
-//           transposing load (ds_read_b64_tr_b16): per group of 16 lanes, lane r supplies the address of four
-//           consecutive bf16 and lane j receives element j % 4 of the four rows supplied by lanes j / 4 + 4 e
-//           (e = 0 .. 3).  With lane r pointing at key 4 kq + r / 4, channels 4 (r % 4) .. + 3 of the hd tile, lane j
-//           receives channel j of keys 4 kq .. 4 kq + 3: one load per half of an operand fragment, no shuffling
-//           of V on the way into LDS.
-//      (K: plus pad slots, see the declaration)
+// Workgroup: 4 waves x 32 queries = 128 queries of one (batch, head); KV tile: 64 keys, two tiles in LDS: the
+// tile after the one being multiplied travels memory -> LDS directly while that goes on, one barrier per tile.
+// The LDS side of such a load is lane-linear (64 lanes x 16 bytes = 1 KiB per instruction), so the layouts below
+// are produced on the memory side, by which 16 bytes each lane asks for.
+// LDS  K  : [key-tile 4][hd-step HD/32][64 lanes][8 bf16]   A operand of S^T = K . Q^T, one conflict-free
+//           ds_read_b128 per fragment
+//      V  : [key 64][hd] row-major, rows HD * 2 bytes apart, the 32-byte units of a row XOR-swizzled by the key so
+//           that 8 neighbouring keys' units of one channel block cover all 64 banks.  The A operand of
+//           O^T = V^T . P^T is read with the LDS transposing load (ds_read_b64_tr_b16): per group of 16 lanes,
+//           lane r supplies the address of four consecutive bf16 and lane j receives element j % 4 of the four
+//           rows supplied by lanes j / 4 + 4 e (e = 0 .. 3).  With lane r pointing at key 4 kq + r / 4, channels
+//           4 (r % 4) .. + 3 of the hd tile, lane j receives channel j of keys 4 kq .. 4 kq + 3: one load per
+//           half of an operand fragment, no shuffling of V on the way into LDS.
 // In the second product the 8 key slots of lane group kq in key-step s are
 //   e<4 : key 32s + 4kq + e        e>=4 : key 32s + 16 + 4kq + (e-4)
 // which is exactly how the S^T accumulators of the two 16-key tiles 2s, 2s+1 sit in a lane, so
@@ -129,6 +132,31 @@ __device__ __forceinline__ float reduce_lane_groups(float v, Op op) {
   return combine_xor32(combine_xor16(v, op), op);
 }
 
+// One wave's requests for a K / V tile of the prefill kernel: HD / 32 instructions of 1 KiB per operand, memory ->
+// LDS directly (kdst / vdst: the wave's first KiB of the tile's buffers).  row: key within the tile, in: byte
+// within the key's row, per instruction and lane.  Only the last tile can reach past the last visible key; rows
+// past it may hold anything, so the last visible row is read in their place.
+template <int HD>
+__device__ __forceinline__ void prefill_request_tile(__amdgpu_buffer_rsrc_t rk, __amdgpu_buffer_rsrc_t rv, unsigned char* kdst,
+                                                     unsigned char* vdst, const int (&k_row)[HD / 32], const int (&k_in)[HD / 32],
+                                                     const int (&v_row)[HD / 32], const int (&v_in)[HD / 32], int k0, int last_pos) {
+  const bool tail = k0 + 63 > last_pos;
+#pragma unroll
+  for (int i = 0; i < HD / 32; ++i) {
+    const int kr = tail ? min(k0 + k_row[i], last_pos) - k0 : k_row[i];
+    const int vr = tail ? min(k0 + v_row[i], last_pos) - k0 : v_row[i];
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, (lds_ptr_t)(kdst + (i << 10)), 16, kr * (HD * 2) + k_in[i], k0 * (HD * 2), 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, (lds_ptr_t)(vdst + (i << 10)), 16, vr * (HD * 2) + v_in[i], k0 * (HD * 2), 0, 0);
+  }
+}
+
+template <int HD>
+struct PrefillLds {
+  static constexpr int KT = 64;
+  static constexpr int TILE = KT * HD * 2;            // bytes of one K (or V) tile
+  static constexpr int BYTES = 4 * TILE + 2 * KT * 4;  // K x 2, V x 2, bias x 2
+};
+
 template <int HD>
 __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_t* __restrict__ q,
                                                                 const uint16_t* __restrict__ kc,
@@ -137,14 +165,16 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
                                                                 uint16_t* __restrict__ out, int T, int H, int Hkv,
                                                                 int Lmax, int past_len, int bias_stride) {
   constexpr int KT = 64;             // keys per tile
-  constexpr int STEPS = HD / 32;     // hd steps of the first product
+  constexpr int STEPS = HD / 32;     // hd steps of the first product = 1 KiB load instructions per wave, tile and operand
   constexpr int HT = HD / 16;        // hd tiles of the second product
   constexpr int QT = 2;              // 16-query tiles per wave
-  // 16-byte slots; a pad slot after every 16 (K) / every 128 (V) spreads the staging writes over the banks
-  __shared__ __align__(16) u32x4 lds_k[4 * STEPS * 4 * 17];
-  constexpr int VROW = HD * 2 + 32;  // bytes per key row of V in LDS
-  __shared__ __align__(16) unsigned char lds_v[KT * VROW];
-  __shared__ float lds_bias[KT];
+  constexpr int TILE = PrefillLds<HD>::TILE;
+  constexpr int CPR = HD / 8;        // 16-byte chunks per key row
+  constexpr int VROW = HD * 2;       // bytes per key row of V in LDS
+  extern __shared__ __align__(16) unsigned char smem[];
+  unsigned char* const lds_k = smem;             // [2][TILE]
+  unsigned char* const lds_v = smem + 2 * TILE;  // [2][TILE]
+  float* const lds_bias = reinterpret_cast<float*>(smem + 4 * TILE);  // [2][KT]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15, kq = lane >> 4;
@@ -159,7 +189,6 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
   const int64_t cbase = ((int64_t)b * Hkv + hk) * Lmax * HD;
   const int half = (nqb + 1) / 2, rank = blockIdx.y;
   const int qblock = rank < half ? nqb - 1 - rank : rank - half;
-  {
   const int q0 = qblock * 128 + wave * 32;
 
   // Q^T fragments: lane (query col, hd 32*step + 8*kq ..)
@@ -174,7 +203,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
     for (int s = 0; s < STEPS; ++s) qf[qt][s] = *reinterpret_cast<const bf16x8*>(src + 32 * s + 8 * kq);
   }
   f32x4 o[QT][HT];
-  float m[QT], l[QT];
+  float m[QT], l[QT];  // l: this lane's share of the denominator (its 16 of a tile's 64 keys); added up at the end
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     m[qt] = -INFINITY, l[qt] = 0.f;
@@ -184,68 +213,65 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
 
   const int last_pos = past_len + min(qblock * 128 + 127, T - 1);   // workgroup-uniform loop bound
   const int wave_last = past_len + min(q0 + 31, T - 1);             // last position this wave needs
-  // K / V of a tile travel memory -> registers -> LDS; the registers of tile k0+KT are requested right
-  // after tile k0 has been written to LDS, so the requests are in flight while tile k0 is multiplied.
-  constexpr int CPR = HD / 8;                     // 16-byte chunks per key row
-  constexpr int KPT = KT * CPR / 256;             // K chunks per thread per tile
-  u32x4 rkk[KPT], rvv[KPT];
-  float rbias = 0.f;
-  // range-checked loads: the tile's base as the scalar offset, a lane's place in the tile worked out once
+  // range-checked loads: the tile's base as the scalar offset, a lane's place in the tile worked out once.
+  // Wave w asks for the K fragments of key tile w (one instruction per hd step) and for V rows
+  // w * KT / 4 .. + KT / 4 - 1 (STEPS instructions of 1 KiB).
   const __amdgpu_buffer_rsrc_t rk_ = make_rsrc(kc + cbase, (int64_t)Lmax * HD * 2);
   const __amdgpu_buffer_rsrc_t rv_ = make_rsrc(vc + cbase, (int64_t)Lmax * HD * 2);
-  int kv_off[KPT];
+  auto v_swz = [](int key) { return HD == 128 ? (key & 7) : ((key >> 1) & 3); };  // on the 32-byte units of a row
+  int k_row[STEPS], k_in[STEPS], v_row[STEPS], v_in[STEPS];  // key within the tile, byte within the row
 #pragma unroll
-  for (int i = 0; i < KPT; ++i) {
-    const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
-    kv_off[i] = (kk * HD + 8 * c) * 2;
+  for (int i = 0; i < STEPS; ++i) {
+    k_row[i] = 16 * wave + col;
+    k_in[i] = (4 * i + kq) * 16;
+    const int slot = (wave * STEPS + i) * 64 + lane;  // 16-byte slot of the V tile this lane fills
+    const int row = slot / CPR, pos = slot % CPR;
+    v_row[i] = row;
+    v_in[i] = ((((pos >> 1) ^ v_swz(row)) << 1) | (pos & 1)) * 16;
   }
-  auto fetch = [&](int k0) {
-    const bool tail = k0 + KT - 1 > last_pos;  // only the last tile can reach past the last visible key
-#pragma unroll
-    for (int i = 0; i < KPT; ++i) {
-      int off = kv_off[i], base = k0 * HD * 2;
-      if (tail) {  // rows past the last visible key may hold anything: read the last visible row instead
-        const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
-        off = (min(k0 + kk, last_pos) * HD + 8 * c) * 2, base = 0;
-      }
-      rkk[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rk_, off, base, 0));
-      rvv[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rv_, off, base, 0));
-    }
+  float rbias = 0.f;
+  auto fetch = [&](int k0, int buf) {
+    prefill_request_tile<HD>(rk_, rv_, lds_k + buf * TILE + wave * (STEPS << 10), lds_v + buf * TILE + wave * (STEPS << 10), k_row,
+                             k_in, v_row, v_in, k0, last_pos);
     if (key_bias && tid < KT) rbias = key_bias[(int64_t)b * bias_stride + min(k0 + tid, last_pos)];
   };
-  auto stash = [&]() {
-#pragma unroll
-    for (int i = 0; i < KPT; ++i) {
-      const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
-      lds_k[(((kk >> 4) * STEPS + (c >> 2)) * 4 + (c & 3)) * 17 + (kk & 15)] = rkk[i];
-    }
-#pragma unroll
-    for (int i = 0; i < KPT; ++i) {
-      const int e = tid + i * 256, kk = e / CPR, c = e % CPR;
-      *reinterpret_cast<u32x4*>(lds_v + kk * VROW + c * 16) = rvv[i];
-    }
-    if (tid < KT) lds_bias[tid] = rbias;
+  auto publish = [&](int buf) {  // own requests landed, then everybody's
+    if (tid < KT) lds_bias[buf * KT + tid] = rbias;  // zeros without a key_bias: the diagonal tiles read it either way
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, true));
+    __builtin_amdgcn_s_barrier();
   };
-  const int v_rd = (4 * kq + (col >> 2)) * VROW + 8 * (col & 3);  // this lane's row of the transposing loads
-  fetch(0);
-  for (int k0 = 0; k0 <= last_pos; k0 += KT) {
-    __syncthreads();  // the previous tile has been read
-    stash();
-    if (k0 + KT <= last_pos) fetch(k0 + KT);
-    __syncthreads();
-    if (k0 > wave_last) continue;  // nothing visible to this wave in the tile (barriers stay uniform)
+  // this lane's row of the transposing loads, per hd tile (the swizzle of the lane's keys is the same for every
+  // key step: they differ by multiples of 16)
+  int v_rd[HT];
+#pragma unroll
+  for (int ht = 0; ht < HT; ++ht) v_rd[ht] = (4 * kq + (col >> 2)) * VROW + ((ht ^ v_swz(4 * kq + (col >> 2))) << 5) + 8 * (col & 3);
+  fetch(0, 0);
+  publish(0);
+  int buf = 0;
+  for (int k0 = 0; k0 <= last_pos; k0 += KT, buf ^= 1) {
+    // the other buffer was read during the previous tile, and everybody is past that tile's barrier
+    if (k0 + KT <= last_pos) fetch(k0 + KT, buf ^ 1);
+    if (k0 <= wave_last) {  // else nothing visible to this wave in the tile (barriers stay uniform)
+    const u32x4* kt_ = reinterpret_cast<const u32x4*>(lds_k + buf * TILE);
+    const unsigned char* vt_ = lds_v + buf * TILE;
+    const float* bias_ = lds_bias + buf * KT;
 
     // ---- S^T = K . Q^T -----------------------------------------------------------------------------
+    // all of the tile's K fragments are asked for before the first product, so that only the first waits out the
+    // LDS latency
     f32x4 s[QT][4];
+    u32x4 kf[4 * STEPS];
+#pragma unroll
+    for (int i = 0; i < 4 * STEPS; ++i) kf[i] = kt_[i * 64 + lane];
+    __builtin_amdgcn_sched_barrier(0);  // or the scheduler moves each read down to its use
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
 #pragma unroll
-      for (int qt = 0; qt < QT; ++qt) s[qt][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
       for (int st = 0; st < STEPS; ++st) {
-        const bf16x8 kf = __builtin_bit_cast(bf16x8, lds_k[((kt * STEPS + st) * 4 + kq) * 17 + col]);
 #pragma unroll
-        for (int qt = 0; qt < QT; ++qt) s[qt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qt][st], s[qt][kt], 0, 0, 0);
+        for (int qt = 0; qt < QT; ++qt)
+          s[qt][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf[kt * STEPS + st]), qf[qt][st],
+                                                              st == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : s[qt][kt], 0, 0, 0);
       }
     }
     // ---- online softmax per query column, in the log2 domain -----------------------------------------------
@@ -263,7 +289,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int kk = kt * 16 + 4 * kq + r;
-            const float bias = lds_bias[kk];
+            const float bias = bias_[kk];
             float v = bias <= kMaskThreshold ? lowest : __builtin_fmaf(s[qt][kt][r], c2, bias * 1.4426950408889634f);
             v = k0 + kk > qpos[qt] ? -INFINITY : v;
             s[qt][kt][r] = v;
@@ -276,12 +302,24 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
           for (int r = 0; r < 4; ++r) tmax = fmaxf(tmax, s[qt][kt][r]);
         tmax *= c2;  // c2 > 0: the maximum commutes with the scaling
       }
-      tmax = reduce_lane_groups(tmax, [](float a, float b) { return fmaxf(a, b); });
       // The reference maximum follows the running maximum lazily: it moves only when the tile's maximum is more than
       // kLazyMax (log2 units) above it, so probabilities stay below 2^kLazyMax and the accumulators are rescaled
       // on a few tiles instead of nearly all (the same ratio o / l comes out; finite: key 0 of the first tile is
-      // visible to every query, and -inf + kLazyMax is -inf)
-      const float mn = tmax > m[qt] + kLazyMax ? tmax : m[qt];
+      // visible to every query, and -inf + kLazyMax is -inf).  m is the same in the four lane groups of a query
+      // column, so when no lane's own maximum is that far above it the column's is not either, and the exchange
+      // between the lane groups is skipped with the rescaling.
+      if (__builtin_amdgcn_ballot_w64(tmax > m[qt] + kLazyMax) != 0) {
+        tmax = reduce_lane_groups(tmax, [](float a, float b) { return fmaxf(a, b); });
+        const float mn = tmax > m[qt] + kLazyMax ? tmax : m[qt];
+        const float alpha = __builtin_amdgcn_exp2f(m[qt] - mn);  // 1 where the column's maximum stays
+        l[qt] *= alpha;
+#pragma unroll
+        for (int ht = 0; ht < HT; ++ht)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[qt][ht][r] *= alpha;
+        m[qt] = mn;
+      }
+      const float mn = m[qt];
       float psum = 0.f;
       float p[4][4];
 #pragma unroll
@@ -291,16 +329,6 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
           p[kt][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[qt][kt][r], cs, -mn));
           psum += p[kt][r];
         }
-      psum = reduce_lane_groups(psum, [](float a, float b) { return a + b; });
-      if (__builtin_amdgcn_ballot_w64(mn != m[qt]) != 0) {  // the running maximum moved for some query of the wave
-        const float alpha = __builtin_amdgcn_exp2f(m[qt] - mn);
-        l[qt] *= alpha;
-#pragma unroll
-        for (int ht = 0; ht < HT; ++ht)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) o[qt][ht][r] *= alpha;
-        m[qt] = mn;
-      }
       l[qt] += psum;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
@@ -313,27 +341,38 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
       }
     }
     // ---- O^T += V^T . P^T ----------------------------------------------------------------------------------
+    // all of the tile's V fragments are asked for before the first product (the compiler lets the first of these
+    // loads wait for the outstanding memory -> LDS requests: it cannot tell that they fill the other buffer; written
+    // as assembly with hand-placed waits the loads lose that wait and the kernel runs no faster)
+    bf16x8 vf[HT][2];
 #pragma unroll
     for (int ht = 0; ht < HT; ++ht)
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
         typedef short s16x4 __attribute__((ext_vector_type(4)));
         typedef s16x4 __attribute__((address_space(3))) * tr_ptr;
-        const unsigned char* vp = lds_v + v_rd + (32 * s2) * VROW + 32 * ht;
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        const unsigned char* vp = vt_ + v_rd[ht] + (32 * s2) * VROW;
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr)vp);
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr)(vp + 16 * VROW));
-        typedef short s16x8 __attribute__((ext_vector_type(8)));
-        const bf16x8 vf = __builtin_bit_cast(bf16x8, s16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
-#pragma unroll
-        for (int qt = 0; qt < QT; ++qt) o[qt][ht] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[qt][s2], o[qt][ht], 0, 0, 0);
+        vf[ht][s2] = __builtin_bit_cast(bf16x8, s16x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]});
       }
+    __builtin_amdgcn_sched_barrier(0);  // or the scheduler moves each load down to its use
+#pragma unroll
+    for (int ht = 0; ht < HT; ++ht)
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) o[qt][ht] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[ht][s2], pf[qt][s2], o[qt][ht], 0, 0, 0);
+    }
+    publish(buf ^ 1);  // the next tile is in LDS and this one has been read by everybody
   }
   // ---- write O[q][hd]: lane holds hd = 16ht + 4kq + r for query col ------------------------------------------
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     const int t = q0 + qt * 16 + col;
+    const float inv = 1.f / reduce_lane_groups(l[qt], [](float a, float b) { return a + b; });
     if (t >= T) continue;
-    const float inv = 1.f / l[qt];
     uint16_t* dst = out + ((int64_t)b * T + t) * H * HD + (int64_t)h * HD;
 #pragma unroll
     for (int ht = 0; ht < HT; ++ht) {
@@ -342,7 +381,6 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
       w.y = pack_bf16x2(o[qt][ht][2] * inv, o[qt][ht][3] * inv);
       *reinterpret_cast<u32x2*>(dst + 16 * ht + 4 * kq) = w;
     }
-  }
   }
 }
 
@@ -1031,14 +1069,18 @@ int attn_prefill_main(const void* q, const void* kcache, const void* vcache, con
   if (key_bias && bias_stride < past_len + T) return O355_EINVAL;
   if (dtype == O355_BF16 && (hd == 128 || hd == 64) && (int64_t)Lmax * hd < (1ll << 31)) {  // 32-bit offsets within a head
     const dim3 grid(H, (T + 127) / 128, B);  // heads fastest, then query blocks by rank (see the kernel)
-    if (hd == 128)
-      hipLaunchKernelGGL(attn_prefill_mfma_kernel<128>, grid, dim3(256), 0, s, (const uint16_t*)q,
+    if (hd == 128) {
+      constexpr int lds = PrefillLds<128>::BYTES;  // more than a launch gets without asking
+      auto kern = attn_prefill_mfma_kernel<128>;
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+        return O355_ELAUNCH;
+      hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, (const uint16_t*)q, (const uint16_t*)kcache,
+                         (const uint16_t*)vcache, key_bias, (uint16_t*)out, T, H, Hkv, Lmax, past_len, bias_stride);
+    } else {
+      hipLaunchKernelGGL(attn_prefill_mfma_kernel<64>, grid, dim3(256), PrefillLds<64>::BYTES, s, (const uint16_t*)q,
                          (const uint16_t*)kcache, (const uint16_t*)vcache, key_bias, (uint16_t*)out, T, H, Hkv, Lmax,
                          past_len, bias_stride);
-    else
-      hipLaunchKernelGGL(attn_prefill_mfma_kernel<64>, grid, dim3(256), 0, s, (const uint16_t*)q,
-                         (const uint16_t*)kcache, (const uint16_t*)vcache, key_bias, (uint16_t*)out, T, H, Hkv, Lmax,
-                         past_len, bias_stride);
+    }
     O355_CHECK_LAUNCH();
   }
 #define GENERIC(DTv, HDv) \

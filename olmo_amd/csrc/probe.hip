@@ -108,6 +108,15 @@ __global__ __launch_bounds__(512) void mfma_bf16_kernel(float* __restrict__ sink
   if (s == 12345.678f) sink[threadIdx.x] = s;
 }
 
+// Every workgroup takes all of a CU's LDS and writes `pattern` over it (one workgroup per CU at a time; the grid is
+// several times the CU count so that every CU gets one).
+__global__ __launch_bounds__(256) void lds_fill_kernel(uint32_t pattern, uint32_t* __restrict__ sink, int words) {
+  extern __shared__ __align__(16) uint32_t lds_all[];
+  for (int i = threadIdx.x; i < words; i += 256) lds_all[i] = pattern;
+  __syncthreads();
+  if (lds_all[(threadIdx.x * 97) % words] != pattern) sink[threadIdx.x] = 1u;  // keeps the stores
+}
+
 }  // namespace
 
 extern "C" int olmo355_probe_stream_read(const void* src, int64_t bytes, void* sink, void* stream) {
@@ -152,5 +161,19 @@ extern "C" int olmo355_probe_mfma_bf16(int iters, void* sink, double* flops, voi
   if (iters <= 0 || !sink) return O355_EINVAL;
   hipLaunchKernelGGL(mfma_bf16_kernel, dim3(256), dim3(512), 0, as_stream(stream), (float*)sink, iters, 77u);
   if (flops) *flops = 256.0 * 8.0 * (double)iters * 16.0 * 16384.0;
+  O355_CHECK_LAUNCH();
+}
+
+// Leaves `pattern` in the LDS of every CU (tests run it before a kernel to show that the kernel reads nothing it has
+// not written: LDS keeps what the last workgroup left there).
+extern "C" int olmo355_probe_fill_lds(uint32_t pattern, void* sink, void* stream) {
+  if (!sink) return O355_EINVAL;
+  int dev = 0, cus = 0, lds = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+      hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess || cus <= 0 || lds < 65536)
+    return O355_ELAUNCH;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(lds_fill_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+    return O355_ELAUNCH;
+  hipLaunchKernelGGL(lds_fill_kernel, dim3((unsigned)(8 * cus)), dim3(256), (size_t)lds, as_stream(stream), pattern, (uint32_t*)sink, lds / 4);
   O355_CHECK_LAUNCH();
 }

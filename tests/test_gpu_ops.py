@@ -28,6 +28,17 @@ def _ops():
     return ops
 
 
+def poison_lds(dev):
+    """NaNs into the LDS of every CU: a kernel that reads LDS it has not written then shows it in its output
+    (LDS keeps what the last workgroup left, often zeros, so such a read can pass unnoticed otherwise)."""
+    from olmo_amd import _lib
+
+    sink = torch.zeros(256, dtype=torch.int32, device=dev)
+    assert _lib.lib().olmo355_probe_fill_lds(0x7FC07FC0, sink.data_ptr(), torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    assert int(sink.sum().item()) == 0
+
+
 def say(*a):
     print(*a, flush=True)
 
@@ -631,6 +642,7 @@ def test_attn_prefill(dev, dtype, B, T, past, H, Hkv, hd):
     kc = torch.zeros(B, Hkv, Lmax, hd, dtype=dtype)
     vc = torch.zeros_like(kc)
     kc[:, :, :L], vc[:, :, :L] = k, v
+    poison_lds(dev)
     out = ops.attn_prefill(q.transpose(1, 2).reshape(B, T, H * hd).contiguous().to(dev), kc.to(dev), vc.to(dev), B, T, H,
                            Hkv, hd, past).cpu()
     if dtype == torch.float32:
@@ -649,6 +661,7 @@ def test_attn_prefill(dev, dtype, B, T, past, H, Hkv, hd):
     fb = fb.to(dtype)
     fb = fb.masked_fill(fb == float("-inf"), torch.finfo(dtype).min)
     ref2 = om.attention(q, k, v, fb, dtype).transpose(1, 2).reshape(B, T, H * hd)
+    poison_lds(dev)
     out2 = ops.attn_prefill(q.transpose(1, 2).reshape(B, T, H * hd).contiguous().to(dev), kc.to(dev), vc.to(dev), B, T,
                             H, Hkv, hd, past, key_bias=bias.to(dev)).cpu()
     valid = slice(5, None) if past == 0 else slice(None)  # rows that see at least one real key
@@ -967,6 +980,7 @@ def test_measuring_probes(dev):
     torch.cuda.synchronize()
     assert fl.value == 256 * 8 * 10 * 8 * 32768.0
     assert int(sink.abs().sum().item()) == 0
+    poison_lds(dev)
 
 
 @pytest.mark.parametrize("M,N,K", [(65, 256, 128), (300, 1024, 384), (2048, 2816, 512), (513, 22016, 256)])
