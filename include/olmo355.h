@@ -236,8 +236,9 @@ int olmo355_attn_prefill(const void* q, const void* kcache, const void* vcache, 
  * launch grid; the true count is past_len + 1 (or *past_len_dev + 1 when given).
  * ws: olmo355_attn_decode_workspace_bytes(B,H,hd,n_keys_max) bytes, zeroed when allocated: it begins with
  * two int32 counters per (batch, head) that olmo355_attn_decode_fused uses to let one workgroup of a head
- * merge the partial results (a ticket counter, which every launch leaves at zero, and a launch counter whose
- * value marks the partials of the current launch); the partials follow, (hd + 2) numbers per 128 keys with
+ * merge the partial results (B * H ticket counters, which every launch leaves at zero, then B * H launch counters
+ * whose value marks the partials of the current launch; the regions are apart, so one workspace may serve
+ * launches that merge either way, for the same B and H); the partials follow, (hd + 2) numbers per 128 keys with
  * room for a flag word each. */
 int64_t olmo355_attn_decode_workspace_bytes(int B, int H, int hd, int n_keys_max);
 int olmo355_attn_decode(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out,

@@ -626,7 +626,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   // on one address take 6 us to drain.)
   int my_epoch = 0;
   if (ll && tid == 0)
-    my_epoch = __hip_atomic_load(tickets + 2 * (b * H + h) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    my_epoch = __hip_atomic_load(tickets + (gridDim.z + b) * H + h, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int sub = lane % LPK, kslot = lane / LPK;
   const float scale = 1.f / sqrtf((float)HD);
@@ -925,7 +925,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     }
     out[((int64_t)b * H + h) * HD + tid] = gave_up ? (uint16_t)0x7FC0 : f32_to_bf16_bits(go / gl);
     if (tid == 0)  // the next launch's flag
-      __hip_atomic_store(tickets + 2 * (b * H + h) + 1, (int)(flag & 0x3FFFFFu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(tickets + (gridDim.z + b) * H + h, (int)(flag & 0x3FFFFFu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
   }
   // ---- 4. the last workgroup of a (batch, head) to finish merges the partials itself ---------------------
@@ -1248,7 +1248,8 @@ extern "C" int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, 
   hipLaunchKernelGGL((attn_decode_combine_kernel<O355_BF16, HDv>), dim3(H, B), dim3(HDv), 0, s, (const float*)ws, out, \
                      H, past_len, past_len_dev, nch)
   // the workspace starts with one ticket counter per (batch, head): zero on entry (zeroed at allocation,
-  // reset by the workgroup that draws the last ticket), then the partials
+  // reset by the workgroup that draws the last ticket), then one launch counter per (batch, head) for the flag
+  // form (a region of its own: a workspace may serve both forms in turn), then the partials
   // (measured at the 7B shapes, context 2048: the in-kernel merge wins while the launch is a single round of
   // workgroups -- 17.0 against 20.4 us at batch 1 -- and loses once workgroups queue up -- 69.7 against 61.6 us
   // at batch 8, where one workgroup per (batch, head) takes 66.9)
