@@ -385,7 +385,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
 }
 
 // =====================================================================================================
-// decode: one query per (batch, head); keys split into chunks of 128 (32 per wave)
+// decode: one query per (batch, head); keys split into chunks of 128, 192 or 256 (32, 48 or 64 per wave)
 // =====================================================================================================
 // A lane owns 8 channels of one key: LPK = HD/8 lanes cover a key row with one 16-byte load each,
 // a wave covers 64/LPK keys per load instruction.  All K and V loads of the wave's 32 keys are
@@ -393,8 +393,22 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
 // over the LPK lanes with DPP adds.
 constexpr int kFlagMergeFromChunks = 24;  // chunks per head from which "choose" takes the flag form of the in-kernel merge
 constexpr int kLLSpinLimit = 1 << 21;  // polls of the merging workgroup before it gives up (seconds)
-constexpr int kDecodeChunk = 128;
-constexpr int kDecodeKeysPerWave = 32;
+constexpr int kDecodeMinChunk = 128;  // the smallest chunk: what the workspace is sized for
+
+// Keys per wave of the decode kernels (a workgroup of four waves takes four times as many).  Measured, us per
+// launch at 32 / 48 / 64 keys per wave (hd 128):
+//   32 heads x 2049 keys  16.1 / 14.5 / 16.3   (64 makes 9 chunks, the last with one key, and 288 workgroups leave CUs idle)
+//   16 heads x 2101 keys  13.6 / 11.6 / 11.9     32 heads x 1001 keys  11.7 / 11.0 / 11.5
+//   16 heads x 1001 keys   9.6 /  9.9 / 10.5     32 heads x  301 keys   9.0 / 10.1 / 11.3
+//   40 heads x 4091 keys  34.1 / 29.4 / 29.1     8 x 32 heads x 2049 keys  65.8 / 67.0 / 63.4
+// So: the longest run of keys per workgroup that still leaves the launch with clearly more workgroups than CUs, and
+// short runs for short contexts, where a workgroup's serial walk over its keys is most of the launch.
+inline int decode_keys_per_wave(int B, int H, int n_keys_max) {
+  const int64_t heads = (int64_t)B * H;
+  if (heads * ((n_keys_max + 255) / 256) >= 320) return 64;
+  if (n_keys_max >= 1536) return 48;
+  return 32;
+}
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v) {
@@ -411,7 +425,7 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
-template <int DT, int HD>
+template <int DT, int HD, int KPW>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const void* __restrict__ q, const void* __restrict__ kc,
                                                           const void* __restrict__ vc,
                                                           const float* __restrict__ key_bias, float* __restrict__ ws,
@@ -421,7 +435,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const void* __restrict
                                                           int src_stride, int prompt_len, int beam) {
   constexpr int LPK = HD / 8;                        // lanes per key (8 channels each)
   constexpr int KPI = 64 / LPK;                      // keys per wave iteration
-  constexpr int ITERS = kDecodeKeysPerWave / KPI;    // iterations per wave
+  constexpr int ITERS = KPW / KPI;                   // iterations per wave
+  constexpr int kDecodeChunk = 4 * KPW, kDecodeKeysPerWave = KPW;
   constexpr int VW = DT == O355_BF16 ? 1 : 2;        // 16-byte vectors per 8 channels
   __shared__ float red_o[4][HD];
   __shared__ float red_ml[4][2];
@@ -556,7 +571,7 @@ template <int DT, int HD>
 __global__ __launch_bounds__(HD) void attn_decode_combine_kernel(const float* __restrict__ ws, void* __restrict__ out,
                                                                  int H, int past_len,
                                                                  const int32_t* __restrict__ past_dev,
-                                                                 int nchunks_max) {
+                                                                 int nchunks_max, int chunk_keys) {
   constexpr int UN = 32;  // partials fetched per round, every load before the first use
   const int h = blockIdx.x, b = blockIdx.y;
   const float* src = ws + ((int64_t)b * H + h) * nchunks_max * (HD + 2);
@@ -573,7 +588,7 @@ __global__ __launch_bounds__(HD) void attn_decode_combine_kernel(const float* __
     }
     if (c0 == 0) {
       const int L = (past_dev ? *past_dev : past_len) + 1;
-      nch = min((L + kDecodeChunk - 1) / kDecodeChunk, nchunks_max);
+      nch = min((L + chunk_keys - 1) / chunk_keys, nchunks_max);
     }
     float rm = mm;
 #pragma unroll
@@ -598,7 +613,7 @@ __global__ __launch_bounds__(HD) void attn_decode_combine_kernel(const float* __
 // 2*(H+Hkv)*HD bytes of q and k while its K/V loads are in flight, rotates its own head's q
 // (olmo/model.py:298-324) into LDS, and the workgroup whose chunk holds the new position also forms
 // the new key / value row, appends it to the cache (olmo/model.py:615-620) and uses it from LDS.
-template <int HD, int QV>  // QV: 16-byte pieces of the q (k) row per thread, H*HD/8 <= QV*256
+template <int HD, int QV, int KPW>  // QV: 16-byte pieces of the q (k) row per thread, H*HD/8 <= QV*256; KPW: keys per wave
 __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     const uint16_t* __restrict__ qkv, const uint16_t* __restrict__ qw, const uint16_t* __restrict__ kw,
     const float* __restrict__ sin_t, const float* __restrict__ cos_t, uint16_t* __restrict__ kc,
@@ -606,7 +621,8 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     int n_pos, int past_len, const int32_t* __restrict__ past_dev, int nchunks_max, int bias_stride, float eps,
     const float* __restrict__ qk_ssq, const float* __restrict__ rope_now, uint16_t* __restrict__ out,
     int* __restrict__ tickets, int ll) {
-  constexpr int LPK = HD / 8, KPI = 64 / LPK, ITERS = kDecodeKeysPerWave / KPI;
+  constexpr int LPK = HD / 8, KPI = 64 / LPK, ITERS = KPW / KPI;
+  constexpr int kDecodeChunk = 4 * KPW, kDecodeKeysPerWave = KPW;
   constexpr int HALF = HD / 2, CPH = HD / 16;  // pair chunks per head
   constexpr int ROWS = 4 * KPI;                 // partial results of the workgroup: one per (wave, key slot)
   __shared__ __align__(16) float red_o[ROWS][HD];
@@ -983,11 +999,17 @@ template <int DT, int HD>
 int launch_decode(const void* q, const void* kc, const void* vc, const float* key_bias, void* out, float* ws, int B,
                   int H, int Hkv, int Lmax, int past_len, const int32_t* past_dev, int n_keys_max, int bias_stride,
                   const int32_t* beam_src, int src_stride, int prompt_len, int beam, hipStream_t stream) {
-  const int nch = (n_keys_max + kDecodeChunk - 1) / kDecodeChunk;
-  hipLaunchKernelGGL((attn_decode_kernel<DT, HD>), dim3(nch, H, B), dim3(256), 0, stream, q, kc, vc, key_bias, ws, H,
-                     Hkv, Lmax, past_len, past_dev, nch, bias_stride, beam_src, src_stride, prompt_len, beam);
+  const int kpw = decode_keys_per_wave(B, H, n_keys_max), chunk = 4 * kpw;
+  const int nch = (n_keys_max + chunk - 1) / chunk;
+#define DECODE(KPWv)                                                                                                  \
+  hipLaunchKernelGGL((attn_decode_kernel<DT, HD, KPWv>), dim3(nch, H, B), dim3(256), 0, stream, q, kc, vc, key_bias, \
+                     ws, H, Hkv, Lmax, past_len, past_dev, nch, bias_stride, beam_src, src_stride, prompt_len, beam)
+  if (kpw == 64) DECODE(64);
+  else if (kpw == 48) DECODE(48);
+  else DECODE(32);
+#undef DECODE
   hipLaunchKernelGGL((attn_decode_combine_kernel<DT, HD>), dim3(H, B), dim3(HD), 0, stream, ws, out, H, past_len,
-                     past_dev, nch);
+                     past_dev, nch, chunk);
   O355_CHECK_LAUNCH();
 }
 
@@ -1122,7 +1144,7 @@ extern "C" int olmo355_rope_advance(int32_t* pos, int delta, const float* sin_ta
 
 extern "C" int64_t olmo355_attn_decode_workspace_bytes(int B, int H, int hd, int n_keys_max) {
   if (B <= 0 || H <= 0 || hd <= 0 || n_keys_max <= 0) return 0;
-  const int64_t nch = (n_keys_max + kDecodeChunk - 1) / kDecodeChunk;
+  const int64_t nch = (n_keys_max + kDecodeMinChunk - 1) / kDecodeMinChunk;  // longer chunks need less
   // two counters per (batch, head), then the partials: (hd + 2) numbers per chunk, each with room for a flag word
   return (int64_t)B * H * 8 + (int64_t)B * H * nch * (hd + 2) * 8;
 }
@@ -1238,15 +1260,18 @@ extern "C" int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, 
   if (key_bias && bias_stride < n_keys_max) return O355_EINVAL;
   if (dtype != O355_BF16 || (hd != 128 && hd != 64) || H * hd > 8 * 4 * 256) return O355_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
-  const int nch = (n_keys_max + kDecodeChunk - 1) / kDecodeChunk;
+  const int kpw = decode_keys_per_wave(B, H, n_keys_max), chunk_keys = 4 * kpw;
+  const int nch = (n_keys_max + chunk_keys - 1) / chunk_keys;
 #define FUSED(HDv, QVv)                                                                                                 \
-  hipLaunchKernelGGL((attn_decode_fused_kernel<HDv, QVv>), dim3(nch, H, B), dim3(256), 0, s, (const uint16_t*)qkv,   \
-                     (const uint16_t*)qw, (const uint16_t*)kw, sin_tab, cos_tab, (uint16_t*)kcache, (uint16_t*)vcache, \
-                     key_bias, (float*)ws, H, Hkv, Lmax, n_pos, past_len, past_len_dev, nch, bias_stride, eps, qk_ssq, \
-                     rope_now, (uint16_t*)out, tickets, ll);                                                                     \
+  if (kpw == 64) { FUSED_KPW(HDv, QVv, 64); } else if (kpw == 48) { FUSED_KPW(HDv, QVv, 48); } else { FUSED_KPW(HDv, QVv, 32); } \
   if (!tickets)                                                                                                        \
   hipLaunchKernelGGL((attn_decode_combine_kernel<O355_BF16, HDv>), dim3(H, B), dim3(HDv), 0, s, (const float*)ws, out, \
-                     H, past_len, past_len_dev, nch)
+                     H, past_len, past_len_dev, nch, chunk_keys)
+#define FUSED_KPW(HDv, QVv, KPWv)                                                                                       \
+  hipLaunchKernelGGL((attn_decode_fused_kernel<HDv, QVv, KPWv>), dim3(nch, H, B), dim3(256), 0, s, (const uint16_t*)qkv,   \
+                     (const uint16_t*)qw, (const uint16_t*)kw, sin_tab, cos_tab, (uint16_t*)kcache, (uint16_t*)vcache, \
+                     key_bias, (float*)ws, H, Hkv, Lmax, n_pos, past_len, past_len_dev, nch, bias_stride, eps, qk_ssq, \
+                     rope_now, (uint16_t*)out, tickets, ll)
   // the workspace starts with one ticket counter per (batch, head): zero on entry (zeroed at allocation,
   // reset by the workgroup that draws the last ticket), then one launch counter per (batch, head) for the flag
   // form (a region of its own: a workspace may serve both forms in turn), then the partials
@@ -1266,6 +1291,7 @@ extern "C" int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, 
     if (qv <= 1) { FUSED(64, 1); } else if (qv <= 2) { FUSED(64, 2); } else { FUSED(64, 4); }
   }
 #undef FUSED
+#undef FUSED_KPW
   O355_CHECK_LAUNCH();
 }
 
