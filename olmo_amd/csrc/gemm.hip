@@ -775,11 +775,13 @@ extern "C" int64_t olmo355_gemm_streamk_workspace_bytes(void) { return kStreamKF
 // 1 when the stream-K form is expected to beat the tiled launch.  Measured on the 7B shapes at 2048 rows: where the
 // 256 x 256 tiles make a whole number of rounds the two are level; with 1.5 or 2.7 tiles per CU stream-K gains
 // 4-15 %; with fewer tiles than CUs every tile is shared and the hand-over (about 15 us of partials written, read
-// and waited for) must be earned by the better rate of the large tile: yes at K = 11008, no at K = 4096.
+// and waited for) must be earned by the better rate of the large tile: yes at K = 11008, no at K = 4096.  With a
+// quarter to a half of the CUs' worth of tiles only a long K pays (1024 rows: N = 4096, K = 11008 94 against 111 us
+// for the best tiled launch; N = K = 4096 51 against 44).
 extern "C" int olmo355_gemm_streamk_plan(int M, int N, int K) {
   if (M <= 0 || N <= 0 || K <= 0 || (K & 255) || (N & 15)) return 0;
   const int64_t tiles = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
-  if (tiles < 128) return 0;
+  if (tiles < 128) return tiles >= 64 && K >= 8192 ? 1 : 0;
   if (tiles < 256) return 2.0 * M * N * K >= 150e9 ? 1 : 0;
   const int64_t rounds = (tiles + 255) / 256;
   return tiles * 100 < rounds * 256 * 92 ? 1 : 0;  // the last round less than 92 % full

@@ -293,7 +293,7 @@ def _streamk_ws(dev):
 
 
 @pytest.mark.parametrize("M,N,K", [(1024, 4096, 1024), (1000, 4080, 1280), (2048, 8192, 512), (700, 6160, 2048),
-                                   (2048, 12288, 1024)])
+                                   (2048, 12288, 1024), (1024, 4096, 8448)])
 def test_w4_gemm_streamk(dev, M, N, K):
     """The stream-K form against the oracle on shapes where a tile's K is shared by four workgroups (one unit of 256
     per CU), by two with uneven pieces, by none (256 tiles of two units: one whole tile per CU), with ragged M and N,
