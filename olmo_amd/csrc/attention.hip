@@ -388,7 +388,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
 // decode: one query per (batch, head); keys split into chunks of 128, 192 or 256 (32, 48 or 64 per wave)
 // =====================================================================================================
 // A lane owns 8 channels of one key: LPK = HD/8 lanes cover a key row with one 16-byte load each,
-// a wave covers 64/LPK keys per load instruction.  All K and V loads of the wave's 32 keys are
+// a wave covers 64/LPK keys per load instruction.  All K and V loads of the wave's keys are
 // issued before the first use (the kernel is latency-bound at batch 1); the dot product is reduced
 // over the LPK lanes with DPP adds.
 constexpr int kFlagMergeFromChunks = 24;  // chunks per head from which "choose" takes the flag form of the in-kernel merge
@@ -1279,8 +1279,9 @@ extern "C" int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, 
   // workgroups -- 17.0 against 20.4 us at batch 1 -- and loses once workgroups queue up -- 69.7 against 61.6 us
   // at batch 8, where one workgroup per (batch, head) takes 66.9)
   const bool merge_in_kernel = merge == 0 || merge == 1 || (merge < 0 && (int64_t)B * H * nch <= 1536);
-  // (measured, batch 1: the flag form is level with the ticket form at 17 chunks per head -- 17.2 against 16.4 us,
-  // 7B at context 2048 -- and ahead from about two dozen -- 34.4 against 36.5 us, 13B at context 4090)
+  // (measured with 128-key chunks, batch 1: the flag form is level with the ticket form at 17 chunks per head -- 17.2
+  // against 16.4 us, 7B at context 2048 -- and ahead from about two dozen -- 34.4 against 36.5 us, 13B at context 4090;
+  // with that launch's 256-key chunks, 17 per head, the two forms are level again at 29.6 us)
   const int ll = merge_in_kernel && (merge == 1 || (merge < 0 && nch >= kFlagMergeFromChunks)) ? 1 : 0;  // needs the counters
   int* tickets = merge_in_kernel ? reinterpret_cast<int*>(ws) : nullptr;
   ws = reinterpret_cast<float*>(ws) + (int64_t)2 * B * H;
