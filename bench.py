@@ -251,6 +251,53 @@ def main() -> int:
     log(f"[bench] yardstick: vendor library, dense bf16 GEMMs of the same shapes (M={ctx}): {tf_lib:.0f} TFLOP/s = "
         f"{tf_lib / MFMA_BF16_PEAK_TF:.1%} of bf16 MFMA peak")
     # ---- what this box gives a kernel that only streams the same weights / only issues MFMAs ----------
+    # ---- the two attention kernels on their own: decode (HBM-bound) and prefill (matrix cores) -----------------
+    H, hd = cfg.n_heads, cfg.head_dim
+    n_lay = 16  # distinct caches, so that no launch finds its keys in a cache
+    qkv1 = torch.randn(1, 3 * H * hd, device=dev).to(torch.bfloat16)
+    ones = torch.ones(H * hd, device=dev).to(torch.bfloat16)
+    sin_t, cos_t = ops.rope_tables(hd, float(cfg.rope_theta), cap, dev)
+    kvs = [(torch.randn(1, H, cap, hd, device=dev).to(torch.bfloat16), torch.randn(1, H, cap, hd, device=dev).to(torch.bfloat16))
+           for _ in range(n_lay)]
+    aws = ops.attn_decode_workspace(1, H, hd, cap, dev)
+    pos_dev = torch.tensor([ctx], dtype=torch.int32, device=dev)
+    ssq1 = torch.rand(1, 3 * H * hd // 16, device=dev) * 16
+    rope_now = torch.cat([sin_t[ctx], cos_t[ctx]]).contiguous()
+
+    def decode_attention_launches():
+        for kc_, vc_ in kvs:
+            ops.attn_decode_fused(qkv1, ones, ones, sin_t, cos_t, kc_, vc_, aws, 1, H, H, hd, 0, cap, cfg.layer_norm_eps,
+                                  past_len_dev=pos_dev, qk_ssq=ssq1, rope_now=rope_now)
+
+    att_s = timed_graph(decode_attention_launches, reps) / n_lay
+    att_bytes = 2.0 * (ctx + 1) * hd * 2 * H + 3 * H * hd * 2  # keys and values of every head, the token's q | k | v
+    extra["decode_attention"] = {"bound": "hbm", "achieved": att_bytes / att_s / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                 "frac": att_bytes / att_s / 1e9 / HBM_PEAK_GBS, "avg_launch_us": att_s * 1e6,
+                                 "what": f"attn_decode_fused_kernel (QK-norm, rotary, cache append, attention, merge), batch 1, "
+                                         f"{ctx + 1} keys, {H} heads, one captured graph of {n_lay} launches over distinct caches"}
+    log(f"[bench] decode attention (batch 1, {ctx + 1} keys): {att_s * 1e6:.2f} us/launch, {att_bytes / att_s / 1e9:.0f} GB/s = "
+        f"{att_bytes / att_s / 1e9 / HBM_PEAK_GBS:.1%} of HBM peak")
+    del kvs
+    qp = torch.randn(1, ctx, H * hd, device=dev).to(torch.bfloat16)
+    kp = torch.randn(1, H, ctx + 16, hd, device=dev).to(torch.bfloat16)
+    vp = torch.randn(1, H, ctx + 16, hd, device=dev).to(torch.bfloat16)
+    ops.attn_prefill(qp, kp, vp, 1, ctx, H, H, hd, 0)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(5):
+        ops.attn_prefill(qp, kp, vp, 1, ctx, H, H, hd, 0)
+    e1.record()
+    torch.cuda.synchronize()
+    pf_s = e0.elapsed_time(e1) * 1e-3 / 5
+    pf_flops = 4.0 * H * hd * ctx * (ctx + 1) / 2
+    extra["prefill_attention"] = {"bound": "mfma", "achieved": pf_flops / pf_s / 1e12, "peak": MFMA_BF16_PEAK_TF, "unit": "TFLOP/s",
+                                  "frac": pf_flops / pf_s / 1e12 / MFMA_BF16_PEAK_TF, "avg_launch_us": pf_s * 1e6,
+                                  "what": f"attn_prefill_mfma_kernel, 1 x {ctx} tokens, {H} heads of {hd}, causal: 4 T (T + 1) hd / 2 "
+                                          "flop per head"}
+    log(f"[bench] prefill attention (1 x {ctx}): {pf_s * 1e6:.1f} us, {pf_flops / pf_s / 1e12:.0f} TFLOP/s = "
+        f"{pf_flops / pf_s / 1e12 / MFMA_BF16_PEAK_TF:.1%} of bf16 MFMA peak")
+    del qp, kp, vp
+
     # Same launches as above (one per block Linear, distinct buffers, one captured graph), but the kernel reads
     # the tiled weight bytes and does nothing else: the distance from here to the published 8 TB/s is not the
     # linear kernel's to close.  The matrix-core probe runs v_mfma_f32_16x16x32_bf16 (the GEMM's instruction) on
