@@ -626,6 +626,16 @@ def test_qknorm_rope_kvwrite(dev, dtype, qknorm, H, Hkv, hd):
     (torch.bfloat16, 1, 300, 0, 4, 4, 128),
     (torch.bfloat16, 2, 130, 70, 4, 2, 128),
     (torch.bfloat16, 1, 257, 0, 2, 2, 64),
+    # one query; a tile short of / exactly / just over one key tile and one query block; a long past; many tiles
+    (torch.bfloat16, 1, 1, 0, 2, 2, 128),
+    (torch.bfloat16, 1, 63, 0, 2, 2, 128),
+    (torch.bfloat16, 2, 64, 0, 2, 1, 64),
+    (torch.bfloat16, 2, 65, 5, 4, 4, 64),
+    (torch.bfloat16, 1, 128, 0, 2, 2, 128),
+    (torch.bfloat16, 1, 129, 127, 2, 1, 128),
+    (torch.bfloat16, 1, 7, 1000, 2, 2, 128),
+    (torch.bfloat16, 1, 1000, 24, 2, 2, 128),
+    (torch.bfloat16, 1, 1000, 24, 2, 2, 64),
     (torch.float32, 2, 100, 0, 8, 8, 32),
     (torch.float32, 1, 70, 30, 2, 2, 32),
 ])
