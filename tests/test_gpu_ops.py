@@ -681,8 +681,10 @@ def test_attn_prefill(dev, dtype, B, T, past, H, Hkv, hd):
 
 
 @pytest.mark.parametrize("dtype,B,L,H,Hkv,hd", [
-    (torch.bfloat16, 1, 2048, 32, 32, 128),
-    (torch.bfloat16, 3, 700, 4, 2, 128),
+    (torch.bfloat16, 1, 2048, 32, 32, 128),   # 48 keys per wave
+    (torch.bfloat16, 3, 700, 4, 2, 128),      # 32 keys per wave
+    (torch.bfloat16, 8, 1300, 32, 32, 128),   # 64 keys per wave (many heads x sequences)
+    (torch.float32, 16, 1100, 8, 8, 32),      # the same in fp32
     (torch.bfloat16, 2, 1, 2, 2, 64),
     (torch.bfloat16, 2, 257, 2, 2, 64),
     (torch.float32, 2, 513, 8, 8, 32),
