@@ -1,9 +1,10 @@
 // Causal attention over the contiguous per-layer KV cache [B, Hkv, Lmax, hd]
 // (olmo/model.py:533-586,627-648): softmax(q k^T / sqrt(hd) + bias) v, fp32 softmax.
 //
-//  * attn_prefill_mfma_kernel  bf16, hd 64/128: flash-style, K and V^T tiles staged in LDS in
-//    MFMA-fragment order, S^T = K.Q^T and O^T = V^T.P^T on the matrix cores so the softmax
-//    statistics of a query stay in one lane column and P never leaves registers.
+//  * attn_prefill_mfma_kernel  bf16, hd 64/128: flash-style, K tiles in LDS in MFMA-fragment order and V
+//    tiles row-major (read with transposing loads), both loaded memory -> LDS directly a tile ahead;
+//    S^T = K.Q^T and O^T = V^T.P^T on the matrix cores so the softmax statistics of a query stay in
+//    one lane column and P never leaves registers.
 //  * attn_decode_kernel        one query per sequence, keys split over workgroups and waves,
 //    DPP / wave reductions, partial (max, sum, o) merged by attn_decode_combine_kernel.
 //  * attn_generic_kernel       any dtype / head size <= 128, one query per thread (used for the
@@ -136,6 +137,9 @@ __device__ __forceinline__ float reduce_lane_groups(float v, Op op) {
 // LDS directly (kdst / vdst: the wave's first KiB of the tile's buffers).  row: key within the tile, in: byte
 // within the key's row, per instruction and lane.  Only the last tile can reach past the last visible key; rows
 // past it may hold anything, so the last visible row is read in their place.
+// (A function and not a lambda of the kernel: with the memory -> LDS builtin inside a lambda that the kernel calls,
+// this toolchain's host pass emits no launch stub for the kernel, without a diagnostic, and the library then fails
+// to load with an undefined symbol.)
 template <int HD>
 __device__ __forceinline__ void prefill_request_tile(__amdgpu_buffer_rsrc_t rk, __amdgpu_buffer_rsrc_t rv, unsigned char* kdst,
                                                      unsigned char* vdst, const int (&k_row)[HD / 32], const int (&k_in)[HD / 32],
