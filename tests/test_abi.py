@@ -58,6 +58,24 @@ def test_argument_checks_return_status_without_launching():
     assert h.olmo355_attn_decode_workspace_bytes(1, 32, 128, 2048) == 32 * 16 * 130 * 8 + 32 * 8
 
 
+def test_gemm_plans_are_host_arithmetic():
+    """Which form a large-M product takes is decided on the host from the shape alone; the decisions that the 7B
+    prefill rests on (measured: see the comments at the plan functions), kept from drifting."""
+    from olmo_amd import _lib
+
+    h = _lib.lib()
+    sk, sp = h.olmo355_gemm_streamk_plan, h.olmo355_gemm_splitk_plan
+    # one prompt of 2048 tokens: 384, 688 and 128 tiles of 256 x 256 -- stream-K where the rounds are uneven or K is long
+    assert sk(2048, 12288, 4096) == 1 and sk(2048, 22016, 4096) == 1 and sk(2048, 4096, 11008) == 1
+    assert sk(2048, 4096, 4096) == 0       # every tile would be shared and K is short: the tiled launch
+    assert sk(8192, 4096, 4096) == 0       # 512 tiles: two full rounds
+    assert sk(1024, 4096, 11008) == 1 and sk(1024, 4096, 4096) == 0   # 64 tiles: only a long K pays
+    assert sk(512, 4096, 11008) == 0       # 32 tiles: split-K's range
+    assert sk(2048, 4096, 4000) == 0       # K must divide into units of 256
+    assert sp(512, 4096, 11008) == 2 and sp(300, 4096, 4096) == 2 and sp(2048, 4096, 4096) == 1
+    assert sk(0, 4096, 4096) == 0 and sp(0, 4096, 4096) == 1
+
+
 def test_ops_refuse_cpu_tensors():
     import torch
 
