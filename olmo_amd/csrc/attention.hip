@@ -617,14 +617,20 @@ __global__ __launch_bounds__(HD) void attn_decode_combine_kernel(const float* __
 // 2*(H+Hkv)*HD bytes of q and k while its K/V loads are in flight, rotates its own head's q
 // (olmo/model.py:298-324) into LDS, and the workgroup whose chunk holds the new position also forms
 // the new key / value row, appends it to the cache (olmo/model.py:615-620) and uses it from LDS.
-template <int HD, int QV, int KPW>  // QV: 16-byte pieces of the q (k) row per thread, H*HD/8 <= QV*256; KPW: keys per wave
+//
+// RELAY: the launch is one leg of the two-stream decode relay (relay.hip).  qkv then holds tagged words (bf16 bits
+// << 16 | epoch & 0xffff), qk_ssq pairs (float bits, epoch) and `out` receives tagged words; the cache rows -- which
+// depend on no other launch of the step -- are requested first, and the few threads that read the token's q | k | v
+// pieces and the sums of squares ask for them until every tag shows this step's epoch (at most spin_limit times).
+template <int HD, int QV, int KPW, bool RELAY = false>  // QV: 16-byte pieces of the q (k) row per thread, H*HD/8 <= QV*256; KPW: keys per wave
 __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     const uint16_t* __restrict__ qkv, const uint16_t* __restrict__ qw, const uint16_t* __restrict__ kw,
     const float* __restrict__ sin_t, const float* __restrict__ cos_t, uint16_t* __restrict__ kc,
     uint16_t* __restrict__ vc, const float* __restrict__ key_bias, float* __restrict__ ws, int H, int Hkv, int Lmax,
     int n_pos, int past_len, const int32_t* __restrict__ past_dev, int nchunks_max, int bias_stride, float eps,
     const float* __restrict__ qk_ssq, const float* __restrict__ rope_now, uint16_t* __restrict__ out,
-    int* __restrict__ tickets, int ll) {
+    int* __restrict__ tickets, int ll, const int32_t* __restrict__ epoch_p = nullptr, int32_t* __restrict__ status = nullptr,
+    int spin_limit = 0) {
   constexpr int LPK = HD / 8, KPI = 64 / LPK, ITERS = KPW / KPI;
   constexpr int kDecodeChunk = 4 * KPW, kDecodeKeysPerWave = KPW;
   constexpr int HALF = HD / 2, CPH = HD / 16;  // pair chunks per head
@@ -678,9 +684,11 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   u32x4 x1, x2, w1, w2, vrow;
   f32x4 cs1[2], cs2[2], sn1[2], sn2[2];
   if (role_q || role_k) {
-    const uint16_t* src = role_q ? row + h * HD : row + dq + hk * HD;
-    x1 = reinterpret_cast<const u32x4*>(src + j)[0];
-    x2 = reinterpret_cast<const u32x4*>(src + j + HALF)[0];
+    if constexpr (!RELAY) {
+      const uint16_t* src = role_q ? row + h * HD : row + dq + hk * HD;
+      x1 = reinterpret_cast<const u32x4*>(src + j)[0];
+      x2 = reinterpret_cast<const u32x4*>(src + j + HALF)[0];
+    }
     if (norm) {
       const uint16_t* wsrc = role_q ? qw + h * HD : kw + hk * HD;
       w1 = reinterpret_cast<const u32x4*>(wsrc + j)[0];
@@ -694,10 +702,12 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
       sn1[v4] = reinterpret_cast<const f32x4*>(sp + j)[v4], sn2[v4] = reinterpret_cast<const f32x4*>(sp + j + HALF)[v4];
     }
   }
-  if (role_v) vrow = reinterpret_cast<const u32x4*>(row + dq + dk + hk * HD)[tid - 64];
+  if constexpr (!RELAY) {
+    if (role_v) vrow = reinterpret_cast<const u32x4*>(row + dq + dk + hk * HD)[tid - 64];
+  }
   float sq = 0.f, sk = 0.f;
   u32x4 qrow[QV], krow[QV];
-  if (norm) {
+  if (norm && !RELAY) {
     if (qk_ssq) {  // per-tile partials left by the projection: wave 0 alone adds them up
       if (wave == 0) {
         const float* pr = qk_ssq + (int64_t)b * ((dq + 2 * dk) >> 4);
@@ -730,6 +740,74 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     bias[it] = key_bias ? key_bias[(int64_t)b * bias_stride + min(min(kbase + it * KPI + kslot, kmax), bias_stride - 1)] : 0.f;  // keys past the row's end are past L
   }
 
+  uint32_t tag16 = 0;
+  if constexpr (RELAY) {
+    // ---- 1'. the token's pieces and the sums of squares, asked for until they carry this step's epoch.  Waves 0 and
+    // 1 hold every role; wave 0 also adds up the per-tile sums of squares (two pairs per lane and request).
+    const uint32_t epoch = (uint32_t)*epoch_p;
+    tag16 = epoch & 0xffffu;
+    // workgroups whose chunk lies past the current length (a captured launch covers the cache's capacity) leave below
+    // without having waited for anything
+    const bool has_work = chunk * kDecodeChunk < pos + 1 || (ll && chunk == nchunks_max - 1);
+    if (wave < 2 && has_work) {
+      const int width = dq + 2 * dk;
+      const __amdgpu_buffer_rsrc_t rt = make_rsrc(reinterpret_cast<const uint32_t*>(qkv) + (int64_t)b * width, (int64_t)width * 4);
+      const __amdgpu_buffer_rsrc_t rs2 = make_rsrc(reinterpret_cast<const uint64_t*>(qk_ssq) + (int64_t)b * (width >> 4), (int64_t)(width >> 4) * 8);
+      const int first = role_q ? h * HD + j : (role_k ? dq + hk * HD + j : dq + dk + hk * HD + (tid - 64) * 8);  // element
+      const bool role = role_q || role_k || role_v;
+      const int nq_p = dq >> 4, nk_p = dk >> 4;  // pairs of the q and the k part
+      u32x4 t[4], pq[3], pk[3];
+      bool gave_up = false;
+      for (int spins = 0;; ++spins) {
+        bool ok = true;
+        if (role) {
+          t[0] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rt, first * 4, 0, 16));
+          t[1] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rt, first * 4 + 16, 0, 16));
+          if (!role_v) {
+            t[2] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rt, (first + HALF) * 4, 0, 16));
+            t[3] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rt, (first + HALF) * 4 + 16, 0, 16));
+          }
+        }
+        if (wave == 0 && norm) {
+#pragma unroll
+          for (int r = 0; r < 3; ++r) {
+            if (r * 128 < nq_p) pq[r] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs2, lane * 16, r * 1024, 16));
+            if (r * 128 < nk_p) pk[r] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs2, lane * 16, nq_p * 8 + r * 1024, 16));
+          }
+#pragma unroll
+          for (int r = 0; r < 3; ++r) {
+            if (r * 128 + lane * 2 < nq_p) ok = ok && pq[r].y == epoch && pq[r].w == epoch;
+            if (r * 128 + lane * 2 < nk_p) ok = ok && pk[r].y == epoch && pk[r].w == epoch;
+          }
+        }
+        if (role) {
+          auto tok = [&](const u32x4& v) { return (((v.x ^ tag16) | (v.y ^ tag16) | (v.z ^ tag16) | (v.w ^ tag16)) & 0xffffu) == 0u; };
+          ok = ok && tok(t[0]) && tok(t[1]);
+          if (!role_v) ok = ok && tok(t[2]) && tok(t[3]);
+        }
+        if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
+        if (spins >= spin_limit) {
+          gave_up = true;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(4);
+      }
+      if (gave_up && lane == 0) __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      auto pack8 = [](const u32x4& a, const u32x4& c) {  // eight tagged words -> eight bf16
+        return u32x4{(a.x >> 16) | (a.y & 0xffff0000u), (a.z >> 16) | (a.w & 0xffff0000u), (c.x >> 16) | (c.y & 0xffff0000u),
+                     (c.z >> 16) | (c.w & 0xffff0000u)};
+      };
+      if (role_q || role_k) x1 = pack8(t[0], t[1]), x2 = pack8(t[2], t[3]);
+      if (role_v) vrow = pack8(t[0], t[1]);
+      if (wave == 0 && norm) {
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+          if (r * 128 + lane * 2 < nq_p) sq += __uint_as_float(pq[r].x) + __uint_as_float(pq[r].z);
+          if (r * 128 + lane * 2 < nk_p) sk += __uint_as_float(pk[r].x) + __uint_as_float(pk[r].z);
+        }
+      }
+    }
+  }
   // ---- 2. QK-norm scale factors, rotary, the new cache row --------------------------------------------------
   float rq = 1.f, rk_ = 1.f;
   u32x4 pk1, pk2;
@@ -943,7 +1021,13 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
       }
       gm = rm;
     }
-    out[((int64_t)b * H + h) * HD + tid] = gave_up ? (uint16_t)0x7FC0 : f32_to_bf16_bits(go / gl);
+    {
+      const uint16_t bits = gave_up ? (uint16_t)0x7FC0 : f32_to_bf16_bits(go / gl);
+      if constexpr (RELAY)
+        __hip_atomic_store(reinterpret_cast<uint32_t*>(out) + ((int64_t)b * H + h) * HD + tid, ((uint32_t)bits << 16) | tag16,
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else out[((int64_t)b * H + h) * HD + tid] = bits;
+    }
     if (tid == 0)  // the next launch's flag
       __hip_atomic_store(tickets + (gridDim.z + b) * H + h, (int)(flag & 0x3FFFFFu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
@@ -996,7 +1080,10 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
       }
     gm = rm;
   }
-  out[((int64_t)b * H + h) * HD + tid] = f32_to_bf16_bits(go / gl);
+  if constexpr (RELAY)
+    __hip_atomic_store(reinterpret_cast<uint32_t*>(out) + ((int64_t)b * H + h) * HD + tid,
+                       ((uint32_t)f32_to_bf16_bits(go / gl) << 16) | tag16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else out[((int64_t)b * H + h) * HD + tid] = f32_to_bf16_bits(go / gl);
 }
 
 template <int DT, int HD>
@@ -1249,12 +1336,31 @@ extern "C" int olmo355_attn_decode_static(const void* q, const void* kcache, con
 // merge: how the key chunks of a (batch, head) are merged: -1 = choose, 0 = in the kernel by the workgroup that
 // finishes last (a ticket drawn after its stores have landed), 1 = in the kernel by the workgroup of the head's last
 // chunk, which polls flags stored with the numbers, 2 = the separate combine kernel
-extern "C" int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
-                                               const float* cos_tab, void* kcache, void* vcache, const float* key_bias,
-                                               void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
-                                               int past_len, const int32_t* past_len_dev, int n_keys_max,
-                                               int bias_stride, float eps, const float* qk_ssq, const float* rope_now,
-                                               int dtype, int merge, void* stream) {
+namespace {
+struct FusedPlan {
+  int kpw, nch, ll;
+  bool merge_in_kernel;
+};
+FusedPlan fused_plan(int B, int H, int n_keys_max, int merge) {
+  FusedPlan p;
+  p.kpw = decode_keys_per_wave(B, H, n_keys_max);
+  p.nch = (n_keys_max + 4 * p.kpw - 1) / (4 * p.kpw);
+  // (measured at the 7B shapes, context 2048: the in-kernel merge wins while the launch is a single round of
+  // workgroups -- 17.0 against 20.4 us at batch 1 -- and loses once workgroups queue up -- 69.7 against 61.6 us
+  // at batch 8, where one workgroup per (batch, head) takes 66.9)
+  p.merge_in_kernel = merge == 0 || merge == 1 || (merge < 0 && (int64_t)B * H * p.nch <= 1536);
+  // (measured with 128-key chunks, batch 1: the flag form is level with the ticket form at 17 chunks per head -- 17.2
+  // against 16.4 us, 7B at context 2048 -- and ahead from about two dozen -- 34.4 against 36.5 us, 13B at context 4090;
+  // with that launch's 256-key chunks, 17 per head, the two forms are level again at 29.6 us)
+  p.ll = p.merge_in_kernel && (merge == 1 || (merge < 0 && p.nch >= kFlagMergeFromChunks)) ? 1 : 0;  // needs the counters
+  return p;
+}
+
+int attn_fused_any(const void* qkv, const void* qw, const void* kw, const float* sin_tab, const float* cos_tab, void* kcache,
+                   void* vcache, const float* key_bias, void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
+                   int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps, const void* qk_ssq,
+                   const float* rope_now, int dtype, int merge, bool relay, const int32_t* epoch, int32_t* status, int spin_limit,
+                   void* stream) {
   if (merge < -1 || merge > 2) return O355_EINVAL;
   if (!qkv || !sin_tab || !cos_tab || !kcache || !vcache || !out || !ws) return O355_EINVAL;
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || past_len < 0 || n_keys_max <= 0 || n_keys_max > Lmax)
@@ -1264,40 +1370,52 @@ extern "C" int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, 
   if (key_bias && bias_stride < n_keys_max) return O355_EINVAL;
   if (dtype != O355_BF16 || (hd != 128 && hd != 64) || H * hd > 8 * 4 * 256) return O355_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
-  const int kpw = decode_keys_per_wave(B, H, n_keys_max), chunk_keys = 4 * kpw;
-  const int nch = (n_keys_max + chunk_keys - 1) / chunk_keys;
+  const FusedPlan plan = fused_plan(B, H, n_keys_max, merge);
+  const int kpw = plan.kpw, chunk_keys = 4 * kpw, nch = plan.nch, ll = plan.ll;
+  if (relay) {
+    if (!epoch || !status || spin_limit < 0 || (qw && !qk_ssq)) return O355_EINVAL;
+    if (!plan.merge_in_kernel || H * hd > 6144 || Hkv * hd > 6144) return O355_EUNSUPPORTED;
+  }
 #define FUSED(HDv, QVv)                                                                                                 \
-  if (kpw == 64) { FUSED_KPW(HDv, QVv, 64); } else if (kpw == 48) { FUSED_KPW(HDv, QVv, 48); } else { FUSED_KPW(HDv, QVv, 32); } \
+  if (kpw == 64) { FUSED_KPW(HDv, QVv, 64, false); } else if (kpw == 48) { FUSED_KPW(HDv, QVv, 48, false); } else { FUSED_KPW(HDv, QVv, 32, false); } \
   if (!tickets)                                                                                                        \
   hipLaunchKernelGGL((attn_decode_combine_kernel<O355_BF16, HDv>), dim3(H, B), dim3(HDv), 0, s, (const float*)ws, out, \
                      H, past_len, past_len_dev, nch, chunk_keys)
-#define FUSED_KPW(HDv, QVv, KPWv)                                                                                       \
-  hipLaunchKernelGGL((attn_decode_fused_kernel<HDv, QVv, KPWv>), dim3(nch, H, B), dim3(256), 0, s, (const uint16_t*)qkv,   \
+#define FUSED_RELAY(HDv)                                                                                                \
+  if (kpw == 64) { FUSED_KPW(HDv, 1, 64, true); } else if (kpw == 48) { FUSED_KPW(HDv, 1, 48, true); } else { FUSED_KPW(HDv, 1, 32, true); }
+#define FUSED_KPW(HDv, QVv, KPWv, RELAYv)                                                                               \
+  hipLaunchKernelGGL((attn_decode_fused_kernel<HDv, QVv, KPWv, RELAYv>), dim3(nch, H, B), dim3(256), 0, s, (const uint16_t*)qkv,   \
                      (const uint16_t*)qw, (const uint16_t*)kw, sin_tab, cos_tab, (uint16_t*)kcache, (uint16_t*)vcache, \
-                     key_bias, (float*)ws, H, Hkv, Lmax, n_pos, past_len, past_len_dev, nch, bias_stride, eps, qk_ssq, \
-                     rope_now, (uint16_t*)out, tickets, ll)
+                     key_bias, (float*)ws, H, Hkv, Lmax, n_pos, past_len, past_len_dev, nch, bias_stride, eps,         \
+                     (const float*)qk_ssq, rope_now, (uint16_t*)out, tickets, ll, epoch, status, spin_limit)
   // the workspace starts with one ticket counter per (batch, head): zero on entry (zeroed at allocation,
   // reset by the workgroup that draws the last ticket), then one launch counter per (batch, head) for the flag
   // form (a region of its own: a workspace may serve both forms in turn), then the partials
-  // (measured at the 7B shapes, context 2048: the in-kernel merge wins while the launch is a single round of
-  // workgroups -- 17.0 against 20.4 us at batch 1 -- and loses once workgroups queue up -- 69.7 against 61.6 us
-  // at batch 8, where one workgroup per (batch, head) takes 66.9)
-  const bool merge_in_kernel = merge == 0 || merge == 1 || (merge < 0 && (int64_t)B * H * nch <= 1536);
-  // (measured with 128-key chunks, batch 1: the flag form is level with the ticket form at 17 chunks per head -- 17.2
-  // against 16.4 us, 7B at context 2048 -- and ahead from about two dozen -- 34.4 against 36.5 us, 13B at context 4090;
-  // with that launch's 256-key chunks, 17 per head, the two forms are level again at 29.6 us)
-  const int ll = merge_in_kernel && (merge == 1 || (merge < 0 && nch >= kFlagMergeFromChunks)) ? 1 : 0;  // needs the counters
-  int* tickets = merge_in_kernel ? reinterpret_cast<int*>(ws) : nullptr;
+  int* tickets = plan.merge_in_kernel ? reinterpret_cast<int*>(ws) : nullptr;
   ws = reinterpret_cast<float*>(ws) + (int64_t)2 * B * H;
   const int qv = (H * hd / 8 + 255) / 256;
-  if (hd == 128) {
+  if (relay) {
+    if (hd == 128) { FUSED_RELAY(128) } else { FUSED_RELAY(64) }
+  } else if (hd == 128) {
     if (qv <= 1) { FUSED(128, 1); } else if (qv <= 2) { FUSED(128, 2); } else { FUSED(128, 4); }
   } else {
     if (qv <= 1) { FUSED(64, 1); } else if (qv <= 2) { FUSED(64, 2); } else { FUSED(64, 4); }
   }
 #undef FUSED
+#undef FUSED_RELAY
 #undef FUSED_KPW
   O355_CHECK_LAUNCH();
+}
+}  // namespace
+
+extern "C" int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
+                                               const float* cos_tab, void* kcache, void* vcache, const float* key_bias,
+                                               void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
+                                               int past_len, const int32_t* past_len_dev, int n_keys_max,
+                                               int bias_stride, float eps, const float* qk_ssq, const float* rope_now,
+                                               int dtype, int merge, void* stream) {
+  return attn_fused_any(qkv, qw, kw, sin_tab, cos_tab, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd, Lmax, n_pos, past_len,
+                        past_len_dev, n_keys_max, bias_stride, eps, qk_ssq, rope_now, dtype, merge, false, nullptr, nullptr, 0, stream);
 }
 
 extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
@@ -1309,4 +1427,37 @@ extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const 
   return olmo355_attn_decode_fused_merge(qkv, qw, kw, sin_tab, cos_tab, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd,
                                          Lmax, n_pos, past_len, past_len_dev, n_keys_max, bias_stride, eps, qk_ssq,
                                          rope_now, dtype, -1, stream);
+}
+
+extern "C" int olmo355_attn_decode_relay(const uint32_t* qkv, const void* qw, const void* kw, const float* sin_tab,
+                                         const float* cos_tab, void* kcache, void* vcache, const float* key_bias,
+                                         uint32_t* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
+                                         int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride,
+                                         float eps, const uint64_t* qk_ssq, const float* rope_now, const int32_t* epoch,
+                                         int32_t* status, int spin_limit, void* stream) {
+  return attn_fused_any(qkv, qw, kw, sin_tab, cos_tab, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd, Lmax, n_pos, past_len,
+                        past_len_dev, n_keys_max, bias_stride, eps, qk_ssq, rope_now, O355_BF16, -1, true, epoch, status,
+                        spin_limit, stream);
+}
+
+// What a launch of olmo355_attn_decode_relay takes of the chip (as olmo355_w4_relay_footprint): out[0] workgroups,
+// out[1] waves per workgroup, out[2] vector registers per lane, out[3] bytes of LDS per workgroup.
+extern "C" int olmo355_attn_decode_relay_footprint(int B, int H, int hd, int n_keys_max, int* out) {
+  if (!out || B <= 0 || H <= 0 || n_keys_max <= 0) return O355_EINVAL;
+  if (hd != 128 && hd != 64) return O355_EUNSUPPORTED;
+  const FusedPlan plan = fused_plan(B, H, n_keys_max, -1);
+  if (!plan.merge_in_kernel) return O355_EUNSUPPORTED;
+  out[0] = plan.nch * H * B, out[1] = 4;
+  const void* fn = nullptr;
+#define FP(HDv, KPWv) fn = reinterpret_cast<const void*>(attn_decode_fused_kernel<HDv, 1, KPWv, true>)
+  if (hd == 128) {
+    if (plan.kpw == 64) FP(128, 64); else if (plan.kpw == 48) FP(128, 48); else FP(128, 32);
+  } else {
+    if (plan.kpw == 64) FP(64, 64); else if (plan.kpw == 48) FP(64, 48); else FP(64, 32);
+  }
+#undef FP
+  hipFuncAttributes fa;
+  if (hipFuncGetAttributes(&fa, fn) != hipSuccess) return O355_ELAUNCH;
+  out[2] = fa.numRegs, out[3] = (int)fa.sharedSizeBytes;
+  return O355_OK;
 }

@@ -376,6 +376,135 @@ def w4_chain(steps, sync: torch.Tensor, status: torch.Tensor, spin_limit: int = 
     return True
 
 
+# ---------------------------------------------------------------------------------------------
+# the decode relay (one row): launches on two streams, the hand-over carried by epoch tags in the data
+# ---------------------------------------------------------------------------------------------
+RELAY_SPIN_LIMIT = 1 << 20  # polls of a waiting wave before it gives up and sets the status word (about a second)
+
+
+def relay_untag(t: torch.Tensor) -> torch.Tensor:
+    """Tagged words (int32: bf16 bits << 16 | epoch) -> the bf16 numbers (a copy)."""
+    return t.contiguous().view(torch.int16).view(*t.shape, 2)[..., 1].contiguous().view(torch.bfloat16)
+
+
+def relay_tags(t: torch.Tensor) -> torch.Tensor:
+    """The 16-bit tags of tagged words."""
+    return t & 0xFFFF
+
+
+def relay_tag(x: torch.Tensor, out: torch.Tensor, epoch: torch.Tensor, stream: Optional[int] = None) -> torch.Tensor:
+    """bf16 numbers -> tagged words carrying the current epoch, into ``out`` (int32, same count)."""
+    _dev(x, out, epoch)
+    if x.dtype != torch.bfloat16 or out.dtype != torch.int32 or out.numel() != x.numel() or epoch.dtype != torch.int32:
+        raise TypeError("relay_tag: bf16 in, int32 out of the same size, int32 epoch")
+    check("olmo355_relay_tag", lib().olmo355_relay_tag(_p(x), _p(out), x.numel(), _p(epoch), _stream() if stream is None else stream))
+    return out
+
+
+def w4_relay(x: torch.Tensor, w: "W4Tiled", y: torch.Tensor, epoch: torch.Tensor, status: torch.Tensor, *,
+             resid: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None, eps: float = 0.0,
+             ssq_in: Optional[torch.Tensor] = None, x_out: Optional[torch.Tensor] = None,
+             ssq_out: Optional[torch.Tensor] = None, swiglu: bool = False, cfg: int = 0,
+             spin_limit: int = RELAY_SPIN_LIMIT, stream: Optional[int] = None) -> bool:
+    """One int4 linear of the decode relay at one row; every buffer is the caller's (nothing is allocated).
+    ``x``: int32 tagged words or bf16; ``y``: int32 (tagged) or bf16, ``N`` (``N/2`` with ``swiglu``) numbers;
+    ``ssq_in`` / ``ssq_out``: int64 pairs per 16-column tile; ``resid`` / ``x_out``: tagged rows; with ``resid`` the
+    activations are ``resid + rmsnorm(x; norm_w, eps)`` and also go to ``x_out``.  Returns ``False`` when the kernel
+    does not cover the shape (nothing launched)."""
+    _dev(x, y, epoch, status, resid, norm_w, ssq_in, x_out, ssq_out, w.wt)
+    if x.numel() != w.K or x.dtype not in (torch.int32, torch.bfloat16) or y.dtype not in (torch.int32, torch.bfloat16):
+        raise ValueError("w4_relay: one row of K tagged words or bf16 numbers in; int32 or bf16 out")
+    if y.numel() != (w.N // 2 if swiglu else w.N):
+        raise ValueError("w4_relay: output size mismatch")
+    for t, n, dt in ((resid, w.K, torch.int32), (x_out, w.K, torch.int32), (norm_w, w.K, torch.bfloat16),
+                     (ssq_in, w.K // 16, torch.int64), (ssq_out, w.N // 16, torch.int64)):
+        if t is not None and (t.numel() != n or t.dtype != dt):
+            raise ValueError("w4_relay: a side buffer has the wrong size or dtype")
+    if epoch.dtype != torch.int32 or status.dtype != torch.int32:
+        raise TypeError("w4_relay: int32 epoch and status words")
+    st = lib().olmo355_w4_relay(_p(x), int(x.dtype == torch.int32), _p(ssq_in), _p(resid), _p(norm_w), float(eps), _p(x_out),
+                                _p(w.wt), _p(w.st), _p(w.zt), _p(y), int(y.dtype == torch.int32), _p(ssq_out), w.N, w.K,
+                                int(swiglu), _p(epoch), _p(status), int(spin_limit), int(cfg),
+                                _stream() if stream is None else stream)
+    if st == 2:
+        return False
+    check("olmo355_w4_relay", st)
+    return True
+
+
+def relay_final(x: torch.Tensor, ssq_in: torch.Tensor, resid: torch.Tensor, norm_w: torch.Tensor, eps: float,
+                out: torch.Tensor, epoch: torch.Tensor, status: torch.Tensor, spin_limit: int = RELAY_SPIN_LIMIT) -> torch.Tensor:
+    """``out = resid + rmsnorm(x; norm_w, eps)`` from tagged rows into a plain bf16 row (the relay's last update)."""
+    _dev(x, ssq_in, resid, norm_w, out, epoch, status)
+    K = x.numel()
+    if (x.dtype != torch.int32 or resid.dtype != torch.int32 or resid.numel() != K or ssq_in.dtype != torch.int64
+            or ssq_in.numel() != K // 16 or norm_w.dtype != torch.bfloat16 or norm_w.numel() != K
+            or out.dtype != torch.bfloat16 or out.numel() != K):
+        raise ValueError("relay_final: tagged rows, int64 pairs, bf16 weight and output of one width expected")
+    check("olmo355_relay_final",
+          lib().olmo355_relay_final(_p(x), _p(ssq_in), _p(resid), _p(norm_w), float(eps), _p(out), K, _p(epoch), _p(status),
+                                    int(spin_limit), _stream()))
+    return out
+
+
+def attn_decode_relay(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, ws, out, H: int, Hkv: int, hd: int,
+                      past_len: int, n_keys_max: int, eps: float, epoch: torch.Tensor, status: torch.Tensor,
+                      key_bias: Optional[torch.Tensor] = None, past_len_dev: Optional[torch.Tensor] = None,
+                      qk_ssq: Optional[torch.Tensor] = None, rope_now: Optional[torch.Tensor] = None,
+                      spin_limit: int = RELAY_SPIN_LIMIT, stream: Optional[int] = None) -> bool:
+    """:func:`attn_decode_fused` for one sequence as a leg of the relay: ``qkv`` tagged words, ``qk_ssq`` int64 pairs,
+    ``out`` tagged words ``[H * hd]``.  Returns ``False`` when the relay form does not cover the shape."""
+    _dev(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, ws, out, key_bias, past_len_dev, qk_ssq, rope_now, epoch, status)
+    width = (H + 2 * Hkv) * hd
+    if qkv.dtype != torch.int32 or qkv.numel() != width or out.dtype != torch.int32 or out.numel() != H * hd:
+        raise ValueError("attn_decode_relay: tagged qkv of one token and a tagged output row expected")
+    if qk_ssq is not None and (qk_ssq.dtype != torch.int64 or qk_ssq.numel() != width // 16):
+        raise ValueError("attn_decode_relay: qk_ssq int64 [(H + 2 Hkv) hd / 16] expected")
+    if kcache.dtype != torch.bfloat16 or kcache.shape != vcache.shape or kcache.shape[1] != Hkv or kcache.shape[3] != hd:
+        raise ValueError("attn_decode_relay: bf16 caches [B, Hkv, Lmax, hd] expected")
+    if rope_now is not None and (rope_now.dtype != torch.float32 or rope_now.numel() != 2 * hd):
+        raise ValueError("rope_now: float32 [2 * hd] expected")
+    Lmax, n_pos = kcache.shape[2], sin_tab.shape[0]
+    if ws.numel() * ws.element_size() < int(lib().olmo355_attn_decode_workspace_bytes(1, H, hd, n_keys_max)):
+        raise ValueError("attention workspace too small")
+    st = lib().olmo355_attn_decode_relay(_p(qkv), _p(q_weight), _p(k_weight), _p(sin_tab), _p(cos_tab), _p(kcache), _p(vcache),
+                                         _p(key_bias), _p(out), _p(ws), 1, H, Hkv, hd, Lmax, n_pos, past_len, _p(past_len_dev),
+                                         n_keys_max, key_bias.shape[1] if key_bias is not None else 0, float(eps), _p(qk_ssq),
+                                         _p(rope_now), _p(epoch), _p(status), int(spin_limit),
+                                         _stream() if stream is None else stream)
+    if st == 2:
+        return False
+    check("olmo355_attn_decode_relay", st)
+    return True
+
+
+def relay_footprint_w4(N: int, K: int, norm: bool, swiglu: bool, cfg: int = 0, x_tagged: bool = True):
+    """(workgroups, waves per workgroup, registers per lane, LDS bytes per workgroup) of a :func:`w4_relay` launch,
+    or ``None`` when the kernel does not cover the shape."""
+    import ctypes
+
+    out = (ctypes.c_int * 4)()
+    st = lib().olmo355_w4_relay_footprint(N, K, int(norm), int(x_tagged), int(swiglu), int(cfg), out)
+    return tuple(out) if st == 0 else None
+
+
+def relay_footprint_attn(H: int, hd: int, n_keys_max: int):
+    import ctypes
+
+    out = (ctypes.c_int * 4)()
+    st = lib().olmo355_attn_decode_relay_footprint(1, H, hd, n_keys_max, out)
+    return tuple(out) if st == 0 else None
+
+
+def relay_pair_ok(older, younger, n_cu: int, lds_per_cu: int) -> bool:
+    """Whether the younger launch, waiting on the older one's output, can never keep a workgroup of the older one
+    from starting (footprints as above)."""
+    import ctypes
+
+    a, b = (ctypes.c_int * 4)(*older), (ctypes.c_int * 4)(*younger)
+    return bool(lib().olmo355_relay_pair_ok(a, b, int(n_cu), int(lds_per_cu)))
+
+
 def f32_linear(x: torch.Tensor, weight_nk: torch.Tensor) -> torch.Tensor:
     _dev(x, weight_nk)
     if x.dtype != torch.float32 or weight_nk.dtype != torch.float32:
