@@ -50,12 +50,13 @@ EXPORTS = {
     "olmo355_w4_chain_grid": (I, []),
     "olmo355_w4_chain_sync_ints": (I, []),
     "olmo355_w4_chain": (I, [ctypes.POINTER(ChainPhase), I, I, P, P, I, P]),
-    "olmo355_w4_relay": (I, [P, I, P, P, P, F, P, P, P, P, P, I, P, I, I, I, P, P, I, I, P]),
+    "olmo355_w4_relay": (I, [P, I, P, P, P, F, P, P, P, P, P, I, P, I, I, I, P, P, P, P, I, I, P]),
     "olmo355_w4_relay_footprint": (I, [I, I, I, I, I, I, P]),
     "olmo355_relay_pair_ok": (I, [P, P, I, I]),
+    "olmo355_relay_device": (I, [P]),
     "olmo355_relay_final": (I, [P, P, P, P, F, P, I, P, P, I, P]),
     "olmo355_relay_tag": (I, [P, P, I, P, P]),
-    "olmo355_attn_decode_relay": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, P, P, P, I, P]),
+    "olmo355_attn_decode_relay": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, P, P, P, P, P, I, P]),
     "olmo355_attn_decode_relay_footprint": (I, [I, I, I, I, P]),
     "olmo355_b16_gemv_fused": (I, [P, P, P, F, P, P, P, I, I, I, I, P]),
     "olmo355_w4_gemm": (I, [P, P, P, P, P, I, I, I, P]),

@@ -19,6 +19,7 @@
 #include "common.h"
 
 #include <mutex>
+#include <type_traits>
 
 namespace {
 
@@ -619,7 +620,7 @@ __global__ __launch_bounds__(HD) void attn_decode_combine_kernel(const float* __
 // the new key / value row, appends it to the cache (olmo/model.py:615-620) and uses it from LDS.
 //
 // RELAY: the launch is one leg of the two-stream decode relay (relay.hip).  qkv then holds tagged words (bf16 bits
-// << 16 | epoch & 0xffff), qk_ssq pairs (float bits, epoch) and `out` receives tagged words; the cache rows -- which
+// << 16 | epoch & 0xffff), qk_ssq tagged sums (float, low 4 bits = epoch & 0xf) and `out` receives tagged words; the cache rows -- which
 // depend on no other launch of the step -- are requested first, and the few threads that read the token's q | k | v
 // pieces and the sums of squares ask for them until every tag shows this step's epoch (at most spin_limit times).
 template <int HD, int QV, int KPW, bool RELAY = false>  // QV: 16-byte pieces of the q (k) row per thread, H*HD/8 <= QV*256; KPW: keys per wave
@@ -630,7 +631,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     int n_pos, int past_len, const int32_t* __restrict__ past_dev, int nchunks_max, int bias_stride, float eps,
     const float* __restrict__ qk_ssq, const float* __restrict__ rope_now, uint16_t* __restrict__ out,
     int* __restrict__ tickets, int ll, const int32_t* __restrict__ epoch_p = nullptr, int32_t* __restrict__ status = nullptr,
-    int spin_limit = 0) {
+    int spin_limit = 0, const int32_t* __restrict__ hint_in = nullptr, int32_t* __restrict__ hint_out = nullptr) {
   constexpr int LPK = HD / 8, KPI = 64 / LPK, ITERS = KPW / KPI;
   constexpr int kDecodeChunk = 4 * KPW, kDecodeKeysPerWave = KPW;
   constexpr int HALF = HD / 2, CPH = HD / 16;  // pair chunks per head
@@ -723,6 +724,47 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
       }
     }
   }
+  // ---- relay: the token's pieces and the sums of squares are tagged; they are asked for once here, BEFORE the cache
+  // rows (when the projection is done already they arrive first and the query is ready while the rows travel) ...
+  uint32_t tag16 = 0, epoch = 0;
+  const int relay_width = dq + 2 * dk;
+  const __amdgpu_buffer_rsrc_t rt = make_rsrc(RELAY ? reinterpret_cast<const uint32_t*>(qkv) + (int64_t)b * relay_width : nullptr,
+                                              RELAY ? (int64_t)relay_width * 4 : 0);
+  const __amdgpu_buffer_rsrc_t rs2 = make_rsrc(RELAY && qk_ssq ? reinterpret_cast<const uint32_t*>(qk_ssq) + (int64_t)b * (relay_width >> 4) : nullptr,
+                                               RELAY && qk_ssq ? (int64_t)(relay_width >> 4) * 4 : 0);
+  const int relay_first = role_q ? h * HD + j : (role_k ? dq + hk * HD + j : dq + dk + hk * HD + (tid - 64) * 8);  // element
+  const bool role = role_q || role_k || role_v;
+  const int nq_p = dq >> 4, nk_p = dk >> 4;  // tagged sums of the q and the k part (float, low 4 bits = epoch & 0xf)
+  u32x4 t[4], pq[2], pk[2];
+  // workgroups whose chunk lies past the current length (a captured launch covers the cache's capacity) leave below
+  // without having waited for anything
+  const bool relay_work = RELAY && (chunk * kDecodeChunk < pos + 1 || (ll && chunk == nchunks_max - 1));
+  // (every request goes past the L2 -- device-coherent -- so that no poll finds a line there that was fetched before
+  // the projection's stores)
+  auto relay_ask = [&]() {
+    auto ld = [&](__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+      return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 16));
+    };
+    if (role) {
+      t[0] = ld(rt, relay_first * 4, 0);
+      t[1] = ld(rt, relay_first * 4 + 16, 0);
+      if (!role_v) {
+        t[2] = ld(rt, (relay_first + HALF) * 4, 0);
+        t[3] = ld(rt, (relay_first + HALF) * 4 + 16, 0);
+      }
+    }
+    if (wave == 0 && norm) {
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        if (r * 256 < nq_p) pq[r] = ld(rs2, lane * 16, r * 1024);
+        if (r * 256 < nk_p) pk[r] = ld(rs2, lane * 16, nq_p * 4 + r * 1024);
+      }
+    }
+  };
+  if constexpr (RELAY) {
+    epoch = (uint32_t)*epoch_p, tag16 = epoch & 0xffffu;
+    if (wave < 2 && relay_work && !hint_in) relay_ask();  // beside a running producer (hint word given) the rows are rarely there yet
+  }
   // first row of the last request that fits; 0 for a cache shorter than one request, whose lanes past the end
   // the range check then sees (the scalar offset is 0)
   const int rowcap = max(kmax + 1 - KPI, 0);
@@ -740,44 +782,19 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     bias[it] = key_bias ? key_bias[(int64_t)b * bias_stride + min(min(kbase + it * KPI + kslot, kmax), bias_stride - 1)] : 0.f;  // keys past the row's end are past L
   }
 
-  uint32_t tag16 = 0;
   if constexpr (RELAY) {
-    // ---- 1'. the token's pieces and the sums of squares, asked for until they carry this step's epoch.  Waves 0 and
-    // 1 hold every role; wave 0 also adds up the per-tile sums of squares (two pairs per lane and request).
-    const uint32_t epoch = (uint32_t)*epoch_p;
-    tag16 = epoch & 0xffffu;
-    // workgroups whose chunk lies past the current length (a captured launch covers the cache's capacity) leave below
-    // without having waited for anything
-    const bool has_work = chunk * kDecodeChunk < pos + 1 || (ll && chunk == nchunks_max - 1);
-    if (wave < 2 && has_work) {
-      const int width = dq + 2 * dk;
-      const __amdgpu_buffer_rsrc_t rt = make_rsrc(reinterpret_cast<const uint32_t*>(qkv) + (int64_t)b * width, (int64_t)width * 4);
-      const __amdgpu_buffer_rsrc_t rs2 = make_rsrc(reinterpret_cast<const uint64_t*>(qk_ssq) + (int64_t)b * (width >> 4), (int64_t)(width >> 4) * 8);
-      const int first = role_q ? h * HD + j : (role_k ? dq + hk * HD + j : dq + dk + hk * HD + (tid - 64) * 8);  // element
-      const bool role = role_q || role_k || role_v;
-      const int nq_p = dq >> 4, nk_p = dk >> 4;  // pairs of the q and the k part
-      u32x4 t[4], pq[3], pk[3];
-      bool gave_up = false;
+    // ---- 1'. ... and until they do, asked for again: these requests queue behind the cache rows, which have to
+    // arrive anyway
+    if (wave < 2 && relay_work) {
+      bool gave_up = false, watched = false;
       for (int spins = 0;; ++spins) {
-        bool ok = true;
-        if (role) {
-          t[0] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rt, first * 4, 0, 16));
-          t[1] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rt, first * 4 + 16, 0, 16));
-          if (!role_v) {
-            t[2] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rt, (first + HALF) * 4, 0, 16));
-            t[3] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rt, (first + HALF) * 4 + 16, 0, 16));
-          }
-        }
+        bool ok = hint_in == nullptr || watched;  // nothing has been asked for before the hint was up
         if (wave == 0 && norm) {
 #pragma unroll
-          for (int r = 0; r < 3; ++r) {
-            if (r * 128 < nq_p) pq[r] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs2, lane * 16, r * 1024, 16));
-            if (r * 128 < nk_p) pk[r] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rs2, lane * 16, nq_p * 8 + r * 1024, 16));
-          }
-#pragma unroll
-          for (int r = 0; r < 3; ++r) {
-            if (r * 128 + lane * 2 < nq_p) ok = ok && pq[r].y == epoch && pq[r].w == epoch;
-            if (r * 128 + lane * 2 < nk_p) ok = ok && pk[r].y == epoch && pk[r].w == epoch;
+          for (int r = 0; r < 2; ++r) {
+            auto sok = [&](const u32x4& v) { return (((v.x ^ epoch) | (v.y ^ epoch) | (v.z ^ epoch) | (v.w ^ epoch)) & 0xfu) == 0u; };
+            if (r * 256 + lane * 4 < nq_p) ok = ok && sok(pq[r]);
+            if (r * 256 + lane * 4 < nk_p) ok = ok && sok(pk[r]);
           }
         }
         if (role) {
@@ -790,9 +807,25 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
           gave_up = true;
           break;
         }
-        __builtin_amdgcn_s_sleep(4);
+        if (hint_in && !watched) {  // the projection is still at work: watch the word its last workgroup sets (a hint; the tags decide)
+          const __amdgpu_buffer_rsrc_t rh = make_rsrc(hint_in, O355_RELAY_HINT_COPIES * O355_RELAY_HINT_STRIDE);
+          const int copy = ((((int)blockIdx.y * (int)gridDim.x + (int)blockIdx.x) * 2 + wave) & (O355_RELAY_HINT_COPIES - 1)) * O355_RELAY_HINT_STRIDE;
+          for (; spins < spin_limit; ++spins) {
+            asm volatile("" ::: "memory");  // the request is made again in every iteration
+            if ((uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rh, 0, copy, 16) == epoch) break;
+            __builtin_amdgcn_s_sleep(16);
+          }
+          watched = true;
+        } else {
+          __builtin_amdgcn_s_sleep(4);
+        }
+        asm volatile("" ::: "memory");  // the requests are made again in every iteration
+        relay_ask();
       }
-      if (gave_up && lane == 0) __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (gave_up && lane == 0) {
+        __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (status[4]) atomicOr(status + 5, 8), atomicAdd(status + 7, 1);
+      }
       auto pack8 = [](const u32x4& a, const u32x4& c) {  // eight tagged words -> eight bf16
         return u32x4{(a.x >> 16) | (a.y & 0xffff0000u), (a.z >> 16) | (a.w & 0xffff0000u), (c.x >> 16) | (c.y & 0xffff0000u),
                      (c.z >> 16) | (c.w & 0xffff0000u)};
@@ -801,9 +834,13 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
       if (role_v) vrow = pack8(t[0], t[1]);
       if (wave == 0 && norm) {
 #pragma unroll
-        for (int r = 0; r < 3; ++r) {
-          if (r * 128 + lane * 2 < nq_p) sq += __uint_as_float(pq[r].x) + __uint_as_float(pq[r].z);
-          if (r * 128 + lane * 2 < nk_p) sk += __uint_as_float(pk[r].x) + __uint_as_float(pk[r].z);
+        for (int r = 0; r < 2; ++r) {
+          auto sm = [](const u32x4& v) {
+            return (__uint_as_float(v.x & 0xfffffff0u) + __uint_as_float(v.y & 0xfffffff0u)) +
+                   (__uint_as_float(v.z & 0xfffffff0u) + __uint_as_float(v.w & 0xfffffff0u));
+          };
+          if (r * 256 + lane * 4 < nq_p) sq += sm(pq[r]);
+          if (r * 256 + lane * 4 < nk_p) sk += sm(pk[r]);
         }
       }
     }
@@ -1028,6 +1065,8 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       else out[((int64_t)b * H + h) * HD + tid] = bits;
     }
+    if (RELAY && hint_out && tid < O355_RELAY_HINT_COPIES && h == H - 1 && b == (int)gridDim.z - 1)
+      __hip_atomic_store(hint_out + tid * (O355_RELAY_HINT_STRIDE / 4), (int32_t)epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (tid == 0)  // the next launch's flag
       __hip_atomic_store(tickets + (gridDim.z + b) * H + h, (int)(flag & 0x3FFFFFu), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return;
@@ -1084,6 +1123,8 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
     __hip_atomic_store(reinterpret_cast<uint32_t*>(out) + ((int64_t)b * H + h) * HD + tid,
                        ((uint32_t)f32_to_bf16_bits(go / gl) << 16) | tag16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   else out[((int64_t)b * H + h) * HD + tid] = f32_to_bf16_bits(go / gl);
+  if (RELAY && hint_out && tid < O355_RELAY_HINT_COPIES && h == H - 1 && b == (int)gridDim.z - 1)
+    __hip_atomic_store(hint_out + tid * (O355_RELAY_HINT_STRIDE / 4), (int32_t)epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <int DT, int HD>
@@ -1360,7 +1401,7 @@ int attn_fused_any(const void* qkv, const void* qw, const void* kw, const float*
                    void* vcache, const float* key_bias, void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
                    int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps, const void* qk_ssq,
                    const float* rope_now, int dtype, int merge, bool relay, const int32_t* epoch, int32_t* status, int spin_limit,
-                   void* stream) {
+                   const int32_t* hint_in, int32_t* hint_out, void* stream) {
   if (merge < -1 || merge > 2) return O355_EINVAL;
   if (!qkv || !sin_tab || !cos_tab || !kcache || !vcache || !out || !ws) return O355_EINVAL;
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || past_len < 0 || n_keys_max <= 0 || n_keys_max > Lmax)
@@ -1374,7 +1415,7 @@ int attn_fused_any(const void* qkv, const void* qw, const void* kw, const float*
   const int kpw = plan.kpw, chunk_keys = 4 * kpw, nch = plan.nch, ll = plan.ll;
   if (relay) {
     if (!epoch || !status || spin_limit < 0 || (qw && !qk_ssq)) return O355_EINVAL;
-    if (!plan.merge_in_kernel || H * hd > 6144 || Hkv * hd > 6144) return O355_EUNSUPPORTED;
+    if (!plan.merge_in_kernel || H * hd > 8192 || Hkv * hd > 8192 || ((H * hd) & 127) || ((Hkv * hd) & 127)) return O355_EUNSUPPORTED;
   }
 #define FUSED(HDv, QVv)                                                                                                 \
   if (kpw == 64) { FUSED_KPW(HDv, QVv, 64, false); } else if (kpw == 48) { FUSED_KPW(HDv, QVv, 48, false); } else { FUSED_KPW(HDv, QVv, 32, false); } \
@@ -1387,7 +1428,7 @@ int attn_fused_any(const void* qkv, const void* qw, const void* kw, const float*
   hipLaunchKernelGGL((attn_decode_fused_kernel<HDv, QVv, KPWv, RELAYv>), dim3(nch, H, B), dim3(256), 0, s, (const uint16_t*)qkv,   \
                      (const uint16_t*)qw, (const uint16_t*)kw, sin_tab, cos_tab, (uint16_t*)kcache, (uint16_t*)vcache, \
                      key_bias, (float*)ws, H, Hkv, Lmax, n_pos, past_len, past_len_dev, nch, bias_stride, eps,         \
-                     (const float*)qk_ssq, rope_now, (uint16_t*)out, tickets, ll, epoch, status, spin_limit)
+                     (const float*)qk_ssq, rope_now, (uint16_t*)out, tickets, ll, epoch, status, spin_limit, hint_in, hint_out)
   // the workspace starts with one ticket counter per (batch, head): zero on entry (zeroed at allocation,
   // reset by the workgroup that draws the last ticket), then one launch counter per (batch, head) for the flag
   // form (a region of its own: a workspace may serve both forms in turn), then the partials
@@ -1415,7 +1456,7 @@ extern "C" int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, 
                                                int bias_stride, float eps, const float* qk_ssq, const float* rope_now,
                                                int dtype, int merge, void* stream) {
   return attn_fused_any(qkv, qw, kw, sin_tab, cos_tab, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd, Lmax, n_pos, past_len,
-                        past_len_dev, n_keys_max, bias_stride, eps, qk_ssq, rope_now, dtype, merge, false, nullptr, nullptr, 0, stream);
+                        past_len_dev, n_keys_max, bias_stride, eps, qk_ssq, rope_now, dtype, merge, false, nullptr, nullptr, 0, nullptr, nullptr, stream);
 }
 
 extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
@@ -1433,11 +1474,12 @@ extern "C" int olmo355_attn_decode_relay(const uint32_t* qkv, const void* qw, co
                                          const float* cos_tab, void* kcache, void* vcache, const float* key_bias,
                                          uint32_t* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
                                          int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride,
-                                         float eps, const uint64_t* qk_ssq, const float* rope_now, const int32_t* epoch,
-                                         int32_t* status, int spin_limit, void* stream) {
+                                         float eps, const uint32_t* qk_ssq, const float* rope_now, const int32_t* epoch,
+                                         int32_t* status, const int32_t* hint_in, int32_t* hint_out, int spin_limit,
+                                         void* stream) {
   return attn_fused_any(qkv, qw, kw, sin_tab, cos_tab, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd, Lmax, n_pos, past_len,
                         past_len_dev, n_keys_max, bias_stride, eps, qk_ssq, rope_now, O355_BF16, -1, true, epoch, status,
-                        spin_limit, stream);
+                        spin_limit, hint_in, hint_out, stream);
 }
 
 // What a launch of olmo355_attn_decode_relay takes of the chip (as olmo355_w4_relay_footprint): out[0] workgroups,

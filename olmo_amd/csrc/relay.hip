@@ -10,7 +10,8 @@
 //
 // The hand-over needs no flag, counter or ticket: every number that crosses from one launch to the next carries
 // the step's epoch.  An output element is one 32-bit word (bf16 bits << 16 | epoch & 0xffff), a per-tile sum of
-// squares is an 8-byte pair (float bits, epoch), both written with one device-scope store.  A consumer loads its
+// squares one 32-bit word too (the float rounded to 20 mantissa bits | epoch & 0xf), each written with one
+// device-scope store.  A consumer loads its
 // slice of the row with device-coherent loads and looks at the tags: all equal to the epoch -> the numbers are
 // this step's; otherwise it asks again.  Every buffer is written exactly once per step and the epoch changes with
 // every step, so a stale word can never pass for a fresh one.  The wait is bounded: after `spin_limit` polls the
@@ -29,28 +30,45 @@
 // residual update from tagged inputs into a plain bf16 row.  The attention launch of the relay is
 // attn_decode_fused_kernel<.., RELAY = true> (attention.hip).
 #include <algorithm>
+#include <type_traits>
 
 #include "common.h"
 
 namespace {
 
 constexpr int kSc1 = 16;  // cache policy of a buffer access: device-coherent (never served from a stale L2 line)
+constexpr int kHintCopies = O355_RELAY_HINT_COPIES, kHintStride = O355_RELAY_HINT_STRIDE;
 
 struct RelayArgs {
   const void* x;           // [K]: tagged words (x_tagged) or plain bf16
-  const uint64_t* ssq_in;  // norm: [K/16] pairs (float bits | epoch << 32) left by the launch that wrote x
+  const uint32_t* ssq_in;  // norm: [K/16] tagged sums (float, low 4 bits = epoch & 0xf) left by the launch that wrote x
   const uint32_t* resid;   // norm: [K] tagged residual stream
   const uint16_t* norm_w;  // norm: [K] bf16
   uint32_t* x_out;         // norm: [K] tagged, resid + rmsnorm(x), written by workgroup 0
   void* y;                 // [N] (SwiGLU: [N/2]): tagged words (y_tagged) or plain bf16
-  uint64_t* ssq_out;       // optional, [N/16] pairs
+  uint32_t* ssq_out;       // optional, [N/16] tagged sums
   const int32_t* epoch;    // the step's epoch (device word)
-  int32_t* status;         // set to 1 when a wait gave up
+  int32_t* status;         // [0] set to 1 when a wait gave up; [1..3] statistics when [4] is set (8 words)
+  const int32_t* hint_in;  // optional: a word the producer sets to the epoch when its last workgroup is done
+  int32_t* hint_out;       // optional: this launch's own such word
   float eps;
   int N, K, x_tagged, y_tagged, spin_limit;
 };
 
+// At the top of every polling loop: the requests below it must be made again in every iteration.  (A buffer load is a
+// plain read to the compiler; without this it may keep the first answer in a register and the loop never ends.)
+__device__ __forceinline__ void poll_fence() { asm volatile("" ::: "memory"); }
+
 __device__ __forceinline__ uint32_t tag_word(float v, uint32_t tag16) { return ((uint32_t)f32_to_bf16_bits(v) << 16) | tag16; }
+// a sum of squares as a tagged word: rounded to 20 mantissa bits (its error then stays below that of adding the
+// 256 .. 512 partials of a row in another order), the low 4 bits carry the epoch -- enough to tell this step's
+// word from the previous step's, which is the only other thing the buffer can hold
+__device__ __forceinline__ uint32_t tag_sum(float v, uint32_t epoch) { return ((__float_as_uint(v) + 0x8u) & 0xfffffff0u) | (epoch & 0xfu); }
+__device__ __forceinline__ float sum_of(uint32_t w) { return __uint_as_float(w & 0xfffffff0u); }
+__device__ __forceinline__ bool sums_ok(const u32x4& v, uint32_t epoch) {
+  const uint32_t t = epoch & 0xfu;
+  return (((v.x ^ t) | (v.y ^ t) | (v.z ^ t) | (v.w ^ t)) & 0xfu) == 0u;
+}
 __device__ __forceinline__ bool tags_ok(const u32x4& v, uint32_t tag16) {
   return (((v.x ^ tag16) | (v.y ^ tag16) | (v.z ^ tag16) | (v.w ^ tag16)) & 0xffffu) == 0u;
 }
@@ -61,8 +79,13 @@ __device__ __forceinline__ u32x2 untag4(const u32x4& v) {
 
 // MODE 0: plain bf16 activations; 1: tagged activations; 2: tagged activations with the chained-norm prologue.
 // NQ: quads of four 128-row groups a wave holds in registers (its whole share of K: ceil(K/128 / WAVES) <= 4 NQ).
+// Registers decide how many launches fit the chip side by side: the two-tile shapes are held to 96 (five waves per
+// SIMD), the others are left to the compiler.
+constexpr int relay_min_waves_per_simd(int NT, int NQ) { return 1; }
+
 template <int NT, int WAVES, int NQ, int MODE, int EPI>
-__global__ __launch_bounds__(WAVES * 64) void w4_relay_kernel(RelayArgs a, const u32x4* __restrict__ wt,
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(relay_min_waves_per_simd(NT, NQ))))
+void w4_relay_kernel(RelayArgs a, const u32x4* __restrict__ wt,
                                                               const uint16_t* __restrict__ st, const uint8_t* __restrict__ zt) {
   static_assert(EPI == 0 || NT == 2, "the SwiGLU epilogue owns one up tile and one gate tile");
   constexpr int XC = 2 * NQ;  // 256-element chunks of a wave's slice, at most
@@ -91,25 +114,31 @@ __global__ __launch_bounds__(WAVES * 64) void w4_relay_kernel(RelayArgs a, const
   const __amdgpu_buffer_rsrc_t rz = make_rsrc(zt, (int64_t)ntiles * G * 8);
   u32x4 w[NQ][4][NT];
   uint32_t s16[NQ][NT], z8[NQ][NT];
+  auto issue_weights = [&]() {
 #pragma unroll
-  for (int q = 0; q < NQ; ++q)
+    for (int q = 0; q < NQ; ++q)
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int gc = min(g_begin + 4 * q + u, G - 1);  // past the wave's share: any valid piece, never multiplied
+      for (int u = 0; u < 4; ++u) {
+        const int gc = min(g_begin + 4 * q + u, G - 1);  // past the wave's share: any valid piece, never multiplied
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-        w[q][u][nt] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, lane * 16, (tg[nt] + gc) * 1024, 2));
-    }
-  // the lanes of row block kq hold the scale and zero of group 4 q + kq of the quad
+        for (int nt = 0; nt < NT; ++nt)
+          w[q][u][nt] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, lane * 16, (tg[nt] + gc) * 1024, 2));
+      }
+    // the lanes of row block kq hold the scale and zero of group 4 q + kq of the quad
 #pragma unroll
-  for (int q = 0; q < NQ; ++q)
+    for (int q = 0; q < NQ; ++q)
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      s16[q][nt] = __builtin_amdgcn_raw_buffer_load_b16(rs, (kq * 16 + col) * 2, (tg[nt] + g_begin + 4 * q) * 32, 0);
-      z8[q][nt] = __builtin_amdgcn_raw_buffer_load_b8(rz, kq * 8 + (col >> 1), (tg[nt] + g_begin + 4 * q) * 8, 0);
-    }
+      for (int nt = 0; nt < NT; ++nt) {
+        s16[q][nt] = __builtin_amdgcn_raw_buffer_load_b16(rs, (kq * 16 + col) * 2, (tg[nt] + g_begin + 4 * q) * 32, 0);
+        z8[q][nt] = __builtin_amdgcn_raw_buffer_load_b8(rz, kq * 8 + (col >> 1), (tg[nt] + g_begin + 4 * q) * 8, 0);
+      }
+  };
 
-  // ---- 2. the activations of this wave's slice of K: wait until the producer's words carry this step's epoch ------
+  // ---- 2. the activations of this wave's slice of K.  On one stream (no hint word) they are asked for BEFORE the
+  // weights: the producer is done, they arrive first and are turned into operands while the weights travel.
+  // Otherwise the wave asks (again) until the words carry this step's epoch -- those requests queue behind the wave's
+  // weights, which have to arrive anyway. -----------------------------------------------------------------------------
+  const int spin_max = a.spin_limit;
   const uint32_t epoch = (uint32_t)*a.epoch, tag16 = epoch & 0xffffu;
   const int k0 = g_begin * 128, k1 = g_end * 128;  // the slice, in elements
   const int nch = (k1 - k0 + 255) >> 8;            // chunks of 256 elements: 4 per lane
@@ -118,20 +147,21 @@ __global__ __launch_bounds__(WAVES * 64) void w4_relay_kernel(RelayArgs a, const
   bool gave_up = false;
   if constexpr (MODE == 0) {
     const __amdgpu_buffer_rsrc_t rx = make_rsrc(a.x, (int64_t)K * 2);
+    u32x2 v[XC];
 #pragma unroll
     for (int c = 0; c < XC; ++c)
-      if (c < nch) {
-        const int e = k0 + c * 256 + lane * 4;
-        const u32x2 v = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rx, lane * 8, (k0 + c * 256) * 2, 0));
-        if (e < k1) *reinterpret_cast<u32x2*>(smem + e * 2) = v;
-      }
+      if (c < nch) v[c] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rx, lane * 8, (k0 + c * 256) * 2, 0));
+    issue_weights();
+#pragma unroll
+    for (int c = 0; c < XC; ++c)
+      if (c < nch && k0 + c * 256 + lane * 4 < k1) *reinterpret_cast<u32x2*>(smem + (k0 + c * 256 + lane * 4) * 2) = v[c];
   } else {
     const __amdgpu_buffer_rsrc_t rx = make_rsrc(a.x, (int64_t)K * 4);
     const __amdgpu_buffer_rsrc_t rr = make_rsrc(a.resid, MODE == 2 ? (int64_t)K * 4 : 0);
     const __amdgpu_buffer_rsrc_t rn = make_rsrc(a.norm_w, MODE == 2 ? (int64_t)K * 2 : 0);
-    const int n_ssq = K >> 4;                       // pairs; 128 per request (two per lane)
-    const __amdgpu_buffer_rsrc_t rq = make_rsrc(a.ssq_in, MODE == 2 ? (int64_t)n_ssq * 8 : 0);
-    constexpr int SL = MODE == 2 ? 3 : 0;           // K <= 6144
+    const int n_ssq = K >> 4;                       // tagged sums; 256 per request (four per lane)
+    const __amdgpu_buffer_rsrc_t rq = make_rsrc(a.ssq_in, MODE == 2 ? (int64_t)n_ssq * 4 : 0);
+    constexpr int SL = MODE == 2 ? 2 : 0;           // K <= 8192
     u32x2 nw[XC];
     if constexpr (MODE == 2) {
 #pragma unroll
@@ -139,10 +169,14 @@ __global__ __launch_bounds__(WAVES * 64) void w4_relay_kernel(RelayArgs a, const
         if (c < nch) nw[c] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rn, lane * 8, (k0 + c * 256) * 2, 0));
     }
     u32x4 xv[XC], rv[XC], sv[SL > 0 ? SL : 1];
-    for (int spins = 0;; ++spins) {
+    // Every request goes past the L2 (device-coherent): a line fetched before the producer's stores must never be
+    // found there again by a later poll.  (A request that MAY be served by the L2, even one the compiler only
+    // speculates, leaves such a line behind, and the device-coherent requests that follow then hit it: the wave
+    // sees the old tags until the line happens to be evicted -- measured as waits of a millisecond.)
+    auto ask = [&]() {
 #pragma unroll
       for (int s = 0; s < SL; ++s)
-        if (s * 128 < n_ssq) sv[s] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rq, lane * 16, s * 1024, kSc1));
+        if (s * 256 < n_ssq) sv[s] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rq, lane * 16, s * 1024, kSc1));
 #pragma unroll
       for (int c = 0; c < XC; ++c)
         if (c < nch) {
@@ -150,32 +184,80 @@ __global__ __launch_bounds__(WAVES * 64) void w4_relay_kernel(RelayArgs a, const
           if constexpr (MODE == 2)
             rv[c] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, lane * 16, (k0 + c * 256) * 4, kSc1));
         }
+    };
+    float ss = 0.f;  // this lane's share of the row's sum of squares (of the last check)
+    auto all_tagged = [&]() {  // wave-uniform: every word of the slice carries this step's epoch
       bool ok = true;
+      ss = 0.f;
 #pragma unroll
       for (int s = 0; s < SL; ++s)
-        if (s * 128 + lane * 2 < n_ssq) ok = ok && sv[s].y == epoch && sv[s].w == epoch;  // n_ssq is even
+        if (s * 256 + lane * 4 < n_ssq) {  // n_ssq is a multiple of 8 (K of 128)
+          ok = ok && sums_ok(sv[s], epoch);
+          ss += (sum_of(sv[s].x) + sum_of(sv[s].y)) + (sum_of(sv[s].z) + sum_of(sv[s].w));
+        }
 #pragma unroll
       for (int c = 0; c < XC; ++c)
         if (c < nch && k0 + c * 256 + lane * 4 < k1) {
           ok = ok && tags_ok(xv[c], tag16);
           if constexpr (MODE == 2) ok = ok && tags_ok(rv[c], tag16);
         }
-      if (__builtin_amdgcn_ballot_w64(!ok) == 0) break;
-      if (spins >= a.spin_limit) {
-        gave_up = true;
-        break;
+      return __builtin_amdgcn_ballot_w64(!ok) == 0;
+    };
+    // With a hint word the launch may be running beside its producer, whose rows are then rarely there yet: a request
+    // made now would be wasted traffic (every workgroup asks for the whole row), so the wave asks only once the hint is up.
+    const bool eager = a.hint_in == nullptr;
+    if (eager) ask();
+    issue_weights();
+    const bool ready = eager && all_tagged();
+    if (a.hint_in && wave == 0 && ready && lane == 0)  // the other waves of the workgroup need not wait for the hint either
+      *reinterpret_cast<volatile uint32_t*>(red + WAVES * NT * 16) = epoch ^ (uint32_t)(uintptr_t)a.hint_in;
+    if (!ready) {
+      int spins = 0, hint_spins = 0;
+      // The producer is still at work.  Asking for the whole slice over and over would cost more traffic than the
+      // weights (every workgroup reads all of the row), so the wave first watches one word that the producer's last
+      // workgroup sets when it is done -- a hint, not a guarantee: the tags decide.
+      // One wave per workgroup watches the hint -- one of kHintCopies copies, kHintStride bytes apart, so that the
+      // pollers of a launch are spread over the memory channels -- and tells the others through LDS.
+      if (a.hint_in) {
+        volatile uint32_t* flag = reinterpret_cast<volatile uint32_t*>(red + WAVES * NT * 16);
+        const uint32_t mine = epoch ^ (uint32_t)(uintptr_t)a.hint_in;
+        if (wave == 0) {
+          const __amdgpu_buffer_rsrc_t rh = make_rsrc(a.hint_in, kHintCopies * kHintStride);
+          const int copy = (blockIdx.x & (kHintCopies - 1)) * kHintStride;
+          for (; spins < spin_max; ++spins) {
+            poll_fence();
+            if ((uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rh, 0, copy, kSc1) == epoch) break;
+            __builtin_amdgcn_s_sleep(16);
+          }
+          if (lane == 0) *flag = mine;
+        } else {
+          for (; spins < spin_max; ++spins) {
+            poll_fence();
+            if (*flag == mine) break;
+            __builtin_amdgcn_s_sleep(16);
+          }
+        }
+        hint_spins = spins;
       }
-      __builtin_amdgcn_s_sleep(4);
+      for (;; ++spins) {
+        poll_fence();
+        ask();
+        if (all_tagged()) break;
+        if (spins >= spin_max) {
+          gave_up = true;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(4);
+      }
+      if (a.status[4] && lane == 0) {  // statistics of a tuning run (status[4] set by the host): waits per launch
+        atomicMax(a.status + 1, hint_spins);
+        atomicMax(a.status + 2, spins - hint_spins);
+        atomicAdd(a.status + 3, 1);
+      }
     }
     float rstd = 0.f;
-    if constexpr (MODE == 2) {  // 1 / rms of the row: the per-tile partials in a fixed order (lane-strided, then the tree)
-      float ss = 0.f;
-#pragma unroll
-      for (int s = 0; s < SL; ++s)
-        if (s * 128 + lane * 2 < n_ssq) ss += __uint_as_float(sv[s].x) + __uint_as_float(sv[s].z);
-      ss = wave_sum(ss);
-      rstd = 1.f / sqrtf(ss / (float)K + a.eps);
-    }
+    if constexpr (MODE == 2)  // 1 / rms of the row: the per-tile partials in a fixed order (lane-strided, then the tree)
+      rstd = 1.f / sqrtf(wave_sum(ss) / (float)K + a.eps);
     const __amdgpu_buffer_rsrc_t ro = make_rsrc(a.x_out, MODE == 2 ? (int64_t)K * 4 : 0);
 #pragma unroll
     for (int c = 0; c < XC; ++c)
@@ -198,7 +280,10 @@ __global__ __launch_bounds__(WAVES * 64) void w4_relay_kernel(RelayArgs a, const
         if (e < k1) *reinterpret_cast<u32x2*>(smem + e * 2) = o;
       }
   }
-  if (gave_up && lane == 0) __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (gave_up && lane == 0) {
+    __hip_atomic_store(a.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (a.status[4]) atomicOr(a.status + 5, 1 << MODE), atomicAdd(a.status + 6, 1);
+  }
 
   // ---- 3. the products: one accumulator per quad of groups, group u of the quad in operand rows 4u (row 0 = the
   // activation row, the others the zero row), so its products land in the lanes of row block u ---------------------
@@ -257,6 +342,8 @@ __global__ __launch_bounds__(WAVES * 64) void w4_relay_kernel(RelayArgs a, const
     for (int wv = 0; wv < WAVES; ++wv) v += red[(wv * NT + nt) * 16 + c];
     return v;
   };
+  if (a.hint_out && blockIdx.x == gridDim.x - 1 && tid < kHintCopies)
+    __hip_atomic_store(a.hint_out + tid * (kHintStride / 4), (int32_t)epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if constexpr (EPI == 0) {
     if (tid < NT * 16) {
       const int c = tid & 15, nt = tid >> 4;
@@ -270,8 +357,7 @@ __global__ __launch_bounds__(WAVES * 64) void w4_relay_kernel(RelayArgs a, const
       if (a.ssq_out) {  // sum of squares of the tile's 16 outputs: one row of 16 lanes
         const float qv = row16_sum(v * v);
         if (live && c == 0)
-          __hip_atomic_store(a.ssq_out + tile[nt], (uint64_t)__float_as_uint(qv) | ((uint64_t)epoch << 32), __ATOMIC_RELAXED,
-                             __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(a.ssq_out + tile[nt], tag_sum(qv, epoch), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
   } else {
@@ -289,7 +375,7 @@ __global__ __launch_bounds__(WAVES * 64) void w4_relay_kernel(RelayArgs a, const
 
 // out = resid + rmsnorm(x; norm_w) for one tagged row (the last block's pending update, olmo/model.py:814-821),
 // written as plain bf16 for the launches after the relay.  One workgroup.
-__global__ __launch_bounds__(256) void relay_final_kernel(const uint32_t* __restrict__ x, const uint64_t* __restrict__ ssq_in,
+__global__ __launch_bounds__(256) void relay_final_kernel(const uint32_t* __restrict__ x, const uint32_t* __restrict__ ssq_in,
                                                           const uint32_t* __restrict__ resid, const uint16_t* __restrict__ norm_w,
                                                           uint16_t* __restrict__ out, int K, float eps,
                                                           const int32_t* __restrict__ epoch_p, int32_t* status, int spin_limit) {
@@ -298,17 +384,15 @@ __global__ __launch_bounds__(256) void relay_final_kernel(const uint32_t* __rest
   const uint32_t epoch = (uint32_t)*epoch_p, tag16 = epoch & 0xffffu;
   const int n_ssq = K >> 4;
   const __amdgpu_buffer_rsrc_t rx = make_rsrc(x, (int64_t)K * 4), rr = make_rsrc(resid, (int64_t)K * 4),
-                               rq = make_rsrc(ssq_in, (int64_t)n_ssq * 8);
+                               rq = make_rsrc(ssq_in, (int64_t)n_ssq * 4);
   constexpr int C = 8;  // K <= 8192: 1024 elements per pass of the workgroup
-  u32x4 xv[C], rv[C], sv[2];
+  u32x4 xv[C], rv[C], sv;
   bool gave_up = false;
   for (int spins = 0;; ++spins) {
     bool ok = true;
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {  // 512 pairs at most: two per thread and request
-      sv[s] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rq, tid * 16, s * 4096, kSc1));
-      if (s * 512 + tid * 2 < n_ssq) ok = ok && sv[s].y == epoch && sv[s].w == epoch;
-    }
+    poll_fence();
+    sv = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rq, tid * 16, 0, kSc1));  // 512 sums at most: four per thread
+    if (tid * 4 < n_ssq) ok = ok && sums_ok(sv, epoch);
 #pragma unroll
     for (int c = 0; c < C; ++c)
       if (c * 1024 < K) {
@@ -323,11 +407,12 @@ __global__ __launch_bounds__(256) void relay_final_kernel(const uint32_t* __rest
     }
     __builtin_amdgcn_s_sleep(4);
   }
-  if (gave_up && tid == 0) __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (gave_up && tid == 0) {
+    __hip_atomic_store(status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (status[4]) atomicOr(status + 5, 16);
+  }
   float ss = 0.f;
-#pragma unroll
-  for (int s = 0; s < 2; ++s)
-    if (s * 512 + tid * 2 < n_ssq) ss += __uint_as_float(sv[s].x) + __uint_as_float(sv[s].z);
+  if (tid * 4 < n_ssq) ss = (sum_of(sv.x) + sum_of(sv.y)) + (sum_of(sv.z) + sum_of(sv.w));
   ss = wave_sum(ss);
   if (lane == 0) part[wave] = ss;
   __syncthreads();
@@ -386,7 +471,7 @@ inline bool relay_cfg(int N, int K, int swiglu, int cfg, RelayCfg* out) {
   return true;
 }
 
-inline size_t relay_lds(int K, const RelayCfg& c) { return (size_t)4 * K + (size_t)c.waves * c.nt * 16 * 4; }
+inline size_t relay_lds(int K, const RelayCfg& c) { return (size_t)4 * K + (size_t)c.waves * c.nt * 16 * 4 + 16; }  // + the hint flag
 
 template <typename F>
 int with_relay_kernel(const RelayCfg& c, int mode, int swiglu, F&& f) {
@@ -406,14 +491,14 @@ int with_relay_kernel(const RelayCfg& c, int mode, int swiglu, F&& f) {
   return O355_EUNSUPPORTED;
 }
 
-int relay_check(const void* x, int x_tagged, const uint64_t* ssq_in, const uint32_t* resid, const uint16_t* norm_w,
+int relay_check(const void* x, int x_tagged, const uint32_t* ssq_in, const uint32_t* resid, const uint16_t* norm_w,
                 const uint32_t* x_out, const void* wt, const void* st, const void* zt, const void* y, int N, int K,
                 int swiglu, const int32_t* epoch, const int32_t* status, int spin_limit, int* mode) {
   if (!x || !wt || !st || !zt || !y || !epoch || !status || N <= 0 || K <= 0 || spin_limit < 0) return O355_EINVAL;
   const bool norm = resid != nullptr;
   if (norm && (!ssq_in || !norm_w || !x_out || !x_tagged)) return O355_EINVAL;
   if (!norm && (ssq_in || norm_w || x_out)) return O355_EINVAL;
-  if ((K & 127) || (N & (swiglu ? 31 : 15)) || K > 6144 * (norm ? 1 : 4)) return O355_EUNSUPPORTED;
+  if ((K & 127) || (N & (swiglu ? 31 : 15)) || K > 8192 * (norm ? 1 : 3)) return O355_EUNSUPPORTED;
   if ((int64_t)(N >> 4) * (K >> 7) * 1024 >= (1ll << 31)) return O355_EUNSUPPORTED;
   if (swiglu && !norm) return O355_EUNSUPPORTED;
   *mode = norm ? 2 : (x_tagged ? 1 : 0);
@@ -422,17 +507,18 @@ int relay_check(const void* x, int x_tagged, const uint64_t* ssq_in, const uint3
 
 }  // namespace
 
-extern "C" int olmo355_w4_relay(const void* x, int x_tagged, const uint64_t* ssq_in, const uint32_t* resid,
+extern "C" int olmo355_w4_relay(const void* x, int x_tagged, const uint32_t* ssq_in, const uint32_t* resid,
                                 const uint16_t* norm_w, float eps, uint32_t* x_out, const uint32_t* wt, const uint16_t* st,
-                                const uint8_t* zt, void* y, int y_tagged, uint64_t* ssq_out, int N, int K, int swiglu,
-                                const int32_t* epoch, int32_t* status, int spin_limit, int cfg, void* stream) {
+                                const uint8_t* zt, void* y, int y_tagged, uint32_t* ssq_out, int N, int K, int swiglu,
+                                const int32_t* epoch, int32_t* status, const int32_t* hint_in, int32_t* hint_out,
+                                int spin_limit, int cfg, void* stream) {
   int mode = 0;
   const int chk = relay_check(x, x_tagged, ssq_in, resid, norm_w, x_out, wt, st, zt, y, N, K, swiglu, epoch, status, spin_limit, &mode);
   if (chk != O355_OK) return chk;
   if (swiglu && ssq_out) return O355_EUNSUPPORTED;
   RelayCfg c;
   if (!relay_cfg(N, K, swiglu, cfg, &c)) return O355_EUNSUPPORTED;
-  RelayArgs a{x, ssq_in, resid, norm_w, x_out, y, ssq_out, epoch, status, eps, N, K, x_tagged, y_tagged, spin_limit};
+  RelayArgs a{x, ssq_in, resid, norm_w, x_out, y, ssq_out, epoch, status, hint_in, hint_out, eps, N, K, x_tagged, y_tagged, spin_limit};
   const size_t lds = relay_lds(K, c);
   const int ntiles = N >> 4;
   const unsigned blocks = swiglu ? (unsigned)(ntiles >> 1) : (unsigned)((ntiles + c.nt - 1) / c.nt);
@@ -486,7 +572,18 @@ extern "C" int olmo355_relay_pair_ok(const int* a, const int* b, int n_cu, int l
   return n > 0 && (int64_t)b[0] < (int64_t)n * n_cu ? 1 : 0;
 }
 
-extern "C" int olmo355_relay_final(const uint32_t* x, const uint64_t* ssq_in, const uint32_t* resid, const uint16_t* norm_w,
+// out[0] = CUs of the current device, out[1] = bytes of LDS per CU: the chip side of olmo355_relay_pair_ok
+extern "C" int olmo355_relay_device(int* out) {
+  int dev = 0, cus = 0, lds = 0;
+  if (!out) return O355_EINVAL;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+      hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, dev) != hipSuccess || cus <= 0 || lds <= 0)
+    return O355_ELAUNCH;
+  out[0] = cus, out[1] = lds;
+  return O355_OK;
+}
+
+extern "C" int olmo355_relay_final(const uint32_t* x, const uint32_t* ssq_in, const uint32_t* resid, const uint16_t* norm_w,
                                    float eps, uint16_t* out, int K, const int32_t* epoch, int32_t* status, int spin_limit,
                                    void* stream) {
   if (!x || !ssq_in || !resid || !norm_w || !out || !epoch || !status || K <= 0 || spin_limit < 0) return O355_EINVAL;

@@ -156,6 +156,7 @@ def greedy_generate(model, input_ids: torch.Tensor, attention_mask: Optional[tor
             if len(pending) >= 64:
                 settle()
     settle()
+    model.relay_check()
     tokens = tokens[:, :steps]
     result = [tokens]
     after = None

@@ -193,6 +193,68 @@ class _Embedding(nn.Module):
         return ops.embedding(ids.contiguous(), self.weight.data)
 
 
+RELAY = False             # opt-in: the one-row decode step as a two-stream relay (measured: not faster than the chained step)
+RELAY_TWO_STREAMS = True  # ... or keep it on one stream inside a captured step
+RELAY_FENCE = ()           # tuning: launches fenced off from the other stream ("pre:attention", "post:ff_out", ...)
+
+
+class _RelayState:
+    """Buffers, epoch and launch plan of the one-row decode relay (``olmo_amd/csrc/relay.hip``): every tensor that
+    passes from one launch of a step to the next lives here, one per block and role, each written exactly once per
+    step -- which is what lets a launch on the second stream start before its producer has finished."""
+
+    # launch shapes tried per linear, in order of preference (0 = the kernel's own choice; waves | tiles << 8)
+    CANDIDATES = {"att_proj": (0, 8 | 2 << 8, 16 | 2 << 8), "attn_out": (0, 8 | 1 << 8), "ff_proj": (0, 16 | 2 << 8),
+                  "ff_out": (0, 8 | 1 << 8)}
+
+    def __init__(self, model: "OLMo"):
+        c, dev = model.config, model.device
+        d, dkv = c.d_model, c.effective_n_kv_heads * c.head_dim
+        width, h2 = d + 2 * dkv, c.act_out_size
+        i32 = lambda n: torch.zeros(n, dtype=torch.int32, device=dev)
+        self.epoch, self.status = i32(1), i32(8)  # status: [0] a wait gave up; [1..3] wait statistics when [4] is set
+        self.x0 = i32(d)  # the token's embedding, tagged: the first residual row
+        self.layers = [dict(qkv=i32(width), ssq_qkv=i32(width // 16), att=i32(d), a=i32(d), ssq_a=i32(d // 16), x1=i32(d),
+                            u=i32(h2), x2=i32(d), f=i32(d), ssq_f=i32(d // 16)) for _ in range(c.n_layers)]
+        # per launch: 64 copies, 1 KiB apart, of a word set to the epoch when the launch's last workgroup is done
+        self.hints = torch.zeros(c.n_layers * 5, 64 * 256, dtype=torch.int32, device=dev)
+        self.side = torch.cuda.Stream(device=dev)
+        self.shapes = {"att_proj": (width, d, True, False), "attn_out": (d, d, False, False),
+                       "ff_proj": (c.hidden_size, d, True, True), "ff_out": (d, h2, False, False)}  # N, K, norm, swiglu
+        self.cfg = {k: 0 for k in self.shapes}
+        self.plans: Dict[int, Optional[Dict[str, int]]] = {}
+        self.attn_ok: Dict[int, bool] = {}
+        self.covered = all(ops.relay_footprint_w4(n, k, nm, sw) is not None for n, k, nm, sw in self.shapes.values()) \
+            and c.head_dim in (64, 128) and d <= 8192 and dkv <= 8192
+
+    def plan(self, model: "OLMo", n_keys_max: int) -> Optional[Dict[str, int]]:
+        """Launch shapes under which every pair of consecutive launches of a step fits the chip side by side (the
+        condition for running them on two streams), or ``None`` when there is no such choice."""
+        if n_keys_max in self.plans:
+            return self.plans[n_keys_max]
+        import itertools
+
+        c = model.config
+        n_cu, lds = ops.relay_device()
+        att = ops.relay_footprint_attn(c.n_heads, c.head_dim, n_keys_max)
+        found = None
+        if att is not None:
+            names = ("att_proj", "attn_out", "ff_proj", "ff_out")
+            for combo in itertools.product(*(self.CANDIDATES[n] for n in names)):
+                fp = {}
+                for n, cf in zip(names, combo):
+                    N, K, nm, sw = self.shapes[n]
+                    fp[n] = ops.relay_footprint_w4(N, K, nm, sw, cf)
+                if any(v is None for v in fp.values()):
+                    continue
+                order = [fp["att_proj"], att, fp["attn_out"], fp["ff_proj"], fp["ff_out"]]
+                if all(ops.relay_pair_ok(order[i], order[(i + 1) % 5], n_cu, lds) for i in range(5)):
+                    found = dict(zip(names, combo))
+                    break
+        self.plans[n_keys_max] = found
+        return found
+
+
 class OLMo(nn.Module):
     def __init__(self, config: ModelConfig, device="cuda", dtype: torch.dtype = torch.bfloat16,
                  max_cache_len: Optional[int] = None, block_weight_device=None):
@@ -265,6 +327,7 @@ class OLMo(nn.Module):
         # not used for such models
         self._act_order = any(isinstance(m, QuantLinear) and (m._perm is not None or m._has_bias) for m in self.modules())
         self._chain_ok = {}  # rows -> whether the chained decode block covers this model
+        self._relay: Optional[_RelayState] = None  # state of the one-row decode relay, made on first use
         self._rope_now = None  # rotary rows of the current position during a captured decode step
         self._beam = None  # the beam cache while a beam-search step runs
         self._prepared = True
@@ -438,6 +501,110 @@ class OLMo(nn.Module):
         f, _, ssq_f = ops.w4_linear_chain(u, blk.ff_out.tiled, want_ssq=True)
         return x, (f, blk.ff_norm.weight.data, ssq_f)
 
+    # The one-row decode step as a relay (olmo_amd/csrc/relay.hip): the chained block above with every hand-over
+    # between launches carried by epoch tags in the data.  On one stream this is the same arithmetic launch for launch;
+    # inside a captured step the launches alternate between two streams, so that each one requests its weights while
+    # its predecessor still computes.  Returns the residual row after the last block (bf16 [1, 1, d]).
+    def _relay_blocks(self, x, cache: KVCache, past_len: int, key_bias, graph_pos, n_keys_max: int) -> torch.Tensor:
+        c, rs = self.config, self._relay
+        eps = c.layer_norm_eps
+        H, Hkv, hd = c.n_heads, c.effective_n_kv_heads, c.head_dim
+        sin, cos = self._rope
+        ws = self._decode_ws(1, n_keys_max)
+        main = torch.cuda.current_stream()
+        # two streams only inside a captured step (eager launches are bound by the host anyway), with the plan made
+        # beforehand (planning queries kernel attributes, which has no place inside a capture)
+        plan = rs.plans.get(n_keys_max) if (RELAY_TWO_STREAMS and torch.cuda.is_current_stream_capturing()) else None
+        cfg = plan if plan is not None else rs.cfg
+        ops.incr_i32(rs.epoch)
+        ops.relay_tag(x.view(-1), rs.x0, rs.epoch)
+        if plan is not None:
+            rs.side.wait_stream(main)
+            lanes = (main.cuda_stream, rs.side.cuda_stream)
+        else:
+            lanes = (main.cuda_stream, main.cuda_stream)
+        n = 0  # launches so far: launch n goes to stream n % 2
+        streams = (main, rs.side)
+
+        def fence(which):  # tuning knob: keep the named launch apart from its neighbours on the other stream
+            if plan is not None and which in RELAY_FENCE:
+                streams[0].wait_stream(streams[1])
+                streams[1].wait_stream(streams[0])
+
+        # hint words only where a launch may run beside its producer: without one a launch asks for its rows at once
+        hint = lambda i: dict(hint_in=rs.hints[i - 1] if (i > 0 and plan is not None) else None, hint_out=rs.hints[i] if plan is not None else None)
+        resid, pend = rs.x0, None
+        rope_now = self._rope_now if graph_pos is not None else None
+        for blk, L in zip(self.transformer["blocks"], rs.layers):
+            qknorm = blk.q_norm is not None
+            ssq_qkv = L["ssq_qkv"] if qknorm else None
+            fence("pre:att_proj")
+            if pend is None:
+                ok = ops.w4_relay(rs.x0, blk.att_proj.tiled, L["qkv"], rs.epoch, rs.status, ssq_out=ssq_qkv,
+                                  cfg=cfg["att_proj"], stream=lanes[n % 2], **hint(n))
+            else:
+                ok = ops.w4_relay(pend[0], blk.att_proj.tiled, L["qkv"], rs.epoch, rs.status, resid=resid, norm_w=pend[1],
+                                  eps=eps, ssq_in=pend[2], x_out=L["x1"], ssq_out=ssq_qkv, cfg=cfg["att_proj"],
+                                  stream=lanes[n % 2], **hint(n))
+                resid = L["x1"]
+            n += 1
+            fence("post:att_proj"), fence("pre:attention")
+            ok = ok and ops.attn_decode_relay(L["qkv"], blk.q_norm.weight.data if qknorm else None,
+                                              blk.k_norm.weight.data if qknorm else None, sin, cos, cache.k[blk.layer_id],
+                                              cache.v[blk.layer_id], ws, L["att"], H, Hkv, hd, past_len, n_keys_max, eps,
+                                              rs.epoch, rs.status, key_bias=key_bias, past_len_dev=graph_pos, qk_ssq=ssq_qkv,
+                                              rope_now=rope_now, stream=lanes[n % 2], **hint(n))
+            n += 1
+            fence("post:attention"), fence("pre:attn_out")
+            ok = ok and ops.w4_relay(L["att"], blk.attn_out.tiled, L["a"], rs.epoch, rs.status, ssq_out=L["ssq_a"],
+                                     cfg=cfg["attn_out"], stream=lanes[n % 2], **hint(n))
+            n += 1
+            fence("post:attn_out"), fence("pre:ff_proj")
+            ok = ok and ops.w4_relay(L["a"], blk.ff_proj.tiled, L["u"], rs.epoch, rs.status, resid=resid,
+                                     norm_w=blk.attn_norm.weight.data, eps=eps, ssq_in=L["ssq_a"], x_out=L["x2"], swiglu=True,
+                                     cfg=cfg["ff_proj"], stream=lanes[n % 2], **hint(n))
+            resid = L["x2"]
+            n += 1
+            fence("post:ff_proj"), fence("pre:ff_out")
+            ok = ok and ops.w4_relay(L["u"], blk.ff_out.tiled, L["f"], rs.epoch, rs.status, ssq_out=L["ssq_f"],
+                                     cfg=cfg["ff_out"], stream=lanes[n % 2], **hint(n))
+            n += 1
+            fence("post:ff_out")
+            if not ok:
+                raise RuntimeError("the decode relay declined a launch it had accepted when it was planned")
+            pend = (L["f"], blk.ff_norm.weight.data, L["ssq_f"])
+        if plan is not None:
+            main.wait_stream(rs.side)
+        out = torch.empty(1, 1, c.d_model, dtype=torch.bfloat16, device=self.device)
+        ops.relay_final(pend[0], pend[2], resid, pend[1], eps, out.view(-1), rs.epoch, rs.status)
+        return out
+
+    def _relay_decode_ok(self, B: int, key_bias, n_keys_max: int) -> bool:
+        """Whether the relay covers this step: one row, the chained block's conditions, every launch shape covered
+        (decided once per model) and an attention launch whose chunks merge inside the kernel."""
+        if not RELAY or B != 1:
+            return False
+        if self._relay is None:
+            if torch.cuda.is_current_stream_capturing():
+                return False  # not decided yet: its buffers are not made inside a capture
+            self._relay = _RelayState(self)
+        rs = self._relay
+        if n_keys_max not in rs.attn_ok:
+            if torch.cuda.is_current_stream_capturing():
+                return False
+            c = self.config
+            rs.attn_ok[n_keys_max] = ops.relay_footprint_attn(c.n_heads, c.head_dim, n_keys_max) is not None
+            rs.plan(self, n_keys_max)
+        return rs.covered and rs.attn_ok[n_keys_max]
+
+    def relay_check(self) -> None:
+        """Raises if a launch of the decode relay gave up waiting for its input since the last call (a host
+        synchronisation; the results of that step are undefined)."""
+        if self._relay is not None and int(self._relay.status[0].item()) != 0:
+            words = self._relay.status.tolist()
+            self._relay.status.zero_()
+            raise RuntimeError(f"a launch of the decode relay gave up waiting for its producer (status words {words})")
+
     def _chain_decode_ok(self, M: int) -> bool:
         """Whether :meth:`_block_decode_chain` covers this model at ``M`` rows: decided once per ``M`` by
         issuing block 0's four linears in chained form on scratch inputs (outside any graph capture)."""
@@ -576,7 +743,12 @@ class OLMo(nn.Module):
         fused = T == 1 and cache is not None and self._beam is None and self._fused_decode_ok(B, collect_hidden)
         chain = fused and self._chain_decode_ok(B)
         pend = None
-        for i, blk in enumerate(self.transformer["blocks"]):
+        if chain and self._relay_decode_ok(B, key_bias, n_keys_max):
+            x = self._relay_blocks(x, cache, past_len, key_bias, graph_pos, n_keys_max)
+            blocks = ()
+        else:
+            blocks = self.transformer["blocks"]
+        for i, blk in enumerate(blocks):
             if collect_hidden:
                 hidden.append(x)
             if cache is not None:

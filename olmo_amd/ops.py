@@ -379,7 +379,11 @@ def w4_chain(steps, sync: torch.Tensor, status: torch.Tensor, spin_limit: int = 
 # ---------------------------------------------------------------------------------------------
 # the decode relay (one row): launches on two streams, the hand-over carried by epoch tags in the data
 # ---------------------------------------------------------------------------------------------
-RELAY_SPIN_LIMIT = 1 << 20  # polls of a waiting wave before it gives up and sets the status word (about a second)
+RELAY_SPIN_LIMIT = 1 << 16  # polls of a waiting wave before it gives up and sets the status word (a tenth of a second)
+
+
+def _spins(spin_limit: Optional[int]) -> int:
+    return int(RELAY_SPIN_LIMIT if spin_limit is None else spin_limit)
 
 
 def relay_untag(t: torch.Tensor) -> torch.Tensor:
@@ -405,10 +409,11 @@ def w4_relay(x: torch.Tensor, w: "W4Tiled", y: torch.Tensor, epoch: torch.Tensor
              resid: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None, eps: float = 0.0,
              ssq_in: Optional[torch.Tensor] = None, x_out: Optional[torch.Tensor] = None,
              ssq_out: Optional[torch.Tensor] = None, swiglu: bool = False, cfg: int = 0,
-             spin_limit: int = RELAY_SPIN_LIMIT, stream: Optional[int] = None) -> bool:
+             hint_in: Optional[torch.Tensor] = None, hint_out: Optional[torch.Tensor] = None,
+             spin_limit: Optional[int] = None, stream: Optional[int] = None) -> bool:
     """One int4 linear of the decode relay at one row; every buffer is the caller's (nothing is allocated).
     ``x``: int32 tagged words or bf16; ``y``: int32 (tagged) or bf16, ``N`` (``N/2`` with ``swiglu``) numbers;
-    ``ssq_in`` / ``ssq_out``: int64 pairs per 16-column tile; ``resid`` / ``x_out``: tagged rows; with ``resid`` the
+    ``ssq_in`` / ``ssq_out``: int32 tagged sums per 16-column tile; ``resid`` / ``x_out``: tagged rows; with ``resid`` the
     activations are ``resid + rmsnorm(x; norm_w, eps)`` and also go to ``x_out``.  Returns ``False`` when the kernel
     does not cover the shape (nothing launched)."""
     _dev(x, y, epoch, status, resid, norm_w, ssq_in, x_out, ssq_out, w.wt)
@@ -417,14 +422,14 @@ def w4_relay(x: torch.Tensor, w: "W4Tiled", y: torch.Tensor, epoch: torch.Tensor
     if y.numel() != (w.N // 2 if swiglu else w.N):
         raise ValueError("w4_relay: output size mismatch")
     for t, n, dt in ((resid, w.K, torch.int32), (x_out, w.K, torch.int32), (norm_w, w.K, torch.bfloat16),
-                     (ssq_in, w.K // 16, torch.int64), (ssq_out, w.N // 16, torch.int64)):
+                     (ssq_in, w.K // 16, torch.int32), (ssq_out, w.N // 16, torch.int32)):
         if t is not None and (t.numel() != n or t.dtype != dt):
             raise ValueError("w4_relay: a side buffer has the wrong size or dtype")
-    if epoch.dtype != torch.int32 or status.dtype != torch.int32:
-        raise TypeError("w4_relay: int32 epoch and status words")
+    if epoch.dtype != torch.int32 or status.dtype != torch.int32 or status.numel() < 8:
+        raise TypeError("w4_relay: an int32 epoch word and 8 int32 status words")
     st = lib().olmo355_w4_relay(_p(x), int(x.dtype == torch.int32), _p(ssq_in), _p(resid), _p(norm_w), float(eps), _p(x_out),
                                 _p(w.wt), _p(w.st), _p(w.zt), _p(y), int(y.dtype == torch.int32), _p(ssq_out), w.N, w.K,
-                                int(swiglu), _p(epoch), _p(status), int(spin_limit), int(cfg),
+                                int(swiglu), _p(epoch), _p(status), _p(hint_in), _p(hint_out), _spins(spin_limit), int(cfg),
                                 _stream() if stream is None else stream)
     if st == 2:
         return False
@@ -433,17 +438,17 @@ def w4_relay(x: torch.Tensor, w: "W4Tiled", y: torch.Tensor, epoch: torch.Tensor
 
 
 def relay_final(x: torch.Tensor, ssq_in: torch.Tensor, resid: torch.Tensor, norm_w: torch.Tensor, eps: float,
-                out: torch.Tensor, epoch: torch.Tensor, status: torch.Tensor, spin_limit: int = RELAY_SPIN_LIMIT) -> torch.Tensor:
+                out: torch.Tensor, epoch: torch.Tensor, status: torch.Tensor, spin_limit: Optional[int] = None) -> torch.Tensor:
     """``out = resid + rmsnorm(x; norm_w, eps)`` from tagged rows into a plain bf16 row (the relay's last update)."""
     _dev(x, ssq_in, resid, norm_w, out, epoch, status)
     K = x.numel()
-    if (x.dtype != torch.int32 or resid.dtype != torch.int32 or resid.numel() != K or ssq_in.dtype != torch.int64
+    if (x.dtype != torch.int32 or resid.dtype != torch.int32 or resid.numel() != K or ssq_in.dtype != torch.int32
             or ssq_in.numel() != K // 16 or norm_w.dtype != torch.bfloat16 or norm_w.numel() != K
             or out.dtype != torch.bfloat16 or out.numel() != K):
-        raise ValueError("relay_final: tagged rows, int64 pairs, bf16 weight and output of one width expected")
+        raise ValueError("relay_final: tagged rows, int32 tagged sums, bf16 weight and output of one width expected")
     check("olmo355_relay_final",
           lib().olmo355_relay_final(_p(x), _p(ssq_in), _p(resid), _p(norm_w), float(eps), _p(out), K, _p(epoch), _p(status),
-                                    int(spin_limit), _stream()))
+                                    _spins(spin_limit), _stream()))
     return out
 
 
@@ -451,15 +456,16 @@ def attn_decode_relay(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache,
                       past_len: int, n_keys_max: int, eps: float, epoch: torch.Tensor, status: torch.Tensor,
                       key_bias: Optional[torch.Tensor] = None, past_len_dev: Optional[torch.Tensor] = None,
                       qk_ssq: Optional[torch.Tensor] = None, rope_now: Optional[torch.Tensor] = None,
-                      spin_limit: int = RELAY_SPIN_LIMIT, stream: Optional[int] = None) -> bool:
-    """:func:`attn_decode_fused` for one sequence as a leg of the relay: ``qkv`` tagged words, ``qk_ssq`` int64 pairs,
+                      hint_in: Optional[torch.Tensor] = None, hint_out: Optional[torch.Tensor] = None,
+                      spin_limit: Optional[int] = None, stream: Optional[int] = None) -> bool:
+    """:func:`attn_decode_fused` for one sequence as a leg of the relay: ``qkv`` tagged words, ``qk_ssq`` int32 tagged sums,
     ``out`` tagged words ``[H * hd]``.  Returns ``False`` when the relay form does not cover the shape."""
     _dev(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache, ws, out, key_bias, past_len_dev, qk_ssq, rope_now, epoch, status)
     width = (H + 2 * Hkv) * hd
     if qkv.dtype != torch.int32 or qkv.numel() != width or out.dtype != torch.int32 or out.numel() != H * hd:
         raise ValueError("attn_decode_relay: tagged qkv of one token and a tagged output row expected")
-    if qk_ssq is not None and (qk_ssq.dtype != torch.int64 or qk_ssq.numel() != width // 16):
-        raise ValueError("attn_decode_relay: qk_ssq int64 [(H + 2 Hkv) hd / 16] expected")
+    if qk_ssq is not None and (qk_ssq.dtype != torch.int32 or qk_ssq.numel() != width // 16):
+        raise ValueError("attn_decode_relay: qk_ssq int32 [(H + 2 Hkv) hd / 16] expected")
     if kcache.dtype != torch.bfloat16 or kcache.shape != vcache.shape or kcache.shape[1] != Hkv or kcache.shape[3] != hd:
         raise ValueError("attn_decode_relay: bf16 caches [B, Hkv, Lmax, hd] expected")
     if rope_now is not None and (rope_now.dtype != torch.float32 or rope_now.numel() != 2 * hd):
@@ -470,7 +476,7 @@ def attn_decode_relay(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache,
     st = lib().olmo355_attn_decode_relay(_p(qkv), _p(q_weight), _p(k_weight), _p(sin_tab), _p(cos_tab), _p(kcache), _p(vcache),
                                          _p(key_bias), _p(out), _p(ws), 1, H, Hkv, hd, Lmax, n_pos, past_len, _p(past_len_dev),
                                          n_keys_max, key_bias.shape[1] if key_bias is not None else 0, float(eps), _p(qk_ssq),
-                                         _p(rope_now), _p(epoch), _p(status), int(spin_limit),
+                                         _p(rope_now), _p(epoch), _p(status), _p(hint_in), _p(hint_out), _spins(spin_limit),
                                          _stream() if stream is None else stream)
     if st == 2:
         return False
@@ -494,6 +500,15 @@ def relay_footprint_attn(H: int, hd: int, n_keys_max: int):
     out = (ctypes.c_int * 4)()
     st = lib().olmo355_attn_decode_relay_footprint(1, H, hd, n_keys_max, out)
     return tuple(out) if st == 0 else None
+
+
+def relay_device():
+    """(CUs, bytes of LDS per CU) of the current device."""
+    import ctypes
+
+    out = (ctypes.c_int * 2)()
+    check("olmo355_relay_device", lib().olmo355_relay_device(out))
+    return int(out[0]), int(out[1])
 
 
 def relay_pair_ok(older, younger, n_cu: int, lds_per_cu: int) -> bool:
