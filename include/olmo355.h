@@ -99,64 +99,6 @@ int olmo355_w4_gemv_chain(const uint16_t* x, const uint16_t* resid, const uint16
                           const float* ssq_in, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
                           float* ssq_out, int M, int N, int K, int swiglu, void* stream);
 
-/* ---- the batch-1 decode step as a relay on two streams ---------------------------------------------------------
- * The launches of a decode step -- att_proj, attention, attn_out, ff_proj, ff_out of every block, i.e. the calls
- * OLMoSequentialBlock.forward makes one after the other (olmo/model.py:746-823), each linear a QuantLinear.forward
- * (AGQ/auto_gptq/nn_modules/qlinear/qlinear_cuda_old.py:192-290) -- form a chain in which every launch needs the whole
- * output of the one before but none of its weights depend on it.  In the relay form launch n+1 may run on a second
- * stream while launch n is still at work: it requests all of its weights (cache rows) first and then waits for its
- * input rows, which carry the hand-over themselves:
- *   tagged row   uint32 per element: bf16 bits << 16 | (epoch & 0xffff)
- *   tagged sums  uint32 per 16-column tile: the tile's sum of squares as a float rounded to 20 mantissa bits,
- *                the low 4 bits = epoch & 0xf
- * `epoch` is a device word that the caller changes before every step (olmo355_incr_i32); every tagged buffer is
- * written exactly once per step, by one launch, and must not be reused for anything else while the step runs.  A
- * consumer polls its inputs with device-coherent loads until every tag equals the epoch, at most `spin_limit` times;
- * then it sets status[0] = 1, uses what it has and ends (results undefined, nothing hangs; `status` is 8 words:
- * with status[4] set by the host, the int4 linears also leave the longest waits of a run in status[1..3]).  On one stream the same
- * calls simply never wait.  hint_out / hint_in (optional, O355_RELAY_HINT_COPIES words O355_RELAY_HINT_STRIDE bytes apart per launch,
- * handed from a launch to its consumer): the producer's last workgroup stores the epoch there when it is done, and a consumer that found its rows
- * unfinished watches that one word before it asks for the rows again -- polling whole rows from every workgroup
- * would cost more traffic than the weights.  A hint only: the tags decide.
- *
- * Two launches of the relay that are in flight together (consecutive ones on the two streams) must fit the chip side
- * by side: olmo355_relay_pair_ok(older, younger, n_cu, lds_per_cu) says whether the younger one, all of its
- * workgroups waiting, can never keep a workgroup of the older one from starting; footprints (workgroups, waves per
- * workgroup, vector registers per lane, LDS bytes per workgroup) come from the *_footprint calls.  Use the second
- * stream only when every consecutive pair passes; never more than two streams.
- *
- * olmo355_w4_relay: y = x' . W at ONE row.  x: tagged row (x_tagged) or bf16 [K].  resid != NULL: x' = resid +
- * rmsnorm(x; norm_w, eps) with the mean square from ssq_in (tagged sums [K/16]), x' also written to x_out (tagged; resid
- * and x_out tagged rows; needs x_tagged, K <= 8192); else x' = x and ssq_in, norm_w, x_out are NULL.  y: tagged (y_tagged)
- * or bf16, [N], or [N/2] = silu(gate) * up with swiglu (olmo/model.py:365-368; needs resid); ssq_out: NULL or tagged sums
- * [N/16] (not with swiglu).  cfg: 0 = choose the launch shape, else waves per workgroup (4, 8, 16) | column tiles
- * per workgroup (1, 2) << 8.  O355_EUNSUPPORTED when a wave's share of K exceeds its registers (K / 128 / waves > 12). */
-#define O355_RELAY_HINT_COPIES 64
-#define O355_RELAY_HINT_STRIDE 1024 /* bytes between the copies: a hint buffer is 64 KiB */
-int olmo355_w4_relay(const void* x, int x_tagged, const uint32_t* ssq_in, const uint32_t* resid, const uint16_t* norm_w,
-                     float eps, uint32_t* x_out, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, void* y,
-                     int y_tagged, uint32_t* ssq_out, int N, int K, int swiglu, const int32_t* epoch, int32_t* status,
-                     const int32_t* hint_in, int32_t* hint_out, int spin_limit, int cfg, void* stream);
-int olmo355_w4_relay_footprint(int N, int K, int norm, int x_tagged, int swiglu, int cfg, int* out4);
-int olmo355_relay_pair_ok(const int* older4, const int* younger4, int n_cu, int lds_per_cu);
-int olmo355_relay_device(int* out2); /* CUs of the current device, bytes of LDS per CU */
-/* olmo355_attn_decode_fused as a leg of the relay: qkv tagged [B, (H + 2 Hkv) hd], qk_ssq tagged sums (required with
- * QK-norm), out tagged [B, H hd]; the cache rows are requested before the wait.  Only launches whose chunks are
- * merged inside the kernel (B * H * chunks <= 1536), H hd <= 8192. */
-int olmo355_attn_decode_relay(const uint32_t* qkv, const void* qw, const void* kw, const float* sin_tab,
-                              const float* cos_tab, void* kcache, void* vcache, const float* key_bias, uint32_t* out,
-                              void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos, int past_len,
-                              const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps,
-                              const uint32_t* qk_ssq, const float* rope_now, const int32_t* epoch, int32_t* status,
-                              const int32_t* hint_in, int32_t* hint_out, int spin_limit, void* stream);
-int olmo355_attn_decode_relay_footprint(int B, int H, int hd, int n_keys_max, int* out4);
-/* out (bf16 [K]) = resid + rmsnorm(x; norm_w, eps) from tagged rows and tagged sums: the last block's pending update
- * (olmo/model.py:814-821) handed to the launches after the relay.  olmo355_relay_tag: bf16 -> tagged row (the
- * step's first residual row, the token's embedding). */
-int olmo355_relay_final(const uint32_t* x, const uint32_t* ssq_in, const uint32_t* resid, const uint16_t* norm_w, float eps,
-                        uint16_t* out, int K, const int32_t* epoch, int32_t* status, int spin_limit, void* stream);
-int olmo355_relay_tag(const uint16_t* x, uint32_t* out, int n, const int32_t* epoch, void* stream);
-
 /* Large-M path: dequantise tiles into LDS as bf16 and multiply on the matrix cores.  Stands
  * in for the reference's dequantise-then-matmul branch (AGQ qlinear_cuda_old.py:236-287) and
  * exllama's reconstruct + cublasHgemm (exllama/cuda_func/q4_matmul.cu:222-260).
@@ -209,43 +151,6 @@ int olmo355_w4_gemm_swiglu(const uint16_t* x, const uint32_t* wt, const uint16_t
  * (lane l: row n = 16*nt + (l&15), columns 32*ks + 8*(l>>4) .. +7); K % 32 == 0, N % 16 == 0.
  * fp32: weight in torch layout [N,K]. */
 int olmo355_b16_repack(const uint16_t* w_nk, uint16_t* wt, int N, int K, void* stream);
-/* Up to four decode-step int4 linears (at most 4 rows) in ONE launch: phase p computes y_p = x_p . W_p where x_p
- * is phase p-1's output, directly or as resid + rmsnorm(y_{p-1}) -- e.g. attn_out -> ff_proj (+ SwiGLU) -> ff_out ->
- * the next block's att_proj, the calls OLMoSequentialBlock.forward makes one after the other (olmo/model.py:786-821,
- * then :746-757 of the following block), each a QuantLinear.forward (AGQ/auto_gptq/nn_modules/qlinear/
- * qlinear_cuda_old.py:192-290).  A persistent grid of olmo355_w4_chain_grid() workgroups (one per CU) with a
- * grid-wide barrier between phases; the weight requests of phase p+1 go out before the wait for phase p.
- * Per phase (all device pointers; argument meaning as olmo355_w4_gemv_chain):
- *   x [M,K]; resid / norm_w / ssq_in / x_out all NULL, or all given: then the phase multiplies
- *   x_out = resid + rmsnorm(x; norm_w, eps) with the mean square from ssq_in [M][K/16];
- *   y [M,N], or [M,N/2] with swiglu; ssq_out NULL or [M][N/16] (not with swiglu);
- *   rot in [0, grid): workgroup b owns the column tiles (b + rot) mod grid, + grid, ... (vary it between phases and
- *   layers so that the workgroups with one tile more are not always the same).
- * sync: olmo355_w4_chain_sync_ints() int32 (an epoch counter, then one arrival flag per workgroup), zeroed once
- * when allocated and then owned by the launches that use it, one at a time: every launch leaves it ready for the
- * next.  status: one int32, set to 1 if a barrier wait gave up after spin_limit polls (the results are then
- * undefined; the launch still ends and sync stays usable).
- * Needs every workgroup resident: nothing else may occupy the device's CUs while it runs. */
-#define O355_CHAIN_MAX_PHASES 4
-typedef struct {
-  const uint16_t* x;
-  const uint16_t* resid;
-  const uint16_t* norm_w;
-  const float* ssq_in;
-  uint16_t* x_out;
-  const uint32_t* wt;
-  const uint16_t* st;
-  const uint8_t* zt;
-  uint16_t* y;
-  float* ssq_out;
-  int N, K, swiglu, rot;
-  float eps;
-} olmo355_chain_phase;
-int olmo355_w4_chain_grid(void);
-int olmo355_w4_chain_sync_ints(void);
-int olmo355_w4_chain(const olmo355_chain_phase* phases, int n_phases, int M, int32_t* sync, int32_t* status,
-                     int spin_limit, void* stream);
-
 /* small-M (<= 64) path */
 int olmo355_b16_gemv(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, void* stream);
 int olmo355_b16_gemv_fused(const uint16_t* x, const uint16_t* resid, const uint16_t* norm_w, float eps,
@@ -402,21 +307,7 @@ int olmo355_sample(const void* logits, int rows, int n, float temperature, int t
 /* *p += 1 for a device int32 (advances the position between captured decode steps). */
 int olmo355_incr_i32(int32_t* p, void* stream);
 
-/* ---- measuring probes (no counterpart in the reference; used by bench.py only) -------------------
- * What a kernel that only streams `bytes` from HBM takes (16-byte non-temporal loads per lane, launch shaped
- * like the small-M linears; nothing is written), and what the matrix cores sustain on random bf16 operands
- * (256 workgroups x 8 waves x iters x 16 v_mfma_f32_16x16x32_bf16, the prefill GEMM's instruction; *flops = total
- * floating-point operations).
- * `sink` is a device buffer of at least 2 KiB that stays unwritten. */
-int olmo355_probe_stream_read(const void* src, int64_t bytes, void* sink, void* stream);
-/* The same over n buffers (host arrays of device pointers and byte counts, n <= 160) in ONE launch of a persistent
- * grid of two workgroups per CU: no launch boundary and no ramp per buffer. */
-int olmo355_probe_stream_read_many(const void* const* srcs, const int64_t* bytes, int n, void* sink, void* stream);
-int olmo355_probe_mfma_bf16(int iters, void* sink, double* flops, void* stream);
-/* For tests: leaves `pattern` in every 32-bit word of the LDS of every CU (LDS keeps what the last workgroup left
- * there, so a kernel that reads LDS it has not written gives results that depend on what ran before it; with a NaN
- * pattern in place such a read shows in the output). */
-int olmo355_probe_fill_lds(uint32_t pattern, void* sink, void* stream);
+
 
 #ifdef __cplusplus
 }

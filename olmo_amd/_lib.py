@@ -14,7 +14,7 @@ from typing import Optional
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "lib", "libolmo355.so")
 
-__all__ = ["lib", "LIB_PATH", "Olmo355Unavailable", "Olmo355Error", "check", "EXPORTS", "ChainPhase"]
+__all__ = ["lib", "LIB_PATH", "Olmo355Unavailable", "Olmo355Error", "check", "EXPORTS"]
 
 
 class Olmo355Unavailable(RuntimeError):
@@ -30,13 +30,6 @@ class Olmo355Error(RuntimeError):
 P, I, L, F = c_void_p, c_int, c_int64, c_float
 
 
-class ChainPhase(ctypes.Structure):
-    """``olmo355_chain_phase`` of include/olmo355.h."""
-
-    _fields_ = [(n, c_void_p) for n in ("x", "resid", "norm_w", "ssq_in", "x_out", "wt", "st", "zt", "y", "ssq_out")] + \
-               [(n, c_int) for n in ("N", "K", "swiglu", "rot")] + [("eps", c_float)]
-
-
 # name -> (restype, argtypes); must list every symbol include/olmo355.h declares
 EXPORTS = {
     "olmo355_version": (I, []),
@@ -47,17 +40,6 @@ EXPORTS = {
     "olmo355_w4_gemv": (I, [P, P, P, P, P, I, I, I, P]),
     "olmo355_w4_gemv_fused": (I, [P, P, P, F, P, P, P, P, P, I, I, I, I, P]),
     "olmo355_w4_gemv_chain": (I, [P, P, P, F, P, P, P, P, P, P, P, I, I, I, I, P]),
-    "olmo355_w4_chain_grid": (I, []),
-    "olmo355_w4_chain_sync_ints": (I, []),
-    "olmo355_w4_chain": (I, [ctypes.POINTER(ChainPhase), I, I, P, P, I, P]),
-    "olmo355_w4_relay": (I, [P, I, P, P, P, F, P, P, P, P, P, I, P, I, I, I, P, P, P, P, I, I, P]),
-    "olmo355_w4_relay_footprint": (I, [I, I, I, I, I, I, P]),
-    "olmo355_relay_pair_ok": (I, [P, P, I, I]),
-    "olmo355_relay_device": (I, [P]),
-    "olmo355_relay_final": (I, [P, P, P, P, F, P, I, P, P, I, P]),
-    "olmo355_relay_tag": (I, [P, P, I, P, P]),
-    "olmo355_attn_decode_relay": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, P, P, P, P, P, I, P]),
-    "olmo355_attn_decode_relay_footprint": (I, [I, I, I, I, P]),
     "olmo355_b16_gemv_fused": (I, [P, P, P, F, P, P, P, I, I, I, I, P]),
     "olmo355_w4_gemm": (I, [P, P, P, P, P, I, I, I, P]),
     "olmo355_w4_gemm_swiglu": (I, [P, P, P, P, P, I, I, I, P]),
@@ -93,10 +75,6 @@ EXPORTS = {
     "olmo355_gather_columns": (I, [P, P, P, I, I, P]),
     "olmo355_clamp": (I, [P, L, F, I, P]),
     "olmo355_sample": (I, [P, I, I, F, I, F, c_uint64, P, I, P, P, I, P]),
-    "olmo355_probe_stream_read": (I, [P, L, P, P]),
-    "olmo355_probe_stream_read_many": (I, [P, P, I, P, P]),
-    "olmo355_probe_mfma_bf16": (I, [I, P, P, P]),
-    "olmo355_probe_fill_lds": (I, [ctypes.c_uint32, P, P]),
     "olmo355_add": (I, [P, P, P, L, I, P]),
     "olmo355_add_bias_bf16": (I, [P, P, P, I, I, P]),
     "olmo355_argmax": (I, [P, P, I, I, I, P]),
@@ -105,11 +83,22 @@ EXPORTS = {
 
 # variant entry points of include/olmo355_debug.h (the dispatcher's choice as an explicit argument; tests and tuning)
 VARIANT_EXPORTS = {
+    "olmo355_w4_relay": (I, [P, I, P, P, P, F, P, P, P, P, P, I, P, I, I, I, P, P, P, P, I, I, P]),
+    "olmo355_w4_relay_footprint": (I, [I, I, I, I, I, I, P]),
+    "olmo355_relay_pair_ok": (I, [P, P, I, I]),
+    "olmo355_relay_device": (I, [P]),
+    "olmo355_relay_final": (I, [P, P, P, P, F, P, I, P, P, I, P]),
+    "olmo355_relay_tag": (I, [P, P, I, P, P]),
+    "olmo355_attn_decode_relay": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, P, P, P, P, P, I, P]),
+    "olmo355_attn_decode_relay_footprint": (I, [I, I, I, I, P]),
+    "olmo355_probe_stream_read": (I, [P, L, P, P]),
+    "olmo355_probe_stream_read_many": (I, [P, P, I, P, P]),
+    "olmo355_probe_mfma_bf16": (I, [I, P, P, P]),
+    "olmo355_probe_fill_lds": (I, [ctypes.c_uint32, P, P]),
     "olmo355_w4_gemm_tile": (I, [P, P, P, P, P, I, I, I, I, P]),
     "olmo355_b16_gemm_tile": (I, [P, P, P, I, I, I, I, P]),
     "olmo355_w4_gemm_streamk_patience": (I, [P, P, P, P, P, I, I, I, P, I, I, P]),
     "olmo355_w4_gemv_form": (I, [P, P, P, P, P, I, I, I, I, P]),
-    "olmo355_w4_chain_trace": (I, [ctypes.POINTER(ChainPhase), I, I, P, P, I, P, P]),
     "olmo355_attn_decode_fused_merge": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, P, I, I, P]),
 }
 

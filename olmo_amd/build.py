@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libolmo355.so")
-SOURCES = ["w4_format.hip", "gemv.hip", "gemv_mid.hip", "chain.hip", "relay.hip", "gemm.hip", "elementwise.hip", "attention.hip", "sample.hip", "beam.hip", "probe.hip"]
+SOURCES = ["w4_format.hip", "gemv.hip", "gemv_mid.hip", "relay.hip", "gemm.hip", "elementwise.hip", "attention.hip", "sample.hip", "beam.hip", "probe.hip"]
 
 # -packed-fp32-ops off: keep the compiler from forming packed-fp32 VALU instructions
 HIPCC_FLAGS = [

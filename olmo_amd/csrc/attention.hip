@@ -17,6 +17,7 @@
 // attn_masked_rows_kernel reproduces after a prefill launch; a decode step's single query (a real
 // token, never masked itself) needs no such pass.
 #include "common.h"
+#include "../../include/olmo355_debug.h"
 
 #include <mutex>
 #include <type_traits>

@@ -3,6 +3,7 @@
 // achieved figures so that "fraction of the published peak" can be read against what is reachable at the
 // same launch sizes on the same box.
 #include "common.h"
+#include "../../include/olmo355_debug.h"
 
 namespace {
 

@@ -33,6 +33,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "../../include/olmo355_debug.h"
 
 namespace {
 

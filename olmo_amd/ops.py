@@ -306,76 +306,6 @@ def w4_linear_chain(x: torch.Tensor, w: "W4Tiled", resid: Optional[torch.Tensor]
     return y, x_new, ssq
 
 
-@dataclass
-class ChainStep:
-    """One phase of :func:`w4_chain`: ``y = x' . W`` with ``x' = x`` or ``resid + rmsnorm(x; norm_w, eps)``."""
-
-    x: torch.Tensor
-    w: "W4Tiled"
-    y: torch.Tensor
-    resid: Optional[torch.Tensor] = None
-    norm_w: Optional[torch.Tensor] = None
-    ssq_in: Optional[torch.Tensor] = None
-    x_out: Optional[torch.Tensor] = None
-    ssq_out: Optional[torch.Tensor] = None
-    swiglu: bool = False
-    eps: float = 0.0
-    rot: int = 0
-
-
-CHAIN_SPIN_LIMIT = 1 << 18
-
-
-def chain_grid() -> int:
-    return int(lib().olmo355_w4_chain_grid())
-
-
-def chain_sync(device) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Barrier state and status word of :func:`w4_chain`: zeroed once, then reused by one launch at a time."""
-    n = int(lib().olmo355_w4_chain_sync_ints())
-    return torch.zeros(n, dtype=torch.int32, device=device), torch.zeros(1, dtype=torch.int32, device=device)
-
-
-def w4_chain(steps, sync: torch.Tensor, status: torch.Tensor, spin_limit: int = CHAIN_SPIN_LIMIT,
-             trace: Optional[torch.Tensor] = None) -> bool:
-    """Up to four decode-step int4 linears (at most 4 rows) in one launch of a persistent grid; every tensor is
-    given by the caller (outputs included: nothing is allocated here).  ``sync``, ``status``: from
-    :func:`chain_sync`; ``status`` becomes 1 if a barrier wait gave up.  Returns ``False`` when the kernel does
-    not cover the shapes (nothing launched)."""
-    from ._lib import ChainPhase
-
-    n = len(steps)
-    M = steps[0].x.numel() // steps[0].w.K
-    arr = (ChainPhase * n)()
-    for i, s in enumerate(steps):
-        _dev(s.x, s.y, s.resid, s.norm_w, s.ssq_in, s.x_out, s.ssq_out, s.w.wt)
-        if s.x.dtype != torch.bfloat16 or s.y.dtype != torch.bfloat16 or s.x.numel() != M * s.w.K:
-            raise ValueError("w4_chain: bfloat16 rows of K elements expected")
-        if s.y.numel() != M * (s.w.N // 2 if s.swiglu else s.w.N):
-            raise ValueError("w4_chain: output size mismatch")
-        if s.ssq_in is not None and (s.ssq_in.dtype != torch.float32 or s.ssq_in.numel() != M * s.w.K // 16):
-            raise ValueError("w4_chain: ssq_in float32 [M, K/16] expected")
-        if s.ssq_out is not None and (s.ssq_out.dtype != torch.float32 or s.ssq_out.numel() != M * s.w.N // 16):
-            raise ValueError("w4_chain: ssq_out float32 [M, N/16] expected")
-        if s.x_out is not None and (s.x_out.dtype != torch.bfloat16 or s.x_out.numel() != M * s.w.K):
-            raise ValueError("w4_chain: x_out bfloat16 [M, K] expected")
-        p = arr[i]
-        p.x, p.resid, p.norm_w, p.ssq_in, p.x_out = _p(s.x), _p(s.resid), _p(s.norm_w), _p(s.ssq_in), _p(s.x_out)
-        p.wt, p.st, p.zt, p.y, p.ssq_out = _p(s.w.wt), _p(s.w.st), _p(s.w.zt), _p(s.y), _p(s.ssq_out)
-        p.N, p.K, p.swiglu, p.rot, p.eps = s.w.N, s.w.K, int(s.swiglu), int(s.rot), float(s.eps)
-    if sync.dtype != torch.int32 or sync.numel() < int(lib().olmo355_w4_chain_sync_ints()) or status.dtype != torch.int32:
-        raise ValueError("w4_chain: sync and status as made by chain_sync expected")
-    _dev(sync, status)
-    if trace is None:
-        st = lib().olmo355_w4_chain(arr, n, M, _p(sync), _p(status), int(spin_limit), _stream())
-    else:  # tuning runs: int64 [grid, 8, 4, 8] time stamps
-        st = lib().olmo355_w4_chain_trace(arr, n, M, _p(sync), _p(status), int(spin_limit), _p(trace), _stream())
-    if st == 2:
-        return False
-    check("olmo355_w4_chain", st)
-    return True
-
-
 # ---------------------------------------------------------------------------------------------
 # the decode relay (one row): launches on two streams, the hand-over carried by epoch tags in the data
 # ---------------------------------------------------------------------------------------------
