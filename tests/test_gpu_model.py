@@ -3,11 +3,19 @@ against the CPU oracle on the same seeded weights and inputs.
 
 Tolerances (BASELINE north_star): bf16 -- max-abs error of softmax(logits) <= 2e-2 and greedy
 agreement >= 99 %; fp32 -- logits within 2e-4.  Greedy agreement is measured under teacher
-forcing (the oracle is fed the device's tokens).  A step agrees when the device token's oracle
-logit equals the oracle maximum (exact ties in a 16-bit logit vector are common with random
-weights and ``topk``'s tie order is unspecified: olmo/beam_search.py:102-113) -- reported as
-"strict" -- or lies within one bf16 ulp of it, the resolution of the reference's own output --
-reported as "ulp"; the 99 % bar is asserted on the latter and both are printed.
+forcing (the oracle is fed the device's tokens) and pinned by rules a wrong kernel fails (``agreement``):
+
+* on every step whose oracle top-2 margin exceeds three bf16 ulps -- the largest distance by which the two sides'
+  16-bit logits of one candidate have been seen apart (both round the head's output to bf16, on hidden states that
+  differ in the last bit of a few elements), so the steps where rounding cannot move the arg-max -- the device's
+  token IS the oracle's arg-max, without exception;
+* on the other steps (an exact tie or near-tie in a 16-bit logit vector, common with random weights and a
+  100 352-token vocabulary; ``topk``'s order among ties is unspecified, olmo/beam_search.py:102-113) the
+  device's token lies within three ulps of the oracle maximum;
+* where a referee is run (the oracle with fp32 activations on the same weights, teacher-forced on the same
+  tokens), the device agrees with the referee's arg-max at least as often as the bf16 oracle itself does,
+  less one step: it is no further from the exact model than the reference's own rounding is;
+* floors on what has been measured: strict agreement >= 95 %, within one ulp >= 98 %, within two >= 99 %.
 """
 import pytest
 import torch
@@ -79,29 +87,47 @@ def softmax_err(a, b):
     return (torch.softmax(a.float(), -1) - torch.softmax(b.float(), -1)).abs().max().item()
 
 
-def agreement(dev_tokens, oracle_logits):
-    """dev_tokens [B,S]; oracle_logits [B,S,V] -> (strict, loose) fractions of steps.
+def agreement_report(dev_tokens, oracle_logits, referee_logits=None):
+    """dev_tokens [B,S]; oracle_logits [B,S,V] (teacher-forced on dev_tokens) -> dict of rates over the B*S steps.
 
-    strict: the device's token is the oracle's arg-max.  loose: its oracle logit is within two bf16 ulps of the
-    oracle's maximum.  Logits leave the head rounded to bf16 on both sides (half an ulp each way), on hidden states
-    that differ in the last bit of many elements (the oracle rounds at the reference's points, e.g. the softmax
-    probabilities to bf16 before P.V, which a kernel that walks the keys in chunks cannot reproduce), and with random
-    N(0, 0.02) weights and 100 352 candidates the top logits of a step lie an ulp or two apart: two candidates whose
-    exact logits are an ulp apart can come out two apart on one side and level on the other.  Any change in the order
-    of an fp32 sum reshuffles which steps are hit.  Measured on the 1B model, 256 steps, four input seeds, two ways
-    of splitting the keys of the decode attention: strict 96.9-98.4 %, within one ulp 98.4-99.2 %, within two
-    99.6-100 %, never more than three."""
+    ulp: one bf16 step at the oracle's maximum logit.  margin: oracle top-1 minus top-2.  A step is *clear* when
+    its margin exceeds three ulps: both sides round the logits to bf16 on hidden states that differ in the last bit
+    of a few elements, and the same candidate's logit has been measured up to three ulps apart on the two sides
+    (never more, over every model and seed of this file), so two candidates can trade places only when they are
+    that close."""
     ol = oracle_logits.float()
-    mx = ol.max(-1).values
+    top2 = ol.topk(2, dim=-1).values
+    mx, margin = top2[..., 0], top2[..., 0] - top2[..., 1]
     chosen = ol.gather(-1, dev_tokens.unsqueeze(-1)).squeeze(-1)
-    strict = (chosen == mx).float().mean().item()
     ulp = 2.0 ** (torch.floor(torch.log2(mx.abs().clamp_min(1e-30))) - 7)
-    loose = (chosen >= mx - 2 * ulp).float().mean().item()
-    off = (chosen < mx)
-    if off.any():
-        say("  steps where the device's token is not the oracle's arg-max: gap to the oracle maximum in bf16 ulps",
-            ((mx - chosen) / ulp)[off].tolist())
-    return strict, loose
+    gap = (mx - chosen) / ulp
+    clear = margin > 3 * ulp
+    rep = {
+        "steps": gap.numel(), "strict": (gap == 0).float().mean().item(), "ulp1": (gap <= 1).float().mean().item(),
+        "ulp2": (gap <= 2).float().mean().item(), "max_gap_ulps": gap.max().item(), "clear_steps": int(clear.sum().item()),
+        "clear_strict": (gap[clear] == 0).float().mean().item() if bool(clear.any()) else 1.0,
+    }
+    if bool((gap > 0).any()):
+        say("  steps where the device's token is not the oracle's arg-max: (gap, oracle margin) in bf16 ulps",
+            [(round(g, 2), round(m, 2)) for g, m in zip(gap[gap > 0].tolist(), (margin / ulp)[gap > 0].tolist())])
+    if referee_logits is not None:
+        ref_arg = referee_logits.float().argmax(-1)
+        rep["device_vs_referee"] = (dev_tokens == ref_arg).float().mean().item()
+        rep["oracle_vs_referee"] = (ol.argmax(-1) == ref_arg).float().mean().item()
+    return rep
+
+
+def agreement(dev_tokens, oracle_logits, referee_logits=None, floors=False):
+    """Asserts the rules of this file's header and returns (strict, within two ulps)."""
+    rep = agreement_report(dev_tokens, oracle_logits, referee_logits)
+    say("  agreement:", {k: (round(v, 4) if isinstance(v, float) else v) for k, v in rep.items()})
+    assert rep["clear_strict"] == 1.0, "a step with a clear oracle margin was decoded differently"
+    assert rep["max_gap_ulps"] <= 3.0, "a device token lies more than three bf16 ulps below the oracle's maximum"
+    if floors:
+        assert rep["strict"] >= 0.95 and rep["ulp1"] >= 0.98 and rep["ulp2"] >= 0.99, rep
+    if referee_logits is not None:
+        assert rep["device_vs_referee"] >= rep["oracle_vs_referee"] - 1.0 / rep["steps"] - 1e-9, rep
+    return rep["strict"], rep["ulp2"]
 
 
 # ------------------------------------------------------------------------------------------------
@@ -447,7 +473,15 @@ def test_config2_1b_bf16_prefill_and_256_greedy_steps(dev):
             say("   oracle step", i)
     ref = torch.stack(refs, dim=1)  # [1,256,V]
     e = softmax_err(logits, ref)
-    strict, loose = agreement(toks, ref)
+    # the referee: the same weights with fp32 activations (no rounding of its own), teacher-forced on the same tokens
+    say("  running the fp32 referee (CPU) ...")
+    referee = om.OracleModel(cfg, oracle.w, torch.float32)
+    f0, kvf = referee.forward(ids, use_cache=True, last_logits_only=True)
+    frefs = [f0[:, -1]]
+    for i in range(255):
+        r, kvf = referee.forward(toks[:, i:i + 1], past_key_values=kvf, use_cache=True)
+        frefs.append(r[:, -1])
+    strict, loose = agreement(toks, ref, referee_logits=torch.stack(frefs, dim=1), floors=True)
     say(f"  softmax max-abs err {e:.3e}; greedy agreement over 256 steps: strict {strict:.4f} within 2 ulps {loose:.4f}")
     assert e <= 2e-2
     assert loose >= 0.99
@@ -665,6 +699,53 @@ def test_13b_decode_at_its_workload_shape(dev):
             worst = max(worst, softmax_err(logits_e[k - 1][b0:b0 + 4], ref))
         say(f"  step {k}: softmax max-abs difference cache vs full forward {worst:.2e}")
         assert worst <= 2e-2
+
+
+@pytest.mark.parametrize("B", [1, 8])
+def test_7b_decode_at_its_workload_shape(dev, B):
+    """BASELINE's third configuration -- the one bench.py times -- at its real shape: OLMo-2 7B int4-g128 at full
+    depth (32 layers), batch 1 and 8, KV context 2048 (random weights).  Size-independent properties, no oracle at
+    this size: (1) a decode step over the cache gives the last row of a full causal forward of the same tokens
+    (reference tests/model_test.py:196-199) -- different kernels on the two sides: the lean / staged int4 kernels
+    with chained norms and the fused decode attention against the MFMA GEMMs and the prefill attention; (2) the
+    captured-graph loop reproduces the eager loop bit for bit."""
+    say("7b decode at context 2048, batch", B)
+    from olmo_amd.generate import DecodeSession, _prefill
+    from olmo_amd.synthetic import build_random_model
+
+    cfg = PRESETS["olmo2-7b"]
+    ctx, steps = 2048, 4
+    model = build_random_model(cfg, torch.bfloat16, quantized=True, seed=4, device=dev, max_cache_len=ctx + 8,
+                               free_checkpoint_buffers=True)
+    ids = torch.randint(0, cfg.vocab_size, (B, ctx), generator=torch.Generator().manual_seed(12)).to(dev)
+
+    def run(use_graph):
+        out, cache, first, kb = _prefill(model, ids, None)
+        sess = DecodeSession(model, cache, first, kb)
+        toks, logits = [first.view(B).clone()], []
+        for i in range(steps):
+            if use_graph and i == 2:
+                sess.capture()
+            sess.step()
+            toks.append(sess.ids.view(B).clone())
+            logits.append(sess.logits.view(B, -1).clone())
+        return torch.stack(toks, 1), logits
+
+    toks_e, logits_e = run(False)
+    toks_g, logits_g = run(True)
+    assert torch.equal(toks_e, toks_g)
+    for a, b in zip(logits_e, logits_g):
+        assert torch.equal(a, b), "graph replay differs from eager decode"
+    for k in (1, 2):  # step k fed token k-1 at position ctx+k-1: the last row of a full forward over ctx+k tokens
+        full = torch.cat((ids, toks_e[:, :k]), dim=1)
+        worst = 0.0
+        for b0 in range(0, B, 4):
+            ref = model(full[b0:b0 + 4], last_logits_only=True).logits
+            worst = max(worst, softmax_err(logits_e[k - 1][b0:b0 + 4], ref.view(ref.shape[0], -1)))
+        say(f"  step {k}: softmax max-abs difference cache vs full forward {worst:.2e}")
+        assert worst <= 2e-2
+    del model
+    torch.cuda.empty_cache()
 
 
 def test_sampled_generation(dev):
