@@ -125,20 +125,29 @@ int olmo355_b16_gemm_splitk(const uint16_t* x, const uint16_t* wt, uint16_t* y, 
  * that ends it adds the others' fp32 partials (in a fixed order: results are reproducible, and differ from the
  * tiled entry only in the order of fp32 additions) and writes the output.  Same product as QuantLinear.forward's
  * matmul (qlinear_cuda_old.py:287-290) / F.linear (olmo/model.py:746-823).
- * `workspace`: olmo355_gemm_streamk_workspace_bytes() bytes, 16-byte aligned, zero before its first use; a launch
- * leaves its first 4096 bytes (the hand-over flags) zero again.  Launches that share a workspace must be ordered on
- * one stream.  A finishing workgroup that does not see a partial announced within about two seconds writes NaN
- * into its tile instead of waiting on (then zero the workspace before the next use).
+ * `workspace`: ws_bytes >= olmo355_gemm_streamk_workspace_bytes() bytes (O355_EINVAL otherwise), 16-byte aligned,
+ * zeroed once when allocated and never cleaned afterwards.  Its first 4096 bytes are int32 words: one hand-over flag
+ * per workgroup, which holds the `epoch` of the launch whose partial the slot carries, and at index
+ * O355_STREAMK_STATUS_WORD a status word.  `epoch`: any non-zero value that differs from the epoch of every earlier
+ * launch on this workspace whose flags may still be set (a counter that skips 0 will do; O355_EINVAL for 0).  A stale
+ * flag of an earlier launch therefore never passes for a partial of this one, whatever state that launch ended in
+ * (for the same reason these launches must not be recorded into a HIP graph: a replay would repeat its epoch).
+ * Launches that share a workspace must be ordered on one stream.  A finishing workgroup that does not see a partial
+ * announced within about two seconds writes NaN into its tile instead of waiting on and stores the launch's epoch
+ * into the status word: a caller that reads a non-zero status word knows that the output of that launch is not
+ * valid; the next launch (with a new epoch) needs no clean-up of the workspace.
  * Needs K % 256 == 0, N % 16 == 0 (SwiGLU form: N % 256 == 0) and at least one unit of 256 per CU; otherwise
  * O355_EUNSUPPORTED.  olmo355_gemm_streamk_plan: 1 when this form is expected to beat the tiled launch. */
+#define O355_STREAMK_STATUS_WORD 513
 int64_t olmo355_gemm_streamk_workspace_bytes(void);
 int olmo355_gemm_streamk_plan(int M, int N, int K);
 int olmo355_w4_gemm_streamk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
-                            int M, int N, int K, void* workspace, void* stream);
+                            int M, int N, int K, void* workspace, int64_t ws_bytes, int epoch, void* stream);
 int olmo355_w4_gemm_swiglu_streamk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
-                                   uint16_t* y, int M, int N, int K, void* workspace, void* stream);
+                                   uint16_t* y, int M, int N, int K, void* workspace, int64_t ws_bytes, int epoch,
+                                   void* stream);
 int olmo355_b16_gemm_streamk(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, void* workspace,
-                             void* stream);
+                             int64_t ws_bytes, int epoch, void* stream);
 
 /* The same product for an ff_proj weight ([up | gate] column halves) with SwiGLU (olmo/model.py:365-368,813-819)
  * in the epilogue: y [M, N/2] = silu(gate) * up, each factor rounded to bf16 first as the separate Linear and
@@ -197,7 +206,8 @@ int olmo355_attn_prefill(const void* q, const void* kcache, const void* vcache, 
 
 /* T == 1 with the keys split over workgroups.  n_keys_max bounds the number of keys for the
  * launch grid; the true count is past_len + 1 (or *past_len_dev + 1 when given).
- * ws: olmo355_attn_decode_workspace_bytes(B,H,hd,n_keys_max) bytes, zeroed when allocated: it begins with
+ * ws: ws_bytes >= olmo355_attn_decode_workspace_bytes(B,H,hd,n_keys_max) bytes (O355_EINVAL, nothing launched,
+ * when smaller: the launch writes one partial per 128 keys of every (batch, head)), zeroed when allocated: it begins with
  * two int32 counters per (batch, head) that olmo355_attn_decode_fused uses to let one workgroup of a head
  * merge the partial results (B * H ticket counters, which every launch leaves at zero, then B * H launch counters
  * whose value marks the partials of the current launch; the regions are apart, so one workspace may serve
@@ -205,7 +215,7 @@ int olmo355_attn_prefill(const void* q, const void* kcache, const void* vcache, 
  * room for a flag word each. */
 int64_t olmo355_attn_decode_workspace_bytes(int B, int H, int hd, int n_keys_max);
 int olmo355_attn_decode(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out,
-                        void* ws, int B, int H, int Hkv, int hd, int Lmax, int past_len,
+                        void* ws, int64_t ws_bytes, int B, int H, int Hkv, int hd, int Lmax, int past_len,
                         const int32_t* past_len_dev, int n_keys_max, int bias_stride, int dtype, void* stream);
 
 /* olmo355_attn_decode for callers that cannot allocate device memory or pass a workspace (code under HIP graph
@@ -215,7 +225,10 @@ int olmo355_attn_decode(const void* q, const void* kcache, const void* vcache, c
  * process ends.  Returns O355_ETOOBIG (nothing launched) when
  * olmo355_attn_decode_workspace_bytes(B, H, hd, n_keys_max) exceeds that.  Calls no hipMalloc / hipFree / allocating
  * library routine.  All calls on one GPU share the array and it keeps the last call's contents: calls that
- * overlap on one GPU (different streams or host threads) race; calls on one stream are ordered. */
+ * overlap on one GPU (different streams or host threads) race; calls on one stream are ordered.
+ * The first call on a GPU looks the array's device address up (hipGetSymbolAddress, a query that is not
+ * permitted while a stream of the process is capturing): make one call on every GPU, e.g. a warm-up step, before
+ * the first capture; later calls only launch kernels. */
 int64_t olmo355_attn_decode_static_max_bytes(void);
 int olmo355_attn_decode_static(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out,
                                int B, int H, int Hkv, int hd, int Lmax, int past_len, const int32_t* past_len_dev,
@@ -229,7 +242,7 @@ int olmo355_attn_decode_static(const void* q, const void* kcache, const void* vc
  * generated token of b's history; entries past the current length must still be valid row numbers).  The
  * search updates beam_src with its backpointers.  Needs prompt_len + src_stride >= n_keys_max. */
 int olmo355_attn_decode_beam(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out,
-                             void* ws, int B, int H, int Hkv, int hd, int Lmax, int past_len,
+                             void* ws, int64_t ws_bytes, int B, int H, int Hkv, int hd, int Lmax, int past_len,
                              const int32_t* past_len_dev, int n_keys_max, int bias_stride, const int32_t* beam_src,
                              int src_stride, int prompt_len, int beam, int dtype, void* stream);
 
@@ -243,8 +256,8 @@ int olmo355_attn_decode_beam(const void* q, const void* kcache, const void* vcac
  * dependent load behind the whole cache stream. */
 int olmo355_attn_decode_fused(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
                               const float* cos_tab, void* kcache, void* vcache, const float* key_bias, void* out,
-                              void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos, int past_len,
-                              const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps,
+                              void* ws, int64_t ws_bytes, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
+                              int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps,
                               const float* qk_ssq, const float* rope_now, int dtype, void* stream);
 /* Between captured decode steps: *pos += delta, then rope_now [2*hd] = sin_tab[*pos] | cos_tab[*pos]
  * (rows of get_rotary_embedding's tables, olmo/model.py:285-296).  delta 0 initialises rope_now. */

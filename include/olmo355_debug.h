@@ -21,7 +21,8 @@ int olmo355_b16_gemm_tile(const uint16_t* x, const uint16_t* wt, uint16_t* y, in
  * given up as NaN) and with publish = 0, which makes the partials' owners leave their flags down: the give-up path
  * forced from the host, every workgroup still exits. */
 int olmo355_w4_gemm_streamk_patience(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
-                                  int M, int N, int K, void* workspace, int spin_limit, int publish, void* stream);
+                                  int M, int N, int K, void* workspace, int64_t ws_bytes, int epoch, int spin_limit,
+                                  int publish, void* stream);
 
 /* olmo355_w4_gemv with the kernel family given: 0 = choose; 1 = the kernels that keep all rows of x in LDS per
  * workgroup (the lean M <= 16 kernel where it applies), never the staged-activation kernel; 2 = the
@@ -36,8 +37,8 @@ int olmo355_w4_gemv_form(const uint16_t* x, const uint32_t* wt, const uint16_t* 
  * wait for nothing), 2 = the separate combine kernel. */
 int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
                                     const float* cos_tab, void* kcache, void* vcache, const float* key_bias, void* out,
-                                    void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos, int past_len,
-                                    const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps,
+                                    void* ws, int64_t ws_bytes, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
+                                    int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps,
                                     const float* qk_ssq, const float* rope_now, int dtype, int merge, void* stream);
 
 #include "olmo355.h"
@@ -88,8 +89,8 @@ int olmo355_relay_device(int* out2); /* CUs of the current device, bytes of LDS 
  * merged inside the kernel (B * H * chunks <= 1536), H hd <= 8192. */
 int olmo355_attn_decode_relay(const uint32_t* qkv, const void* qw, const void* kw, const float* sin_tab,
                               const float* cos_tab, void* kcache, void* vcache, const float* key_bias, uint32_t* out,
-                              void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos, int past_len,
-                              const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps,
+                              void* ws, int64_t ws_bytes, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
+                              int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps,
                               const uint32_t* qk_ssq, const float* rope_now, const int32_t* epoch, int32_t* status,
                               const int32_t* hint_in, int32_t* hint_out, int spin_limit, void* stream);
 int olmo355_attn_decode_relay_footprint(int B, int H, int hd, int n_keys_max, int* out4);

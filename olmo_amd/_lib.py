@@ -52,11 +52,11 @@ EXPORTS = {
     "olmo355_qknorm_rope_kvwrite": (I, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P, F, I, P]),
     "olmo355_attn_prefill": (I, [P, P, P, P, P, I, I, I, I, I, I, I, I, I, P]),
     "olmo355_attn_decode_workspace_bytes": (L, [I, I, I, I]),
-    "olmo355_attn_decode": (I, [P, P, P, P, P, P, I, I, I, I, I, I, P, I, I, I, P]),
+    "olmo355_attn_decode": (I, [P, P, P, P, P, P, L, I, I, I, I, I, I, P, I, I, I, P]),
     "olmo355_attn_decode_static_max_bytes": (L, []),
     "olmo355_attn_decode_static": (I, [P, P, P, P, P, I, I, I, I, I, I, P, I, I, I, P]),
-    "olmo355_attn_decode_fused": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, P, I, P]),
-    "olmo355_attn_decode_beam": (I, [P, P, P, P, P, P, I, I, I, I, I, I, P, I, I, P, I, I, I, I, P]),
+    "olmo355_attn_decode_fused": (I, [P, P, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, I, P, I, I, F, P, P, I, P]),
+    "olmo355_attn_decode_beam": (I, [P, P, P, P, P, P, L, I, I, I, I, I, I, P, I, I, P, I, I, I, I, P]),
     "olmo355_log_softmax": (I, [P, P, I, I, I, P]),
     "olmo355_topk": (I, [P, I, I, I, P, P, P]),
     "olmo355_gumbel_perturb": (I, [P, P, I, I, F, c_uint64, c_uint64, P]),
@@ -66,9 +66,9 @@ EXPORTS = {
     "olmo355_b16_gemm_splitk": (I, [P, P, P, I, I, I, I, P, P]),
     "olmo355_gemm_streamk_workspace_bytes": (L, []),
     "olmo355_gemm_streamk_plan": (I, [I, I, I]),
-    "olmo355_w4_gemm_streamk": (I, [P, P, P, P, P, I, I, I, P, P]),
-    "olmo355_w4_gemm_swiglu_streamk": (I, [P, P, P, P, P, I, I, I, P, P]),
-    "olmo355_b16_gemm_streamk": (I, [P, P, P, I, I, I, P, P]),
+    "olmo355_w4_gemm_streamk": (I, [P, P, P, P, P, I, I, I, P, L, I, P]),
+    "olmo355_w4_gemm_swiglu_streamk": (I, [P, P, P, P, P, I, I, I, P, L, I, P]),
+    "olmo355_b16_gemm_streamk": (I, [P, P, P, I, I, I, P, L, I, P]),
     "olmo355_rope_advance": (I, [P, I, P, P, P, I, I, P]),
     "olmo355_swiglu": (I, [P, P, I, I, I, P]),
     "olmo355_embedding": (I, [P, P, P, I, I, I, I, P]),
@@ -89,7 +89,7 @@ VARIANT_EXPORTS = {
     "olmo355_relay_device": (I, [P]),
     "olmo355_relay_final": (I, [P, P, P, P, F, P, I, P, P, I, P]),
     "olmo355_relay_tag": (I, [P, P, I, P, P]),
-    "olmo355_attn_decode_relay": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, P, P, P, P, P, I, P]),
+    "olmo355_attn_decode_relay": (I, [P, P, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, I, P, I, I, F, P, P, P, P, P, P, I, P]),
     "olmo355_attn_decode_relay_footprint": (I, [I, I, I, I, P]),
     "olmo355_probe_stream_read": (I, [P, L, P, P]),
     "olmo355_probe_stream_read_many": (I, [P, P, I, P, P]),
@@ -97,9 +97,9 @@ VARIANT_EXPORTS = {
     "olmo355_probe_fill_lds": (I, [ctypes.c_uint32, P, P]),
     "olmo355_w4_gemm_tile": (I, [P, P, P, P, P, I, I, I, I, P]),
     "olmo355_b16_gemm_tile": (I, [P, P, P, I, I, I, I, P]),
-    "olmo355_w4_gemm_streamk_patience": (I, [P, P, P, P, P, I, I, I, P, I, I, P]),
+    "olmo355_w4_gemm_streamk_patience": (I, [P, P, P, P, P, I, I, I, P, L, I, I, I, P]),
     "olmo355_w4_gemv_form": (I, [P, P, P, P, P, I, I, I, I, P]),
-    "olmo355_attn_decode_fused_merge": (I, [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, P, I, I, F, P, P, I, I, P]),
+    "olmo355_attn_decode_fused_merge": (I, [P, P, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, I, P, I, I, F, P, P, I, I, P]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

@@ -1284,12 +1284,14 @@ extern "C" int64_t olmo355_attn_decode_workspace_bytes(int B, int H, int hd, int
 
 namespace {
 int attn_decode_any(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out, void* ws,
-                    int B, int H, int Hkv, int hd, int Lmax, int past_len, const int32_t* past_len_dev,
+                    int64_t ws_bytes, int B, int H, int Hkv, int hd, int Lmax, int past_len, const int32_t* past_len_dev,
                     int n_keys_max, int bias_stride, const int32_t* beam_src, int src_stride, int prompt_len, int beam,
                     int dtype, void* stream) {
   if (!q || !kcache || !vcache || !out || !ws) return O355_EINVAL;
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || past_len < 0 || n_keys_max <= 0 || n_keys_max > Lmax)
     return O355_EINVAL;
+  // the launch writes one partial per (sequence, head, chunk): the workspace must hold them all
+  if (ws_bytes < olmo355_attn_decode_workspace_bytes(B, H, hd, n_keys_max)) return O355_EINVAL;
   if (!past_len_dev && past_len + 1 > n_keys_max) return O355_EINVAL;
   if (key_bias && bias_stride < n_keys_max) return O355_EINVAL;
   if (beam_src && (beam <= 0 || B % beam || prompt_len < 0 || src_stride <= 0 || prompt_len + src_stride < n_keys_max))
@@ -1313,20 +1315,20 @@ int attn_decode_any(const void* q, const void* kcache, const void* vcache, const
 }  // namespace
 
 extern "C" int olmo355_attn_decode(const void* q, const void* kcache, const void* vcache, const float* key_bias,
-                                   void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int past_len,
+                                   void* out, void* ws, int64_t ws_bytes, int B, int H, int Hkv, int hd, int Lmax, int past_len,
                                    const int32_t* past_len_dev, int n_keys_max, int bias_stride, int dtype,
                                    void* stream) {
-  return attn_decode_any(q, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd, Lmax, past_len, past_len_dev, n_keys_max,
+  return attn_decode_any(q, kcache, vcache, key_bias, out, ws, ws_bytes, B, H, Hkv, hd, Lmax, past_len, past_len_dev, n_keys_max,
                          bias_stride, nullptr, 0, 0, 1, dtype, stream);
 }
 
 extern "C" int olmo355_attn_decode_beam(const void* q, const void* kcache, const void* vcache, const float* key_bias,
-                                        void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int past_len,
+                                        void* out, void* ws, int64_t ws_bytes, int B, int H, int Hkv, int hd, int Lmax, int past_len,
                                         const int32_t* past_len_dev, int n_keys_max, int bias_stride,
                                         const int32_t* beam_src, int src_stride, int prompt_len, int beam, int dtype,
                                         void* stream) {
   if (!beam_src) return O355_EINVAL;
-  return attn_decode_any(q, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd, Lmax, past_len, past_len_dev, n_keys_max,
+  return attn_decode_any(q, kcache, vcache, key_bias, out, ws, ws_bytes, B, H, Hkv, hd, Lmax, past_len, past_len_dev, n_keys_max,
                          bias_stride, beam_src, src_stride, prompt_len, beam, dtype, stream);
 }
 
@@ -1371,8 +1373,8 @@ extern "C" int olmo355_attn_decode_static(const void* q, const void* kcache, con
   void* ws = nullptr;
   const int st = scratch_of_current_device(&ws);
   if (st != O355_OK) return st;
-  return attn_decode_any(q, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd, Lmax, past_len, past_len_dev, n_keys_max,
-                         bias_stride, nullptr, 0, 0, 1, dtype, stream);
+  return attn_decode_any(q, kcache, vcache, key_bias, out, ws, kStaticScratchBytes, B, H, Hkv, hd, Lmax, past_len, past_len_dev,
+                         n_keys_max, bias_stride, nullptr, 0, 0, 1, dtype, stream);
 }
 
 // merge: how the key chunks of a (batch, head) are merged: -1 = choose, 0 = in the kernel by the workgroup that
@@ -1399,8 +1401,8 @@ FusedPlan fused_plan(int B, int H, int n_keys_max, int merge) {
 }
 
 int attn_fused_any(const void* qkv, const void* qw, const void* kw, const float* sin_tab, const float* cos_tab, void* kcache,
-                   void* vcache, const float* key_bias, void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
-                   int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps, const void* qk_ssq,
+                   void* vcache, const float* key_bias, void* out, void* ws, int64_t ws_bytes, int B, int H, int Hkv, int hd, int Lmax,
+                   int n_pos, int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride, float eps, const void* qk_ssq,
                    const float* rope_now, int dtype, int merge, bool relay, const int32_t* epoch, int32_t* status, int spin_limit,
                    const int32_t* hint_in, int32_t* hint_out, void* stream) {
   if (merge < -1 || merge > 2) return O355_EINVAL;
@@ -1408,6 +1410,7 @@ int attn_fused_any(const void* qkv, const void* qw, const void* kw, const float*
   if (B <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || past_len < 0 || n_keys_max <= 0 || n_keys_max > Lmax)
     return O355_EINVAL;
   if ((qw == nullptr) != (kw == nullptr)) return O355_EINVAL;
+  if (ws_bytes < olmo355_attn_decode_workspace_bytes(B, H, hd, n_keys_max)) return O355_EINVAL;
   if (!past_len_dev && (past_len + 1 > n_keys_max || past_len + 1 > n_pos)) return O355_EINVAL;
   if (key_bias && bias_stride < n_keys_max) return O355_EINVAL;
   if (dtype != O355_BF16 || (hd != 128 && hd != 64) || H * hd > 8 * 4 * 256) return O355_EUNSUPPORTED;
@@ -1452,33 +1455,33 @@ int attn_fused_any(const void* qkv, const void* qw, const void* kw, const float*
 
 extern "C" int olmo355_attn_decode_fused_merge(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
                                                const float* cos_tab, void* kcache, void* vcache, const float* key_bias,
-                                               void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
+                                               void* out, void* ws, int64_t ws_bytes, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
                                                int past_len, const int32_t* past_len_dev, int n_keys_max,
                                                int bias_stride, float eps, const float* qk_ssq, const float* rope_now,
                                                int dtype, int merge, void* stream) {
-  return attn_fused_any(qkv, qw, kw, sin_tab, cos_tab, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd, Lmax, n_pos, past_len,
+  return attn_fused_any(qkv, qw, kw, sin_tab, cos_tab, kcache, vcache, key_bias, out, ws, ws_bytes, B, H, Hkv, hd, Lmax, n_pos, past_len,
                         past_len_dev, n_keys_max, bias_stride, eps, qk_ssq, rope_now, dtype, merge, false, nullptr, nullptr, 0, nullptr, nullptr, stream);
 }
 
 extern "C" int olmo355_attn_decode_fused(const void* qkv, const void* qw, const void* kw, const float* sin_tab,
                                          const float* cos_tab, void* kcache, void* vcache, const float* key_bias,
-                                         void* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
+                                         void* out, void* ws, int64_t ws_bytes, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
                                          int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride,
                                          float eps, const float* qk_ssq, const float* rope_now, int dtype,
                                          void* stream) {
-  return olmo355_attn_decode_fused_merge(qkv, qw, kw, sin_tab, cos_tab, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd,
+  return olmo355_attn_decode_fused_merge(qkv, qw, kw, sin_tab, cos_tab, kcache, vcache, key_bias, out, ws, ws_bytes, B, H, Hkv, hd,
                                          Lmax, n_pos, past_len, past_len_dev, n_keys_max, bias_stride, eps, qk_ssq,
                                          rope_now, dtype, -1, stream);
 }
 
 extern "C" int olmo355_attn_decode_relay(const uint32_t* qkv, const void* qw, const void* kw, const float* sin_tab,
                                          const float* cos_tab, void* kcache, void* vcache, const float* key_bias,
-                                         uint32_t* out, void* ws, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
+                                         uint32_t* out, void* ws, int64_t ws_bytes, int B, int H, int Hkv, int hd, int Lmax, int n_pos,
                                          int past_len, const int32_t* past_len_dev, int n_keys_max, int bias_stride,
                                          float eps, const uint32_t* qk_ssq, const float* rope_now, const int32_t* epoch,
                                          int32_t* status, const int32_t* hint_in, int32_t* hint_out, int spin_limit,
                                          void* stream) {
-  return attn_fused_any(qkv, qw, kw, sin_tab, cos_tab, kcache, vcache, key_bias, out, ws, B, H, Hkv, hd, Lmax, n_pos, past_len,
+  return attn_fused_any(qkv, qw, kw, sin_tab, cos_tab, kcache, vcache, key_bias, out, ws, ws_bytes, B, H, Hkv, hd, Lmax, n_pos, past_len,
                         past_len_dev, n_keys_max, bias_stride, eps, qk_ssq, rope_now, O355_BF16, -1, true, epoch, status,
                         spin_limit, hint_in, hint_out, stream);
 }

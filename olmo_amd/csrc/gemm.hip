@@ -95,10 +95,11 @@ struct StreamKArgs {
   const uint8_t* zt;
   uint16_t* y;
   float* slots;    // [grid][8 waves][128 registers / 4][64 lanes] float4: a wave's accumulators as they stand
-  int* flags;      // [grid], zero between launches
+  int* flags;      // [grid]: the epoch of the launch whose partial the slot holds; word 513: status
   int M, N, K, tiles_n, tiles;
   int spin_limit;  // polls of a flag before a finishing workgroup gives up and writes NaN
   int publish;     // 0 (tests of the give-up path only): leave the flag down
+  int epoch;       // this launch's flag value: differs from that of the launch before on the same workspace, never 0
 };
 typedef const __attribute__((address_space(4))) StreamKArgs* StreamKArgsPtr;
 __device__ __forceinline__ StreamKArgsPtr streamk_args() {
@@ -107,6 +108,7 @@ __device__ __forceinline__ StreamKArgsPtr streamk_args() {
   return p;
 }
 enum { GEMM_PLAIN = 0, GEMM_SPLIT = 1, GEMM_STREAMK = 2 };
+constexpr int kStreamKStatusWord = O355_STREAMK_STATUS_WORD;  // int32 index in the workspace: epoch of a launch that gave up
 
 template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false, int KIND = GEMM_PLAIN>  // wave grid, 32 x 32 blocks (of four 16 x 16 MFMA tiles) per wave
 __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wt,
@@ -364,7 +366,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     // operations, those stores among them, so the flag can go up without a wait of its own
     if (sk_raise && tid == 0) {
       const StreamKArgsPtr ka = streamk_args();
-      if (ka->publish) __hip_atomic_store(ka->flags + sk_self, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (ka->publish) __hip_atomic_store(ka->flags + sk_self, ka->epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
 #pragma unroll
@@ -406,23 +408,25 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
       const StreamKArgsPtr ka = streamk_args();
       float* const slots = ka->slots;
       int* const flags = ka->flags;
-      const int spin_limit = ka->spin_limit;
+      const int spin_limit = ka->spin_limit, epoch = ka->epoch;
       // the workgroups first .. self - 1 hold the earlier runs of this tile's K and finished them before anything
       // else they had to do; their partials are added in a fixed order.  The wait is bounded: a flag that does
-      // not come up in spin_limit polls turns the tile into NaN instead of hanging the grid.
+      // not show this launch's epoch within spin_limit polls turns the tile into NaN instead of hanging the grid,
+      // and the status word of the workspace says so.  Flags are never cleared: the next launch waits for its
+      // own epoch, so a flag raised late by a workgroup nobody waited for any more cannot be mistaken for news.
       int* s_ok = reinterpret_cast<int*>(smem);  // the operand buffers are done with once every wave is past the K loop
       for (int pc = sk_self - 1; pc >= sk_first; --pc) {
         __syncthreads();
         if (tid == 0) {
           int ok = 0;
           for (int spin = 0; spin <= spin_limit; ++spin) {
-            if (__hip_atomic_load(flags + pc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+            if (__hip_atomic_load(flags + pc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == epoch) {
               ok = 1;
               break;
             }
             __builtin_amdgcn_s_sleep(8);
           }
-          if (ok) __hip_atomic_store(flags + pc, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+          if (!ok) __hip_atomic_store(flags + kStreamKStatusWord, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           *s_ok = ok;
         }
         __syncthreads();
@@ -462,7 +466,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     const int publish = ka->publish;
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, false));
     __syncthreads();
-    if (tid == 0 && publish) __hip_atomic_store(flags + sk_self, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0 && publish) __hip_atomic_store(flags + sk_self, ka->epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   };
   // va, vb: this lane's four outputs (columns 4 kq4 .. + 3 of row m) of two blocks whose first columns are nb and nb + 16
   auto store_pair = [&](const f32x4& va, const f32x4& vb, uint16_t* __restrict__ dst, int m, int nb, int ncols, int ld) {
@@ -628,7 +632,8 @@ constexpr int kStreamKSpinLimit = 1 << 21;
 
 template <bool W4, bool SWIGLU>
 int launch_streamk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M, int N,
-                   int K, void* ws, int spin_limit, int publish, hipStream_t stream) {
+                   int K, void* ws, int64_t ws_bytes, int epoch, int spin_limit, int publish, hipStream_t stream) {
+  if (ws_bytes < olmo355_gemm_streamk_workspace_bytes() || epoch == 0) return O355_EINVAL;
   int dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
     return O355_ELAUNCH;
@@ -643,7 +648,7 @@ int launch_streamk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, co
   int* flags = reinterpret_cast<int*>(ws);
   float* slots = reinterpret_cast<float*>(reinterpret_cast<char*>(ws) + kStreamKFlagBytes);
   if ((int64_t)tiles_m * tiles_n * (K >> 8) * grid >= (1ll << 31)) return O355_EUNSUPPORTED;
-  const StreamKArgs args{x, wt, st, zt, y, slots, flags, M, N, K, tiles_n, tiles_m * tiles_n, spin_limit, publish};
+  const StreamKArgs args{x, wt, st, zt, y, slots, flags, M, N, K, tiles_n, tiles_m * tiles_n, spin_limit, publish, epoch};
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, stream, args);
   O355_CHECK_LAUNCH();
 }
@@ -795,34 +800,34 @@ static int streamk_args_ok(const void* x, const void* wt, const void* y, const v
 }
 
 extern "C" int olmo355_w4_gemm_streamk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
-                                       uint16_t* y, int M, int N, int K, void* workspace, void* stream) {
+                                       uint16_t* y, int M, int N, int K, void* workspace, int64_t ws_bytes, int epoch, void* stream) {
   if (!st || !zt) return O355_EINVAL;
   if (const int rc = streamk_args_ok(x, wt, y, workspace, M, N, K)) return rc;
-  return launch_streamk<true, false>(x, wt, st, zt, y, M, N, K, workspace, kStreamKSpinLimit, 1, as_stream(stream));
+  return launch_streamk<true, false>(x, wt, st, zt, y, M, N, K, workspace, ws_bytes, epoch, kStreamKSpinLimit, 1, as_stream(stream));
 }
 
 extern "C" int olmo355_w4_gemm_swiglu_streamk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
-                                              uint16_t* y, int M, int N, int K, void* workspace, void* stream) {
+                                              uint16_t* y, int M, int N, int K, void* workspace, int64_t ws_bytes, int epoch, void* stream) {
   if (!st || !zt) return O355_EINVAL;
   if (const int rc = streamk_args_ok(x, wt, y, workspace, M, N, K)) return rc;
   if ((N & 255) || (int64_t)(N >> 4) * (K >> 7) * 1024 >= (1ll << 32)) return O355_EUNSUPPORTED;
-  return launch_streamk<true, true>(x, wt, st, zt, y, M, N, K, workspace, kStreamKSpinLimit, 1, as_stream(stream));
+  return launch_streamk<true, true>(x, wt, st, zt, y, M, N, K, workspace, ws_bytes, epoch, kStreamKSpinLimit, 1, as_stream(stream));
 }
 
 extern "C" int olmo355_b16_gemm_streamk(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K,
-                                        void* workspace, void* stream) {
+                                        void* workspace, int64_t ws_bytes, int epoch, void* stream) {
   if (const int rc = streamk_args_ok(x, wt, y, workspace, M, N, K)) return rc;
   return launch_streamk<false, false>(x, reinterpret_cast<const uint32_t*>(wt), nullptr, nullptr, y, M, N, K, workspace,
-                                      kStreamKSpinLimit, 1, as_stream(stream));
+                                      ws_bytes, epoch, kStreamKSpinLimit, 1, as_stream(stream));
 }
 
 // test hook: the finishing workgroups' patience and whether partials are announced at all
 extern "C" int olmo355_w4_gemm_streamk_patience(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
-                                             uint16_t* y, int M, int N, int K, void* workspace, int spin_limit, int publish,
-                                             void* stream) {
+                                             uint16_t* y, int M, int N, int K, void* workspace, int64_t ws_bytes, int epoch,
+                                             int spin_limit, int publish, void* stream) {
   if (!st || !zt || spin_limit < 0) return O355_EINVAL;
   if (const int rc = streamk_args_ok(x, wt, y, workspace, M, N, K)) return rc;
-  return launch_streamk<true, false>(x, wt, st, zt, y, M, N, K, workspace, spin_limit, publish, as_stream(stream));
+  return launch_streamk<true, false>(x, wt, st, zt, y, M, N, K, workspace, ws_bytes, epoch, spin_limit, publish, as_stream(stream));
 }
 
 extern "C" int olmo355_w4_gemm_splitk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,

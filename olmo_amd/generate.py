@@ -157,6 +157,7 @@ def greedy_generate(model, input_ids: torch.Tensor, attention_mask: Optional[tor
                 settle()
     settle()
     model.relay_check()
+    ops.streamk_check()  # a prefill GEMM that gave a tile up as NaN is an error here, not a silent bad token
     tokens = tokens[:, :steps]
     result = [tokens]
     after = None

@@ -143,10 +143,11 @@ def w4_linear(x: torch.Tensor, w: W4Tiled) -> torch.Tensor:
         check("olmo355_w4_gemv",
               lib().olmo355_w4_gemv(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream()))
     else:
-        ws = _streamk(M, w.N, w.K, x.device)
+        sk = _streamk(M, w.N, w.K, x.device)
         st = 2
-        if ws is not None:
-            st = lib().olmo355_w4_gemm_streamk(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _p(ws), _stream())
+        if sk is not None:
+            st = lib().olmo355_w4_gemm_streamk(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _p(sk[0]),
+                                               sk[0].numel(), sk[1], _stream())
             if st != 2:
                 check("olmo355_w4_gemm_streamk", st)
         if st == 2:
@@ -163,21 +164,41 @@ def _splitk(M: int, N: int, K: int) -> int:
     return int(lib().olmo355_gemm_splitk_plan(M, N, K)) if SPLITK else 1
 
 
-_streamk_ws = {}
+_streamk_ws = {}  # (device, stream) -> [workspace, epoch of its last launch]
 
 
 def _streamk(M: int, N: int, K: int, device: torch.device):
-    """The stream-K workspace to use for this shape on the current stream, or None when the tiled launch is the better
-    one.  One zeroed buffer per (device, stream), kept for the life of the process: launches that share it are
-    ordered on their stream, and every launch leaves its flags zero again."""
+    """``(workspace, epoch)`` for a stream-K launch of this shape on the current stream, or None when the tiled
+    launch is the better one.  One buffer per (device, stream), zeroed once and kept for the life of the process:
+    launches that share it are ordered on their stream, and each gets an epoch of its own (a counter that skips 0),
+    so flags left by an earlier launch, finished or not, never pass for this one's."""
     if not STREAMK or not lib().olmo355_gemm_streamk_plan(M, N, K):
         return None
+    if torch.cuda.is_current_stream_capturing():
+        return None  # a captured launch would replay its epoch, and the flags of the last replay would pass for news
     key = (device.index if device.index is not None else torch.cuda.current_device(), _stream())
-    ws = _streamk_ws.get(key)
-    if ws is None:
-        ws = torch.zeros(int(lib().olmo355_gemm_streamk_workspace_bytes()), dtype=torch.uint8, device=device)
-        _streamk_ws[key] = ws
-    return ws
+    slot = _streamk_ws.get(key)
+    if slot is None:
+        slot = [torch.zeros(int(lib().olmo355_gemm_streamk_workspace_bytes()), dtype=torch.uint8, device=device), 0]
+        _streamk_ws[key] = slot
+    slot[1] = slot[1] % 0x7FFFFFFF + 1
+    return slot[0], slot[1]
+
+
+def streamk_check() -> None:
+    """Raise if a stream-K launch issued through this module gave up waiting for a partial (its tile then holds NaN).
+    Reads one word per workspace back to the host (a synchronisation): for the end of a generation or a test, not
+    for the path between launches.  The word is cleared, so one failure is reported once."""
+    for (dev, _), (ws, _) in _streamk_ws.items():
+        word = ws.view(torch.int32)[STREAMK_STATUS_WORD]
+        epoch = int(word.item())
+        if epoch:
+            word.zero_()
+            raise RuntimeError(f"a stream-K GEMM on device {dev} gave up waiting for a partial (launch epoch {epoch}): "
+                               "its output holds NaN")
+
+
+STREAMK_STATUS_WORD = 513  # O355_STREAMK_STATUS_WORD of the C header
 
 
 # ---------------------------------------------------------------------------------------------
@@ -221,10 +242,11 @@ def b16_linear(x: torch.Tensor, w: B16Tiled) -> torch.Tensor:
             check("olmo355_b16_gemm_splitk",
                   lib().olmo355_b16_gemm_splitk(_p(x), _p(w.wt), _p(y), M, w.N, w.K, splits, _p(part), _stream()))
         else:
-            ws = _streamk(M, w.N, w.K, x.device)
+            sk = _streamk(M, w.N, w.K, x.device)
             st = 2
-            if ws is not None:
-                st = lib().olmo355_b16_gemm_streamk(_p(x), _p(w.wt), _p(y), M, w.N, w.K, _p(ws), _stream())
+            if sk is not None:
+                st = lib().olmo355_b16_gemm_streamk(_p(x), _p(w.wt), _p(y), M, w.N, w.K, _p(sk[0]), sk[0].numel(), sk[1],
+                                                    _stream())
                 if st != 2:
                     check("olmo355_b16_gemm_streamk", st)
             if st == 2:
@@ -262,11 +284,11 @@ def linear_fused(x: torch.Tensor, w, resid: Optional[torch.Tensor] = None, norm_
     x_new = rmsnorm(x, norm_w, eps, residual=resid) if resid is not None else x
     if swiglu_out and isinstance(w, W4Tiled) and M > GEMV_MAX_M:  # many rows: SwiGLU in the GEMM's epilogue
         y = torch.empty(*x.shape[:-1], n_out, dtype=torch.bfloat16, device=x.device)
-        ws = _streamk(M, w.N, w.K, x.device)
+        sk = _streamk(M, w.N, w.K, x.device)
         st = 2
-        if ws is not None:
-            st = lib().olmo355_w4_gemm_swiglu_streamk(_p(x_new), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _p(ws),
-                                                     _stream())
+        if sk is not None:
+            st = lib().olmo355_w4_gemm_swiglu_streamk(_p(x_new), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K,
+                                                     _p(sk[0]), sk[0].numel(), sk[1], _stream())
             if st not in (0, 2):
                 check("olmo355_w4_gemm_swiglu_streamk", st)
         if st == 2:
@@ -404,7 +426,8 @@ def attn_decode_relay(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache,
     if ws.numel() * ws.element_size() < int(lib().olmo355_attn_decode_workspace_bytes(1, H, hd, n_keys_max)):
         raise ValueError("attention workspace too small")
     st = lib().olmo355_attn_decode_relay(_p(qkv), _p(q_weight), _p(k_weight), _p(sin_tab), _p(cos_tab), _p(kcache), _p(vcache),
-                                         _p(key_bias), _p(out), _p(ws), 1, H, Hkv, hd, Lmax, n_pos, past_len, _p(past_len_dev),
+                                         _p(key_bias), _p(out), _p(ws), _nbytes(ws), 1, H, Hkv, hd, Lmax, n_pos, past_len,
+                                         _p(past_len_dev),
                                          n_keys_max, key_bias.shape[1] if key_bias is not None else 0, float(eps), _p(qk_ssq),
                                          _p(rope_now), _p(epoch), _p(status), _p(hint_in), _p(hint_out), _spins(spin_limit),
                                          _stream() if stream is None else stream)
@@ -706,6 +729,10 @@ def attn_prefill(q, kcache, vcache, B: int, T: int, H: int, Hkv: int, hd: int, p
     return out
 
 
+def _nbytes(t: torch.Tensor) -> int:
+    return t.numel() * t.element_size()
+
+
 def attn_decode_workspace(B: int, H: int, hd: int, n_keys_max: int, device) -> torch.Tensor:
     n = int(lib().olmo355_attn_decode_workspace_bytes(B, H, hd, n_keys_max))
     return torch.zeros(n // 4, dtype=torch.float32, device=device)  # the ticket counters at its start begin at zero
@@ -728,13 +755,13 @@ def attn_decode(q, kcache, vcache, ws, B: int, H: int, Hkv: int, hd: int, past_l
         if beam_src.dtype != torch.int32 or beam_src.dim() != 2 or beam_src.shape[0] != B or not beam_src.is_contiguous():
             raise ValueError("beam_src: contiguous int32 [B, steps] expected")
         check("olmo355_attn_decode_beam",
-              lib().olmo355_attn_decode_beam(_p(q), _p(kcache), _p(vcache), _p(key_bias), _p(out), _p(ws), B, H, Hkv, hd,
+              lib().olmo355_attn_decode_beam(_p(q), _p(kcache), _p(vcache), _p(key_bias), _p(out), _p(ws), _nbytes(ws), B, H, Hkv, hd,
                                              Lmax, past_len, _p(past_len_dev), n_keys_max,
                                              key_bias.shape[1] if key_bias is not None else 0, _p(beam_src),
                                              beam_src.shape[1], int(prompt_len), int(beam), _dt(q), _stream()))
         return out
     check("olmo355_attn_decode",
-          lib().olmo355_attn_decode(_p(q), _p(kcache), _p(vcache), _p(key_bias), _p(out), _p(ws), B, H, Hkv, hd, Lmax,
+          lib().olmo355_attn_decode(_p(q), _p(kcache), _p(vcache), _p(key_bias), _p(out), _p(ws), _nbytes(ws), B, H, Hkv, hd, Lmax,
                                     past_len, _p(past_len_dev), n_keys_max,
                                     key_bias.shape[1] if key_bias is not None else 0, _dt(q), _stream()))
     return out
@@ -762,7 +789,7 @@ def attn_decode_fused(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcache,
         raise ValueError("attention workspace too small")
     out = torch.empty(B, 1, H * hd, dtype=qkv.dtype, device=qkv.device)
     args = (_p(qkv), _p(q_weight), _p(k_weight), _p(sin_tab), _p(cos_tab), _p(kcache), _p(vcache), _p(key_bias), _p(out),
-            _p(ws), B, H, Hkv, hd, Lmax, n_pos, past_len, _p(past_len_dev), n_keys_max,
+            _p(ws), _nbytes(ws), B, H, Hkv, hd, Lmax, n_pos, past_len, _p(past_len_dev), n_keys_max,
             key_bias.shape[1] if key_bias is not None else 0, float(eps), _p(qk_ssq), _p(rope_now), _dt(qkv))
     if merge == -1:
         st = lib().olmo355_attn_decode_fused(*args, _stream())

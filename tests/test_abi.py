@@ -58,6 +58,39 @@ def test_argument_checks_return_status_without_launching():
     assert h.olmo355_attn_decode_workspace_bytes(1, 32, 128, 2048) == 32 * 16 * 130 * 8 + 32 * 8
 
 
+def test_sized_workspaces_are_checked_before_any_device_call():
+    """Every entry that writes into a caller's workspace takes its size and refuses one that is too small with
+    O355_EINVAL before touching the device (so this runs without a GPU; the pointers are never dereferenced).  The
+    same calls with the full size are the GPU tests' business."""
+    import ctypes
+
+    from olmo_amd import _lib
+
+    h = _lib.lib()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    B, H, Hkv, hd, Lmax, keys = 2, 32, 32, 128, 4096, 2048
+    need = h.olmo355_attn_decode_workspace_bytes(B, H, hd, keys)
+    assert need > 0
+    for short in (0, need - 1):
+        assert h.olmo355_attn_decode(p, p, p, None, p, p, short, B, H, Hkv, hd, Lmax, 10, None, keys, 0, 0, None) == 1
+        assert h.olmo355_attn_decode_beam(p, p, p, None, p, p, short, B, H, Hkv, hd, Lmax, 10, None, keys, 0, p, Lmax, 0, 2,
+                                          0, None) == 1
+        assert h.olmo355_attn_decode_fused(p, None, None, p, p, p, p, None, p, p, short, B, H, Hkv, hd, Lmax, Lmax, 10, None,
+                                           keys, 0, 1e-6, None, None, 0, None) == 1
+        assert h.olmo355_attn_decode_fused_merge(p, None, None, p, p, p, p, None, p, p, short, B, H, Hkv, hd, Lmax, Lmax, 10,
+                                                 None, keys, 0, 1e-6, None, None, 0, 2, None) == 1
+        assert h.olmo355_attn_decode_relay(p, None, None, p, p, p, p, None, p, p, short // B, 1, H, Hkv, hd, Lmax, Lmax, 10, None,
+                                           keys, 0, 1e-6, None, None, p, p, None, None, 16, None) == 1
+    need = h.olmo355_gemm_streamk_workspace_bytes()
+    assert need == 4096 + 256 * 256 * 256 * 4
+    for short, epoch in ((0, 1), (need - 1, 1), (need, 0)):  # epoch 0 is the value of a workspace never written: refused
+        assert h.olmo355_w4_gemm_streamk(p, p, p, p, p, 2048, 12288, 4096, p, short, epoch, None) == 1
+        assert h.olmo355_w4_gemm_swiglu_streamk(p, p, p, p, p, 2048, 22016, 4096, p, short, epoch, None) == 1
+        assert h.olmo355_b16_gemm_streamk(p, p, p, 2048, 12288, 4096, p, short, epoch, None) == 1
+        assert h.olmo355_w4_gemm_streamk_patience(p, p, p, p, p, 2048, 12288, 4096, p, short, epoch, 4, 0, None) == 1
+
+
 def test_gemm_plans_are_host_arithmetic():
     """Which form a large-M product takes is decided on the host from the shape alone; the decisions that the 7B
     prefill rests on (measured: see the comments at the plan functions), kept from drifting."""

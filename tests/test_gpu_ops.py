@@ -287,6 +287,9 @@ def test_w4_gemm_every_tile_width(dev, width, M, N, K):
     assert (y.float().cpu() - ref).abs().max().item() <= 2 ** -7 * scale
 
 
+STREAMK_STATUS_WORD = 513  # O355_STREAMK_STATUS_WORD of include/olmo355.h
+
+
 def _streamk_ws(dev):
     from olmo_amd import _lib
     return torch.zeros(_lib.lib().olmo355_gemm_streamk_workspace_bytes(), dtype=torch.uint8, device=dev)
@@ -297,8 +300,9 @@ def _streamk_ws(dev):
 def test_w4_gemm_streamk(dev, M, N, K):
     """The stream-K form against the oracle on shapes where a tile's K is shared by four workgroups (one unit of 256
     per CU), by two with uneven pieces, by none (256 tiles of two units: one whole tile per CU), with ragged M and N,
-    and with 1.5 tiles per CU; the flags are zero again afterwards and a second launch on the same
-    workspace gives the same bits."""
+    and with 1.5 tiles per CU; a second launch on the same workspace, which still holds every flag of the first, with
+    the next epoch gives the same bits, and so does a third on a workspace whose flag words were all overwritten with
+    a stale epoch (what a launch that was cut short would leave)."""
     say("w4_gemm_streamk", M, N, K)
     from olmo_amd import _lib
     ops = _ops()
@@ -310,15 +314,23 @@ def test_w4_gemm_streamk(dev, M, N, K):
     ws = _streamk_ws(dev)
     s = torch.cuda.current_stream().cuda_stream
     ys = []
-    for _ in range(2):
+    words = ws.view(torch.int32)
+    for epoch in (1, 2, 9):
+        if epoch == 9:
+            words[:256] = 8  # every hand-over flag left up by an earlier launch
         y = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=dev)
         st = _lib.lib().olmo355_w4_gemm_streamk(xd.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y.data_ptr(),
-                                                M, N, K, ws.data_ptr(), s)
+                                                M, N, K, ws.data_ptr(), ws.numel(), epoch, s)
         torch.cuda.synchronize()
         assert st == 0
-        assert not ws[:4096].any()
+        assert words[STREAMK_STATUS_WORD].item() == 0
+        assert set(words[:256].unique().tolist()) <= {0, 8, epoch - 1, epoch}  # flags hold epochs; nothing is cleaned
         ys.append(y)
-    assert torch.equal(ys[0], ys[1])
+    assert torch.equal(ys[0], ys[1]) and torch.equal(ys[0], ys[2])
+    # a workspace that is too small, or epoch 0, is refused before anything is launched
+    args = (xd.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), ys[0].data_ptr(), M, N, K, ws.data_ptr())
+    assert _lib.lib().olmo355_w4_gemm_streamk(*args, ws.numel() - 1, 10, s) == 1
+    assert _lib.lib().olmo355_w4_gemm_streamk(*args, ws.numel(), 0, s) == 1
     scale = ref.abs().max().item()
     assert (ys[0].float().cpu() - ref).abs().max().item() <= 2 ** -7 * scale
     # against the tiled launch: the same fp32 products added in another order
@@ -345,18 +357,19 @@ def test_w4_gemm_swiglu_streamk_and_dense_streamk(dev):
     y1 = torch.full_like(y0, float("nan"))
     assert L.olmo355_w4_gemm_swiglu(x.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y0.data_ptr(), M, N, K, s) == 0
     assert L.olmo355_w4_gemm_swiglu_streamk(x.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y1.data_ptr(), M, N, K,
-                                            ws.data_ptr(), s) == 0
+                                            ws.data_ptr(), ws.numel(), 1, s) == 0
     torch.cuda.synchronize()
     a, b = y1.float(), y0.float()
     # silu(gate) * up of two bf16-rounded factors: one rounding step of either factor moves the product by 2^-7
     assert ((a - b).abs() <= 2 ** -6 * torch.maximum(a.abs(), b.abs()) + 2 ** -14 * b.abs().max()).all()
-    assert not ws[:4096].any()
+    assert ws.view(torch.int32)[STREAMK_STATUS_WORD].item() == 0
     w = (torch.randn(N, K, generator=torch.Generator().manual_seed(13)) * 0.02).to(torch.bfloat16).to(dev)
     tw = ops.b16_repack(w)
     z0 = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
     z1 = torch.full_like(z0, float("nan"))
     assert L.olmo355_b16_gemm(x.data_ptr(), tw.wt.data_ptr(), z0.data_ptr(), M, N, K, s) == 0
-    assert L.olmo355_b16_gemm_streamk(x.data_ptr(), tw.wt.data_ptr(), z1.data_ptr(), M, N, K, ws.data_ptr(), s) == 0
+    assert L.olmo355_b16_gemm_streamk(x.data_ptr(), tw.wt.data_ptr(), z1.data_ptr(), M, N, K, ws.data_ptr(), ws.numel(), 2,
+                                      s) == 0
     torch.cuda.synchronize()
     a, b = z1.float(), z0.float()
     assert ((a - b).abs() <= 2 ** -7 * torch.maximum(a.abs(), b.abs()) + 2 ** -16 * b.abs().max()).all()
@@ -367,7 +380,8 @@ def test_w4_gemm_swiglu_streamk_and_dense_streamk(dev):
 def test_w4_gemm_streamk_gives_up_instead_of_hanging(dev):
     """With the partials' owners told not to raise their flags (a host-side switch of the variant entry) and a
     patience of four polls, every finishing workgroup gives its tile up as NaN, the tiles that were never shared are
-    right, the launch ends, and the workspace needs no cleaning (no flag was raised)."""
+    right, the launch ends with its epoch in the status word, and the next launch on the same workspace, not cleaned,
+    is right."""
     say("w4_gemm_streamk give-up")
     from olmo_amd import _lib
     ops = _ops()
@@ -380,10 +394,10 @@ def test_w4_gemm_streamk_gives_up_instead_of_hanging(dev):
     s = torch.cuda.current_stream().cuda_stream
     y = torch.zeros(M, N, dtype=torch.bfloat16, device=dev)
     st = L.olmo355_w4_gemm_streamk_patience(x.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y.data_ptr(),
-                                            M, N, K, ws.data_ptr(), 4, 0, s)
+                                            M, N, K, ws.data_ptr(), ws.numel(), 5, 4, 0, s)
     torch.cuda.synchronize()
     assert st == 0
-    assert not ws[:4096].any()
+    assert ws.view(torch.int32)[STREAMK_STATUS_WORD].item() == 5
     y0 = torch.empty_like(y)
     assert L.olmo355_w4_gemm(x.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y0.data_ptr(), M, N, K, s) == 0
     torch.cuda.synchronize()
@@ -394,6 +408,14 @@ def test_w4_gemm_streamk_gives_up_instead_of_hanging(dev):
     assert (nan_tiles | clean).all()                     # a tile is given up whole or not at all
     assert nan_tiles.sum().item() == 128 and clean.sum().item() == 256
     assert torch.equal(tiles[clean], ref_tiles[clean])   # whole tiles: the same additions in the same order as the tiled launch
+    # the workspace as the failed launch left it serves the next one
+    y2 = torch.full_like(y, float("nan"))
+    assert L.olmo355_w4_gemm_streamk(x.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), y2.data_ptr(), M, N, K,
+                                     ws.data_ptr(), ws.numel(), 6, s) == 0
+    torch.cuda.synchronize()
+    a, b = y2.float(), y0.float()
+    assert ((a - b).abs() <= 2 ** -7 * torch.maximum(a.abs(), b.abs()) + 2 ** -16 * b.abs().max()).all()
+    assert ws.view(torch.int32)[STREAMK_STATUS_WORD].item() == 5  # kept until its reader clears it
 
 
 def test_gemm_rejects_misaligned_output(dev):

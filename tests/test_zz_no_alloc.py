@@ -23,8 +23,8 @@ def _case(L, dev, B, H, Hkv, hd, Lctx, seed, dtype=torch.bfloat16):
     s = torch.cuda.current_stream().cuda_stream
     dt = 1 if dtype == torch.bfloat16 else 0
     print("no_alloc case", B, H, Hkv, hd, Lctx, flush=True)
-    assert L.olmo355_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), None, ref.data_ptr(), ws.data_ptr(), B, H, Hkv,
-                                 hd, Lmax, 0, pos.data_ptr(), Lmax, 0, dt, s) == 0
+    assert L.olmo355_attn_decode(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), None, ref.data_ptr(), ws.data_ptr(),
+                                 ws.numel() * ws.element_size(), B, H, Hkv, hd, Lmax, 0, pos.data_ptr(), Lmax, 0, dt, s) == 0
     free_before = torch.cuda.mem_get_info()[0]
     assert L.olmo355_attn_decode_static(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), None, out.data_ptr(), B, H, Hkv, hd, Lmax,
                                         0, pos.data_ptr(), Lmax, 0, dt, s) == 0
