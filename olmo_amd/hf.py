@@ -340,20 +340,52 @@ class OLMoForCausalLM(*_ModelBase):
     _CAPTURED_ARGS = frozenset(("attention_mask", "max_new_tokens", "do_sample", "num_beams", "eos_token_id",
                                 "pad_token_id", "use_graph", "temperature", "top_k", "top_p", "seed"))
 
+    def _route(self, input_ids, args, kwargs) -> Tuple[str, Dict[str, Any]]:
+        """Which loop a ``generate`` call without ``loop=`` takes, and with which arguments.  HF's ``generate`` is the
+        reference wrapper's (``hf_olmo/modeling_olmo.py`` inherits it), so whatever the captured loop would do
+        differently goes to transformers: anything but plain greedy decoding of a given number of new tokens
+        (sampling draws from another random stream, ``num_beams > 1`` is HF's length-normalised search there and
+        OLMo's own here), several end tokens, arguments the captured loop does not know.  For the calls it keeps, the
+        captured loop takes the end and padding tokens from ``generation_config`` where the call does not name
+        them, as HF does, and ends once every sequence has ended."""
+        if not HAVE_TRANSFORMERS:
+            return "captured", kwargs
+        gc = getattr(self, "generation_config", None)
+        if input_ids is None or args or not set(kwargs) <= self._CAPTURED_ARGS or "max_new_tokens" not in kwargs:
+            return "transformers", kwargs
+
+        def setting(name, default):
+            if name in kwargs:
+                return kwargs[name]
+            return default if gc is None or getattr(gc, name, None) is None else getattr(gc, name)
+
+        if setting("do_sample", False) or setting("num_beams", 1) != 1:
+            return "transformers", kwargs
+        eos = setting("eos_token_id", None)
+        if isinstance(eos, (list, tuple)):
+            if len(eos) > 1:
+                return "transformers", kwargs
+            eos = eos[0] if eos else None
+        filled = dict(kwargs, eos_token_id=eos, pad_token_id=setting("pad_token_id", None))
+        return "captured", filled
+
     @torch.no_grad()
     def generate(self, input_ids: Optional[torch.LongTensor] = None, *args, loop: Optional[str] = None, **kwargs):
         """Continuation ``[B, prompt + new tokens]`` like HF ``generate``.
 
-        ``loop="captured"``: this package's loop -- prefill, then one captured decode step per token, greedy or
+        ``loop="transformers"``: ``GenerationMixin.generate`` with all of its arguments, calling ``forward`` once per
+        token.  ``loop="captured"``: this package's loop -- prefill, then one captured decode step per token, greedy or
         sampled on the device (temperature, top-k, top-p in HF's order; ``top_k=0`` / ``top_p=1.0`` switch a filter
         off; ``seed`` fixes the draw); ``num_beams > 1`` runs OLMo's own beam search (``olmo/beam_search.py``: summed
         log-probabilities, no length penalty, the best beam, fewer than ``max_new_tokens`` columns when every beam
-        ended early).  ``loop="transformers"``: ``GenerationMixin.generate`` with all of its arguments, calling
-        ``forward`` once per token.  Default: the captured loop when it understands every argument given,
-        transformers' otherwise."""
+        ended early) -- named explicitly, it does exactly what its arguments say and reads nothing from
+        ``generation_config``.  Default (see :meth:`_route`): the captured loop for plain greedy decoding, where it
+        returns the tokens HF's loop would (end and padding tokens from ``generation_config``), transformers'
+        loop for everything else."""
         if loop is None:
-            simple = input_ids is not None and not args and set(kwargs) <= self._CAPTURED_ARGS
-            loop = "captured" if (simple or not HAVE_TRANSFORMERS) else "transformers"
+            loop, kwargs = self._route(input_ids, args, kwargs)
+            if loop == "captured" and HAVE_TRANSFORMERS:
+                kwargs["_hf_stop"] = True
         if loop == "transformers":
             if not HAVE_TRANSFORMERS:
                 raise RuntimeError("transformers is not importable")
@@ -363,7 +395,7 @@ class OLMoForCausalLM(*_ModelBase):
             return super().generate(input_ids, *args, **kwargs)
         if loop != "captured":
             raise ValueError(f"loop must be 'captured' or 'transformers', not {loop!r}")
-        unknown = set(kwargs) - self._CAPTURED_ARGS
+        unknown = set(kwargs) - self._CAPTURED_ARGS - {"_hf_stop"}
         if args or unknown:
             raise TypeError(f"the captured loop does not take {sorted(unknown) or 'positional arguments'}")
         return self._generate_captured(input_ids, **kwargs)
@@ -371,7 +403,8 @@ class OLMoForCausalLM(*_ModelBase):
     def _generate_captured(self, input_ids: torch.LongTensor, attention_mask: Optional[torch.Tensor] = None,
                            max_new_tokens: int = 20, do_sample: bool = False, num_beams: int = 1,
                            eos_token_id: Optional[int] = None, pad_token_id: Optional[int] = None, use_graph: bool = True,
-                           temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0) -> torch.Tensor:
+                           temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0, seed: int = 0,
+                           _hf_stop: bool = False) -> torch.Tensor:
         if num_beams != 1:
             sampler = None
             if do_sample:  # per-node candidates drawn instead of taken from the top (olmo/beam_search.py samplers)
@@ -388,7 +421,8 @@ class OLMoForCausalLM(*_ModelBase):
             return torch.cat((input_ids.to(out.token_ids.device), out.token_ids[:, 0]), dim=1)
         sampling = dict(temperature=temperature, top_k=top_k or 0, top_p=top_p, seed=seed) if do_sample else None
         new = greedy_generate(self.model, input_ids, attention_mask, max_new_tokens, use_graph=use_graph,
-                              eos_token_id=eos_token_id, pad_token_id=pad_token_id, sampling=sampling)
+                              eos_token_id=eos_token_id, pad_token_id=pad_token_id, sampling=sampling,
+                              stop_when_all_ended=_hf_stop)
         return torch.cat((input_ids.to(new.device), new), dim=1)
 
     # ------------------------------------------------------------------------------------------

@@ -416,7 +416,7 @@ def test_generate_with_beams_bf16_consistency(dev):
         from olmo_amd.hf import OLMoConfig, OLMoForCausalLM
 
         hf = OLMoForCausalLM(OLMoConfig.from_model_config(cfg), model=model)
-        assert torch.equal(hf.generate(ids, max_new_tokens=6, num_beams=4), torch.cat([ids, out.token_ids[:, 0]], dim=1))
+        assert torch.equal(hf.generate(ids, max_new_tokens=6, num_beams=4, loop="captured"), torch.cat([ids, out.token_ids[:, 0]], dim=1))
         for b in range(B):
             assert abs(teacher_forced(b, one.token_ids[b, 0]) - one.scores[b, 0].item()) < 0.05 * T
             for j in range(K):

@@ -251,8 +251,8 @@ def test_hf_wrapper_and_greedy_generate(dev, quantized):
     with pytest.raises(ValueError):
         hf(ids, output_attentions=True)
     steps = 128
-    g = hf.generate(ids, max_new_tokens=steps, use_graph=True)
-    e = hf.generate(ids, max_new_tokens=steps, use_graph=False)
+    g = hf.generate(ids, max_new_tokens=steps, use_graph=True, loop="captured")
+    e = hf.generate(ids, max_new_tokens=steps, use_graph=False, loop="captured")
     assert g.shape == (4, 40 + steps) and torch.equal(g[:, :40], ids)
     assert torch.equal(g, e), "graph replay differs from eager decode"
     # step-by-step through the HF forward with prepare_inputs_for_generation
@@ -759,7 +759,7 @@ def test_sampled_generation(dev):
     model, _ = build_pair(cfg, torch.bfloat16, dev, seed=11)
     hf = OLMoForCausalLM(OLMoConfig.from_model_config(cfg), model=model)
     ids = torch.randint(0, cfg.vocab_size, (3, 9), generator=torch.Generator().manual_seed(1)).to(dev)
-    kw = dict(max_new_tokens=12, do_sample=True, temperature=1.5, top_k=50, top_p=0.95, seed=42)
+    kw = dict(max_new_tokens=12, do_sample=True, temperature=1.5, top_k=50, top_p=0.95, seed=42, loop="captured")
     a = hf.generate(ids, use_graph=True, **kw)
     b = hf.generate(ids, use_graph=False, **kw)
     assert a.shape == (3, 21) and torch.equal(a, b)

@@ -176,6 +176,36 @@ def test_prepare_inputs_for_generation():
     assert torch.equal(inp["input_ids"], ids[:, 8:11]) and "next_sequence_length" not in inp
 
 
+def test_default_loop_is_the_captured_one_only_where_it_decodes_as_transformers_would():
+    """A ``generate`` call that names no loop: plain greedy decoding of a stated number of tokens goes to the captured
+    loop with the end and padding tokens of ``generation_config`` filled in; sampling, beams, a default length, several
+    end tokens or any argument the captured loop does not know go to transformers' loop."""
+    case, seed, ours, _, _ = wrapped("olmo1")
+    ids, _ = R.inputs(case, seed)
+    gc = ours.generation_config
+    gc.eos_token_id, gc.pad_token_id = 7, 3
+    loop, kw = ours._route(ids, (), dict(max_new_tokens=4))
+    assert loop == "captured" and kw["eos_token_id"] == 7 and kw["pad_token_id"] == 3
+    loop, kw = ours._route(ids, (), dict(max_new_tokens=4, eos_token_id=None, pad_token_id=9))
+    assert loop == "captured" and kw["eos_token_id"] is None and kw["pad_token_id"] == 9
+    gc.eos_token_id = [7]
+    assert ours._route(ids, (), dict(max_new_tokens=4))[1]["eos_token_id"] == 7
+    gc.eos_token_id = [7, 8]
+    assert ours._route(ids, (), dict(max_new_tokens=4))[0] == "transformers"
+    gc.eos_token_id = 7
+    for kw in (dict(), dict(max_new_tokens=4, do_sample=True), dict(max_new_tokens=4, num_beams=2),
+               dict(max_new_tokens=4, repetition_penalty=1.1), dict(max_length=30)):
+        assert ours._route(ids, (), kw)[0] == "transformers", kw
+    gc.do_sample = True
+    assert ours._route(ids, (), dict(max_new_tokens=4))[0] == "transformers"
+    gc.do_sample = False
+    assert ours._route(None, (), dict(max_new_tokens=4))[0] == "transformers"
+    # on the CPU model of this file the default route must therefore be runnable for a sampled call: transformers' loop
+    gc.eos_token_id = None
+    out = ours.generate(ids[:, :6], attention_mask=torch.ones_like(ids[:, :6]), max_new_tokens=3, do_sample=True, top_k=5)
+    assert out.shape == (ids.shape[0], 9)
+
+
 def test_captured_loop_rejects_what_it_does_not_know():
     case, seed, ours, _, _ = wrapped("olmo1")
     ids, _ = R.inputs(case, seed)
@@ -212,8 +242,25 @@ def test_gpu_transformers_loops_match_independent_model_and_captured_loop(name):
     want = theirs.generate(ids, attention_mask=mask, **kw)
     got = ours.generate(ids.cuda(), attention_mask=mask.cuda(), loop="transformers", **kw)
     assert torch.equal(got.cpu(), want)
-    cap = ours.generate(ids.cuda(), attention_mask=mask.cuda(), max_new_tokens=12)  # the captured loop
+    assert ours._route(ids, (), dict(kw, attention_mask=mask))[0] == "captured"
+    cap = ours.generate(ids.cuda(), attention_mask=mask.cuda(), **kw)  # no loop named: the captured one
     assert torch.equal(cap.cpu(), want)
+    # an end token that does occur, set where HF keeps it (generation_config), named by neither call: both loops stop
+    # a sequence there, pad after it and end once every sequence has ended, and give what the independent model gives
+    new = want[:, ids.shape[1]:]
+    eos = int(new[0, 3])
+    for m in (ours, theirs):
+        m.generation_config.eos_token_id, m.generation_config.pad_token_id = eos, 0
+    want_e = theirs.generate(ids, attention_mask=mask, max_new_tokens=12)
+    assert (want_e[0, ids.shape[1]:] == eos).sum() == 1 and (want_e[0, ids.shape[1]:] == 0).any()
+    via_hf = ours.generate(ids.cuda(), attention_mask=mask.cuda(), max_new_tokens=12, loop="transformers")
+    default = ours.generate(ids.cuda(), attention_mask=mask.cuda(), max_new_tokens=12)
+    assert torch.equal(via_hf.cpu(), want_e) and torch.equal(default.cpu(), want_e)
+    one = ours.generate(ids[:1].cuda(), attention_mask=mask[:1].cuda(), max_new_tokens=12)  # ends early: cut after the end token
+    assert torch.equal(one.cpu(), theirs.generate(ids[:1], attention_mask=mask[:1], max_new_tokens=12))
+    assert one.shape[1] < ids.shape[1] + 12
+    for m in (ours, theirs):
+        m.generation_config.eos_token_id = None
     kw = dict(max_new_tokens=10, num_beams=3, do_sample=False, eos_token_id=None, length_penalty=1.0, early_stopping=False)
     want = theirs.generate(ids[:2, 11:], attention_mask=torch.ones_like(ids[:2, 11:]), **kw)
     got = ours.generate(ids[:2, 11:].cuda(), attention_mask=torch.ones_like(ids[:2, 11:]).cuda(), loop="transformers", **kw)
