@@ -88,13 +88,15 @@ int olmo355_w4_gemv_fused(const uint16_t* x, const uint16_t* resid, const uint16
                           uint16_t* x_out, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
                           int M, int N, int K, int swiglu, void* stream);
 
-/* olmo355_w4_gemv_fused for M <= 4 with the norms chained between launches: RMSNorm needs the sum
+/* olmo355_w4_gemv_fused for M <= 8 with the norms chained between launches: RMSNorm needs the sum
  * of squares of a whole row, and the launch that *produces* that row can leave it behind per 16-column
  * tile, so the consumer's prologue neither re-reads the row nor synchronises its workgroup.
  *   ssq_out != NULL (swiglu == 0): ssq_out[m][N/16] = sum of squares of the bf16 outputs of row m, per tile;
  *   resid != NULL: ssq_in[m][K/16] (left by the launch that wrote x) must be given; x' as above.
  * Used for the three norms of a decode block (olmo/model.py:786-794 attention/MLP post-norms and the
- * full-width QK-norm of :711-716 via olmo355_attn_decode_fused).  O355_EUNSUPPORTED: use the calls above. */
+ * full-width QK-norm of :711-716 via olmo355_attn_decode_fused).  Up to 4 rows keep the activations in LDS; 5 to 8 rows
+ * take them as matrix-core operand fragments straight from memory (no size limit from LDS; K up to 12288 without a
+ * prologue, 8192 with one).  O355_EUNSUPPORTED: use the calls above. */
 int olmo355_w4_gemv_chain(const uint16_t* x, const uint16_t* resid, const uint16_t* norm_w, float eps, uint16_t* x_out,
                           const float* ssq_in, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
                           float* ssq_out, int M, int N, int K, int swiglu, void* stream);

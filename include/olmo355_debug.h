@@ -31,6 +31,12 @@ int olmo355_w4_gemm_streamk_patience(const uint16_t* x, const uint32_t* wt, cons
 int olmo355_w4_gemv_form(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
                          int M, int N, int K, int form, void* stream);
 
+/* olmo355_w4_gemv_chain through the kernel for 5 to 8 rows (any M <= 8 is accepted here) with the column tiles per
+ * workgroup (nt: 1, 2 or 3; with swiglu 2 or 4; 0 = choose) and the waves per workgroup (8, 16; 0 = choose) given. */
+int olmo355_w4_gemv_r8_form(const uint16_t* x, const uint16_t* resid, const uint16_t* norm_w, float eps, uint16_t* x_out,
+                            const float* ssq_in, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y,
+                            float* ssq_out, int M, int N, int K, int swiglu, int nt, int waves, void* stream);
+
 /* olmo355_attn_decode_fused with the merge of a head's key chunks given: -1 = choose, 0 = in the kernel (the last
  * workgroup of a (batch, head) to finish, found by a ticket drawn after its stores have landed), 1 = in the kernel by
  * the workgroup of the head's last chunk, which polls flag words stored together with the numbers (the writers

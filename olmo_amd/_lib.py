@@ -99,6 +99,7 @@ VARIANT_EXPORTS = {
     "olmo355_b16_gemm_tile": (I, [P, P, P, I, I, I, I, P]),
     "olmo355_w4_gemm_streamk_patience": (I, [P, P, P, P, P, I, I, I, P, L, I, I, I, P]),
     "olmo355_w4_gemv_form": (I, [P, P, P, P, P, I, I, I, I, P]),
+    "olmo355_w4_gemv_r8_form": (I, [P, P, P, F, P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
     "olmo355_attn_decode_fused_merge": (I, [P, P, P, P, P, P, P, P, P, P, L, I, I, I, I, I, I, I, P, I, I, F, P, P, I, I, P]),
 }
 

@@ -709,12 +709,19 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   }
   float sq = 0.f, sk = 0.f;
   u32x4 qrow[QV], krow[QV];
+  f32x4 ssq_q[2], ssq_k[2];  // added up where the scale factors are formed, after the cache rows have been asked for
   if (norm && !RELAY) {
-    if (qk_ssq) {  // per-tile partials left by the projection: wave 0 alone adds them up
+    if (qk_ssq) {
+      // per-tile partials left by the projection: wave 0 alone adds them up.  At most 512 per row (H * HD <= 8192):
+      // two 16-byte requests per lane and row, all four on their way at once (a loop of single loads is a chain of
+      // round trips to L2 ahead of the cache rows: 8 us per launch at batch 8), zeros past the row's end
       if (wave == 0) {
         const float* pr = qk_ssq + (int64_t)b * ((dq + 2 * dk) >> 4);
-        for (int i = lane; i < (dq >> 4); i += 64) sq += pr[i];
-        for (int i = lane; i < (dk >> 4); i += 64) sk += pr[(dq >> 4) + i];
+        const __amdgpu_buffer_rsrc_t rpq = make_rsrc(pr, (int64_t)(dq >> 4) * 4), rpk = make_rsrc(pr + (dq >> 4), (int64_t)(dk >> 4) * 4);
+        ssq_q[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rpq, lane * 16, 0, 0));
+        ssq_q[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rpq, lane * 16 + 1024, 0, 0));
+        ssq_k[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rpk, lane * 16, 0, 0));
+        ssq_k[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rpk, lane * 16 + 1024, 0, 0));
       }
     } else {
 #pragma unroll
@@ -852,6 +859,10 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   if (norm) {
     if (qk_ssq) {
       if (wave == 0) {
+        if constexpr (!RELAY) {
+          sq = ((ssq_q[0][0] + ssq_q[0][1]) + (ssq_q[0][2] + ssq_q[0][3])) + ((ssq_q[1][0] + ssq_q[1][1]) + (ssq_q[1][2] + ssq_q[1][3]));
+          sk = ((ssq_k[0][0] + ssq_k[0][1]) + (ssq_k[0][2] + ssq_k[0][3])) + ((ssq_k[1][0] + ssq_k[1][1]) + (ssq_k[1][2] + ssq_k[1][3]));
+        }
         sq = wave_sum(sq), sk = wave_sum(sk);
         rq = 1.f / sqrtf(sq / (float)dq + eps);
         rk_ = 1.f / sqrtf(sk / (float)dk + eps);

@@ -835,6 +835,295 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_small_kernel(GemvArgs args
   w4_gemv_small_body<GPA, NT, WAVES, PRO, EPI>(args, wt, st, zt);
 }
 
+// ---- int4, 5 .. 8 rows: the activations as operand fragments, never whole in LDS ------------------------------
+// With eight rows the two groups of 128 that share a matrix instruction fill its 16 operand rows exactly
+// (rows 0-7: group g, rows 8-15: group g + 1), so a wave keeps the fragments of its own run of K in registers: no
+// copy of all of x in LDS (eight rows of K = 11008 would not fit), no zero row, no barrier before the first product,
+// and all of a wave's requests -- weights, scales, activations -- leave before anything is waited for.  The rows
+// are asked for as they lie in memory (half a wave per row, 16 bytes per lane: a lane of the operand layout would ask
+// for 16 bytes of a line of its own, and the texture path handles a quad of lanes at a time) and turned into
+// fragments through 4 KiB of LDS that belong to the wave alone (written and read by the same wave, in order, so
+// without a barrier; blocks of 256 bytes 272 apart, so that both the writes and the fragment reads touch every
+// bank once).  The operand is shared by both groups, so group g's weights also multiply rows 8-15 (and the other way
+// round): each group of the pair accumulates into registers of its own and a lane keeps the half that means
+// something (rows 0-7 of the first, 8-15 of the second) when scale and zero are applied.  A workgroup owns NT
+// column tiles (NT / 2 up-and-gate pairs with the SwiGLU epilogue) and all of K, split over its waves in runs of at
+// most PMAX pairs of groups.
+// PRO: the chained norm prologue x := resid + rmsnorm(a; w, eps): wave r adds up the sums of squares of row r
+// and leaves 1 / rms in LDS (the one barrier, while everything else is in flight), and a lane normalises the pieces
+// it has asked for before they go through LDS; workgroup 0 writes x_out.
+constexpr int kR8BlockBytes = 272, kR8WaveBytes = 16 * kR8BlockBytes;
+
+template <int NT, int PMAX>
+struct R8Weights {  // one set of NT column tiles over a wave's run of K: packed pieces, scales, zeros as they arrive
+  u32x4 w[PMAX][2][NT];
+  uint32_t s16[PMAX][NT], z8[PMAX][NT];
+};
+
+// The grid stays (at most one workgroup per CU) and a workgroup walks the sets of NT tiles blockIdx.x,
+// blockIdx.x + gridDim.x, ...: the fragments of x -- and with PRO the work of normalising them -- are paid for once
+// per workgroup, not once per set, and the next set's weights are on their way while this one is multiplied.
+// PF: with more sets than workgroups, ask for the next set's weights before this one is multiplied (a second
+// set of registers); without it a workgroup still walks its sets, each waiting for its own requests.
+template <int NT, int WAVES, int PMAX, bool PRO, int EPI, bool PF>
+__global__ __launch_bounds__(WAVES * 64) void w4_gemv_r8_kernel(GemvArgs args, const u32x4* __restrict__ wt,
+                                                                const uint16_t* __restrict__ st,
+                                                                const uint8_t* __restrict__ zt) {
+  static_assert(EPI == 0 || (NT & 1) == 0, "the SwiGLU epilogue owns up-and-gate pairs of tiles");
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* red = reinterpret_cast<float*>(smem);  // [2][WAVES][NT][8 rows][16 columns]: sets alternate between the halves
+  float* rstd_l = red + 2 * WAVES * NT * 128;   // [8]
+  const int M = args.M, K = args.K;
+  const int G = K >> 7, ntiles = args.N >> 4;
+  const int n_sets = EPI == 1 ? ((ntiles >> 1) + NT / 2 - 1) / (NT / 2) : (ntiles + NT - 1) / NT;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  unsigned char* xs = smem + (2 * WAVES * NT * 128 + 8) * 4 + wave * kR8WaveBytes;  // this wave's own 16 blocks
+  const int col = lane & 15, kq = lane >> 4;
+  const int ul = kq >> 1;  // the group of a pair whose results this lane keeps
+  const int g_begin = (G * wave) / WAVES, g_end = (G * (wave + 1)) / WAVES;
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc(wt, (int64_t)ntiles * G * 1024);
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(st, (int64_t)ntiles * G * 32);
+  const __amdgpu_buffer_rsrc_t rz = make_rsrc(zt, (int64_t)ntiles * G * 8);
+  const __amdgpu_buffer_rsrc_t rx = make_rsrc(args.x, (int64_t)M * K * 2);
+  constexpr int kNowhere = 0x40000000;  // past every buffer here: such a request returns zeros
+  const int wvoff = lane * 16;
+  // as asked for: request i of a pair covers rows 2 i and 2 i + 1, a lane 16 bytes = 8 of the pair's 256 columns
+  const int half = lane >> 5, c32 = lane & 31, cu = c32 >> 4;  // cu: which group of the pair the lane's columns lie in
+
+  auto tile_of_set = [&](int set, int nt) {
+    if constexpr (EPI == 1) return set * (NT / 2) + (nt >> 1) + ((nt & 1) ? (ntiles >> 1) : 0);
+    else return set * NT + nt;
+  };
+  auto tile_live = [&](int set, int nt) {
+    if constexpr (EPI == 1) return set * (NT / 2) + (nt >> 1) < (ntiles >> 1);
+    else return set * NT + nt < ntiles;
+  };
+  auto request = [&](auto& r, int set) {
+    int tg[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) tg[nt] = min(tile_of_set(set, nt), ntiles - 1) * G;  // out-of-range tiles: computed, dropped
+#pragma unroll
+    for (int p = 0; p < PMAX; ++p) {
+      const int g = g_begin + 2 * p;
+      if (g < g_end) {  // wave-uniform
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int gc = min(g + u, G - 1);  // a second group past the matrix: any valid piece, its rows of x are zero
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            r.w[p][u][nt] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, wvoff, (tg[nt] + gc) * 1024, 2));
+        }
+        // the lanes that keep group g + ul hold its scale and zero (zeros past the matrix: the range check looks at
+        // the per-lane offset, so that is where "nowhere" has to stand)
+        const int svoff = g + ul < G ? (ul * 16 + col) * 2 : kNowhere, zvoff = g + ul < G ? ul * 8 + (col >> 1) : kNowhere;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          r.s16[p][nt] = __builtin_amdgcn_raw_buffer_load_b16(rs, svoff, (tg[nt] + g) * 32, 0);
+          r.z8[p][nt] = __builtin_amdgcn_raw_buffer_load_b8(rz, zvoff, (tg[nt] + g) * 8, 0);
+        }
+      }
+    }
+  };
+
+  u32x4 xa[PMAX][4];  // first the rows as asked for (PRO: of the tensor to be normalised), then the operand fragments
+  // rows past M lie past the buffer and read as zeros; so must the second group of a pair that reaches past the run
+  auto x_voff = [&](int g) { return (g + cu < g_end) ? half * K * 2 + 256 * g + 16 * c32 : kNowhere; };
+#pragma unroll
+  for (int p = 0; p < PMAX; ++p) {
+    const int g = g_begin + 2 * p;
+    if (g < g_end) {
+      const int xo = x_voff(g);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        xa[p][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, xo + 2 * i * K * 2, 0, 0));
+    }
+  }
+  u32x4 xr[PRO ? PMAX : 1][4], xw[PRO ? PMAX : 1];
+  f32x4 pv[4];
+  if constexpr (PRO) {
+    const __amdgpu_buffer_rsrc_t rr = make_rsrc(args.resid, (int64_t)M * K * 2), rn = make_rsrc(args.norm_w, (int64_t)K * 2);
+    const int n_ssq = K >> 4;
+    if (wave < M) {  // the sum of squares of row `wave`: n_ssq partials, lane-strided
+      const __amdgpu_buffer_rsrc_t rp = make_rsrc(args.ssq_in + (int64_t)wave * n_ssq, (int64_t)n_ssq * 4);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        pv[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (c * 256 < n_ssq) pv[c] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rp, lane * 16, c * 1024, 0));
+      }
+    }
+#pragma unroll
+    for (int p = 0; p < PMAX; ++p) {
+      const int g = g_begin + 2 * p;
+      if (g < g_end) {
+        const int xo = x_voff(g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          xr[p][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, xo + 2 * i * K * 2, 0, 0));
+        xw[p] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rn, (g + cu < g_end) ? 256 * g + 16 * c32 : kNowhere, 0, 0));
+      }
+    }
+  }
+  R8Weights<NT, PMAX> cur;
+  R8Weights<NT, PF ? PMAX : 1> nxt;
+  int set = blockIdx.x;
+  if (set < n_sets) request(cur, set);
+
+  if constexpr (PRO) {
+    if (wave < M) {
+      const int n_ssq = K >> 4;
+      float ss = (pv[0][0] + pv[0][1]) + (pv[0][2] + pv[0][3]);
+#pragma unroll
+      for (int c = 1; c < 4; ++c)
+        if (c * 256 < n_ssq) ss += (pv[c][0] + pv[c][1]) + (pv[c][2] + pv[c][3]);
+      ss = wave_sum_dpp(ss);
+      if (lane == 0) rstd_l[wave] = 1.f / sqrtf(ss / (float)K + args.eps);
+    }
+    __syncthreads();
+    float rstd[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) rstd[i] = 2 * i + half < M ? rstd_l[2 * i + half] : 0.f;
+#pragma unroll
+    for (int p = 0; p < PMAX; ++p) {
+      const int g = g_begin + 2 * p;
+      if (g < g_end) {
+        float wn[8];
+        unpack8(xw[p], wn);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (2 * i >= M) continue;  // both rows of the request lie past M: zeros came back, zeros stay
+          const int row = 2 * i + half;
+          const bool mine = row < M && g + cu < g_end;
+          float f[8], r[8];
+          unpack8(xa[p][i], f);
+          unpack8(xr[p][i], r);
+          u32x4 o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float y0 = round_bf16(wn[2 * e] * round_bf16(f[2 * e] * rstd[i]));
+            const float y1 = round_bf16(wn[2 * e + 1] * round_bf16(f[2 * e + 1] * rstd[i]));
+            o[e] = pack_bf16x2(r[2 * e] + y0, r[2 * e + 1] + y1);
+          }
+          xa[p][i] = mine ? o : u32x4{0u, 0u, 0u, 0u};
+          if (blockIdx.x == 0 && mine)
+            *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(args.x_out) + (int64_t)row * K * 2 + 256 * g + 16 * c32) = o;
+        }
+      }
+    }
+  }
+  // rows as asked for -> operand fragments, a pair at a time through the wave's own blocks: block (row, group of the
+  // pair) holds that row's 128 columns; the fragment of k-step j is chunk 4 j + kq of block (col & 7, col >> 3)
+#pragma unroll
+  for (int p = 0; p < PMAX; ++p) {
+    const int g = g_begin + 2 * p;
+    if (g < g_end) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        *reinterpret_cast<u32x4*>(xs + (2 * (2 * i + half) + cu) * kR8BlockBytes + (c32 & 15) * 16) = xa[p][i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        xa[p][j] = *reinterpret_cast<const u32x4*>(xs + (2 * (col & 7) + (col >> 3)) * kR8BlockBytes + (4 * j + kq) * 16);
+    }
+  }
+
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  const bf16x8 ones = ones_bf16x8();
+  const UnpackConsts uc;
+  // the sums of the activations over each group do not depend on the tile: once, before the sets
+  f32x4 xsum[PMAX];
+#pragma unroll
+  for (int p = 0; p < PMAX; ++p) {
+    xsum[p] = zero4;
+    if (g_begin + 2 * p < g_end) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        xsum[p] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[p][j]), ones, xsum[p], 0, 0, 0);
+    }
+  }
+  int parity = 0;
+  for (; set < n_sets; set += gridDim.x, parity ^= 1) {
+    const int next = set + gridDim.x;
+    if constexpr (PF) {
+      if (next < n_sets) request(nxt, next);
+    }
+    f32x4 acc[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[nt] = zero4;
+#pragma unroll
+    for (int p = 0; p < PMAX; ++p) {
+      const int g = g_begin + 2 * p;
+      if (g < g_end) {
+        f32x4 t[2][NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) t[0][nt] = zero4, t[1][nt] = zero4;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const bf16x8 af = __builtin_bit_cast(bf16x8, xa[p][j]);
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+              t[u][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, unpack_w4_bias128(cur.w[p][u][nt][j], uc), t[u][nt], 0, 0, 0);
+        }
+        // this lane's rows are 4 kq + r of the operand: group g for kq < 2, group g + 1 otherwise
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+          const float sc = (float)__builtin_bit_cast(_Float16, (uint16_t)cur.s16[p][nt]);
+          const float nzc = -(float)(129 + (int)((cur.z8[p][nt] >> (4 * (col & 1))) & 15u));  // -(128 + (stored + 1))
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float tv = ul ? t[1][nt][r] : t[0][nt][r];
+            acc[nt][r] = __builtin_fmaf(sc, __builtin_fmaf(nzc, xsum[p][r], tv), acc[nt][r]);
+          }
+        }
+      }
+    }
+    // ---- reduce: the two groups of a pair inside the wave, then the waves through LDS, in fixed order ----------
+    float* redp = red + parity * (WAVES * NT * 128);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float v = combine_xor32(acc[nt][r], AddOp{});
+        if (kq < 2) redp[((wave * NT + nt) * 8 + 4 * kq + r) * 16 + col] = v;
+      }
+    __syncthreads();  // the only one per set: the next set writes the other half of `red`
+    auto total_of = [&](int nt, int mm, int c) {
+      float v = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < WAVES; ++wv) v += redp[((wv * NT + nt) * 8 + mm) * 16 + c];
+      return v;
+    };
+    if constexpr (EPI == 0) {
+      for (int i = tid; i < NT * 128; i += WAVES * 64) {  // whole waves: 16 lanes = one (row, tile)
+        const int c = i & 15, mm = (i >> 4) & 7, nt = i >> 7;
+        const int tl = tile_of_set(set, nt);
+        const bool live = tile_live(set, nt) && mm < M;
+        const float v = live ? round_bf16(total_of(nt, mm, c)) : 0.f;
+        if (live) args.y[(int64_t)mm * args.N + tl * 16 + c] = f32_to_bf16_bits(v);
+        if (args.ssq_out) {  // sum of squares of the 16 outputs of (row, tile): one row of 16 lanes
+          const float q = row16_sum(v * v);
+          if (live && c == 0) args.ssq_out[(int64_t)mm * ntiles + tl] = q;
+        }
+      }
+    } else {
+      for (int i = tid; i < (NT / 2) * 128; i += WAVES * 64) {
+        const int c = i & 15, mm = (i >> 4) & 7, pr = i >> 7;
+        if (mm < M && tile_live(set, 2 * pr)) {
+          const float up = round_bf16(total_of(2 * pr, mm, c));  // the Linear's bf16 output
+          const float gate = round_bf16(total_of(2 * pr + 1, mm, c));
+          const float sg = round_bf16(gate / (1.f + expf(-gate)));
+          args.y[(int64_t)mm * (args.N >> 1) + tile_of_set(set, 2 * pr) * 16 + c] = f32_to_bf16_bits(sg * up);
+        }
+      }
+    }
+    if (next < n_sets) {
+      if constexpr (PF) cur = nxt;
+      else request(cur, next);
+    }
+  }
+}
+
 // ---- dense bf16 --------------------------------------------------------------------------------------------
 template <int MT, int NT, int WAVES, int U, bool XLDS, int PRO, int EPI>
 __global__ __launch_bounds__(WAVES * 64) void b16_gemv_kernel(GemvArgs args, const bf16x8* __restrict__ wt) {
@@ -1008,6 +1297,88 @@ int launch_small(Kern kern, const GemvPlan& p, const GemvArgs& a, hipStream_t st
   ROT_WAVES(GPAv, 1, 0, 0) ROT_WAVES(GPAv, 1, 1, 0) ROT_WAVES(GPAv, 1, 4, 0) ROT_WAVES(GPAv, 2, 0, 1) \
   ROT_WAVES(GPAv, 2, 1, 1) ROT_WAVES(GPAv, 2, 4, 1)
 
+// 5 .. 8 rows through w4_gemv_r8_kernel.  nt / waves 0: chosen here (measured on the 7B shapes at 8 rows: three tiles
+// per workgroup where that still leaves a workgroup per CU, two up-and-gate pairs for the SwiGLU form).
+template <typename Kern>
+int launch_r8(Kern kern, int nt, int waves, bool epi, int n_cu, const GemvArgs& a, hipStream_t stream, const u32x4* w,
+              const uint16_t* st, const uint8_t* zt) {
+  const size_t lds = (size_t)2 * waves * nt * 128 * 4 + 32 + (size_t)waves * kR8WaveBytes;
+  if (lds > 48 * 1024 &&
+      hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    return O355_ELAUNCH;
+  const int ntiles = a.N >> 4;
+  const int sets = epi ? ((ntiles >> 1) + (nt >> 1) - 1) / (nt >> 1) : (ntiles + nt - 1) / nt;
+  hipLaunchKernelGGL(kern, dim3((unsigned)std::min(sets, n_cu)), dim3(waves * 64), lds, stream, a, w, st, zt);
+  O355_CHECK_LAUNCH();
+}
+
+#define R8_CASE(NTv, Wv, Pv, PROv, Ev, PFv)                                                            \
+  if (nt == NTv && waves == Wv && pmax == Pv && pro == PROv && epi == (Ev == 1) && pf == PFv)           \
+    return launch_r8(w4_gemv_r8_kernel<NTv, Wv, Pv, PROv, Ev, PFv>, nt, waves, epi, n_cu, a, as_stream(stream), w, st, zt);
+
+// The instantiations that exist: those that fit the register file of their workgroup size without spilling
+// (16 waves: 128 registers per lane; 8 waves: 256).  pmax pairs of groups per wave, all requested up front; pf: a
+// second set of weight registers.
+constexpr bool r8_exists(int nt, int waves, int pmax, bool pro, bool epi, bool pf) {
+  if (pmax < 1 || pmax > (pro ? 2 : 3)) return false;
+  if (epi ? (nt != 2 && nt != 4) : (nt < 1 || nt > 3)) return false;
+  if (waves == 8) {
+    if (pf) return nt <= 2 && pmax <= 2;
+    return !(nt == 4 && pmax == 3);
+  }
+  if (waves != 16) return false;
+  if (pf) return pmax == 1 && nt <= 2;
+  if (pro) return pmax == 1;
+  return nt == 1 || pmax == 1;
+}
+
+int w4_r8_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, bool pro, bool epi, int nt,
+                   int waves, void* stream) {
+  const int G = a.K >> 7, ntiles = a.N >> 4;
+  if (a.M < 1 || a.M > 8 || (a.K & 127) || (a.N & 15) || (epi && (a.N & 31))) return O355_EUNSUPPORTED;
+  if ((int64_t)a.M * a.K * 2 >= 0x40000000 || (int64_t)ntiles * G * 1024 >= (1ll << 31)) return O355_EUNSUPPORTED;
+  if (pro && (!a.ssq_in || !a.resid || !a.norm_w || !a.x_out || (a.K >> 4) > 1024)) return O355_EUNSUPPORTED;
+  if (a.ssq_out && epi) return O355_EUNSUPPORTED;
+  static int n_cu = 0;  // of the device first used: the grid only has to be about as large as the machine
+  if (n_cu == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      return O355_ELAUNCH;
+    n_cu = cus;
+  }
+  if (nt == 0) nt = epi ? 2 : 1;  // a workgroup walks its sets of tiles one after the other: small sets, few registers
+  const int sets = epi ? ((ntiles >> 1) + (nt >> 1) - 1) / (nt >> 1) : (ntiles + nt - 1) / nt;
+  const bool want_pf = sets > n_cu;
+  auto pairs_of = [&](int wv) { return std::max(1, ((G + wv - 1) / wv + 1) >> 1); };  // of the wave with the longest run
+  if (waves == 0) {
+    waves = 16;
+    if (G < 32 || !r8_exists(nt, 16, pairs_of(16), pro, epi, want_pf)) waves = 8;
+  }
+  const int pmax = pairs_of(waves);
+  bool pf = want_pf;
+  if (pf && !r8_exists(nt, waves, pmax, pro, epi, true)) pf = false;
+  if (!r8_exists(nt, waves, pmax, pro, epi, pf)) return O355_EUNSUPPORTED;
+  const u32x4* w = (const u32x4*)wt;
+  // 16 waves
+  R8_CASE(1, 16, 1, false, 0, false) R8_CASE(1, 16, 2, false, 0, false) R8_CASE(1, 16, 3, false, 0, false) R8_CASE(1, 16, 1, true, 0, false)
+  R8_CASE(2, 16, 1, false, 0, false) R8_CASE(2, 16, 1, true, 0, false)
+  R8_CASE(3, 16, 1, false, 0, false) R8_CASE(3, 16, 1, true, 0, false)
+  R8_CASE(2, 16, 1, false, 1, false) R8_CASE(2, 16, 1, true, 1, false)
+  R8_CASE(4, 16, 1, false, 1, false) R8_CASE(4, 16, 1, true, 1, false)
+  R8_CASE(1, 16, 1, false, 0, true) R8_CASE(1, 16, 1, true, 0, true) R8_CASE(2, 16, 1, false, 0, true) R8_CASE(2, 16, 1, true, 0, true)
+  R8_CASE(2, 16, 1, false, 1, true) R8_CASE(2, 16, 1, true, 1, true)
+  // 8 waves
+  R8_CASE(1, 8, 1, false, 0, false) R8_CASE(1, 8, 2, false, 0, false) R8_CASE(1, 8, 3, false, 0, false) R8_CASE(1, 8, 1, true, 0, false) R8_CASE(1, 8, 2, true, 0, false)
+  R8_CASE(2, 8, 1, false, 0, false) R8_CASE(2, 8, 2, false, 0, false) R8_CASE(2, 8, 3, false, 0, false) R8_CASE(2, 8, 1, true, 0, false) R8_CASE(2, 8, 2, true, 0, false)
+  R8_CASE(3, 8, 1, false, 0, false) R8_CASE(3, 8, 2, false, 0, false) R8_CASE(3, 8, 3, false, 0, false) R8_CASE(3, 8, 1, true, 0, false) R8_CASE(3, 8, 2, true, 0, false)
+  R8_CASE(2, 8, 1, false, 1, false) R8_CASE(2, 8, 2, false, 1, false) R8_CASE(2, 8, 3, false, 1, false) R8_CASE(2, 8, 1, true, 1, false) R8_CASE(2, 8, 2, true, 1, false)
+  R8_CASE(4, 8, 1, false, 1, false) R8_CASE(4, 8, 2, false, 1, false) R8_CASE(4, 8, 1, true, 1, false) R8_CASE(4, 8, 2, true, 1, false)
+  R8_CASE(1, 8, 1, false, 0, true) R8_CASE(1, 8, 2, false, 0, true) R8_CASE(1, 8, 1, true, 0, true) R8_CASE(1, 8, 2, true, 0, true)
+  R8_CASE(2, 8, 1, false, 0, true) R8_CASE(2, 8, 2, false, 0, true) R8_CASE(2, 8, 1, true, 0, true) R8_CASE(2, 8, 2, true, 0, true)
+  R8_CASE(2, 8, 1, false, 1, true) R8_CASE(2, 8, 2, false, 1, true) R8_CASE(2, 8, 1, true, 1, true) R8_CASE(2, 8, 2, true, 1, true)
+  return O355_EUNSUPPORTED;
+}
+
 int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, bool pro, bool epi,
                      void* stream, int form = kFormChoose) {
   GemvPlan p = plan_gemv(a.M, a.N, a.K, true, pro, epi);
@@ -1020,12 +1391,23 @@ int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, 
   const bool plain = !pro && !epi && !a.ssq_in && !a.ssq_out;
   const bool mid_wins = a.M > 16 || (a.M > 8 && a.N >= 8192) || (a.M > 7 && a.N >= 12288);
   const bool force_mid = form == kFormMid || form == kFormMid1 || form == kFormMid2;
+  if (plain && a.M > 4 && a.M <= 8 && form == kFormChoose) {  // measured at 8 rows: 8.7 / 4.8 / 8.6 us against 11.0 / 4.9 / 10.6
+    const int st8 = w4_r8_dispatch(a, wt, st, zt, false, false, 0, 0, stream);
+    if (st8 != O355_EUNSUPPORTED) return st8;
+  }
   if (plain && ((mid_wins && form == kFormChoose) || force_mid)) {
     const int pairs = form == kFormMid1 ? 1 : (form == kFormMid2 ? 2 : 0);
     const int st_mid = o355_w4_mid_dispatch(a.x, wt, st, zt, a.y, a.M, a.N, a.K, pairs, stream);
     if (st_mid != O355_EUNSUPPORTED || force_mid) return st_mid;  // else: sizes beyond its 32-bit offsets
   }
-  if (a.ssq_in || a.ssq_out) {  // chained norms: only the lean kernel speaks that protocol
+  if ((a.ssq_in || a.ssq_out) && a.M > 4) return w4_r8_dispatch(a, wt, st, zt, pro, epi, 0, 0, stream);
+  if (a.ssq_in && a.M > 2) {
+    // three and four rows with the chained prologue: the kernel below needs four pieces of x per lane for them and
+    // with those registers only one of its workgroups fits a CU (measured, 4 rows: att_proj 37 against 11 us)
+    const int st8 = w4_r8_dispatch(a, wt, st, zt, pro, epi, 0, 0, stream);
+    if (st8 != O355_EUNSUPPORTED) return st8;
+  }
+  if (a.ssq_in || a.ssq_out) {  // chained norms: only the lean kernels speak that protocol
     if (!small_ok || a.M > 4 || (a.ssq_out && epi)) return O355_EUNSUPPORTED;
     if (a.ssq_in) {
       const int slice_kib = ((((a.K >> 7) + p.waves - 1) / p.waves) * 256 + 1023) >> 10;  // per row, largest wave
@@ -1112,13 +1494,26 @@ extern "C" int olmo355_w4_gemv_chain(const uint16_t* x, const uint16_t* resid, c
                                      void* stream) {
   if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
   if ((resid != nullptr) != (ssq_in != nullptr)) return O355_EINVAL;  // the prologue here is the chained one
-  if (M > 4 || (K & 127) || (N & 15)) return O355_EUNSUPPORTED;
+  if (M > 8 || (K & 127) || (N & 15)) return O355_EUNSUPPORTED;
   GemvArgs a{x, resid, norm_w, x_out, y, eps, M, N, K};
   a.ssq_in = ssq_in, a.ssq_out = ssq_out;
   const bool pro = resid != nullptr, epi = swiglu != 0;
+  if (M > 4) return w4_r8_dispatch(a, wt, st, zt, pro, epi, 0, 0, stream);
   const int chk = check_fused(a, pro, epi);
   if (chk != O355_OK) return chk;
   return w4_gemv_dispatch(a, wt, st, zt, pro, epi, stream);
+}
+
+extern "C" int olmo355_w4_gemv_r8_form(const uint16_t* x, const uint16_t* resid, const uint16_t* norm_w, float eps,
+                                       uint16_t* x_out, const float* ssq_in, const uint32_t* wt, const uint16_t* st,
+                                       const uint8_t* zt, uint16_t* y, float* ssq_out, int M, int N, int K, int swiglu,
+                                       int nt, int waves, void* stream) {
+  if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0 || nt < 0 || (waves != 0 && waves != 8 && waves != 16))
+    return O355_EINVAL;
+  if ((resid != nullptr) != (ssq_in != nullptr)) return O355_EINVAL;
+  GemvArgs a{x, resid, norm_w, x_out, y, eps, M, N, K};
+  a.ssq_in = ssq_in, a.ssq_out = ssq_out;
+  return w4_r8_dispatch(a, wt, st, zt, resid != nullptr, swiglu != 0, nt, waves, stream);
 }
 
 extern "C" int olmo355_b16_gemv_fused(const uint16_t* x, const uint16_t* resid, const uint16_t* norm_w, float eps,

@@ -458,10 +458,15 @@ class OLMo(nn.Module):
     #   x      residual stream entering the block, *before* the previous block's pending update
     #   pend   (f_prev, ff_norm weight of the previous block) or None: x := x + norm(f_prev) is applied
     #          inside this block's att_proj launch
-    def _fused_decode_ok(self, M: int, collect_hidden: bool) -> bool:
+    def _fused_decode_ok(self, M: int, collect_hidden: bool, rows_in_lds: bool = True) -> bool:
+        """Whether a decode step of ``M`` rows may fold the norms into its linears.  ``rows_in_lds``: for the kernels
+        that keep all rows of the activations in LDS (the chained form for 5 to 8 rows does not)."""
         c = self.config
-        return (M <= 16 and self.dtype == torch.bfloat16 and c.norm_after and c.layer_norm_type == "rms"
-                and not collect_hidden and not self._act_order and c.clip_qkv is None and c.d_model * 2 * (M + 1) <= 64 * 1024 and c.d_model <= 5120)
+        ok = (M <= 16 and self.dtype == torch.bfloat16 and c.norm_after and c.layer_norm_type == "rms"
+              and not collect_hidden and not self._act_order and c.clip_qkv is None)
+        if rows_in_lds:
+            ok = ok and c.d_model * 2 * (M + 1) <= 64 * 1024 and c.d_model <= 5120
+        return ok
 
     @staticmethod
     def _tiled(m: nn.Module):
@@ -613,7 +618,7 @@ class OLMo(nn.Module):
             return cached
         blk = self.transformer["blocks"][0]
         lin = (blk.att_proj, blk.attn_out, blk.ff_proj, blk.ff_out)
-        ok = M <= 4 and all(isinstance(m, QuantLinear) for m in lin) and not torch.cuda.is_current_stream_capturing()
+        ok = M <= 8 and all(isinstance(m, QuantLinear) for m in lin) and not torch.cuda.is_current_stream_capturing()
         if ok:
             d = self.config.d_model
             x = torch.zeros(M, 1, d, dtype=torch.bfloat16, device=self.device)
@@ -740,8 +745,9 @@ class OLMo(nn.Module):
         self._beam = cache if isinstance(cache, BeamKVCache) else None
         if self._beam is not None and T != 1:
             raise ValueError("a beam cache takes one token per row")
-        fused = T == 1 and cache is not None and self._beam is None and self._fused_decode_ok(B, collect_hidden)
-        chain = fused and self._chain_decode_ok(B)
+        decode = T == 1 and cache is not None and self._beam is None
+        fused = decode and self._fused_decode_ok(B, collect_hidden)
+        chain = decode and self._fused_decode_ok(B, collect_hidden, rows_in_lds=False) and self._chain_decode_ok(B)
         pend = None
         if chain and self._relay_decode_ok(B, key_bias, n_keys_max):
             x = self._relay_blocks(x, cache, past_len, key_bias, graph_pos, n_keys_max)

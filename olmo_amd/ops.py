@@ -143,6 +143,7 @@ def w4_linear(x: torch.Tensor, w: W4Tiled) -> torch.Tensor:
         check("olmo355_w4_gemv",
               lib().olmo355_w4_gemv(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream()))
     else:
+        ev = _gemm_begin()
         sk = _streamk(M, w.N, w.K, x.device)
         st = 2
         if sk is not None:
@@ -153,7 +154,43 @@ def w4_linear(x: torch.Tensor, w: W4Tiled) -> torch.Tensor:
         if st == 2:
             check("olmo355_w4_gemm",
                   lib().olmo355_w4_gemm(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream()))
+        _gemm_end(ev, w.N, w.K, M)
     return y
+
+
+class gemm_events:
+    """``with gemm_events() as rec:`` puts a pair of HIP events around every many-row (M > 64) int4 linear issued
+    meanwhile, on the stream it is issued on; after a synchronisation ``rec.rows()`` gives ``(N, K, M, seconds)`` per
+    launch.  For measuring the GEMMs inside a real prefill; off (no events, no cost) otherwise."""
+    active: Optional["gemm_events"] = None
+
+    def __init__(self):
+        self.items = []
+
+    def __enter__(self):
+        gemm_events.active = self
+        return self
+
+    def __exit__(self, *exc):
+        gemm_events.active = None
+
+    def rows(self):
+        return [(n, k, m, e0.elapsed_time(e1) * 1e-3) for n, k, m, e0, e1 in self.items]
+
+
+def _gemm_begin():
+    if gemm_events.active is None:
+        return None
+    e0 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    return e0
+
+
+def _gemm_end(e0, N: int, K: int, M: int) -> None:
+    if e0 is not None and gemm_events.active is not None:
+        e1 = torch.cuda.Event(enable_timing=True)
+        e1.record()
+        gemm_events.active.items.append((N, K, M, e0, e1))
 
 
 SPLITK = True  # tests switch it off to compare the two forms
@@ -284,6 +321,7 @@ def linear_fused(x: torch.Tensor, w, resid: Optional[torch.Tensor] = None, norm_
     x_new = rmsnorm(x, norm_w, eps, residual=resid) if resid is not None else x
     if swiglu_out and isinstance(w, W4Tiled) and M > GEMV_MAX_M:  # many rows: SwiGLU in the GEMM's epilogue
         y = torch.empty(*x.shape[:-1], n_out, dtype=torch.bfloat16, device=x.device)
+        ev = _gemm_begin()
         sk = _streamk(M, w.N, w.K, x.device)
         st = 2
         if sk is not None:
@@ -294,6 +332,7 @@ def linear_fused(x: torch.Tensor, w, resid: Optional[torch.Tensor] = None, norm_
         if st == 2:
             st = lib().olmo355_w4_gemm_swiglu(_p(x_new), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream())
         if st == 0:
+            _gemm_end(ev, w.N, w.K, M)
             return y, x_new
         if st != 2:
             check("olmo355_w4_gemm_swiglu", st)
@@ -303,34 +342,36 @@ def linear_fused(x: torch.Tensor, w, resid: Optional[torch.Tensor] = None, norm_
 
 def w4_linear_chain(x: torch.Tensor, w: "W4Tiled", resid: Optional[torch.Tensor] = None,
                     norm_w: Optional[torch.Tensor] = None, eps: float = 0.0, ssq_in: Optional[torch.Tensor] = None,
-                    swiglu_out: bool = False, want_ssq: bool = False):
-    """Decode-step int4 linear (at most 4 rows) with the norms chained between launches.  Returns
+                    swiglu_out: bool = False, want_ssq: bool = False, r8_form: Optional[Tuple[int, int]] = None):
+    """Decode-step int4 linear (at most 8 rows) with the norms chained between launches.  Returns
     ``(y, x_new, ssq)`` or ``None`` when the kernel does not cover the shape.  ``ssq`` (float32
     ``[M, N/16]``, only with ``want_ssq``) holds the sum of squares of every 16-column tile of ``y``: hand
     it to the launch that normalises ``y`` (``ssq_in`` here, ``qk_ssq`` of :func:`attn_decode_fused`).
-    With ``resid``: ``x_new = resid + rmsnorm(x; norm_w, eps)`` using ``ssq_in`` for the mean square."""
+    With ``resid``: ``x_new = resid + rmsnorm(x; norm_w, eps)`` using ``ssq_in`` for the mean square.
+    ``r8_form=(tiles per workgroup, waves)`` (0 = choose) sends the call through the variant entry of the kernel for
+    5 to 8 rows, for tests and tuning."""
     _dev(x, resid, norm_w, ssq_in)
     if x.dtype != torch.bfloat16 or not isinstance(w, W4Tiled):
         return None
     M = x.numel() // w.K
-    if M < 1 or M > 4 or (resid is None) != (ssq_in is None) or (want_ssq and swiglu_out):
+    if M < 1 or M > 8 or (resid is None) != (ssq_in is None) or (want_ssq and swiglu_out):
         return None
     n_out = w.N // 2 if swiglu_out else w.N
     y = torch.empty(*x.shape[:-1], n_out, dtype=torch.bfloat16, device=x.device)
     x_new = torch.empty_like(x) if resid is not None else x
     ssq = torch.empty(M, w.N // 16, dtype=torch.float32, device=x.device) if want_ssq else None
-    st = lib().olmo355_w4_gemv_chain(_p(x), _p(resid), _p(norm_w), float(eps), _p(x_new) if resid is not None else None,
-                                     _p(ssq_in), _p(w.wt), _p(w.st), _p(w.zt), _p(y), _p(ssq), M, w.N, w.K,
-                                     int(swiglu_out), _stream())
+    args = (_p(x), _p(resid), _p(norm_w), float(eps), _p(x_new) if resid is not None else None, _p(ssq_in), _p(w.wt),
+            _p(w.st), _p(w.zt), _p(y), _p(ssq), M, w.N, w.K, int(swiglu_out))
+    if r8_form is None:
+        st = lib().olmo355_w4_gemv_chain(*args, _stream())
+    else:
+        st = lib().olmo355_w4_gemv_r8_form(*args, int(r8_form[0]), int(r8_form[1]), _stream())
     if st == 2:
         return None
     check("olmo355_w4_gemv_chain", st)
     return y, x_new, ssq
 
 
-# ---------------------------------------------------------------------------------------------
-# the decode relay (one row): launches on two streams, the hand-over carried by epoch tags in the data
-# ---------------------------------------------------------------------------------------------
 RELAY_SPIN_LIMIT = 1 << 16  # polls of a waiting wave before it gives up and sets the status word (a tenth of a second)
 
 

@@ -894,12 +894,14 @@ def test_attn_decode_fused_both_merges(dev, merge, B, past, H, Hkv, hd):
     assert torch.allclose(out_auto.float(), out.float(), rtol=2 ** -7, atol=2 ** -10)
 
 
-@pytest.mark.parametrize("M", [1, 2, 4])
+@pytest.mark.parametrize("M", [1, 2, 4, 5, 7, 8])
 @pytest.mark.parametrize("N,K,epi", [(4096, 4096, False), (12288, 4096, False), (22016, 4096, True), (768, 512, False),
-                                     (4096, 11264, False), (1024, 1024, True)])
+                                     (4096, 11264, False), (1024, 1024, True), (4096, 11008, False), (15360, 5120, False)])
 def test_w4_gemv_chain(dev, M, N, K, epi):
     """Norms chained between launches: the producer's per-tile sums of squares equal those of its output,
-    and a consumer fed with them gives the same x' and y as the oracle's norm + linear (+ SwiGLU)."""
+    and a consumer fed with them gives the same x' and y as the oracle's norm + linear (+ SwiGLU).  Up to 4 rows
+    go through the kernel that keeps the activations in LDS, 5 to 8 through the one that takes them as operand
+    fragments from memory."""
     say("w4_gemv_chain", M, N, K, epi)
     ops = _ops()
     gen = torch.Generator().manual_seed(M + N + K)
@@ -909,7 +911,7 @@ def test_w4_gemv_chain(dev, M, N, K, epi):
     qw, qz, sc = ow4.random_quantized(K, N, 128, seed=N + K)
     Wf = ow4.dequantize(qw, qz, sc, 128).float()
     w = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
-    if (M + 1) * K * 2 > 128 * 1024:
+    if M <= 4 and (M + 1) * K * 2 > 128 * 1024:
         # the activations (plus a zero row) no longer fit the kernel's LDS budget: the call declines
         assert ops.w4_linear_chain(a.to(dev), w, want_ssq=not epi, swiglu_out=epi) is None
         return
@@ -942,6 +944,52 @@ def test_w4_gemv_chain(dev, M, N, K, epi):
     if ssq is not None:
         want = (y.float().cpu() ** 2).view(M, -1, 16).sum(-1)
         assert torch.allclose(ssq.cpu(), want, rtol=1e-5, atol=1e-6 * want.max().item())
+
+
+@pytest.mark.parametrize("M", [3, 8])
+@pytest.mark.parametrize("N,K,epi,pro", [(12288, 4096, False, True), (4096, 4096, False, False), (22016, 4096, True, True),
+                                         (4096, 11008, False, False), (2064, 640, False, True)])
+def test_w4_gemv_r8_forms(dev, M, N, K, epi, pro):
+    """The kernel for 5 to 8 rows in every tiling the variant entry offers (column tiles per workgroup, 8 or 16 waves):
+    each against the oracle; tilings that split K over the same number of waves add the same numbers in the same
+    order and must agree bit for bit."""
+    say("w4_gemv_r8_forms", M, N, K, epi, pro)
+    ops = _ops()
+    gen = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    resid = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    nw = (1 + 0.1 * torch.randn(K, generator=gen)).to(torch.bfloat16)
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=N + K)
+    Wf = ow4.dequantize(qw, qz, sc, 128).float()
+    w = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    x_ref = resid + om.rms_norm(a, nw, 1e-6) if pro else a
+    y_ref = (x_ref.float() @ Wf).to(torch.bfloat16)
+    if epi:
+        y_ref = om.swiglu(y_ref)
+    scale = y_ref.float().abs().max().item()
+    ssq_in = (a.float() ** 2).view(M, -1, 16).sum(-1).to(dev)
+    kw = dict(resid=resid.to(dev), norm_w=nw.to(dev), eps=1e-6, ssq_in=ssq_in) if pro else {}
+    ran = 0
+    for waves in (8, 16):
+        first = None
+        for nt in ((2, 4) if epi else (1, 2, 3)):
+            r = ops.w4_linear_chain(a.to(dev), w, swiglu_out=epi, want_ssq=not epi, r8_form=(nt, waves), **kw)
+            if r is None:  # a tiling whose registers would not fit is not built: the entry declines
+                continue
+            ran += 1
+            y, x_new, ssq = r
+            assert (y.cpu().float() - y_ref.float()).abs().max().item() <= 2 ** -6 * scale, (nt, waves)
+            if pro:
+                dx = (x_new.cpu().float() - x_ref.float()).abs()
+                assert (dx <= 2.0 ** (torch.floor(torch.log2(x_ref.float().abs().clamp_min(1e-30))) - 7)).all()
+            if ssq is not None:
+                want = (y.float().cpu() ** 2).view(M, -1, 16).sum(-1)
+                assert torch.allclose(ssq.cpu(), want, rtol=1e-5, atol=1e-6 * want.max().item())
+            if first is None:
+                first = y
+            else:
+                assert torch.equal(first, y), (nt, waves)
+    assert ran >= (1 if K > 8192 else 2)  # a long K leaves one tiling whose requests fit the registers
 
 
 # ------------------------------------------------------------------------------------------------
