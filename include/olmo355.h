@@ -151,6 +151,16 @@ int olmo355_w4_gemm_swiglu_streamk(const uint16_t* x, const uint32_t* wt, const 
 int olmo355_b16_gemm_streamk(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, void* workspace,
                              int64_t ws_bytes, int epoch, void* stream);
 
+/* The product for fp16 activations, the arithmetic of the reference's own QuantLinear (qlinear_cuda_old.py:253-265,
+ * 287-290: weights fp16(scale * (q - zero)), fp16 activations, here with fp32 accumulation; its known-answer vectors,
+ * AGQ tests/test_q4.py:1071-1104, are met to 2 fp16 ulp).  x [M,K] and y [M,N] are fp16.  olmo355_w4_gemv_f16: up to 16
+ * rows whose K fits LDS (the decode kernel on the fp16 matrix instruction, nibbles as 1024 + q, scale and zero applied
+ * in fp32); olmo355_w4_gemm_f16: any M (tiled launches).  O355_EUNSUPPORTED: use the other. */
+int olmo355_w4_gemv_f16(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M,
+                        int N, int K, void* stream);
+int olmo355_w4_gemm_f16(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M,
+                        int N, int K, void* stream);
+
 /* The same product for an ff_proj weight ([up | gate] column halves) with SwiGLU (olmo/model.py:365-368,813-819)
  * in the epilogue: y [M, N/2] = silu(gate) * up, each factor rounded to bf16 first as the separate Linear and
  * activation would.  N a multiple of 256; O355_EUNSUPPORTED otherwise: olmo355_w4_gemm + olmo355_swiglu. */
@@ -287,6 +297,7 @@ int olmo355_add(const void* a, const void* b, void* out, int64_t n, int dtype, v
  * (AGQ/auto_gptq/nn_modules/qlinear/qlinear_cuda_old.py:288-290); x, out bf16 [M, N], bias fp16 [N] as the
  * checkpoint stores it, sum in fp32, one rounding. */
 int olmo355_add_bias_bf16(const uint16_t* x, const uint16_t* bias_f16, uint16_t* out, int M, int N, void* stream);
+int olmo355_add_bias_f16(const uint16_t* x, const uint16_t* bias_f16, uint16_t* out, int M, int N, void* stream); /* fp16 rows */
 /* Greedy step (olmo/beam_search.py:102-113 with beam 1): first index of the row maximum,
  * written as int64 to out[r], and the same value appended at ids_next when non-NULL. */
 int olmo355_argmax(const void* logits, int64_t* out, int rows, int n, int dtype, void* stream);

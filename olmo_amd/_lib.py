@@ -64,6 +64,8 @@ EXPORTS = {
     "olmo355_gemm_splitk_plan": (I, [I, I, I]),
     "olmo355_w4_gemm_splitk": (I, [P, P, P, P, P, I, I, I, I, P, P]),
     "olmo355_b16_gemm_splitk": (I, [P, P, P, I, I, I, I, P, P]),
+    "olmo355_w4_gemv_f16": (I, [P, P, P, P, P, I, I, I, P]),
+    "olmo355_w4_gemm_f16": (I, [P, P, P, P, P, I, I, I, P]),
     "olmo355_gemm_streamk_workspace_bytes": (L, []),
     "olmo355_gemm_streamk_plan": (I, [I, I, I]),
     "olmo355_w4_gemm_streamk": (I, [P, P, P, P, P, I, I, I, P, L, I, P]),
@@ -77,6 +79,7 @@ EXPORTS = {
     "olmo355_sample": (I, [P, I, I, F, I, F, c_uint64, P, I, P, P, I, P]),
     "olmo355_add": (I, [P, P, P, L, I, P]),
     "olmo355_add_bias_bf16": (I, [P, P, P, I, I, P]),
+    "olmo355_add_bias_f16": (I, [P, P, P, I, I, P]),
     "olmo355_argmax": (I, [P, P, I, I, I, P]),
     "olmo355_incr_i32": (I, [P, P]),
 }

@@ -217,3 +217,30 @@ __device__ __forceinline__ bf16x8 unpack_w4_bias128(uint32_t w, const UnpackCons
   return __builtin_bit_cast(bf16x8, r);
 }
 
+// The same word as 8 fp16 numbers for fp16 activations: fp16(scale * (q - zero)), the arithmetic of the reference's own
+// dequantisation (qlinear_cuda_old.py:253-265: integer difference, one product, one rounding).  (1024 + q) - (1024 +
+// zero) is exact in fp16, the product with the scale rounds once.
+struct DequantConstsF16 {
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  f16x2 s2, nz2;
+};
+__device__ __forceinline__ DequantConstsF16 dequant_consts_f16(uint16_t scale_bits, int zero) {
+  const _Float16 s = __builtin_bit_cast(_Float16, scale_bits), nz = (_Float16)(-(float)(1024 + zero));
+  return {{s, s}, {nz, nz}};
+}
+__device__ __forceinline__ u32x4 dequant_word_f16(uint32_t w, const DequantConstsF16& d) {
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  u32x4 o;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const f16x2 h = __builtin_bit_cast(f16x2, ((w >> (4 * i)) & 0x000f000fu) | 0x64006400u);
+    o[i] = __builtin_bit_cast(uint32_t, (f16x2)((h + d.nz2) * d.s2));
+  }
+  return o;
+}
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {  // round to nearest even, as a cast does
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  const f16x2 p = {(_Float16)lo, (_Float16)hi};
+  return __builtin_bit_cast(uint32_t, p);
+}
+

@@ -377,6 +377,16 @@ __global__ __launch_bounds__(256) void add_bias_bf16_kernel(const uint16_t* __re
   }
 }
 
+// the same for fp16 rows (QuantLinear.forward on fp16 input: out + bias, qlinear_cuda_old.py:288-290)
+__global__ __launch_bounds__(256) void add_bias_f16_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ bias,
+                                                           uint16_t* __restrict__ out, int64_t total, int N) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < total) {
+    const float b = (float)__builtin_bit_cast(_Float16, bias[i % N]);
+    out[i] = __builtin_bit_cast(uint16_t, (_Float16)((float)__builtin_bit_cast(_Float16, x[i]) + b));
+  }
+}
+
 // first index of the maximum of each row (torch.argmax tie rule); all loads of a thread issued
 // up front when the row is 16-byte divisible
 template <int DT>
@@ -573,6 +583,14 @@ extern "C" int olmo355_add_bias_bf16(const uint16_t* x, const uint16_t* bias_f16
   if (!x || !bias_f16 || !out || M <= 0 || N <= 0) return O355_EINVAL;
   const int64_t total = (int64_t)M * N;
   hipLaunchKernelGGL(add_bias_bf16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, as_stream(stream), x,
+                     bias_f16, out, total, N);
+  O355_CHECK_LAUNCH();
+}
+
+extern "C" int olmo355_add_bias_f16(const uint16_t* x, const uint16_t* bias_f16, uint16_t* out, int M, int N, void* stream) {
+  if (!x || !bias_f16 || !out || M <= 0 || N <= 0) return O355_EINVAL;
+  const int64_t total = (int64_t)M * N;
+  hipLaunchKernelGGL(add_bias_f16_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, as_stream(stream), x,
                      bias_f16, out, total, N);
   O355_CHECK_LAUNCH();
 }

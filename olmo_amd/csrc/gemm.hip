@@ -26,6 +26,8 @@
 
 namespace {
 
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
 constexpr int BK = 64;      // K per stage
 constexpr int KSTEPS = 2;   // MFMA k-steps of 32 per stage
 
@@ -58,6 +60,12 @@ __device__ __forceinline__ u32x4 dequant_word_bf16(uint32_t w, const DequantCons
   o[2] = pair(and_or(w8, 0x000f000fu, magic), d.s, d.c0);
   o[3] = pair(and_or(w8, 0x00f000f0u, magic), d.s16, d.c1);
   return o;
+}
+
+template <bool F16>
+__device__ __forceinline__ f32x4 mma16(const bf16x8& a, const bf16x8& b, const f32x4& c) {
+  if constexpr (F16) return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  else return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
 // Tile order: consecutive workgroup ids go round-robin over the 8 XCDs.  XCD x works on the row
@@ -110,7 +118,8 @@ __device__ __forceinline__ StreamKArgsPtr streamk_args() {
 enum { GEMM_PLAIN = 0, GEMM_SPLIT = 1, GEMM_STREAMK = 2 };
 constexpr int kStreamKStatusWord = O355_STREAMK_STATUS_WORD;  // int32 index in the workspace: epoch of a launch that gave up
 
-template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false, int KIND = GEMM_PLAIN>  // wave grid, 32 x 32 blocks (of four 16 x 16 MFMA tiles) per wave
+// F16: the activations, the dequantised weights and the output are fp16 instead of bf16 (int4 weights, plain tiles only)
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false, int KIND = GEMM_PLAIN, bool F16 = false>  // wave grid, 32 x 32 blocks (of four 16 x 16 MFMA tiles) per wave
 __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wt,
                                           const uint16_t* __restrict__ st, const uint8_t* __restrict__ zt,
                                           uint16_t* __restrict__ y, int M, int N, int K, int tile_m, int tile_n,
@@ -118,6 +127,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
                                           float* __restrict__ part = nullptr, int sk_mode = 0, int sk_self = 0,
                                           int sk_first = 0, bool sk_raise = false, bool sk_defer = false) {
   constexpr bool SPLIT = KIND == GEMM_SPLIT;
+  static_assert(!F16 || (W4 && !SWIGLU && KIND == GEMM_PLAIN), "fp16 activations: the plain int4 tiles");
   constexpr int NW = WAVES_M * WAVES_N, NT = 64 * NW;
   constexpr int BM = 32 * WMT * WAVES_M, BN = 32 * WNT * WAVES_N;
   constexpr int MT = 2 * WMT, NT16 = 2 * WNT;  // 16 x 16 MFMA tiles per wave
@@ -218,10 +228,14 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
   auto stash_b_word = [&](int buf, int set, int i, int j) {  // word j (32-row step j of the group) of item i
     const int ntl = wave + NW * i;
     if (B_RAGGED && ntl >= BN / 16) return;  // wave-uniform
-    const float sc = (float)__builtin_bit_cast(_Float16, (uint16_t)rsb[set][i]);
-    const DequantConsts dc = dequant_consts(sc, 1 + (int)((rzb[set][i] >> (4 * (lane & 1))) & 15u));  // stored zero points are one less
+    const int zero = 1 + (int)((rzb[set][i] >> (4 * (lane & 1))) & 15u);  // stored zero points are one less
     // a tiled word is already the lane's piece of a 16-column x 32-row operand fragment: it stays in its lane
-    lds_b[(buf * B_BLK + ntl * KSTEPS + (j & 1)) * 64 + lane] = dequant_word_bf16(rbw[set][i][j], dc);
+    if constexpr (F16) {
+      lds_b[(buf * B_BLK + ntl * KSTEPS + (j & 1)) * 64 + lane] = dequant_word_f16(rbw[set][i][j], dequant_consts_f16((uint16_t)rsb[set][i], zero));
+    } else {
+      const float sc = (float)__builtin_bit_cast(_Float16, (uint16_t)rsb[set][i]);
+      lds_b[(buf * B_BLK + ntl * KSTEPS + (j & 1)) * 64 + lane] = dequant_word_bf16(rbw[set][i][j], dequant_consts(sc, zero));
+    }
   };
   // dense: the tiled pieces [16-column tile][32-row step][64][16 B] are copied as they are
   int bd_voff[W4 ? 1 : B_PW];
@@ -321,8 +335,8 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
         const int slot = (ks * OUT + r) % OS;  // rounds are numbered through the stage: slots rotate across its k-steps
 #pragma unroll
         for (int q = 0; q < INN; ++q) {
-          if constexpr (OUTER_A) acc[r][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fi[q], fo[slot], acc[r][q], 0, 0, 0);
-          else acc[q][r] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fo[slot], fi[q], acc[q][r], 0, 0, 0);
+          if constexpr (OUTER_A) acc[r][q] = mma16<F16>(fi[q], fo[slot], acc[r][q]);
+          else acc[q][r] = mma16<F16>(fo[slot], fi[q], acc[q][r]);
           if (r == OUT - 1) fi[q] = read_inner(nab, nh, q, nks);
         }
         const int rn = r + OS;  // the round this slot serves next
@@ -473,8 +487,8 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
     uint32_t o[2][2];
 #pragma unroll
     for (int x = 0; x < 2; ++x) {
-      const auto sw = __builtin_amdgcn_permlane16_swap(pack_bf16x2(va[2 * x], va[2 * x + 1]), pack_bf16x2(vb[2 * x], vb[2 * x + 1]),
-                                                       false, false);
+      const auto sw = F16 ? __builtin_amdgcn_permlane16_swap(pack_f16x2(va[2 * x], va[2 * x + 1]), pack_f16x2(vb[2 * x], vb[2 * x + 1]), false, false)
+                          : __builtin_amdgcn_permlane16_swap(pack_bf16x2(va[2 * x], va[2 * x + 1]), pack_bf16x2(vb[2 * x], vb[2 * x + 1]), false, false);
       o[0][x] = sw[0], o[1][x] = sw[1];
     }
     const int n = nb + 16 * (kq4 & 1) + 8 * (kq4 >> 1);
@@ -559,7 +573,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const f32x4* __restr
   y[i] = u32x2{pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3])};
 }
 
-template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false>
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false, bool F16 = false>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const uint16_t* __restrict__ x,
                                                                      const uint32_t* __restrict__ wt,
                                                                      const uint16_t* __restrict__ st,
@@ -568,7 +582,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_kernel(const uint
                                                                      int tiles_m, int tiles_n) {
   int tile_m, tile_n;
   tile_of(blockIdx.x, tiles_m, tiles_n, tile_m, tile_n);
-  gemm_body<WAVES_M, WAVES_N, WMT, WNT, W4, SWIGLU>(x, wt, st, zt, y, M, N, K, tile_m, tile_n, 0, K);
+  gemm_body<WAVES_M, WAVES_N, WMT, WNT, W4, SWIGLU, GEMM_PLAIN, F16>(x, wt, st, zt, y, M, N, K, tile_m, tile_n, 0, K);
 }
 
 // Stream-K: a grid that stays, one workgroup per CU.  The tiles' K runs, in units of 256, form one sequence (tile
@@ -653,13 +667,13 @@ int launch_streamk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, co
   O355_CHECK_LAUNCH();
 }
 
-template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false>
+template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false, bool F16 = false>
 int launch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M, int N,
                 int K, hipStream_t stream) {
   constexpr int BM = 32 * WMT * WAVES_M, BN = 32 * WNT * WAVES_N;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;  // fused SwiGLU: N/2 divides by BN/2
   const size_t lds = (size_t)(3 * (BM / 8) + 2 * (BN / 8)) * 1024;
-  auto kern = gemm_kernel<WAVES_M, WAVES_N, WMT, WNT, W4, SWIGLU>;
+  auto kern = gemm_kernel<WAVES_M, WAVES_N, WMT, WNT, W4, SWIGLU, F16>;
   if (lds > 48 * 1024) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) !=
         hipSuccess)
@@ -716,7 +730,7 @@ int launch_splitk(const uint16_t* x, const uint32_t* wt, const uint16_t* st, con
 // is far from proportional to the tile's area: a K-stage costs about 0.5 us of latency however small
 // the tile.  The table holds measured microseconds per round at K = 4096 with int4 weights (the ratios
 // are what matters); the shape with the smallest rounds x time wins.
-template <bool W4>
+template <bool W4, bool F16 = false>
 int dispatch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, uint16_t* y, int M,
                   int N, int K, hipStream_t stream, int force_tile = 0) {  // force_tile: 1000 * rows + columns, 0 = choose
   const int cus = 256;
@@ -733,11 +747,11 @@ int dispatch_gemm(const uint16_t* x, const uint32_t* wt, const uint16_t* st, con
   }
   if (force_tile) best = force_tile < 1000 ? 256000 + force_tile : force_tile;
   switch (best) {
-    case 256256: return launch_gemm<2, 4, 4, 2, W4>(x, wt, st, zt, y, M, N, K, stream);
-    case 256192: return launch_gemm<4, 2, 2, 3, W4>(x, wt, st, zt, y, M, N, K, stream);
-    case 256128: return launch_gemm<4, 2, 2, 2, W4>(x, wt, st, zt, y, M, N, K, stream);
-    case 128128: return launch_gemm<2, 4, 2, 1, W4>(x, wt, st, zt, y, M, N, K, stream);
-    case 128064: return launch_gemm<4, 2, 1, 1, W4>(x, wt, st, zt, y, M, N, K, stream);
+    case 256256: return launch_gemm<2, 4, 4, 2, W4, false, F16>(x, wt, st, zt, y, M, N, K, stream);
+    case 256192: return launch_gemm<4, 2, 2, 3, W4, false, F16>(x, wt, st, zt, y, M, N, K, stream);
+    case 256128: return launch_gemm<4, 2, 2, 2, W4, false, F16>(x, wt, st, zt, y, M, N, K, stream);
+    case 128128: return launch_gemm<2, 4, 2, 1, W4, false, F16>(x, wt, st, zt, y, M, N, K, stream);
+    case 128064: return launch_gemm<4, 2, 1, 1, W4, false, F16>(x, wt, st, zt, y, M, N, K, stream);
   }
   return O355_EINVAL;
 }
@@ -770,6 +784,16 @@ extern "C" int olmo355_w4_gemm(const uint16_t* x, const uint32_t* wt, const uint
   if (misaligned16(y)) return O355_EINVAL;
   if ((K & 127) || (N & 15)) return O355_EUNSUPPORTED;
   return dispatch_gemm<true>(x, wt, st, zt, y, M, N, K, as_stream(stream));
+}
+
+// fp16 activations in, fp16 out; the weights dequantised to fp16 as the reference's QuantLinear does
+// (qlinear_cuda_old.py:253-265,287-290).  Any M; tiled launches only (no split-K or stream-K form).
+extern "C" int olmo355_w4_gemm_f16(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
+                                   uint16_t* y, int M, int N, int K, void* stream) {
+  if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
+  if (misaligned16(y)) return O355_EINVAL;
+  if ((K & 127) || (N & 15)) return O355_EUNSUPPORTED;
+  return dispatch_gemm<true, true>(x, wt, st, zt, y, M, N, K, as_stream(stream));
 }
 
 extern "C" int olmo355_gemm_splitk_plan(int M, int N, int K) { return splitk_plan(M, N, K); }

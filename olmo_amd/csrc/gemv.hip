@@ -652,12 +652,17 @@ struct ChainNorm {
 // no VALU), all weight requests of the wave issued before anything else is waited for, the sums of
 // the activations from the matrix cores (B = ones) instead of a staging pass.  GPA = 4, 2 or 1 groups
 // share an accumulator as in w4_gemv_rot_kernel (M <= 4, 8, 16); the norm prologues exist for GPA = 4.
-template <int GPA, int NT, int WAVES, int PRO, int EPI>
+// F16 (plain products only): fp16 activations and output on the fp16 matrix instruction.  The weights are then what
+// the reference's QuantLinear multiplies with, fp16(scale * (q - zero)), formed per word before the product (no sums
+// of the activations, no correction afterwards): every lane also fetches scale and zero of its own column for each
+// group in flight.
+template <int GPA, int NT, int WAVES, int PRO, int EPI, bool F16 = false>
 __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u32x4* __restrict__ wt,
                                                    const uint16_t* __restrict__ st, const uint8_t* __restrict__ zt) {
   constexpr int RP = 16 / GPA;  // operand rows per group slot
   constexpr int KQS = 4 / GPA;  // lane row blocks per slot
   static_assert(PRO == 0 || GPA == 4, "the norm prologues are written for M <= 4");
+  static_assert(!F16 || (PRO == 0 && EPI == 0), "fp16 activations: plain products");
   extern __shared__ __align__(16) unsigned char smem[];
   const int M = args.M, K = args.K;
   const int G = K >> 7, ntiles = args.N >> 4, nvec = K >> 3;
@@ -720,16 +725,30 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
   ChainNorm<CHAIN ? (1 << (PRO - 8)) : 1> chain;
   if constexpr (CHAIN) chain.begin(args, g_begin * 256, g_end * 256);
   else if constexpr (PRO != 0) norm.begin(args, wave);
+  uint32_t sq[F16 ? GPA : 1][NT], zq[F16 ? GPA : 1][NT];  // F16: scale and zero of (group in slot u, this lane's column)
+  auto issue_szq = [&](int u, int g) {
+    const int gc = min(g, G - 1);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      sq[F16 ? u : 0][nt] = __builtin_amdgcn_raw_buffer_load_b16(rs, col * 2, (tg[nt] + gc) * 32, 0);
+      zq[F16 ? u : 0][nt] = __builtin_amdgcn_raw_buffer_load_b8(rz, col >> 1, (tg[nt] + gc) * 8, 0);
+    }
+  };
 #pragma unroll
   for (int u = 0; u < GPA; ++u) issue_w(u, g_begin + u);
-  issue_sz(s16c, z8c, g_begin);
+  if constexpr (F16) {
+#pragma unroll
+    for (int u = 0; u < GPA; ++u) issue_szq(u, g_begin + u);
+  } else {
+    issue_sz(s16c, z8c, g_begin);
+  }
   if constexpr (PRO == 0 || CHAIN) {
     // zero row, this wave's slice of it
     for (int off = g_begin * 256 + lane * 16; off < g_end * 256; off += 1024)
       *reinterpret_cast<u32x4*>(smem + xbytes + off) = u32x4{0u, 0u, 0u, 0u};
     if constexpr (CHAIN) chain.finish(args, smem, g_begin * 256, g_end * 256);
     // everything but the GPA*NT weight and 2*NT scale/zero requests has arrived: the slice is in LDS
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(GPA * NT + 2 * NT, true));
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(F16 ? 3 * GPA * NT : GPA * NT + 2 * NT, true));
   } else {
     norm.finish(args, xl, red, wave);
   }
@@ -744,11 +763,42 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
   const bf16x8 ones = ones_bf16x8();
   const UnpackConsts uc;
+  auto mma = [](const bf16x8& a_, const bf16x8& b_, const f32x4& c_) {
+    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+    if constexpr (F16) return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a_), __builtin_bit_cast(f16x8, b_), c_, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_, b_, c_, 0, 0, 0);
+  };
   f32x4 acc[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) acc[nt] = zero4;
 
-  for (int base = g_begin; base < g_end; base += GPA) {
+  if constexpr (F16) {
+    for (int base = g_begin; base < g_end; base += GPA) {
+#pragma unroll
+      for (int u = 0; u < GPA; ++u) {
+        const int g = base + u;
+        if (g < g_end) {
+          const uint16_t* xp = xl + xoff[u] + 128 * g;
+          DequantConstsF16 dc[NT];
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            dc[nt] = dequant_consts_f16((uint16_t)sq[u][nt], 1 + (int)((zq[u][nt] >> (4 * (col & 1))) & 15u));  // stored zero points are one less
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const bf16x8 af = *reinterpret_cast<const bf16x8*>(xp + 32 * j);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+              acc[nt] = mma(af, __builtin_bit_cast(bf16x8, dequant_word_f16(w[u][nt][j], dc[nt])), acc[nt]);
+          }
+          if (g + GPA < g_end) {  // refill the slot just consumed
+            issue_w(u, g + GPA);
+            issue_szq(u, g + GPA);
+          }
+        }
+      }
+    }
+  }
+  for (int base = g_begin; !F16 && base < g_end; base += GPA) {
     const bool more = base + GPA < g_end;
     if (more) issue_sz(s16n, z8n, base + GPA);
     f32x4 t[NT], xsum = zero4;
@@ -762,10 +812,9 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const bf16x8 af = *reinterpret_cast<const bf16x8*>(xp + 32 * j);
-          xsum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, ones, xsum, 0, 0, 0);
+          xsum = mma(af, ones, xsum);
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
-            t[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, unpack_w4_bias128(w[u][nt][j], uc), t[nt], 0, 0, 0);
+          for (int nt = 0; nt < NT; ++nt) t[nt] = mma(af, unpack_w4_bias128(w[u][nt][j], uc), t[nt]);
         }
         if (g + GPA < g_end) issue_w(u, g + GPA);  // refill the slot just consumed
       }
@@ -807,8 +856,15 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
     for (int i = tid; i < NT * RP * 16; i += WAVES * 64) {  // whole waves: 16 lanes = one (row, tile)
       const int c = i & 15, m = (i >> 4) % RP, nt = (i >> 4) / RP;
       const bool live = tile[nt] < ntiles && m < M;
-      const float v = live ? round_bf16(total_of(nt, m, c)) : 0.f;
-      if (live) args.y[(int64_t)m * args.N + tile[nt] * 16 + c] = f32_to_bf16_bits(v);
+      float v = 0.f;
+      if constexpr (F16) {
+        const _Float16 hv = (_Float16)(live ? total_of(nt, m, c) : 0.f);
+        v = (float)hv;
+        if (live) args.y[(int64_t)m * args.N + tile[nt] * 16 + c] = __builtin_bit_cast(uint16_t, hv);
+      } else {
+        v = live ? round_bf16(total_of(nt, m, c)) : 0.f;
+        if (live) args.y[(int64_t)m * args.N + tile[nt] * 16 + c] = f32_to_bf16_bits(v);
+      }
       if (args.ssq_out) {  // sum of squares of the 16 outputs of (row, tile): one row of 16 lanes
         const float q = row16_sum(v * v);
         if (live && c == 0) args.ssq_out[(int64_t)m * ntiles + tile[nt]] = q;
@@ -828,11 +884,11 @@ __device__ __forceinline__ void w4_gemv_small_body(const GemvArgs& args, const u
   }
 }
 
-template <int GPA, int NT, int WAVES, int PRO, int EPI>
+template <int GPA, int NT, int WAVES, int PRO, int EPI, bool F16 = false>
 __global__ __launch_bounds__(WAVES * 64) void w4_gemv_small_kernel(GemvArgs args, const u32x4* __restrict__ wt,
                                                                    const uint16_t* __restrict__ st,
                                                                    const uint8_t* __restrict__ zt) {
-  w4_gemv_small_body<GPA, NT, WAVES, PRO, EPI>(args, wt, st, zt);
+  w4_gemv_small_body<GPA, NT, WAVES, PRO, EPI, F16>(args, wt, st, zt);
 }
 
 // ---- int4, 5 .. 8 rows: the activations as operand fragments, never whole in LDS ------------------------------
@@ -1401,9 +1457,10 @@ int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, 
     if (st_mid != O355_EUNSUPPORTED || force_mid) return st_mid;  // else: sizes beyond its 32-bit offsets
   }
   if ((a.ssq_in || a.ssq_out) && a.M > 4) return w4_r8_dispatch(a, wt, st, zt, pro, epi, 0, 0, stream);
-  if (a.ssq_in && a.M > 2) {
-    // three and four rows with the chained prologue: the kernel below needs four pieces of x per lane for them and
-    // with those registers only one of its workgroups fits a CU (measured, 4 rows: att_proj 37 against 11 us)
+  if (a.ssq_in && a.M > 1) {
+    // two to four rows with the chained prologue: the kernel below needs two or four pieces of x per lane for them
+    // and with those registers one or two of its workgroups fit a CU (measured, att_proj / ff_proj: 2 rows 16.4 /
+    // 21.7 against 8.9 / 12.6 us, 4 rows 37 / 64 against 9.6 / 13.2)
     const int st8 = w4_r8_dispatch(a, wt, st, zt, pro, epi, 0, 0, stream);
     if (st8 != O355_EUNSUPPORTED) return st8;
   }
@@ -1466,6 +1523,26 @@ extern "C" int olmo355_w4_gemv(const uint16_t* x, const uint32_t* wt, const uint
   if (M > 64 || (K & 127) || (N & 15)) return O355_EUNSUPPORTED;
   const GemvArgs a{x, nullptr, nullptr, nullptr, y, 0.f, M, N, K};
   return w4_gemv_dispatch(a, wt, st, zt, false, false, stream);
+}
+
+// fp16 activations in, fp16 out (QuantLinear.forward on fp16 input, qlinear_cuda_old.py:287-290), up to 16 rows that fit
+// LDS with a zero row; O355_EUNSUPPORTED otherwise (olmo355_w4_gemm_f16 takes any M).
+extern "C" int olmo355_w4_gemv_f16(const uint16_t* x, const uint32_t* wt, const uint16_t* st, const uint8_t* zt,
+                                   uint16_t* y, int M, int N, int K, void* stream) {
+  if (!x || !wt || !st || !zt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
+  if (M > 16 || (K & 127) || (N & 15)) return O355_EUNSUPPORTED;
+  if ((int64_t)(M + 1) * K * 2 > kSmallMaxBytes || (int64_t)(N >> 4) * (K >> 7) * 1024 >= (1ll << 31)) return O355_EUNSUPPORTED;
+  const GemvArgs a{x, nullptr, nullptr, nullptr, y, 0.f, M, N, K};
+  const GemvPlan p = plan_gemv(M, N, K, true, false, false);
+  const u32x4* w = (const u32x4*)wt;
+  const int sgpa = M <= 4 ? 4 : (M <= 8 ? 2 : 1);
+#define SMALL_F16(GPAv, Wv)                          \
+  if (sgpa == GPAv && p.waves == Wv)                 \
+    return launch_small(w4_gemv_small_kernel<GPAv, 1, Wv, 0, 0, true>, p, a, as_stream(stream), w, st, zt);
+  SMALL_F16(4, 4) SMALL_F16(4, 8) SMALL_F16(4, 16) SMALL_F16(2, 4) SMALL_F16(2, 8) SMALL_F16(2, 16) SMALL_F16(1, 4) SMALL_F16(1, 8)
+  SMALL_F16(1, 16)
+#undef SMALL_F16
+  return O355_EUNSUPPORTED;
 }
 
 extern "C" int olmo355_b16_gemv(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K,

@@ -122,11 +122,35 @@ def w4t_dequant_fp16(w: W4Tiled) -> torch.Tensor:
     return out
 
 
-def w4_linear(x: torch.Tensor, w: W4Tiled) -> torch.Tensor:
-    """``x[..., K] @ W[K, N]`` for a tiled int4 weight; bf16 in, bf16 out."""
+def w4_linear_f16(x: torch.Tensor, w: W4Tiled) -> torch.Tensor:
+    """``x[..., K] @ W[K, N]`` for a tiled int4 weight in the reference QuantLinear's own arithmetic: fp16 activations,
+    weights dequantised to fp16, fp16 out (fp32 accumulation)."""
     _dev(x, w.wt)
+    if x.dtype != torch.float16:
+        raise TypeError("float16 activations expected")
+    if x.shape[-1] != w.K:
+        raise ValueError(f"x last dim {x.shape[-1]} != K {w.K}")
+    M = x.numel() // w.K
+    y = torch.empty(*x.shape[:-1], w.N, dtype=torch.float16, device=x.device)
+    if M == 0:
+        return y
+    st = 2
+    if M <= 16:
+        st = lib().olmo355_w4_gemv_f16(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream())
+        if st != 2:
+            check("olmo355_w4_gemv_f16", st)
+    if st == 2:
+        check("olmo355_w4_gemm_f16", lib().olmo355_w4_gemm_f16(_p(x), _p(w.wt), _p(w.st), _p(w.zt), _p(y), M, w.N, w.K, _stream()))
+    return y
+
+
+def w4_linear(x: torch.Tensor, w: W4Tiled) -> torch.Tensor:
+    """``x[..., K] @ W[K, N]`` for a tiled int4 weight; bf16 in, bf16 out (fp16 in, fp16 out: :func:`w4_linear_f16`)."""
+    _dev(x, w.wt)
+    if x.dtype == torch.float16:
+        return w4_linear_f16(x, w)
     if x.dtype != torch.bfloat16:
-        raise TypeError("int4 linear takes bfloat16 activations")
+        raise TypeError("int4 linear takes bfloat16 or float16 activations")
     if x.shape[-1] != w.K:
         raise ValueError(f"x last dim {x.shape[-1]} != K {w.K}")
     M = x.numel() // w.K
@@ -615,16 +639,16 @@ def add(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
 
 
 def add_bias(x: torch.Tensor, bias_f16: torch.Tensor) -> torch.Tensor:
-    """``x + bias`` over the last axis: bf16 rows, the fp16 bias buffer of a quantised Linear."""
+    """``x + bias`` over the last axis: bf16 or fp16 rows, the fp16 bias buffer of a quantised Linear."""
     _dev(x, bias_f16)
     N = x.shape[-1]
-    if x.dtype != torch.bfloat16 or bias_f16.dtype != torch.float16 or bias_f16.shape != (N,):
-        raise ValueError("add_bias takes bf16 rows and an fp16 bias of the row length")
+    if x.dtype not in (torch.bfloat16, torch.float16) or bias_f16.dtype != torch.float16 or bias_f16.shape != (N,):
+        raise ValueError("add_bias takes bf16 or fp16 rows and an fp16 bias of the row length")
     x = x.contiguous()
     out = torch.empty_like(x)
     if x.numel():
-        check("olmo355_add_bias_bf16",
-              lib().olmo355_add_bias_bf16(_p(x), _p(bias_f16.contiguous()), _p(out), x.numel() // N, N, _stream()))
+        fn = lib().olmo355_add_bias_bf16 if x.dtype == torch.bfloat16 else lib().olmo355_add_bias_f16
+        check("olmo355_add_bias", fn(_p(x), _p(bias_f16.contiguous()), _p(out), x.numel() // N, N, _stream()))
     return out
 
 

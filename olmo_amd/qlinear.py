@@ -146,9 +146,11 @@ class QuantLinear(nn.Module):
 
     # -- forward ---------------------------------------------------------------------------------
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        # bf16 rows (the model's own activations) stay bf16; anything else goes through the reference's own arithmetic:
+        # cast to fp16, fp16 weights, result cast back (qlinear_cuda_old.py:287-290)
         in_dtype = x.dtype
-        if in_dtype != torch.bfloat16:
-            x = x.to(torch.bfloat16)  # the reference casts to float16 here (qlinear_cuda_old.py:287)
+        if in_dtype not in (torch.bfloat16, torch.float16):
+            x = x.to(torch.float16)
         t = self.tiled
         x = x.contiguous()
         if self._perm is not None:
@@ -156,7 +158,7 @@ class QuantLinear(nn.Module):
         y = ops.w4_linear(x, t)
         if self._has_bias:  # qlinear_cuda_old.py:288-290
             y = ops.add_bias(y, self.bias)
-        return y if in_dtype == torch.bfloat16 else y.to(in_dtype)
+        return y if y.dtype == in_dtype else y.to(in_dtype)
 
     def extra_repr(self):
         return f"in={self.infeatures}, out={self.outfeatures}, bits={self.bits}, group_size={self.group_size}"

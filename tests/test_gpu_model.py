@@ -402,6 +402,16 @@ def test_quantlinear_bias(dev):
         y = ql(x.to(dev)).cpu()
         assert (y.float() - ref.float()).abs().max().item() <= 2 ** -7 * ref.float().abs().max().item()
         assert (y.float() - prod.float() - bias.float()).abs().max().item() <= 2 ** -6 * ref.float().abs().max().item()
+        # fp16 and fp32 inputs take the reference's own route (qlinear_cuda_old.py:287-290): cast to fp16, fp16 weights,
+        # bias added in fp16, result cast back to the input's type
+        for dt in (torch.float16, torch.float32):
+            xh = x.to(dt)
+            prod16 = ow4.linear_fp32(xh.half(), ow4.dequantize(qw, qz, sc, 128)).half()
+            ref16 = (prod16.float() + bias.float()).half()
+            yh = ql(xh.to(dev)).cpu()
+            assert yh.dtype == dt
+            tol = 2 ** -10 * ref16.float().abs().max().item()  # two roundings of at most half an fp16 ulp of the largest entry
+            assert (yh.float() - ref16.float()).abs().max().item() <= tol
 
     cfg = small_cfg("olmo2")
     w = om.random_weights(cfg, torch.bfloat16, seed=31, quantized=True, norm_weight_std=0.1)

@@ -94,10 +94,20 @@ def test_w4_dequant_g_idx_general(dev):
     assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
 
 
+def _ulp16(ref):
+    """One fp16 unit in the last place at the magnitude of ``ref`` (normal range)."""
+    return torch.maximum(torch.tensor(2.0 ** -24), 2.0 ** (torch.floor(torch.log2(ref.abs().clamp_min(2.0 ** -14))) - 10))
+
+
 def test_w4_golden_vectors_through_gemv(dev, golden_dir):
-    """The reference's own kernel KATs (AGQ tests/test_q4.py) through the HIP GEMV."""
+    """The reference's own kernel KATs (AGQ tests/test_q4.py:1071-1104, :1757-1764) through the HIP kernels in the
+    reference's own arithmetic -- fp16 activations, fp16(scale * (q - zero)) weights: the decode kernel and, for the same
+    single row, the tiled GEMM must both give the stored outputs to 2 fp16 ulp, with no allowance for input rounding.
+    The bf16 path (the model's) is held to the oracle on the same bf16-rounded inputs."""
     import json
     import os
+
+    from olmo_amd import _lib
 
     ops = _ops()
     kats = json.load(open(os.path.join(golden_dir, "q4_kat.json")))
@@ -110,16 +120,37 @@ def test_w4_golden_vectors_through_gemv(dev, golden_dir):
         qzeros = torch.zeros(k // 128, n // 8, dtype=torch.int32)
         inp = torch.rand(1, 1, k, dtype=torch.float16)
         t = ops.w4_repack(qweight.to(dev), qzeros.to(dev), scales.to(dev), 128)
-        # inputs are fp16 values in [0,1): representable in bf16 only after rounding, so compare
-        # against the oracle on the same bf16 inputs, and against the stored vector with the
-        # input-rounding error budget (|dx| <= 2^-9, sum |w| <= k*0.2)
+        stored = torch.tensor(kat["out"])
+        x16 = inp[0].to(dev)
+        y16 = ops.w4_linear(x16, t)
+        assert y16.dtype == torch.float16
+        assert ((y16.float().cpu()[0] - stored).abs() <= 2 * _ulp16(stored)).all(), name
+        yg = torch.empty_like(y16)
+        assert _lib.lib().olmo355_w4_gemm_f16(x16.data_ptr(), t.wt.data_ptr(), t.st.data_ptr(), t.zt.data_ptr(), yg.data_ptr(), 1, n, k,
+                                              torch.cuda.current_stream().cuda_stream) == 0
+        assert ((yg.float().cpu()[0] - stored).abs() <= 2 * _ulp16(stored)).all(), name
+        W = ow4.dequantize(qweight, qzeros, scales, 128)
         xb = inp[0].to(torch.bfloat16)
         y = ops.w4_linear(xb.to(dev), t).float().cpu()[0]
-        W = ow4.dequantize(qweight, qzeros, scales, 128)
-        ref_same_inputs = ow4.linear_fp32(xb, W)[0]
-        assert torch.allclose(y, ref_same_inputs, rtol=2 ** -8, atol=1e-3), name
-        stored = torch.tensor(kat["out"])
-        assert (y - stored).abs().max() < 0.15, name  # bf16 rounding of the inputs dominates
+        assert torch.allclose(y, ow4.linear_fp32(xb, W)[0], rtol=2 ** -8, atol=1e-3), name
+
+
+@pytest.mark.parametrize("M", [1, 3, 4, 5, 8, 9, 16, 17, 40, 300, 2048])
+@pytest.mark.parametrize("N,K", [(4096, 4096), (1024, 11008), (272, 384)])
+def test_w4_linear_fp16(dev, M, N, K):
+    """fp16 activations (the reference QuantLinear's arithmetic) against the oracle on the same fp16 inputs and the
+    fp16 dequantised table: one fp16 rounding of the result plus what fp32 sums of this length differ by."""
+    say("w4_linear_fp16", M, N, K)
+    ops = _ops()
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=M + N + K)
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(7)).to(torch.float16)
+    W = ow4.dequantize(qw, qz, sc, 128)
+    ref = ow4.linear_fp32(x, W)
+    t = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    y = ops.w4_linear(x.to(dev), t)
+    assert y.dtype == torch.float16 and torch.equal(y, ops.w4_linear(x.to(dev), t))
+    err = (y.float().cpu() - ref).abs()
+    assert (err <= 2 * _ulp16(ref) + 2 ** -13 * ref.abs().max()).all(), float(err.max())
 
 
 # ------------------------------------------------------------------------------------------------
