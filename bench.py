@@ -40,6 +40,60 @@ def linear_shapes(cfg):
     return [(d + 2 * dkv, d), (d, d), (cfg.hidden_size, d), (d, cfg.act_out_size)]  # (N, K)
 
 
+def relay_compare(cfg, dev, ctx: int, steps: int) -> int:
+    """Batch-1 decode of the 7B int4 model at KV context ``ctx``: the chained step against the opt-in relay
+    (``olmo_amd.model.RELAY``: every hand-over between launches carried by tags in the data, launches alternating
+    between two streams inside the captured step).  Same prompt, same weights; three repetitions of each form."""
+    import torch
+
+    from olmo_amd import model as M
+    from olmo_amd.generate import DecodeSession, _prefill
+    from olmo_amd.synthetic import build_random_model
+
+    model = build_random_model(cfg, torch.bfloat16, quantized=True, seed=0, device=dev, max_cache_len=ctx + 4 * steps + 64,
+                               free_checkpoint_buffers=True)
+    ids = torch.randint(0, cfg.vocab_size, (1, ctx), generator=torch.Generator().manual_seed(0)).to(dev)
+
+    def run(relay: bool, two: bool):
+        M.RELAY, M.RELAY_TWO_STREAMS = relay, two
+        _, cache, first, kb = _prefill(model, ids, None)
+        sess = DecodeSession(model, cache, first, kb)
+        sess.step()
+        sess.step()
+        sess.capture()
+        toks = []
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            sess.step()
+            toks.append(sess.ids.view(-1).clone())
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        model.relay_check()
+        return dt * 1e3, torch.stack(toks)
+
+    forms = {"chained": (False, False), "relay_one_stream": (True, False), "relay_two_streams": (True, True)}
+    ms = {k: [] for k in forms}
+    toks = {}
+    try:
+        for rep in range(3):
+            for name, (relay, two) in forms.items():
+                t, tk = run(relay, two)
+                ms[name].append(t)
+                toks[name] = tk
+                log(f"[bench --relay] {name}: {t:.3f} ms/step")
+    finally:
+        M.RELAY, M.RELAY_TWO_STREAMS = False, True
+    same = bool(torch.equal(toks["relay_one_stream"], toks["relay_two_streams"]))
+    agree = float((toks["chained"] == toks["relay_one_stream"]).float().mean())
+    out = {"workload": f"olmo2-7b int4-g128 greedy decode, batch 1, KV context {ctx}, {steps} captured steps",
+           "ms_per_step": {k: min(v) for k, v in ms.items()}, "ms_per_step_all": ms,
+           "relay_streams_same_tokens": same, "relay_vs_chained_token_agreement": agree,
+           "relay_plan": {k: {n: hex(c) for n, c in v.items()} for k, v in getattr(model._relay, "plans", {}).items()} if model._relay else None}
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -62,6 +116,10 @@ def main() -> int:
     ap.add_argument("--counters-probe", action="store_true",
                     help="for rocprofv3 --pmc over every kernel of the path: a 256 MiB device copy (the yardstick), one "
                          "prefill 1 x context and four eager batch-1 decode steps of the 7B int4 model; nothing is timed")
+    ap.add_argument("--relay", action="store_true",
+                    help="the batch-1 decode step of the 7B int4 model three ways in one run: the chained launches (the "
+                         "product's path), the relay on one stream and the relay on two streams inside the captured step; "
+                         "prints ms per step and whether the three gave the same tokens; one JSON object on stdout")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this build runs the whole model on ONE GPU; --gpus N with N > 1 is not supported.")
@@ -88,6 +146,8 @@ def main() -> int:
         return linear_sweep(dev)
     if args.config4:
         return config4(dev, args.steps if args.steps != 128 else 32)
+    if args.relay:
+        return relay_compare(cfg, dev, args.context, args.steps if args.steps != 128 else 64)
     ctx, K, W = args.context, args.steps, args.warmup
     cap = ctx + K + W + 8
     t0 = time.time()

@@ -491,8 +491,10 @@ def test_config2_1b_bf16_prefill_and_256_greedy_steps(dev):
     for i in range(255):
         r, kvf = referee.forward(toks[:, i:i + 1], past_key_values=kvf, use_cache=True)
         frefs.append(r[:, -1])
-    strict, loose = agreement(toks, ref, referee_logits=torch.stack(frefs, dim=1), floors=True)
+    fref = torch.stack(frefs, dim=1)
+    strict, loose = agreement(toks, ref, referee_logits=fref, floors=True)
     say(f"  softmax max-abs err {e:.3e}; greedy agreement over 256 steps: strict {strict:.4f} within 2 ulps {loose:.4f}")
+    say("  " + ", ".join(f"{k} {v:.4f}" if isinstance(v, float) else f"{k} {v}" for k, v in agreement_report(toks, ref, fref).items()))
     assert e <= 2e-2
     assert loose >= 0.99
 
