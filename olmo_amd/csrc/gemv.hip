@@ -1383,6 +1383,7 @@ constexpr bool r8_exists(int nt, int waves, int pmax, bool pro, bool epi, bool p
     return !(nt == 4 && pmax == 3);
   }
   if (waves != 16) return false;
+  if (nt == 1 && !epi && pmax <= 2) return true;  // one tile: two pairs fit with the prologue and with the second set
   if (pf) return pmax == 1 && nt <= 2;
   if (pro) return pmax == 1;
   return nt == 1 || pmax == 1;
@@ -1404,14 +1405,27 @@ int w4_r8_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, co
   }
   // a workgroup walks its sets of tiles one after the other: small sets, few registers; two tiles per set once a
   // workgroup would walk more than eight sets (measured at 8 rows, N = 100352: 41.7 against 47.6 us)
-  if (nt == 0) nt = epi ? 2 : (ntiles > 8 * n_cu ? 2 : 1);
-  const int sets = epi ? ((ntiles >> 1) + (nt >> 1) - 1) / (nt >> 1) : (ntiles + nt - 1) / nt;
-  const bool want_pf = sets > n_cu;
+  const bool auto_nt = nt == 0;
+  if (auto_nt) nt = epi ? 2 : (ntiles > 8 * n_cu ? 2 : 1);
   auto pairs_of = [&](int wv) { return std::max(1, ((G + wv - 1) / wv + 1) >> 1); };  // of the wave with the longest run
-  if (waves == 0) {  // 16 waves where an instantiation exists, with the second set of weight registers or without
-    const int p16 = pairs_of(16);
-    waves = (G >= 32 && (r8_exists(nt, 16, p16, pro, epi, want_pf) || r8_exists(nt, 16, p16, pro, epi, false))) ? 16 : 8;
+  auto sets_of = [&](int t) { return epi ? ((ntiles >> 1) + (t >> 1) - 1) / (t >> 1) : (ntiles + t - 1) / t; };
+  auto any16 = [&](int t) { return r8_exists(t, 16, pairs_of(16), pro, epi, sets_of(t) > n_cu) || r8_exists(t, 16, pairs_of(16), pro, epi, false); };
+  auto any8 = [&](int t) { return r8_exists(t, 8, pairs_of(8), pro, epi, sets_of(t) > n_cu) || r8_exists(t, 8, pairs_of(8), pro, epi, false); };
+  if (waves == 0) {
+    // 16 waves where an instantiation exists, unless the groups split much more evenly into pairs over 8 (K = 5120:
+    // 40 groups are 16 runs of 2 or 3 -- two pairs each, a third of them empty -- or 8 runs of 5; measured at 8 rows,
+    // N = 13824: 14.2 against 12.8 us with two tiles per set)
+    const double fill16 = (double)G / (2.0 * pairs_of(16) * 16), fill8 = (double)G / (2.0 * pairs_of(8) * 8);
+    const int nt8 = (auto_nt && !epi && nt == 1 && any8(2)) ? 2 : nt;
+    if (G >= 32 && any16(nt) && !(fill8 > fill16 + 0.15 && any8(nt8))) {
+      waves = 16;
+    } else {
+      waves = 8;
+      nt = nt8;
+    }
   }
+  const int sets = sets_of(nt);
+  const bool want_pf = sets > n_cu;
   const int pmax = pairs_of(waves);
   bool pf = want_pf;
   if (pf && !r8_exists(nt, waves, pmax, pro, epi, true)) pf = false;
@@ -1423,6 +1437,7 @@ int w4_r8_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, co
   R8_CASE(3, 16, 1, false, 0, false) R8_CASE(3, 16, 1, true, 0, false)
   R8_CASE(2, 16, 1, false, 1, false) R8_CASE(2, 16, 1, true, 1, false)
   R8_CASE(4, 16, 1, false, 1, false) R8_CASE(4, 16, 1, true, 1, false)
+  R8_CASE(1, 16, 2, true, 0, false) R8_CASE(1, 16, 2, true, 0, true) R8_CASE(1, 16, 2, false, 0, true)
   R8_CASE(1, 16, 1, false, 0, true) R8_CASE(1, 16, 1, true, 0, true) R8_CASE(2, 16, 1, false, 0, true) R8_CASE(2, 16, 1, true, 0, true)
   R8_CASE(2, 16, 1, false, 1, true) R8_CASE(2, 16, 1, true, 1, true)
   // 8 waves
