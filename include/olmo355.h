@@ -215,6 +215,18 @@ int olmo355_qknorm_rope_kvwrite(const void* qkv, const void* qw, const void* kw,
 int olmo355_attn_prefill(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out,
                          int B, int T, int H, int Hkv, int hd, int Lmax, int past_len, int bias_stride, int dtype,
                          void* stream);
+/* The same with a workspace.  A launch with fewer workgroups than the chip has places -- one prompt of 1152 to 4096
+ * tokens from scratch with few heads -- lasts as long as its longest query block (causal work grows with the block's
+ * position); with a workspace the blocks whose keys run past 1024 are shared between workgroups along the keys, and
+ * the one that finishes a block last combines all partial results and writes the rows (no workgroup waits for
+ * another; same products, the partial sums of a row combined in the order of their keys whoever comes last).
+ * olmo355_attn_prefill_workspace_bytes: the bytes that form needs for this call, 0 where the plain launch is the one
+ * to use (ws may then be NULL).  ws: zeroed when allocated (its first 4096 bytes are int32 counters, one per (batch,
+ * head, query block), which every launch leaves at zero again, so one workspace may serve calls of different shapes); O355_EINVAL when ws_bytes is smaller than needed. */
+int64_t olmo355_attn_prefill_workspace_bytes(int B, int T, int H, int hd, int past_len, int dtype);
+int olmo355_attn_prefill_ws(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out,
+                            void* ws, int64_t ws_bytes, int B, int T, int H, int Hkv, int hd, int Lmax, int past_len,
+                            int bias_stride, int dtype, void* stream);
 
 /* T == 1 with the keys split over workgroups.  n_keys_max bounds the number of keys for the
  * launch grid; the true count is past_len + 1 (or *past_len_dev + 1 when given).

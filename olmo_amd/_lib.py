@@ -51,6 +51,8 @@ EXPORTS = {
     "olmo355_layernorm_np": (I, [P, P, I, I, F, I, P]),
     "olmo355_qknorm_rope_kvwrite": (I, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P, F, I, P]),
     "olmo355_attn_prefill": (I, [P, P, P, P, P, I, I, I, I, I, I, I, I, I, P]),
+    "olmo355_attn_prefill_workspace_bytes": (L, [I, I, I, I, I, I]),
+    "olmo355_attn_prefill_ws": (I, [P, P, P, P, P, P, L, I, I, I, I, I, I, I, I, I, P]),
     "olmo355_attn_decode_workspace_bytes": (L, [I, I, I, I]),
     "olmo355_attn_decode": (I, [P, P, P, P, P, P, L, I, I, I, I, I, I, P, I, I, I, P]),
     "olmo355_attn_decode_static_max_bytes": (L, []),

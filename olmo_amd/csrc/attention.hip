@@ -142,10 +142,11 @@ __device__ __forceinline__ float reduce_lane_groups(float v, Op op) {
 // (A function and not a lambda of the kernel: with the memory -> LDS builtin inside a lambda that the kernel calls,
 // this toolchain's host pass emits no launch stub for the kernel, without a diagnostic, and the library then fails
 // to load with an undefined symbol.)
-template <int HD>
+template <int S>  // S = HD / 32, deduced from the arrays
 __device__ __forceinline__ void prefill_request_tile(__amdgpu_buffer_rsrc_t rk, __amdgpu_buffer_rsrc_t rv, unsigned char* kdst,
-                                                     unsigned char* vdst, const int (&k_row)[HD / 32], const int (&k_in)[HD / 32],
-                                                     const int (&v_row)[HD / 32], const int (&v_in)[HD / 32], int k0, int last_pos) {
+                                                     unsigned char* vdst, const int (&k_row)[S], const int (&k_in)[S],
+                                                     const int (&v_row)[S], const int (&v_in)[S], int k0, int last_pos) {
+  constexpr int HD = 32 * S;
   const bool tail = k0 + 63 > last_pos;
 #pragma unroll
   for (int i = 0; i < HD / 32; ++i) {
@@ -163,13 +164,32 @@ struct PrefillLds {
   static constexpr int BYTES = 4 * TILE + 2 * KT * 4;  // K x 2, V x 2, bias x 2
 };
 
+// SPLIT (past_len == 0, at most kPrefillMaxChunks x kPrefillChunkBlocks query blocks): a query block whose keys run
+// past kPrefillChunkBlocks x 128 is shared by several workgroups, one per run of that many keys.  One prompt of 2048
+// tokens and 16 heads is 256 workgroups of 1 to 16 units of work each for the chip's 512 places: the launch lasts as
+// long as its longest workgroup while most places stand empty; cut at 8 units the same work is 384 workgroups of at
+// most half that length, all resident at once.  A workgroup that does not hold all of its block's keys
+// leaves its accumulators, reference maximum and denominator as they stand in its slot of the workspace
+// (device-scope stores) and draws a ticket; the one that draws the block's last ticket adds the others' to its own
+// registers and writes the output.  Nobody waits for anybody.
+constexpr int kPrefillChunkBlocks = 8, kPrefillMaxChunks = 4;
+constexpr int kPrefillMaxTriples = 384, kPrefillTicketBytes = 4096;  // (batch, head, query block) triples of a split launch
+template <int HD>
+struct PrefillSplit {
+  static constexpr int O_BYTES = 4 * 2 * (HD / 16) * 64 * 16;  // waves x query tiles x channel tiles x lanes x float4
+  static constexpr int ML_BYTES = 4 * 2 * 64 * 8;              // (reference maximum, denominator) per wave, query tile, lane
+  static constexpr int SLOT_BYTES = O_BYTES + ML_BYTES;
+};
+
 template <int HD>
 __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_t* __restrict__ q,
                                                                 const uint16_t* __restrict__ kc,
                                                                 const uint16_t* __restrict__ vc,
                                                                 const float* __restrict__ key_bias,
                                                                 uint16_t* __restrict__ out, int T, int H, int Hkv,
-                                                                int Lmax, int past_len, int bias_stride) {
+                                                                int Lmax, int past_len, int bias_stride,
+                                                                unsigned char* __restrict__ ws, int max_chunks) {
+  const bool SPLIT = ws != nullptr;  // uniform over the launch
   constexpr int KT = 64;             // keys per tile
   constexpr int STEPS = HD / 32;     // hd steps of the first product = 1 KiB load instructions per wave, tile and operand
   constexpr int HT = HD / 16;        // hd tiles of the second product
@@ -194,7 +214,26 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
   const float c2 = 1.4426950408889634f / sqrtf((float)HD);  // scores live in the log2 domain: exp2(s*c2 + bias*log2e - m)
   const int64_t cbase = ((int64_t)b * Hkv + hk) * Lmax * HD;
   const int half = (nqb + 1) / 2, rank = blockIdx.y;
-  const int qblock = rank < half ? nqb - 1 - rank : rank - half;
+  int qblock = rank < half ? nqb - 1 - rank : rank - half;
+  int chunk = 0, nchunks = 1;
+  if (SPLIT) {
+    // blockIdx.y counts the (block, run of keys) pairs longest first: the full runs (block b has b / 8 of them), then
+    // the blocks' last runs by length, 8 units down to 1 (block b's last run is b % 8 + 1 units long)
+    constexpr int CB = kPrefillChunkBlocks;
+    int r = rank;
+    qblock = -1;
+    for (int bb = nqb - 1; bb >= CB && qblock < 0; --bb) {
+      const int f = bb / CB;
+      if (r < f) qblock = bb, chunk = r;
+      else r -= f;
+    }
+    for (int sz = CB; sz >= 1 && qblock < 0; --sz) {
+      const int cnt = sz - 1 < nqb ? (nqb - (sz - 1) + CB - 1) / CB : 0;
+      if (r < cnt) qblock = sz - 1 + r * CB, chunk = qblock / CB;
+      else r -= cnt;
+    }
+    nchunks = qblock / CB + 1;
+  }
   const int q0 = qblock * 128 + wave * 32;
 
   // Q^T fragments: lane (query col, hd 32*step + 8*kq ..)
@@ -237,7 +276,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
   }
   float rbias = 0.f;
   auto fetch = [&](int k0, int buf) {
-    prefill_request_tile<HD>(rk_, rv_, lds_k + buf * TILE + wave * (STEPS << 10), lds_v + buf * TILE + wave * (STEPS << 10), k_row,
+    prefill_request_tile(rk_, rv_, lds_k + buf * TILE + wave * (STEPS << 10), lds_v + buf * TILE + wave * (STEPS << 10), k_row,
                              k_in, v_row, v_in, k0, last_pos);
     if (key_bias && tid < KT) rbias = key_bias[(int64_t)b * bias_stride + min(k0 + tid, last_pos)];
   };
@@ -251,12 +290,14 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
   int v_rd[HT];
 #pragma unroll
   for (int ht = 0; ht < HT; ++ht) v_rd[ht] = (4 * kq + (col >> 2)) * VROW + ((ht ^ v_swz(4 * kq + (col >> 2))) << 5) + 8 * (col & 3);
-  fetch(0, 0);
+  const int k_first = SPLIT ? chunk * (kPrefillChunkBlocks * 128) : 0;
+  const int k_last = SPLIT ? min(last_pos, k_first + kPrefillChunkBlocks * 128 - 1) : last_pos;  // this workgroup's run of keys
+  fetch(k_first, 0);
   publish(0);
   int buf = 0;
-  for (int k0 = 0; k0 <= last_pos; k0 += KT, buf ^= 1) {
+  for (int k0 = k_first; k0 <= k_last; k0 += KT, buf ^= 1) {
     // the other buffer was read during the previous tile, and everybody is past that tile's barrier
-    if (k0 + KT <= last_pos) fetch(k0 + KT, buf ^ 1);
+    if (k0 + KT <= k_last) fetch(k0 + KT, buf ^ 1);
     if (k0 <= wave_last) {  // else nothing visible to this wave in the tile (barriers stay uniform)
     const u32x4* kt_ = reinterpret_cast<const u32x4*>(lds_k + buf * TILE);
     const unsigned char* vt_ = lds_v + buf * TILE;
@@ -373,11 +414,67 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
     }
     publish(buf ^ 1);  // the next tile is in LDS and this one has been read by everybody
   }
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) l[qt] = reduce_lane_groups(l[qt], [](float a, float b) { return a + b; });
+  if (SPLIT) {
+    if (nchunks > 1) {
+      using PS = PrefillSplit<HD>;
+      // the workspace: one ticket counter per (batch, head, block), then the slots [batch][head][block - 8][run]
+      // (the counters' region has one size for every shape: a workspace that served another shape must not be
+      // found holding that launch's partial results where this launch keeps its counters)
+      int* const tickets = reinterpret_cast<int*>(ws);
+      unsigned char* const slots = ws + kPrefillTicketBytes;
+      const int64_t bh = (int64_t)b * H + h;
+      unsigned char* const base = slots + ((bh * (nqb - kPrefillChunkBlocks) + (qblock - kPrefillChunkBlocks)) * max_chunks) * (int64_t)PS::SLOT_BYTES;
+      {
+        const __amdgpu_buffer_rsrc_t rs = make_rsrc(base + (int64_t)chunk * PS::SLOT_BYTES, PS::SLOT_BYTES);
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+#pragma unroll
+          for (int ht = 0; ht < HT; ++ht)
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o[qt][ht]), rs, (((wave * QT + qt) * HT + ht) * 64 + lane) * 16, 0, 16 /* sc1 */);
+          __builtin_amdgcn_raw_buffer_store_b64(u32x2{__float_as_uint(m[qt]), __float_as_uint(l[qt])}, rs,
+                                                PS::O_BYTES + ((wave * QT + qt) * 64 + lane) * 8, 0, 16 /* sc1 */);
+        }
+      }
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, false));  // vmcnt(0): this wave's stores have landed
+      __syncthreads();
+      int* const s_last = reinterpret_cast<int*>(smem);  // the tiles are done with
+      if (tid == 0) {
+        int* tk = tickets + bh * nqb + qblock;
+        const int t = __hip_atomic_fetch_add(tk, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *s_last = (t == nchunks - 1);
+        if (t == nchunks - 1) __hip_atomic_store(tk, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+      }
+      __syncthreads();
+      if (!*s_last) return;
+      // all runs in the order of their keys, this workgroup's own re-read like the others: which workgroup comes
+      // last varies from launch to launch, the order of the additions must not
+      for (int c = 0; c < nchunks; ++c) {
+        const __amdgpu_buffer_rsrc_t rs = make_rsrc(base + (int64_t)c * PS::SLOT_BYTES, PS::SLOT_BYTES);
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+          const u32x2 ml = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rs, PS::O_BYTES + ((wave * QT + qt) * 64 + lane) * 8, 0, 16));
+          const float mo = __uint_as_float(ml.x), lo = __uint_as_float(ml.y);
+          const float mn = c == 0 ? mo : fmaxf(m[qt], mo);
+          const float a_acc = c == 0 ? 0.f : __builtin_amdgcn_exp2f(m[qt] - mn), a_new = __builtin_amdgcn_exp2f(mo - mn);
+          l[qt] = c == 0 ? lo : l[qt] * a_acc + lo * a_new;
+          m[qt] = mn;
+#pragma unroll
+          for (int ht = 0; ht < HT; ++ht) {
+            const f32x4 oo = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, (((wave * QT + qt) * HT + ht) * 64 + lane) * 16, 0, 16));
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[qt][ht][r] = c == 0 ? oo[r] : o[qt][ht][r] * a_acc + oo[r] * a_new;
+          }
+        }
+      }
+    }
+  }
   // ---- write O[q][hd]: lane holds hd = 16ht + 4kq + r for query col ------------------------------------------
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     const int t = q0 + qt * 16 + col;
-    const float inv = 1.f / reduce_lane_groups(l[qt], [](float a, float b) { return a + b; });
+    const float inv = 1.f / l[qt];
     if (t >= T) continue;
     uint16_t* dst = out + ((int64_t)b * T + t) * H * HD + (int64_t)h * HD;
 #pragma unroll
@@ -1208,16 +1305,18 @@ __global__ __launch_bounds__(256) void attn_masked_rows_kernel(const void* __res
 }
 
 int attn_prefill_main(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out, int B, int T,
-                      int H, int Hkv, int hd, int Lmax, int past_len, int bias_stride, int dtype, hipStream_t s);
-}  // namespace
+                      int H, int Hkv, int hd, int Lmax, int past_len, int bias_stride, int dtype, hipStream_t s, void* ws,
+                      int64_t ws_bytes);
+bool prefill_split_applies(int B, int T, int H, int hd, int past_len, int dtype);
+int64_t prefill_split_bytes(int B, int T, int H, int hd);
 
-extern "C" int olmo355_attn_prefill(const void* q, const void* kcache, const void* vcache, const float* key_bias,
-                                    void* out, int B, int T, int H, int Hkv, int hd, int Lmax, int past_len,
-                                    int bias_stride, int dtype, void* stream) {
+int attn_prefill_any(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out, void* ws,
+                     int64_t ws_bytes, int B, int T, int H, int Hkv, int hd, int Lmax, int past_len, int bias_stride, int dtype,
+                     void* stream) {
   if (!q || !kcache || !vcache || !out) return O355_EINVAL;
   if (hd <= 0 || hd > 256) return O355_EUNSUPPORTED;
   hipStream_t s = as_stream(stream);
-  const int rc = attn_prefill_main(q, kcache, vcache, key_bias, out, B, T, H, Hkv, hd, Lmax, past_len, bias_stride, dtype, s);
+  const int rc = attn_prefill_main(q, kcache, vcache, key_bias, out, B, T, H, Hkv, hd, Lmax, past_len, bias_stride, dtype, s, ws, ws_bytes);
   if (rc != O355_OK || !key_bias) return rc;
   if (dtype == O355_BF16)
     hipLaunchKernelGGL(attn_masked_rows_kernel<O355_BF16>, dim3(Hkv, B), dim3(256), 0, s, vcache, key_bias, out, T, H, Hkv,
@@ -1227,25 +1326,86 @@ extern "C" int olmo355_attn_prefill(const void* q, const void* kcache, const voi
                        hd, Lmax, past_len, bias_stride);
   O355_CHECK_LAUNCH();
 }
+}  // namespace
+
+extern "C" int olmo355_attn_prefill(const void* q, const void* kcache, const void* vcache, const float* key_bias,
+                                    void* out, int B, int T, int H, int Hkv, int hd, int Lmax, int past_len,
+                                    int bias_stride, int dtype, void* stream) {
+  return attn_prefill_any(q, kcache, vcache, key_bias, out, nullptr, 0, B, T, H, Hkv, hd, Lmax, past_len, bias_stride, dtype, stream);
+}
+
+// olmo355_attn_prefill with a workspace: where olmo355_attn_prefill_workspace_bytes(...) is not 0 the launch shares the
+// long query blocks between workgroups along the keys (see attn_prefill_mfma_kernel) and needs that many bytes, zeroed
+// when allocated (it starts with one int32 counter per (batch, head, query block), which every launch leaves at zero
+// again); O355_EINVAL when ws_bytes is smaller.  ws == NULL or a size of 0: the plain launch.
+extern "C" int64_t olmo355_attn_prefill_workspace_bytes(int B, int T, int H, int hd, int past_len, int dtype) {
+  if (B <= 0 || T <= 0 || H <= 0 || !prefill_split_applies(B, T, H, hd, past_len, dtype)) return 0;
+  return prefill_split_bytes(B, T, H, hd);
+}
+extern "C" int olmo355_attn_prefill_ws(const void* q, const void* kcache, const void* vcache, const float* key_bias,
+                                       void* out, void* ws, int64_t ws_bytes, int B, int T, int H, int Hkv, int hd, int Lmax,
+                                       int past_len, int bias_stride, int dtype, void* stream) {
+  return attn_prefill_any(q, kcache, vcache, key_bias, out, ws, ws_bytes, B, T, H, Hkv, hd, Lmax, past_len, bias_stride, dtype, stream);
+}
 
 namespace {
+// The key-split form pays when the plain launch leaves places on the chip empty (two workgroups per CU) while its
+// longest workgroups run: a prompt from scratch (past_len == 0) of 9 to 32 query blocks with at most 384 (batch, head,
+// block) triples.  Measured, 2048 tokens, hd 128: 16 heads (256 triples) 52.6 -> 37.7 us; 32 heads (512 triples, every
+// place taken) 61.4 -> 65.6 us: with the chip full a CU finishes a key tile of a workgroup every 1.3 us whatever the
+// split, and the hand-over is extra.
+bool prefill_split_applies(int B, int T, int H, int hd, int past_len, int dtype) {
+  const int nqb = (T + 127) / 128;
+  return dtype == O355_BF16 && (hd == 128 || hd == 64) && past_len == 0 && nqb > kPrefillChunkBlocks &&
+         nqb <= kPrefillChunkBlocks * kPrefillMaxChunks && (int64_t)B * H * nqb <= kPrefillMaxTriples;
+}
+int64_t prefill_split_bytes(int B, int T, int H, int hd) {
+  const int nqb = (T + 127) / 128, maxc = (nqb - 1) / kPrefillChunkBlocks + 1;
+  static_assert(kPrefillMaxTriples * 4 <= kPrefillTicketBytes, "one counter per triple");
+  const int64_t tickets = kPrefillTicketBytes;
+  const int64_t slot = hd == 128 ? PrefillSplit<128>::SLOT_BYTES : PrefillSplit<64>::SLOT_BYTES;
+  return tickets + (int64_t)B * H * (nqb - kPrefillChunkBlocks) * maxc * slot;
+}
+
 int attn_prefill_main(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out, int B, int T,
-                      int H, int Hkv, int hd, int Lmax, int past_len, int bias_stride, int dtype, hipStream_t s) {
+                      int H, int Hkv, int hd, int Lmax, int past_len, int bias_stride, int dtype, hipStream_t s, void* ws,
+                      int64_t ws_bytes) {
   if (B <= 0 || T <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || past_len < 0 || past_len + T > Lmax) return O355_EINVAL;
   if (key_bias && bias_stride < past_len + T) return O355_EINVAL;
   if (dtype == O355_BF16 && (hd == 128 || hd == 64) && (int64_t)Lmax * hd < (1ll << 31)) {  // 32-bit offsets within a head
-    const dim3 grid(H, (T + 127) / 128, B);  // heads fastest, then query blocks by rank (see the kernel)
+    const int nqb = (T + 127) / 128;
+    if (ws && prefill_split_applies(B, T, H, hd, past_len, dtype)) {
+      if (ws_bytes < prefill_split_bytes(B, T, H, hd)) return O355_EINVAL;
+      int n_wg = 0;
+      for (int b = 0; b < nqb; ++b) n_wg += b / kPrefillChunkBlocks + 1;
+      const int maxc = (nqb - 1) / kPrefillChunkBlocks + 1;
+      const dim3 grid(H, n_wg, B);  // heads fastest, then (block, run of keys) longest first (see the kernel)
+      if (hd == 128) {
+        constexpr int lds = PrefillLds<128>::BYTES;
+        auto kern = attn_prefill_mfma_kernel<128>;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+          return O355_ELAUNCH;
+        hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, (const uint16_t*)q, (const uint16_t*)kcache, (const uint16_t*)vcache,
+                           key_bias, (uint16_t*)out, T, H, Hkv, Lmax, past_len, bias_stride, (unsigned char*)ws, maxc);
+      } else {
+        hipLaunchKernelGGL(attn_prefill_mfma_kernel<64>, grid, dim3(256), PrefillLds<64>::BYTES, s, (const uint16_t*)q,
+                           (const uint16_t*)kcache, (const uint16_t*)vcache, key_bias, (uint16_t*)out, T, H, Hkv, Lmax,
+                           past_len, bias_stride, (unsigned char*)ws, maxc);
+      }
+      O355_CHECK_LAUNCH();
+    }
+    const dim3 grid(H, nqb, B);  // heads fastest, then query blocks by rank (see the kernel)
     if (hd == 128) {
       constexpr int lds = PrefillLds<128>::BYTES;  // more than a launch gets without asking
       auto kern = attn_prefill_mfma_kernel<128>;
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
         return O355_ELAUNCH;
       hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, (const uint16_t*)q, (const uint16_t*)kcache,
-                         (const uint16_t*)vcache, key_bias, (uint16_t*)out, T, H, Hkv, Lmax, past_len, bias_stride);
+                         (const uint16_t*)vcache, key_bias, (uint16_t*)out, T, H, Hkv, Lmax, past_len, bias_stride, nullptr, 1);
     } else {
       hipLaunchKernelGGL(attn_prefill_mfma_kernel<64>, grid, dim3(256), PrefillLds<64>::BYTES, s, (const uint16_t*)q,
                          (const uint16_t*)kcache, (const uint16_t*)vcache, key_bias, (uint16_t*)out, T, H, Hkv, Lmax,
-                         past_len, bias_stride);
+                         past_len, bias_stride, nullptr, 1);
     }
     O355_CHECK_LAUNCH();
   }

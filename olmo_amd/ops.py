@@ -779,8 +779,16 @@ def qknorm_rope_kvwrite(qkv, q_weight, k_weight, sin_tab, cos_tab, kcache, vcach
     return q
 
 
+PREFILL_SPLIT = True  # tests switch it off to compare the two forms
+_prefill_ws = {}  # (device, stream) -> zeroed workspace of the key-split prefill attention, grown on demand
+
+
 def attn_prefill(q, kcache, vcache, B: int, T: int, H: int, Hkv: int, hd: int, past_len: int,
                  key_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal attention of ``T`` new tokens per sequence over the cache rows ``0 .. past_len + T - 1``.  Where the
+    library says the key-split form pays (a launch of one or two rounds of very unequal workgroups) it gets a
+    workspace, one per device and stream, kept for the life of the process (launches on a stream are ordered and
+    each leaves its counters at zero)."""
     _dev(q, kcache, vcache, key_bias)
     Lmax = kcache.shape[2]
     if q.numel() != B * T * H * hd or kcache.dtype != q.dtype:
@@ -788,9 +796,21 @@ def attn_prefill(q, kcache, vcache, B: int, T: int, H: int, Hkv: int, hd: int, p
     if key_bias is not None and (key_bias.dtype != torch.float32 or key_bias.dim() != 2 or key_bias.shape[0] < B):
         raise ValueError("key_bias must be float32 [B, n]")
     out = torch.empty(B, T, H * hd, dtype=q.dtype, device=q.device)
+    stride = key_bias.shape[1] if key_bias is not None else 0
+    need = int(lib().olmo355_attn_prefill_workspace_bytes(B, T, H, hd, past_len, _dt(q))) if PREFILL_SPLIT else 0
+    if need and not torch.cuda.is_current_stream_capturing():
+        key = (q.device.index if q.device.index is not None else torch.cuda.current_device(), _stream())
+        ws = _prefill_ws.get(key)
+        if ws is None or ws.numel() < need:
+            ws = torch.zeros(need, dtype=torch.uint8, device=q.device)
+            _prefill_ws[key] = ws
+        check("olmo355_attn_prefill_ws",
+              lib().olmo355_attn_prefill_ws(_p(q), _p(kcache), _p(vcache), _p(key_bias), _p(out), _p(ws), ws.numel(), B, T, H, Hkv,
+                                            hd, Lmax, past_len, stride, _dt(q), _stream()))
+        return out
     check("olmo355_attn_prefill",
           lib().olmo355_attn_prefill(_p(q), _p(kcache), _p(vcache), _p(key_bias), _p(out), B, T, H, Hkv, hd, Lmax,
-                                     past_len, key_bias.shape[1] if key_bias is not None else 0, _dt(q), _stream()))
+                                     past_len, stride, _dt(q), _stream()))
     return out
 
 

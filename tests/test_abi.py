@@ -82,6 +82,13 @@ def test_sized_workspaces_are_checked_before_any_device_call():
                                                  None, keys, 0, 1e-6, None, None, 0, 2, None) == 1
         assert h.olmo355_attn_decode_relay(p, None, None, p, p, p, p, None, p, p, short // B, 1, H, Hkv, hd, Lmax, Lmax, 10, None,
                                            keys, 0, 1e-6, None, None, p, p, None, None, 16, None) == 1
+    # the key-split prefill attention: a workspace only where that form is taken; too small a one is refused
+    pw = h.olmo355_attn_prefill_workspace_bytes
+    assert pw(1, 2048, 16, 128, 0, 1) == 4096 + 16 * 8 * 2 * (4 * 2 * 8 * 64 * 16 + 4 * 2 * 64 * 8)
+    assert pw(1, 2048, 32, 128, 0, 1) == 0 and pw(1, 1024, 16, 128, 0, 1) == 0 and pw(1, 2048, 16, 128, 5, 1) == 0
+    assert pw(1, 2048, 16, 128, 0, 0) == 0 and pw(1, 2048, 16, 32, 0, 1) == 0 and pw(1, 8192, 2, 128, 0, 1) == 0
+    assert h.olmo355_attn_prefill_ws(p, p, p, None, p, p, pw(1, 2048, 16, 128, 0, 1) - 1, 1, 2048, 16, 16, 128, 4096, 0, 0, 1,
+                                     None) == 1
     need = h.olmo355_gemm_streamk_workspace_bytes()
     assert need == 4096 + 256 * 256 * 256 * 4
     for short, epoch in ((0, 1), (need - 1, 1), (need, 0)):  # epoch 0 is the value of a workspace never written: refused

@@ -691,6 +691,12 @@ def test_qknorm_rope_kvwrite(dev, dtype, qknorm, H, Hkv, hd):
     (torch.bfloat16, 1, 1000, 24, 2, 2, 64),
     (torch.float32, 2, 100, 0, 8, 8, 32),
     (torch.float32, 1, 70, 30, 2, 2, 32),
+    # prompts from scratch of more than 1024 tokens: the long query blocks are shared between workgroups along the keys
+    # (two, two with a ragged last block, three and four runs of keys per block)
+    (torch.bfloat16, 1, 2048, 0, 4, 4, 128),
+    (torch.bfloat16, 1, 1153, 0, 2, 1, 128),
+    (torch.bfloat16, 2, 3000, 0, 2, 2, 64),
+    (torch.bfloat16, 1, 4096, 0, 2, 2, 128),
 ])
 def test_attn_prefill(dev, dtype, B, T, past, H, Hkv, hd):
     say("attn_prefill", dtype, B, T, past, H, Hkv, hd)
@@ -731,6 +737,21 @@ def test_attn_prefill(dev, dtype, B, T, past, H, Hkv, hd):
     tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=0, atol=2.5e-2)
     assert torch.allclose(out2[:, valid].float(), ref2[:, valid].float(), **tol)
     assert torch.isfinite(out2.float()).all()
+    from olmo_amd import _lib
+    if _lib.lib().olmo355_attn_prefill_workspace_bytes(B, T, H, hd, past, 1 if dtype == torch.bfloat16 else 0):
+        # the key-split form ran above (twice on one workspace: its counters must have come back to zero); the plain
+        # launch forms the same products and differs only in how a row's partial sums are combined
+        qd = q.transpose(1, 2).reshape(B, T, H * hd).contiguous().to(dev)
+        again = ops.attn_prefill(qd, kc.to(dev), vc.to(dev), B, T, H, Hkv, hd, past).cpu()
+        assert torch.equal(again, out)
+        ops.PREFILL_SPLIT = False
+        try:
+            plain = ops.attn_prefill(qd, kc.to(dev), vc.to(dev), B, T, H, Hkv, hd, past).cpu()
+        finally:
+            ops.PREFILL_SPLIT = True
+        a, b = out.float(), plain.float()
+        assert ((a - b).abs() <= 2 ** -7 * torch.maximum(a.abs(), b.abs()) + 2 ** -9).all()
+        assert not torch.equal(a, b) or T <= 1024  # the two forms really are different launches
 
 
 @pytest.mark.parametrize("dtype,B,L,H,Hkv,hd", [
