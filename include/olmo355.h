@@ -215,9 +215,9 @@ int olmo355_qknorm_rope_kvwrite(const void* qkv, const void* qw, const void* kw,
 int olmo355_attn_prefill(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out,
                          int B, int T, int H, int Hkv, int hd, int Lmax, int past_len, int bias_stride, int dtype,
                          void* stream);
-/* The same with a workspace.  A launch with fewer workgroups than the chip has places -- one prompt of 1152 to 4096
- * tokens from scratch with few heads -- lasts as long as its longest query block (causal work grows with the block's
- * position); with a workspace the blocks whose keys run past 1024 are shared between workgroups along the keys, and
+/* The same with a workspace.  A launch of a single round of workgroups -- one prompt from scratch -- lasts as long as
+ * its longest query block (causal work grows with the block's position); with a workspace the blocks whose keys run
+ * past 1024 (1536 when the plain launch would fill the chip) are shared between workgroups along the keys, and
  * the one that finishes a block last combines all partial results and writes the rows (no workgroup waits for
  * another; same products, the partial sums of a row combined in the order of their keys whoever comes last).
  * olmo355_attn_prefill_workspace_bytes: the bytes that form needs for this call, 0 where the plain launch is the one

@@ -164,16 +164,16 @@ struct PrefillLds {
   static constexpr int BYTES = 4 * TILE + 2 * KT * 4;  // K x 2, V x 2, bias x 2
 };
 
-// SPLIT (past_len == 0, at most kPrefillMaxChunks x kPrefillChunkBlocks query blocks): a query block whose keys run
-// past kPrefillChunkBlocks x 128 is shared by several workgroups, one per run of that many keys.  One prompt of 2048
+// SPLIT (past_len == 0, at most kPrefillMaxChunks x chunk_blocks query blocks): a query block whose keys run
+// past chunk_blocks x 128 is shared by several workgroups, one per run of that many keys.  One prompt of 2048
 // tokens and 16 heads is 256 workgroups of 1 to 16 units of work each for the chip's 512 places: the launch lasts as
 // long as its longest workgroup while most places stand empty; cut at 8 units the same work is 384 workgroups of at
 // most half that length, all resident at once.  A workgroup that does not hold all of its block's keys
 // leaves its accumulators, reference maximum and denominator as they stand in its slot of the workspace
 // (device-scope stores) and draws a ticket; the one that draws the block's last ticket adds the others' to its own
 // registers and writes the output.  Nobody waits for anybody.
-constexpr int kPrefillChunkBlocks = 8, kPrefillMaxChunks = 4;
-constexpr int kPrefillMaxTriples = 384, kPrefillTicketBytes = 4096;  // (batch, head, query block) triples of a split launch
+constexpr int kPrefillMaxChunks = 4;
+constexpr int kPrefillMaxTriples = 1024, kPrefillTicketBytes = 4096;  // (batch, head, query block) triples of a split launch
 template <int HD>
 struct PrefillSplit {
   static constexpr int O_BYTES = 4 * 2 * (HD / 16) * 64 * 16;  // waves x query tiles x channel tiles x lanes x float4
@@ -188,8 +188,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
                                                                 const float* __restrict__ key_bias,
                                                                 uint16_t* __restrict__ out, int T, int H, int Hkv,
                                                                 int Lmax, int past_len, int bias_stride,
-                                                                unsigned char* __restrict__ ws, int max_chunks) {
+                                                                unsigned char* __restrict__ ws, int max_chunks, int chunk_blocks) {
   const bool SPLIT = ws != nullptr;  // uniform over the launch
+  const int kPrefillChunkBlocks = chunk_blocks;  // query blocks' worth of keys (x 128) per run
   constexpr int KT = 64;             // keys per tile
   constexpr int STEPS = HD / 32;     // hd steps of the first product = 1 KiB load instructions per wave, tile and operand
   constexpr int HT = HD / 16;        // hd tiles of the second product
@@ -217,9 +218,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const uint16_
   int qblock = rank < half ? nqb - 1 - rank : rank - half;
   int chunk = 0, nchunks = 1;
   if (SPLIT) {
-    // blockIdx.y counts the (block, run of keys) pairs longest first: the full runs (block b has b / 8 of them), then
-    // the blocks' last runs by length, 8 units down to 1 (block b's last run is b % 8 + 1 units long)
-    constexpr int CB = kPrefillChunkBlocks;
+    // blockIdx.y counts the (block, run of keys) pairs longest first: the full runs (block b has b / CB of them), then
+    // the blocks' last runs by length, CB units down to 1 (block b's last run is b % CB + 1 units long)
+    const int CB = kPrefillChunkBlocks;
     int r = rank;
     qblock = -1;
     for (int bb = nqb - 1; bb >= CB && qblock < 0; --bb) {
@@ -1349,22 +1350,26 @@ extern "C" int olmo355_attn_prefill_ws(const void* q, const void* kcache, const 
 }
 
 namespace {
-// The key-split form pays when the plain launch leaves places on the chip empty (two workgroups per CU) while its
-// longest workgroups run: a prompt from scratch (past_len == 0) of 9 to 32 query blocks with at most 384 (batch, head,
-// block) triples.  Measured, 2048 tokens, hd 128: 16 heads (256 triples) 52.6 -> 37.7 us; 32 heads (512 triples, every
-// place taken) 61.4 -> 65.6 us: with the chip full a CU finishes a key tile of a workgroup every 1.3 us whatever the
-// split, and the hand-over is extra.
-bool prefill_split_applies(int B, int T, int H, int hd, int past_len, int dtype) {
+// The key-split form pays when the plain launch is a single round of workgroups of very unequal length: a prompt from
+// scratch (past_len == 0) with at most 1024 (batch, head, query block) triples.  The run length: 8 query blocks' worth
+// of keys while the plain launch would leave places on the chip empty (two workgroups per CU), 12 once every place is
+// taken (then only the few longest blocks are worth a hand-over).  Measured, 2048 tokens, us per launch, plain / runs
+// of 8 / 10 / 12 / 14: 16 heads of 128 (256 triples) 52.6 / 37.7-39.5 / 40.7 / 45.4 / 49.9; 32 heads of 128 (512 triples)
+// 61.4 / 65.6 / 61.0 / 56.8 / 60.6; 32 heads of 64 41.8 / - / 34.4 / 35.7 / 37.9.
+int prefill_chunk_blocks(int B, int T, int H) {
   const int nqb = (T + 127) / 128;
-  return dtype == O355_BF16 && (hd == 128 || hd == 64) && past_len == 0 && nqb > kPrefillChunkBlocks &&
-         nqb <= kPrefillChunkBlocks * kPrefillMaxChunks && (int64_t)B * H * nqb <= kPrefillMaxTriples;
+  return (int64_t)B * H * nqb <= 384 ? 8 : 12;
+}
+bool prefill_split_applies(int B, int T, int H, int hd, int past_len, int dtype) {
+  const int nqb = (T + 127) / 128, cb = prefill_chunk_blocks(B, T, H);
+  return dtype == O355_BF16 && (hd == 128 || hd == 64) && past_len == 0 && nqb > cb && nqb <= cb * kPrefillMaxChunks &&
+         (int64_t)B * H * nqb <= kPrefillMaxTriples;
 }
 int64_t prefill_split_bytes(int B, int T, int H, int hd) {
-  const int nqb = (T + 127) / 128, maxc = (nqb - 1) / kPrefillChunkBlocks + 1;
+  const int nqb = (T + 127) / 128, cb = prefill_chunk_blocks(B, T, H), maxc = (nqb - 1) / cb + 1;
   static_assert(kPrefillMaxTriples * 4 <= kPrefillTicketBytes, "one counter per triple");
-  const int64_t tickets = kPrefillTicketBytes;
   const int64_t slot = hd == 128 ? PrefillSplit<128>::SLOT_BYTES : PrefillSplit<64>::SLOT_BYTES;
-  return tickets + (int64_t)B * H * (nqb - kPrefillChunkBlocks) * maxc * slot;
+  return kPrefillTicketBytes + (int64_t)B * H * (nqb - cb) * maxc * slot;
 }
 
 int attn_prefill_main(const void* q, const void* kcache, const void* vcache, const float* key_bias, void* out, int B, int T,
@@ -1376,9 +1381,10 @@ int attn_prefill_main(const void* q, const void* kcache, const void* vcache, con
     const int nqb = (T + 127) / 128;
     if (ws && prefill_split_applies(B, T, H, hd, past_len, dtype)) {
       if (ws_bytes < prefill_split_bytes(B, T, H, hd)) return O355_EINVAL;
+      const int cb = prefill_chunk_blocks(B, T, H);
       int n_wg = 0;
-      for (int b = 0; b < nqb; ++b) n_wg += b / kPrefillChunkBlocks + 1;
-      const int maxc = (nqb - 1) / kPrefillChunkBlocks + 1;
+      for (int b = 0; b < nqb; ++b) n_wg += b / cb + 1;
+      const int maxc = (nqb - 1) / cb + 1;
       const dim3 grid(H, n_wg, B);  // heads fastest, then (block, run of keys) longest first (see the kernel)
       if (hd == 128) {
         constexpr int lds = PrefillLds<128>::BYTES;
@@ -1386,11 +1392,11 @@ int attn_prefill_main(const void* q, const void* kcache, const void* vcache, con
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
           return O355_ELAUNCH;
         hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, (const uint16_t*)q, (const uint16_t*)kcache, (const uint16_t*)vcache,
-                           key_bias, (uint16_t*)out, T, H, Hkv, Lmax, past_len, bias_stride, (unsigned char*)ws, maxc);
+                           key_bias, (uint16_t*)out, T, H, Hkv, Lmax, past_len, bias_stride, (unsigned char*)ws, maxc, cb);
       } else {
         hipLaunchKernelGGL(attn_prefill_mfma_kernel<64>, grid, dim3(256), PrefillLds<64>::BYTES, s, (const uint16_t*)q,
                            (const uint16_t*)kcache, (const uint16_t*)vcache, key_bias, (uint16_t*)out, T, H, Hkv, Lmax,
-                           past_len, bias_stride, (unsigned char*)ws, maxc);
+                           past_len, bias_stride, (unsigned char*)ws, maxc, cb);
       }
       O355_CHECK_LAUNCH();
     }
@@ -1401,11 +1407,11 @@ int attn_prefill_main(const void* q, const void* kcache, const void* vcache, con
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
         return O355_ELAUNCH;
       hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, (const uint16_t*)q, (const uint16_t*)kcache,
-                         (const uint16_t*)vcache, key_bias, (uint16_t*)out, T, H, Hkv, Lmax, past_len, bias_stride, nullptr, 1);
+                         (const uint16_t*)vcache, key_bias, (uint16_t*)out, T, H, Hkv, Lmax, past_len, bias_stride, nullptr, 1, 8);
     } else {
       hipLaunchKernelGGL(attn_prefill_mfma_kernel<64>, grid, dim3(256), PrefillLds<64>::BYTES, s, (const uint16_t*)q,
                          (const uint16_t*)kcache, (const uint16_t*)vcache, key_bias, (uint16_t*)out, T, H, Hkv, Lmax,
-                         past_len, bias_stride, nullptr, 1);
+                         past_len, bias_stride, nullptr, 1, 8);
     }
     O355_CHECK_LAUNCH();
   }

@@ -85,7 +85,9 @@ def test_sized_workspaces_are_checked_before_any_device_call():
     # the key-split prefill attention: a workspace only where that form is taken; too small a one is refused
     pw = h.olmo355_attn_prefill_workspace_bytes
     assert pw(1, 2048, 16, 128, 0, 1) == 4096 + 16 * 8 * 2 * (4 * 2 * 8 * 64 * 16 + 4 * 2 * 64 * 8)
-    assert pw(1, 2048, 32, 128, 0, 1) == 0 and pw(1, 1024, 16, 128, 0, 1) == 0 and pw(1, 2048, 16, 128, 5, 1) == 0
+    assert pw(1, 2048, 32, 128, 0, 1) == 4096 + 32 * 4 * 2 * (4 * 2 * 8 * 64 * 16 + 4 * 2 * 64 * 8)  # every place taken: runs of 12
+    assert pw(1, 1536, 40, 128, 0, 1) == 0 and pw(1, 1024, 16, 128, 0, 1) == 0 and pw(1, 2048, 16, 128, 5, 1) == 0
+    assert pw(8, 2048, 32, 128, 0, 1) == 0  # several rounds of workgroups balance themselves
     assert pw(1, 2048, 16, 128, 0, 0) == 0 and pw(1, 2048, 16, 32, 0, 1) == 0 and pw(1, 8192, 2, 128, 0, 1) == 0
     assert h.olmo355_attn_prefill_ws(p, p, p, None, p, p, pw(1, 2048, 16, 128, 0, 1) - 1, 1, 2048, 16, 16, 128, 4096, 0, 0, 1,
                                      None) == 1
