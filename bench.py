@@ -110,6 +110,8 @@ def main() -> int:
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: one plain copy of known size, then the four "
                          "int4 linears of a layer at one row; nothing is timed or printed")
+    ap.add_argument("--probe-rows", type=int, default=1,
+                    help="rows of the activations in --traffic-probe (8: the kernel for 5 to 8 rows)")
     ap.add_argument("--gemm-probe", action="store_true",
                     help="for rocprofv3 --pmc matrix-core counters: the four int4 block linears of a layer at 2048 "
                          "rows, three times each over distinct weights; nothing is timed or printed")
@@ -139,7 +141,7 @@ def main() -> int:
     dev = torch.device("cuda:0")
     cfg = PRESETS["olmo2-7b"]
     if args.traffic_probe:
-        return traffic_probe(cfg, dev)
+        return traffic_probe(cfg, dev, rows=args.probe_rows)
     if args.gemm_probe:
         return traffic_probe(cfg, dev, rows=2048)
     if args.sweep:
