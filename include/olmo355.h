@@ -10,8 +10,9 @@
  *     kernel is launched when an argument check fails;
  *   - no process-global state: safe from any host thread that has made its device current
  *     (one stated exception: olmo355_attn_decode_static, which owns a fixed device scratch array);
- *   - `dtype` is O355_F32 or O355_BF16 (the activation dtype); fp16 appears only as the
- *     scale / dequant-table type of the int4 format.
+ *   - `dtype` is the activation dtype: O355_F32, O355_BF16 or O355_F16.  Every element-wise, attention,
+ *     sampling and beam entry point takes all three; the fused decode forms (chained norms, relay,
+ *     fused merge, key-split prefill attention) are bf16 only and say so where they are declared.
  *
  * Each declaration cites the reference interface it stands in for.  Paths are relative to
  * the reference tree; "AGQ/" = inference/compression/dependencies/AutoGPTQ/.
@@ -33,6 +34,7 @@ extern "C" {
 
 #define O355_F32 0
 #define O355_BF16 1
+#define O355_F16 2
 
 int olmo355_version(void);
 const char* olmo355_status_string(int status);
@@ -178,6 +180,9 @@ int olmo355_b16_gemv_fused(const uint16_t* x, const uint16_t* resid, const uint1
                            uint16_t* x_out, const uint16_t* wt, uint16_t* y, int M, int N, int K, int swiglu,
                            void* stream);
 int olmo355_b16_gemm(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, void* stream);
+/* fp16 activations and fp16 weights (tiled by olmo355_b16_repack, which moves 16-bit elements of
+ * either type), fp32 accumulate, fp16 out: the same nn.Linear under `model.half()`.  Any M. */
+int olmo355_f16_gemm(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K, void* stream);
 int olmo355_f32_linear(const float* x, const float* w_nk, float* y, int M, int N, int K, void* stream);
 
 /* ---- norms ------------------------------------------------------------------------------ */

@@ -46,6 +46,7 @@ EXPORTS = {
     "olmo355_b16_repack": (I, [P, P, I, I, P]),
     "olmo355_b16_gemv": (I, [P, P, P, I, I, I, P]),
     "olmo355_b16_gemm": (I, [P, P, P, I, I, I, P]),
+    "olmo355_f16_gemm": (I, [P, P, P, I, I, I, P]),
     "olmo355_f32_linear": (I, [P, P, P, I, I, I, P]),
     "olmo355_rmsnorm": (I, [P, P, P, P, I, I, F, I, P]),
     "olmo355_layernorm_np": (I, [P, P, I, I, F, I, P]),

@@ -39,6 +39,19 @@ template <> struct Vec8<O355_BF16> {
     unpack(r, f);
   }
 };
+template <> struct Vec8<O355_F16> {
+  static __device__ __forceinline__ void unpack(const u32x4 (&r)[1], float (&f)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const f16x2 h = __builtin_bit_cast(f16x2, (uint32_t)r[0][i]);
+      f[2 * i] = (float)h[0], f[2 * i + 1] = (float)h[1];
+    }
+  }
+  static __device__ __forceinline__ void ld(const void* p, int64_t elem, float (&f)[8]) {
+    u32x4 r[1] = {reinterpret_cast<const u32x4*>(p)[elem >> 3]};
+    unpack(r, f);
+  }
+};
 template <> struct Vec8<O355_F32> {
   static __device__ __forceinline__ void unpack(const u32x4 (&r)[2], float (&f)[8]) {
 #pragma unroll
@@ -541,7 +554,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const void* __restrict
   constexpr int KPI = 64 / LPK;                      // keys per wave iteration
   constexpr int ITERS = KPW / KPI;                   // iterations per wave
   constexpr int kDecodeChunk = 4 * KPW, kDecodeKeysPerWave = KPW;
-  constexpr int VW = DT == O355_BF16 ? 1 : 2;        // 16-byte vectors per 8 channels
+  constexpr int VW = DT == O355_F32 ? 2 : 1;         // 16-byte vectors per 8 channels
   __shared__ float red_o[4][HD];
   __shared__ float red_ml[4][2];
   const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z, hk = h / (H / Hkv);
@@ -1322,6 +1335,9 @@ int attn_prefill_any(const void* q, const void* kcache, const void* vcache, cons
   if (dtype == O355_BF16)
     hipLaunchKernelGGL(attn_masked_rows_kernel<O355_BF16>, dim3(Hkv, B), dim3(256), 0, s, vcache, key_bias, out, T, H, Hkv,
                        hd, Lmax, past_len, bias_stride);
+  else if (dtype == O355_F16)
+    hipLaunchKernelGGL(attn_masked_rows_kernel<O355_F16>, dim3(Hkv, B), dim3(256), 0, s, vcache, key_bias, out, T, H, Hkv,
+                       hd, Lmax, past_len, bias_stride);
   else
     hipLaunchKernelGGL(attn_masked_rows_kernel<O355_F32>, dim3(Hkv, B), dim3(256), 0, s, vcache, key_bias, out, T, H, Hkv,
                        hd, Lmax, past_len, bias_stride);
@@ -1423,6 +1439,10 @@ int attn_prefill_main(const void* q, const void* kcache, const void* vcache, con
     if (hd == 128) GENERIC(O355_F32, 128);
   } else if (dtype == O355_BF16) {
     if (hd == 32) GENERIC(O355_BF16, 32);
+  } else if (dtype == O355_F16) {
+    if (hd == 32) GENERIC(O355_F16, 32);
+    if (hd == 64) GENERIC(O355_F16, 64);
+    if (hd == 128) GENERIC(O355_F16, 128);
   }
 #undef GENERIC
   return O355_EUNSUPPORTED;
@@ -1485,6 +1505,10 @@ int attn_decode_any(const void* q, const void* kcache, const void* vcache, const
     if (hd == 128) DECODE(O355_F32, 128);
     if (hd == 64) DECODE(O355_F32, 64);
     if (hd == 32) DECODE(O355_F32, 32);
+  } else if (dtype == O355_F16) {
+    if (hd == 128) DECODE(O355_F16, 128);
+    if (hd == 64) DECODE(O355_F16, 64);
+    if (hd == 32) DECODE(O355_F16, 32);
   }
 #undef DECODE
   return O355_EUNSUPPORTED;

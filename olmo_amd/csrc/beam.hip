@@ -165,6 +165,7 @@ extern "C" int olmo355_log_softmax(const void* logits, float* out, int rows, int
   switch (dtype) {
     case O355_F32: hipLaunchKernelGGL(log_softmax_kernel<O355_F32>, dim3(rows), dim3(kThreads), 0, s, logits, out, n); break;
     case O355_BF16: hipLaunchKernelGGL(log_softmax_kernel<O355_BF16>, dim3(rows), dim3(kThreads), 0, s, logits, out, n); break;
+    case O355_F16: hipLaunchKernelGGL(log_softmax_kernel<O355_F16>, dim3(rows), dim3(kThreads), 0, s, logits, out, n); break;
     default: return O355_EUNSUPPORTED;
   }
   O355_CHECK_LAUNCH();

@@ -8,6 +8,7 @@
 
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -61,6 +62,13 @@ template <> struct Act<O355_BF16> {
   static __device__ __forceinline__ void st(void* p, int64_t i, float v) { ((uint16_t*)p)[i] = f32_to_bf16_bits(v); }
   static __device__ __forceinline__ float rnd(float v) { return round_bf16(v); }
   static __device__ __forceinline__ float lowest() { return -3.3895313892515355e38f; }
+};
+template <> struct Act<O355_F16> {
+  typedef uint16_t T;
+  static __device__ __forceinline__ float ld(const void* p, int64_t i) { return (float)((const _Float16*)p)[i]; }
+  static __device__ __forceinline__ void st(void* p, int64_t i, float v) { ((_Float16*)p)[i] = (_Float16)v; }
+  static __device__ __forceinline__ float rnd(float v) { return (float)(_Float16)v; }
+  static __device__ __forceinline__ float lowest() { return -65504.f; }
 };
 
 // Workgroup barrier that orders LDS traffic only: global loads issued before it stay in flight

@@ -27,6 +27,23 @@ template <> struct Vec<O355_BF16> {
     reinterpret_cast<u32x4*>(p)[vec_idx] = v;
   }
 };
+template <> struct Vec<O355_F16> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void ld(const void* p, int64_t vec_idx, float (&f)[8]) {
+    const u32x4 v = reinterpret_cast<const u32x4*>(p)[vec_idx];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const f16x2 h = __builtin_bit_cast(f16x2, (uint32_t)v[i]);
+      f[2 * i] = (float)h[0], f[2 * i + 1] = (float)h[1];
+    }
+  }
+  static __device__ __forceinline__ void st(void* p, int64_t vec_idx, const float (&f)[8]) {
+    u32x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = pack_f16x2(f[2 * i], f[2 * i + 1]);
+    reinterpret_cast<u32x4*>(p)[vec_idx] = v;
+  }
+};
 template <> struct Vec<O355_F32> {
   static constexpr int N = 4;
   static __device__ __forceinline__ void ld(const void* p, int64_t vec_idx, float (&f)[4]) {
@@ -444,6 +461,9 @@ __global__ void incr_kernel(int32_t* p) { *p += 1; }
   } else if ((dtype) == O355_BF16) {                        \
     constexpr int DT = O355_BF16;                           \
     __VA_ARGS__;                                            \
+  } else if ((dtype) == O355_F16) {                         \
+    constexpr int DT = O355_F16;                            \
+    __VA_ARGS__;                                            \
   } else {                                                  \
     return O355_EUNSUPPORTED;                               \
   }
@@ -452,7 +472,7 @@ extern "C" int olmo355_rmsnorm(const void* x, const void* weight, const void* re
                                float eps, int dtype, void* stream) {
   if (!x || !out || rows <= 0 || d <= 0) return O355_EINVAL;
   hipStream_t s = as_stream(stream);
-  const int vn = dtype == O355_BF16 ? 8 : 4;
+  const int vn = dtype == O355_F32 ? 4 : 8;
   const int nvec = d / vn;
   if (d % vn == 0 && nvec <= 4 * 256) {
     if (nvec <= 256) {
@@ -509,7 +529,7 @@ extern "C" int olmo355_qknorm_rope_kvwrite(const void* qkv, const void* qw, cons
 
 extern "C" int olmo355_swiglu(const void* x, void* out, int rows, int h, int dtype, void* stream) {
   if (!x || !out || rows <= 0 || h <= 0) return O355_EINVAL;
-  const int vn = dtype == O355_BF16 ? 8 : 4;
+  const int vn = dtype == O355_F32 ? 4 : 8;
   if (h % vn == 0) {
     const int64_t total = (int64_t)rows * (h / vn);
     DT_SWITCH(dtype, hipLaunchKernelGGL(swiglu_vec_kernel<DT>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,

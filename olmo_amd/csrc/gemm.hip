@@ -118,7 +118,7 @@ __device__ __forceinline__ StreamKArgsPtr streamk_args() {
 enum { GEMM_PLAIN = 0, GEMM_SPLIT = 1, GEMM_STREAMK = 2 };
 constexpr int kStreamKStatusWord = O355_STREAMK_STATUS_WORD;  // int32 index in the workspace: epoch of a launch that gave up
 
-// F16: the activations, the dequantised weights and the output are fp16 instead of bf16 (int4 weights, plain tiles only)
+// F16: the activations, the weights (dense, or int4 dequantised) and the output are fp16 instead of bf16 (plain tiles only)
 template <int WAVES_M, int WAVES_N, int WMT, int WNT, bool W4, bool SWIGLU = false, int KIND = GEMM_PLAIN, bool F16 = false>  // wave grid, 32 x 32 blocks (of four 16 x 16 MFMA tiles) per wave
 __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const uint32_t* __restrict__ wt,
                                           const uint16_t* __restrict__ st, const uint8_t* __restrict__ zt,
@@ -127,7 +127,7 @@ __device__ __forceinline__ void gemm_body(const uint16_t* __restrict__ x, const 
                                           float* __restrict__ part = nullptr, int sk_mode = 0, int sk_self = 0,
                                           int sk_first = 0, bool sk_raise = false, bool sk_defer = false) {
   constexpr bool SPLIT = KIND == GEMM_SPLIT;
-  static_assert(!F16 || (W4 && !SWIGLU && KIND == GEMM_PLAIN), "fp16 activations: the plain int4 tiles");
+  static_assert(!F16 || (!SWIGLU && KIND == GEMM_PLAIN), "fp16 activations: the plain tiles only");
   constexpr int NW = WAVES_M * WAVES_N, NT = 64 * NW;
   constexpr int BM = 32 * WMT * WAVES_M, BN = 32 * WNT * WAVES_N;
   constexpr int MT = 2 * WMT, NT16 = 2 * WNT;  // 16 x 16 MFMA tiles per wave
@@ -890,6 +890,17 @@ extern "C" int olmo355_b16_gemm(const uint16_t* x, const uint16_t* wt, uint16_t*
   if ((K & 63) || (N & 15)) return O355_EUNSUPPORTED;
   return dispatch_gemm<false>(x, reinterpret_cast<const uint32_t*>(wt), nullptr, nullptr, y, M, N, K,
                               as_stream(stream));
+}
+
+// fp16 activations, dense fp16 weights in the tiled layout of olmo355_b16_repack (a 16-bit shuffle: either type), fp16
+// out.  Any M; tiled launches only.
+extern "C" int olmo355_f16_gemm(const uint16_t* x, const uint16_t* wt, uint16_t* y, int M, int N, int K,
+                                void* stream) {
+  if (!x || !wt || !y || M <= 0 || N <= 0 || K <= 0) return O355_EINVAL;
+  if (misaligned16(y)) return O355_EINVAL;
+  if ((K & 63) || (N & 15)) return O355_EUNSUPPORTED;
+  return dispatch_gemm<false, true>(x, reinterpret_cast<const uint32_t*>(wt), nullptr, nullptr, y, M, N, K,
+                                    as_stream(stream));
 }
 
 // ---- dense bf16 weight re-tiling: [N,K] row-major -> [N/16][K/32][64 lanes][8] -----------------

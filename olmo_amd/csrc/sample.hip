@@ -320,6 +320,9 @@ extern "C" int olmo355_sample(const void* logits, int rows, int n, float tempera
   else if (dtype == O355_BF16)
     hipLaunchKernelGGL(sample_kernel<O355_BF16>, dim3(rows), dim3(kThreads), 0, as_stream(stream), logits, n, inv_temp,
                        top_k, top_p, seed, counter_dev, counter, out, logprob);
+  else if (dtype == O355_F16)
+    hipLaunchKernelGGL(sample_kernel<O355_F16>, dim3(rows), dim3(kThreads), 0, as_stream(stream), logits, n, inv_temp,
+                       top_k, top_p, seed, counter_dev, counter, out, logprob);
   else
     return O355_EUNSUPPORTED;
   O355_CHECK_LAUNCH();

@@ -247,7 +247,7 @@ class OLMoForCausalLM(*_ModelBase):
         if model is None:
             if dtype is None:  # what the directory being loaded says (``from_pretrained``), else bfloat16
                 dtype = getattr(config, "dtype", None)
-                dtype = dtype if dtype in (torch.bfloat16, torch.float32) else torch.bfloat16
+                dtype = dtype if dtype in (torch.bfloat16, torch.float16, torch.float32) else torch.bfloat16
             model = OLMo(config.to_model_config(), device=device, dtype=dtype, **model_kwargs)
             if init_params:
                 model.reset_parameters()

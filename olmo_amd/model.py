@@ -100,7 +100,7 @@ class LayerKV(tuple):
 
 
 class DenseLinear(nn.Linear):
-    """``nn.Linear`` without bias whose product runs on the HIP kernels (bf16: re-tiled copy on
+    """``nn.Linear`` without bias whose product runs on the HIP kernels (bf16, fp16: re-tiled copy on
     the matrix cores; fp32: FMA kernel).  Parameters are left uninitialised: weights come from a
     state dict or from ``OLMo.reset_parameters``."""
 
@@ -116,7 +116,7 @@ class DenseLinear(nn.Linear):
         pass
 
     def post_init(self):
-        if self.weight.dtype == torch.bfloat16:
+        if self.weight.dtype in (torch.bfloat16, torch.float16):
             self._tiled = ops.b16_repack(self.weight.data.contiguous())
         return self
 
@@ -262,8 +262,8 @@ class OLMo(nn.Module):
         (for models whose block Linears are about to be replaced by ``QuantLinear``)."""
         super().__init__()
         config.validate_for_inference()
-        if dtype not in (torch.bfloat16, torch.float32):
-            raise OLMoConfigurationError("activation dtype must be bfloat16 or float32")
+        if dtype not in (torch.bfloat16, torch.float16, torch.float32):
+            raise OLMoConfigurationError("activation dtype must be bfloat16, float16 or float32")
         self.config = config
         self.device = torch.device(device)
         self.dtype = dtype
@@ -277,7 +277,7 @@ class OLMo(nn.Module):
         ))
         if not config.weight_tying:  # olmo/model.py:1129-1137
             self.transformer.update({"ff_out": DenseLinear(config.d_model, V, device, dtype)})
-        self._tied_head: Optional[ops.B16Tiled] = None  # weight tying, bf16: the embedding re-tiled as the output matrix
+        self._tied_head: Optional[ops.B16Tiled] = None  # weight tying, 16-bit: the embedding re-tiled as the output matrix
         self._prepared = False
         self._act_order = False
         self._rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
@@ -318,7 +318,7 @@ class OLMo(nn.Module):
                     raise RuntimeError("a block Linear is still on the meta device: swap it or load weights first")
                 m.post_init()
         c = self.config
-        if c.weight_tying and self.dtype == torch.bfloat16:
+        if c.weight_tying and self.dtype != torch.float32:
             self._tied_head = ops.b16_repack(self.transformer["wte"].weight.data.contiguous())
         n_pos = max(self.max_cache_len, c.max_sequence_length)
         self._rope = ops.rope_tables(c.head_dim, float(c.rope_theta), n_pos, self.device)

@@ -14,8 +14,8 @@ import torch
 
 from ._lib import check, lib
 
-F32, BF16 = 0, 1
-_DT = {torch.float32: F32, torch.bfloat16: BF16}
+F32, BF16, F16 = 0, 1, 2
+_DT = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
 GEMV_MAX_M = 64
 
 
@@ -23,7 +23,7 @@ def _dt(t: torch.Tensor) -> int:
     try:
         return _DT[t.dtype]
     except KeyError:
-        raise TypeError(f"unsupported activation dtype {t.dtype}; float32 or bfloat16") from None
+        raise TypeError(f"unsupported activation dtype {t.dtype}; float32, bfloat16 or float16") from None
 
 
 def _dev(*ts: Optional[torch.Tensor]) -> None:
@@ -267,25 +267,41 @@ STREAMK_STATUS_WORD = 513  # O355_STREAMK_STATUS_WORD of the C header
 # ---------------------------------------------------------------------------------------------
 @dataclass
 class B16Tiled:
-    wt: torch.Tensor  # bf16 [N/16, K/32, 64, 8]
+    wt: torch.Tensor  # bf16 or fp16 [N/16, K/32, 64, 8]
     K: int
     N: int
 
 
 def b16_repack(weight_nk: torch.Tensor) -> B16Tiled:
     _dev(weight_nk)
-    if weight_nk.dtype != torch.bfloat16 or weight_nk.dim() != 2:
-        raise TypeError("expects a bfloat16 [N, K] weight")
+    if weight_nk.dtype not in (torch.bfloat16, torch.float16) or weight_nk.dim() != 2:
+        raise TypeError("expects a bfloat16 or float16 [N, K] weight")
     N, K = weight_nk.shape
     if K % 64 or N % 16:
-        raise ValueError(f"dense bf16 path needs K % 64 == 0 and N % 16 == 0 (got N={N}, K={K})")
-    wt = torch.empty(N // 16, K // 32, 64, 8, dtype=torch.bfloat16, device=weight_nk.device)
+        raise ValueError(f"dense 16-bit path needs K % 64 == 0 and N % 16 == 0 (got N={N}, K={K})")
+    wt = torch.empty(N // 16, K // 32, 64, 8, dtype=weight_nk.dtype, device=weight_nk.device)
     check("olmo355_b16_repack", lib().olmo355_b16_repack(_p(weight_nk), _p(wt), N, K, _stream()))
     return B16Tiled(wt, K, N)
 
 
+def f16_linear(x: torch.Tensor, w: B16Tiled) -> torch.Tensor:
+    """``x @ W.T`` for fp16 activations and fp16 weights (fp32 accumulate, one rounding to fp16)."""
+    _dev(x, w.wt)
+    if x.dtype != torch.float16 or w.wt.dtype != torch.float16:
+        raise TypeError("dense fp16 linear takes float16 activations and weights")
+    if x.shape[-1] != w.K:
+        raise ValueError(f"x last dim {x.shape[-1]} != K {w.K}")
+    M = x.numel() // w.K
+    y = torch.empty(*x.shape[:-1], w.N, dtype=torch.float16, device=x.device)
+    if M:
+        check("olmo355_f16_gemm", lib().olmo355_f16_gemm(_p(x), _p(w.wt), _p(y), M, w.N, w.K, _stream()))
+    return y
+
+
 def b16_linear(x: torch.Tensor, w: B16Tiled) -> torch.Tensor:
     _dev(x, w.wt)
+    if w.wt.dtype == torch.float16:
+        return f16_linear(x, w)
     if x.dtype != torch.bfloat16:
         raise TypeError("dense bf16 linear takes bfloat16 activations")
     if x.shape[-1] != w.K:

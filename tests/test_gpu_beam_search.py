@@ -28,7 +28,7 @@ def dev():
 
 
 @pytest.mark.parametrize("rows,n", [(1, 6), (3, 1000), (4, 100352), (2, 50281)])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_log_softmax(dev, rows, n, dtype):
     say("log_softmax", rows, n, dtype)
     from olmo_amd import ops
@@ -251,7 +251,7 @@ def test_gumbel_sampler_stochastic_beam_search(dev):
     assert worst < 4.5, worst
 
 
-@pytest.mark.parametrize("dtype,hd", [(torch.bfloat16, 128), (torch.float32, 32), (torch.bfloat16, 64)])
+@pytest.mark.parametrize("dtype,hd", [(torch.bfloat16, 128), (torch.float32, 32), (torch.bfloat16, 64), (torch.float16, 64)])
 def test_attn_decode_beam_equals_gathered_caches(dev, dtype, hd):
     """The row table must give what the reference's per-step cache gather gives: the plain kernel on caches
     materialised row by row from (prompt of the first beam, generated rows by table) -- bit for bit."""

@@ -296,6 +296,24 @@ def test_b16_linear(dev, M, N, K):
     assert torch.allclose(y, ref, rtol=2 ** -8, atol=2 ** -8 * ref.abs().max().item())
 
 
+@pytest.mark.parametrize("M", [1, 8, 65, 300, 1024])
+@pytest.mark.parametrize("N,K", [(256, 256), (2048, 2048), (1008, 1408)])
+def test_f16_linear(dev, M, N, K):
+    say("f16_linear", M, N, K)
+    ops = _ops()
+    gen = torch.Generator().manual_seed(M + N + K)
+    w = (torch.randn(N, K, generator=gen) * 0.02).to(torch.float16)
+    x = torch.randn(M, K, generator=gen).to(torch.float16)
+    ref = x.float() @ w.float().t()
+    t = ops.b16_repack(w.to(dev))
+    y = ops.b16_linear(x.to(dev), t)
+    assert y.dtype == torch.float16
+    # exact fp16 products, fp32 accumulation, one fp16 rounding of the result
+    assert torch.allclose(y.float().cpu(), ref, rtol=2 ** -11, atol=2 ** -11 * ref.abs().max().item())
+    with pytest.raises(TypeError):
+        ops.b16_linear(x.to(dev).bfloat16(), t)
+
+
 @pytest.mark.parametrize("width", [256, 192, 128, 128128, 128064])
 @pytest.mark.parametrize("M,N,K", [(65, 208, 128), (300, 1008, 384), (513, 400, 1408), (256, 768, 256), (1, 16, 640)])
 def test_w4_gemm_every_tile_width(dev, width, M, N, K):
@@ -572,7 +590,11 @@ def test_f32_linear(dev, M, N, K):
 # ------------------------------------------------------------------------------------------------
 # row kernels
 # ------------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+_MANT = {torch.bfloat16: 7, torch.float16: 10}  # stored mantissa bits of the 16-bit activation dtypes
+_ACT_DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+
+
+@pytest.mark.parametrize("dtype", _ACT_DTYPES)
 @pytest.mark.parametrize("rows,d", [(1, 4096), (37, 2048), (5, 5120), (3, 256)])
 def test_rmsnorm(dev, dtype, rows, d):
     ops = _ops()
@@ -588,9 +610,9 @@ def test_rmsnorm(dev, dtype, rows, d):
         assert torch.allclose(out_r, r + ref, rtol=1e-5, atol=1e-5)
     else:
         # same rounding points; the fp32 sum of squares may differ in the last bit, which can
-        # flip a bf16 rounding: allow 1 bf16 ulp on at most 0.5% of the elements
+        # flip a rounding: allow 1 ulp of the dtype on at most 0.5% of the elements
         diff = (out.float() - ref.float()).abs()
-        ulp = 2.0 ** (torch.floor(torch.log2(ref.float().abs().clamp_min(1e-30))) - 7)
+        ulp = 2.0 ** (torch.floor(torch.log2(ref.float().abs().clamp_min(1e-30))) - _MANT[dtype])
         assert (diff <= ulp).all()
         assert (diff > 0).float().mean().item() < 5e-3
         assert (out_r.float() - (r + ref).float()).abs().max().item() <= 2 * ulp.max().item()
@@ -605,7 +627,7 @@ def test_layernorm_np(dev, rows, d):
     assert torch.allclose(out, ref, rtol=1e-5, atol=2e-6)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", _ACT_DTYPES)
 def test_swiglu(dev, dtype):
     ops = _ops()
     x = (torch.randn(33, 2 * 1376, generator=torch.Generator().manual_seed(4)) * 2).to(dtype)
@@ -615,7 +637,7 @@ def test_swiglu(dev, dtype):
         assert torch.allclose(out, ref, rtol=1e-5, atol=1e-6)
     else:
         diff = (out.float() - ref.float()).abs()
-        ulp = 2.0 ** (torch.floor(torch.log2(ref.float().abs().clamp_min(1e-30))) - 7)
+        ulp = 2.0 ** (torch.floor(torch.log2(ref.float().abs().clamp_min(1e-30))) - _MANT[dtype])
         assert (diff <= ulp).all() and (diff > 0).float().mean().item() < 5e-3
 
 
@@ -631,6 +653,13 @@ def test_embedding_add_argmax(dev):
     lg[1, 77] = lg[1, 5000] = 9.0  # tie: first index wins
     assert torch.equal(ops.argmax(lg.to(dev)).cpu(), torch.argmax(lg.float(), dim=-1))
     assert int(ops.argmax(lg.to(dev))[1]) == 77
+    # the same in fp16
+    th, ah, bh, lh = tab.half(), a.half(), b.half(), lg.half()
+    assert torch.equal(ops.embedding(ids.to(dev), th.to(dev)).cpu(), th[ids])
+    assert torch.equal(ops.add(ah.to(dev), bh.to(dev)).cpu(), (ah.float() + bh.float()).half())
+    assert torch.equal(ops.argmax(lh.to(dev)).cpu(), torch.argmax(lh.float(), dim=-1))
+    xc = (torch.randn(7, 300, generator=gen) * 3).half()
+    assert torch.equal(ops.clamp_(xc.to(dev), 1.5).cpu(), xc.clamp(-1.5, 1.5))
 
 
 # ------------------------------------------------------------------------------------------------
@@ -651,7 +680,8 @@ def _rope_ref(qkv, qw, kw, B, T, H, Hkv, hd, past, theta, eps, n_pos):
 
 
 @pytest.mark.parametrize("dtype,qknorm,H,Hkv,hd", [(torch.bfloat16, True, 16, 16, 128), (torch.bfloat16, True, 8, 2, 64),
-                                                    (torch.float32, False, 8, 8, 32)])
+                                                    (torch.float32, False, 8, 8, 32), (torch.float16, True, 8, 2, 64),
+                                                    (torch.float16, False, 4, 4, 128)])
 def test_qknorm_rope_kvwrite(dev, dtype, qknorm, H, Hkv, hd):
     ops = _ops()
     B, T, past, Lmax, theta, eps = 2, 5, 3, 16, 500000.0, 1e-6
@@ -666,12 +696,13 @@ def test_qknorm_rope_kvwrite(dev, dtype, qknorm, H, Hkv, hd):
     q = ops.qknorm_rope_kvwrite(qkv.to(dev), None if qw is None else qw.to(dev), None if kw is None else kw.to(dev),
                                 sin, cos, kc, vc, B, T, H, Hkv, hd, past, eps)
     q = q.view(B, T, H, hd).transpose(1, 2).cpu()
-    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -7)
+    tol = {torch.float32: dict(rtol=1e-5, atol=1e-5), torch.bfloat16: dict(rtol=2 ** -7, atol=2 ** -7),
+           torch.float16: dict(rtol=2 ** -10, atol=2 ** -10)}[dtype]
     assert torch.allclose(q.float(), qr.float(), **tol)
     assert torch.allclose(kc[:, :, past:past + T].cpu().float(), kr.float(), **tol)
     assert torch.equal(vc[:, :, past:past + T].cpu(), vr)
     assert (kc[:, :, :past] == 0).all() and (kc[:, :, past + T:] == 0).all()
-    if dtype == torch.bfloat16:  # same rounding points: almost every element identical
+    if dtype != torch.float32:  # same rounding points: almost every element identical
         assert (q.float() != qr.float()).float().mean().item() < 1e-2
 
 
@@ -697,6 +728,11 @@ def test_qknorm_rope_kvwrite(dev, dtype, qknorm, H, Hkv, hd):
     (torch.bfloat16, 1, 1153, 0, 2, 1, 128),
     (torch.bfloat16, 2, 3000, 0, 2, 2, 64),
     (torch.bfloat16, 1, 4096, 0, 2, 2, 128),
+    # fp16 activations: every head size on the one-thread-per-row kernel
+    (torch.float16, 1, 300, 0, 4, 4, 128),
+    (torch.float16, 2, 130, 70, 4, 2, 64),
+    (torch.float16, 1, 70, 30, 2, 2, 32),
+    (torch.float16, 1, 1500, 0, 2, 2, 128),
 ])
 def test_attn_prefill(dev, dtype, B, T, past, H, Hkv, hd):
     say("attn_prefill", dtype, B, T, past, H, Hkv, hd)
@@ -716,6 +752,8 @@ def test_attn_prefill(dev, dtype, B, T, past, H, Hkv, hd):
                            Hkv, hd, past).cpu()
     if dtype == torch.float32:
         assert torch.allclose(out, ref, rtol=1e-4, atol=1e-5)
+    elif dtype == torch.float16:  # fp32 arithmetic on the widened operands, one rounding of the output
+        assert torch.allclose(out.float(), ref.float(), rtol=2 ** -10, atol=2 ** -12)
     else:
         # P is rounded to bf16 before the second product (2^-9 relative), output rounded to bf16
         assert torch.allclose(out.float(), ref.float(), rtol=0, atol=2.5e-2)
@@ -734,11 +772,12 @@ def test_attn_prefill(dev, dtype, B, T, past, H, Hkv, hd):
     out2 = ops.attn_prefill(q.transpose(1, 2).reshape(B, T, H * hd).contiguous().to(dev), kc.to(dev), vc.to(dev), B, T,
                             H, Hkv, hd, past, key_bias=bias.to(dev)).cpu()
     valid = slice(5, None) if past == 0 else slice(None)  # rows that see at least one real key
-    tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=0, atol=2.5e-2)
+    tol = {torch.float32: dict(rtol=1e-4, atol=1e-5), torch.bfloat16: dict(rtol=0, atol=2.5e-2),
+           torch.float16: dict(rtol=2 ** -10, atol=2 ** -12)}[dtype]
     assert torch.allclose(out2[:, valid].float(), ref2[:, valid].float(), **tol)
     assert torch.isfinite(out2.float()).all()
     from olmo_amd import _lib
-    if _lib.lib().olmo355_attn_prefill_workspace_bytes(B, T, H, hd, past, 1 if dtype == torch.bfloat16 else 0):
+    if _lib.lib().olmo355_attn_prefill_workspace_bytes(B, T, H, hd, past, ops._DT[dtype]):
         # the key-split form ran above (twice on one workspace: its counters must have come back to zero); the plain
         # launch forms the same products and differs only in how a row's partial sums are combined
         qd = q.transpose(1, 2).reshape(B, T, H * hd).contiguous().to(dev)
@@ -762,6 +801,9 @@ def test_attn_prefill(dev, dtype, B, T, past, H, Hkv, hd):
     (torch.bfloat16, 2, 1, 2, 2, 64),
     (torch.bfloat16, 2, 257, 2, 2, 64),
     (torch.float32, 2, 513, 8, 8, 32),
+    (torch.float16, 3, 700, 4, 2, 128),
+    (torch.float16, 2, 257, 2, 2, 64),
+    (torch.float16, 16, 1100, 8, 8, 32),
 ])
 def test_attn_decode(dev, dtype, B, L, H, Hkv, hd):
     say("attn_decode", dtype, B, L, H, Hkv, hd)
@@ -778,7 +820,8 @@ def test_attn_decode(dev, dtype, B, L, H, Hkv, hd):
     kc, vc = kc.to(dev), vc.to(dev)
     qd = q.reshape(B, 1, H * hd).contiguous().to(dev)
     ws = ops.attn_decode_workspace(B, H, hd, Lmax, dev)
-    tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -8)
+    tol = {torch.float32: dict(rtol=1e-4, atol=1e-5), torch.bfloat16: dict(rtol=2 ** -7, atol=2 ** -8),
+           torch.float16: dict(rtol=2 ** -10, atol=2 ** -12)}[dtype]
     out = ops.attn_decode(qd, kc, vc, ws, B, H, Hkv, hd, L - 1, L).cpu()
     assert torch.allclose(out.float(), ref.float(), **tol)
     # position read from device memory, launch grid sized for the whole cache
@@ -1194,6 +1237,15 @@ def test_sample_distribution_small_vocab(dev, temperature, top_k, top_p):
         cd = torch.tensor([8], dtype=torch.int32, device=dev)
         tok3, _ = ops.sample(logits, temperature, top_k, top_p, seed=123, counter_dev=cd)
         assert not torch.equal(tok3.cpu(), tok)
+
+
+def test_sample_fp16_rows_equal_the_same_values_in_fp32(dev):
+    """The sampler widens a row to fp32 first: fp16 logits give the draws of the same values stored as fp32."""
+    ops = _ops()
+    logits = (torch.randn(64, 5000, generator=torch.Generator().manual_seed(2)) * 3).half()
+    th, lh = ops.sample(logits.to(dev), 0.9, 40, 0.95, seed=11, counter=2)
+    tf, lf = ops.sample(logits.float().to(dev), 0.9, 40, 0.95, seed=11, counter=2)
+    assert torch.equal(th, tf) and torch.equal(lh, lf) and len(set(th.tolist())) > 1
 
 
 @pytest.mark.parametrize("scale,top_k,top_p", [(3.0, 50, 0.9), (3.0, 0, 0.95), (0.3, 40, 1.0), (0.3, 0, 0.5), (6.0, 20000, 0.999)])
