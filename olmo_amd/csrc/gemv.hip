@@ -891,6 +891,232 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_small_kernel(GemvArgs args
   w4_gemv_small_body<GPA, NT, WAVES, PRO, EPI, F16>(args, wt, st, zt);
 }
 
+// ---- int4, one row: the batch-1 decode step ----------------------------------------------------------------
+// Time stamps inside w4_gemv_small_kernel at one row (the four linears of a 7B layer) showed a kernel bound by the
+// number of instructions its waves issue, not by memory: six waves per SIMD of ~900 instructions each, the weights of
+// a wave (4 KiB) already there when its activations are, a median wave 2.4 us into an 8 us launch before its own
+// requests are out.  This kernel is the same product with the row count, the tile count per workgroup and the length
+// of a wave's run of K fixed at compile time, so that what is left is close to what the format needs (per 16-byte
+// piece of weights: four fragment reads, 28 unpack instructions, four matrix instructions):
+//   * sizes come precomputed from the host (32-bit buffer ranges, group counts): no 64-bit clamps on the device;
+//   * a wave's run of K is QUADS pieces of 1 KiB = QUADS x 4 groups; the row's pieces travel through registers in
+//     either mode (copied, or normalised with the producer's sums of squares: ChainNorm's arithmetic), so the
+//     compiler places every wait, and the per-group sums of the activations for the zero-point term are four
+//     two-element dot products and a 16-lane sum on the piece a lane already holds (row i of 16 lanes = group i of the
+//     quad = the accumulator rows of slot i);
+//   * fragment reads address LDS with one base per slot and immediate offsets; every weight request of the wave is
+//     issued before anything is waited for.
+// Same accumulation order as the kernel above (groups in order inside a quad, quads in order, slots by the two
+// half-wave exchanges, waves in order), same rounding points.
+struct OneArgs {
+  const uint16_t* x;       // [K] activations; with the prologue: the row to be normalised
+  const uint16_t* resid;   // [K] residual stream (prologue)
+  const uint16_t* norm_w;  // [K] RMSNorm weight (prologue)
+  uint16_t* x_out;         // [K] resid + norm(x), written by workgroup 0 (prologue)
+  const float* ssq_in;     // [K/16] per-tile sums of squares of x (prologue)
+  const u32x4* wt;
+  const uint16_t* st;
+  const uint8_t* zt;
+  uint16_t* y;             // [N], or [N/2] with the SwiGLU epilogue
+  float* ssq_out;          // [N/16] or null
+  float eps, k_float;
+  int K, G, half_tiles;    // half_tiles: N/32 (SwiGLU: distance between an up tile and its gate tile)
+  uint32_t wt_bytes, st_bytes, zt_bytes;
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc32(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+// PRO: 0 plain; 1, 2: chained norm prologue with one or two 16-byte requests per lane for the sums of squares
+// (K <= 4096, K <= 8192).  NG: groups of the wave with the longest run of K (every wave has NG or NG - 1).  NT column
+// tiles per workgroup: consecutive ones, or with EPI 1 (SwiGLU) NT/2 consecutive up tiles and their gate tiles.  More
+// tiles per workgroup = fewer workgroups that each read the whole row (and, with the prologue, the residual and the
+// norm weight) out of L2: at N = 12288 those reads are as many bytes as the weights.
+// Every wave issues the same requests in the same order (the compiler counts them to place its waits, and requests
+// inside branches make it wait for everything): the one slot a shorter wave does not have is asked for past the end of
+// the buffer, which answers with zeros and moves nothing.
+template <int WAVES, int PRO, int EPI, int NG, int NT>
+__global__ __launch_bounds__(WAVES * 64) void w4_gemv_one_kernel(OneArgs a) {
+  static_assert(EPI == 0 || (NT & 1) == 0, "SwiGLU: tiles in (up, gate) pairs");
+  constexpr int QUADS = (NG + 3) / 4;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int K2 = a.K * 2;  // LDS: the row, a row of zeros, [WAVES][NT][16] partial results
+  float* red = reinterpret_cast<float*>(smem + 2 * K2);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 15, kq = lane >> 4;
+  const int G = a.G;
+  const int g_begin = (G * wave) / WAVES, g_end = (G * (wave + 1)) / WAVES;
+  const bool full = g_end - g_begin == NG;  // else NG - 1 groups (the host checks)
+  const int run = (g_end - g_begin) * 256;  // bytes of the wave's run of the row
+  const int lo = g_begin * 256;             // where it starts
+  int tg[NT];  // first group of tile nt in the tiled weights; EPI: nt = 2 pair + (0 up, 1 gate)
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+    tg[nt] = (EPI ? (int)blockIdx.x * (NT / 2) + (nt >> 1) + (nt & 1) * a.half_tiles : (int)blockIdx.x * NT + nt) * G;
+  const int wvoff = lane * 16;
+
+  // ---- 1. the row's pieces (from L2: asked for first), then every weight request of the wave ------------
+  // (a lane past the wave's run reads the neighbour's bytes, or zeros past the row, and is dropped below)
+  u32x4 av[QUADS], rv[QUADS], nv[QUADS];
+  f32x4 pv[PRO == 2 ? 2 : 1];
+  {
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc32(a.x, (uint32_t)K2);
+    if constexpr (PRO != 0) {
+      const __amdgpu_buffer_rsrc_t rp = make_rsrc32(a.ssq_in, (uint32_t)(a.K >> 2));  // K/16 floats; zeros past the end
+      pv[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rp, wvoff, 0, 0));
+      if constexpr (PRO == 2) pv[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rp, wvoff, 1024, 0));
+    }
+#pragma unroll
+    for (int q = 0; q < QUADS; ++q)
+      av[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, wvoff, lo + q * 1024, 0));
+    if constexpr (PRO != 0) {
+      const __amdgpu_buffer_rsrc_t rr = make_rsrc32(a.resid, (uint32_t)K2), rn = make_rsrc32(a.norm_w, (uint32_t)K2);
+#pragma unroll
+      for (int q = 0; q < QUADS; ++q) {
+        rv[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, wvoff, lo + q * 1024, 0));
+        nv[q] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rn, wvoff, lo + q * 1024, 0));
+      }
+    }
+  }
+  u32x4 w[NG][NT];
+  uint16_t s16[QUADS][NT];
+  uint8_t z8[QUADS][NT];
+  {
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc32(a.wt, a.wt_bytes), rs = make_rsrc32(a.st, a.st_bytes),
+                                 rz = make_rsrc32(a.zt, a.zt_bytes);
+    const int svoff = (kq * 16 + col) * 2, zvoff = kq * 8 + (col >> 1);  // the lanes of slot kq: scale and zero of group kq of the quad
+    const int last_voff = full ? wvoff : (int)0x80000000u;             // past every buffer: zeros, no traffic
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        w[g][nt] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, g == NG - 1 ? last_voff : wvoff, (tg[nt] + g_begin + g) * 1024, 2));
+    // (groups past the wave's run: another group's finite numbers or the range check's zeros, times zero)
+#pragma unroll
+    for (int q = 0; q < QUADS; ++q)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        s16[q][nt] = __builtin_amdgcn_raw_buffer_load_b16(rs, svoff, (tg[nt] + g_begin + 4 * q) * 32, 0);
+        z8[q][nt] = __builtin_amdgcn_raw_buffer_load_b8(rz, zvoff, (tg[nt] + g_begin + 4 * q) * 8, 0);
+      }
+  }
+  // the wave's run of the zero row
+#pragma unroll
+  for (int q = 0; q < QUADS; ++q)
+    if (q * 1024 + wvoff < run) *reinterpret_cast<u32x4*>(smem + K2 + lo + q * 1024 + wvoff) = u32x4{0u, 0u, 0u, 0u};
+
+  // ---- 2. the row: normalised (ChainNorm's arithmetic and order of additions) or as it is, into LDS ---------
+  float rstd = 0.f;
+  if constexpr (PRO != 0) {
+    float ss = (pv[0][0] + pv[0][1]) + (pv[0][2] + pv[0][3]);
+    if constexpr (PRO == 2) ss += (pv[1][0] + pv[1][1]) + (pv[1][2] + pv[1][3]);
+    ss = wave_sum_dpp(ss);
+    rstd = 1.f / sqrtf(ss / a.k_float + a.eps);
+  }
+  typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
+  const bf16x2v one2 = {(__bf16)1.f, (__bf16)1.f};
+  float xsum[QUADS];  // of this lane's group (slot kq) of quad q
+#pragma unroll
+  for (int q = 0; q < QUADS; ++q) {
+    u32x4 o = av[q];
+    if constexpr (PRO != 0) {
+      float f[8], r[8], wn[8];
+      unpack8(av[q], f);
+      unpack8(rv[q], r);
+      unpack8(nv[q], wn);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float y0 = round_bf16(wn[2 * e] * round_bf16(f[2 * e] * rstd));
+        const float y1 = round_bf16(wn[2 * e + 1] * round_bf16(f[2 * e + 1] * rstd));
+        o[e] = pack_bf16x2(r[2 * e] + y0, r[2 * e + 1] + y1);
+      }
+    }
+    const bool in = q * 1024 + wvoff < run;  // whole rows of 16 lanes
+    if (in) {
+      *reinterpret_cast<u32x4*>(smem + lo + q * 1024 + wvoff) = o;
+      if constexpr (PRO != 0) {
+        if (blockIdx.x == 0) *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(a.x_out) + lo + q * 1024 + wvoff) = o;
+      }
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2v, (uint32_t)o[e]), one2, sum, false);
+    sum = row16_sum(sum);
+    xsum[q] = in ? sum : 0.f;
+  }
+
+  // ---- 3. products.  Operand row `col` of slot u is the row itself for col == 4 u and zeros otherwise; a wave reads
+  // only what it wrote ----------------------------------------------------------------------------------------
+  const unsigned char* xb[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) xb[u] = smem + (col == 4 * u ? 0 : K2) + lo + 16 * kq;
+  const UnpackConsts uc;
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  float acc[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) acc[nt] = 0.f;
+#pragma unroll
+  for (int q = 0; q < QUADS; ++q) {
+    f32x4 t[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) t[nt] = zero4;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int g = 4 * q + u;
+      if (g < NG && (g < NG - 1 || full)) {  // compile-time but for the last slot (uniform)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const bf16x8 af = *reinterpret_cast<const bf16x8*>(xb[u] + g * 256 + 64 * j);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+            t[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, unpack_w4_bias128(w[g < NG ? g : 0][nt][j], uc), t[nt], 0, 0, 0);
+        }
+      }
+    }
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      const float sc = (float)__builtin_bit_cast(_Float16, s16[q][nt]);
+      const float nzc = -(float)(129 + (int)(((uint32_t)z8[q][nt] >> (4 * (col & 1))) & 15u));  // -(128 + (stored + 1))
+      acc[nt] = __builtin_fmaf(sc, __builtin_fmaf(nzc, xsum[q], t[nt][0]), acc[nt]);
+    }
+  }
+
+  // ---- 4. the four slots of a wave, then the waves through LDS, in fixed order ---------------------------------
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    float v = combine_xor32(combine_xor16(acc[nt], AddOp{}), AddOp{});
+    if (kq == 0) red[(wave * NT + nt) * 16 + col] = v;
+  }
+  __syncthreads();
+  auto total_of = [&](int nt, int c) {
+    float v = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv) v += red[(wv * NT + nt) * 16 + c];
+    return v;
+  };
+  if constexpr (EPI == 0) {
+    if (tid < NT * 16) {  // whole rows of 16 lanes: one tile each
+      const int c = tid & 15, tile = (int)blockIdx.x * NT + (tid >> 4);
+      const float v = round_bf16(total_of(tid >> 4, c));
+      a.y[tile * 16 + c] = f32_to_bf16_bits(v);
+      if (a.ssq_out) {
+        const float sq = row16_sum(v * v);
+        if (c == 0) a.ssq_out[tile] = sq;
+      }
+    }
+  } else {
+    if (tid < (NT / 2) * 16) {
+      const int c = tid & 15, p = tid >> 4;
+      const float up = round_bf16(total_of(2 * p, c));  // the Linear's bf16 output
+      const float gate = round_bf16(total_of(2 * p + 1, c));
+      const float sg = round_bf16(gate / (1.f + expf(-gate)));
+      a.y[((int)blockIdx.x * (NT / 2) + p) * 16 + c] = f32_to_bf16_bits(sg * up);
+    }
+  }
+}
+
 // ---- int4, 5 .. 8 rows: the activations as operand fragments, never whole in LDS ------------------------------
 // With eight rows the two groups of 128 that share a matrix instruction fill its 16 operand rows exactly
 // (rows 0-7: group g, rows 8-15: group g + 1), so a wave keeps the fragments of its own run of K in registers: no
@@ -1452,8 +1678,72 @@ int w4_r8_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, co
   return O355_EUNSUPPORTED;
 }
 
+// CUs of the device first used (a grid only has to be about as large as the machine); 0 if the query fails
+int cu_count() {
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0)
+      n_cu = cus;
+  }
+  return n_cu;
+}
+
+// One row through w4_gemv_one_kernel; O355_EUNSUPPORTED for what it does not cover (the caller goes on to the
+// general kernels).  `pro`: chained norm prologue (ssq_in given).
+int w4_one_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, bool pro, bool epi,
+                    void* stream) {
+  const int G = a.K >> 7, ntiles = a.N >> 4;
+  if (a.M != 1 || (a.K & 127) || a.K < 512 || (a.N & 15) || (epi && (a.N & 31)) || (pro && !a.ssq_in) || (epi && a.ssq_out))
+    return O355_EUNSUPPORTED;
+  if ((int64_t)ntiles * G * 1024 >= (1ll << 31)) return O355_EUNSUPPORTED;  // 32-bit offsets into the weights
+  const int waves = (epi ? ntiles >> 1 : ntiles) <= 512 && G >= 16 ? 16 : 8;  // as measured for the kernel above: narrow outputs take 16
+  if (G < waves) return O355_EUNSUPPORTED;
+  const int ngv = (G + waves - 1) / waves;  // groups of the longest run; the others have one less or as many
+  const int prov = !pro ? 0 : (a.K <= 4096 ? 1 : (a.K <= 8192 ? 2 : -1));
+  if (ngv > 8 || prov < 0) return O355_EUNSUPPORTED;
+  // tiles (pairs) per workgroup: the count that leaves the busiest CU the fewest tiles when the workgroups are dealt
+  // out evenly, the larger on ties (7B att_proj: 768 tiles = 256 workgroups of three)
+  const int units = epi ? ntiles >> 1 : ntiles, n_cu = std::max(cu_count(), 1);
+  int per = 1;
+  if (!epi && waves == 8 && ngv <= 4 && units % 3 == 0 && ((units / 3 + n_cu - 1) / n_cu) * 3 <= (units + n_cu - 1) / n_cu) per = 3;
+  const int nt = epi ? 2 * per : per;
+  const size_t lds = (size_t)a.K * 4 + (size_t)waves * nt * 64;
+  if (lds > 160 * 1024) return O355_EUNSUPPORTED;
+  OneArgs o{a.x, a.resid, a.norm_w, a.x_out, a.ssq_in, (const u32x4*)wt, st, zt, a.y, a.ssq_out, a.eps, (float)a.K, a.K, G,
+            ntiles >> 1, (uint32_t)((int64_t)ntiles * G * 1024), (uint32_t)((int64_t)ntiles * G * 32), (uint32_t)((int64_t)ntiles * G * 8)};
+  const unsigned blocks = (unsigned)(units / per);
+  hipStream_t s = as_stream(stream);
+#define ONE_CASE(Wv, Pv, Ev, Gv, Nv)                                                                                   \
+  if (waves == Wv && prov == Pv && (int)epi == Ev && ngv == Gv && nt == Nv) {                                          \
+    auto kern = w4_gemv_one_kernel<Wv, Pv, Ev, Gv, Nv>;                                                                \
+    if (lds > 48 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                               (int)lds) != hipSuccess)                                                \
+      return O355_ELAUNCH;                                                                                             \
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(Wv * 64), lds, s, o);                                                  \
+    O355_CHECK_LAUNCH();                                                                                               \
+  }
+  // per (waves, groups): plain and SwiGLU, each without and with the prologue that the K of that split can have
+  // (K <= 4096: one request for the sums of squares, K <= 8192: two); three tiles per workgroup for 8 waves of <= 4 groups
+#define ONE_PAIR(Wv, Pv, Gv) ONE_CASE(Wv, Pv, 0, Gv, 1) ONE_CASE(Wv, Pv, 1, Gv, 2)
+#define ONE_W8_LOW(Gv) ONE_PAIR(8, 0, Gv) ONE_PAIR(8, 1, Gv) ONE_CASE(8, 0, 0, Gv, 3) ONE_CASE(8, 1, 0, Gv, 3)
+#define ONE_W8_HIGH(Gv) ONE_PAIR(8, 0, Gv) ONE_PAIR(8, 2, Gv)
+  ONE_W8_LOW(1) ONE_W8_LOW(2) ONE_W8_LOW(3) ONE_W8_LOW(4) ONE_W8_HIGH(5) ONE_W8_HIGH(6) ONE_W8_HIGH(7) ONE_W8_HIGH(8)
+  ONE_PAIR(16, 0, 1) ONE_PAIR(16, 1, 1) ONE_PAIR(16, 0, 2) ONE_PAIR(16, 1, 2) ONE_PAIR(16, 0, 3) ONE_PAIR(16, 2, 3)
+  ONE_PAIR(16, 0, 4) ONE_PAIR(16, 2, 4) ONE_PAIR(16, 0, 5) ONE_PAIR(16, 0, 6) ONE_PAIR(16, 0, 7) ONE_PAIR(16, 0, 8)
+#undef ONE_W8_HIGH
+#undef ONE_W8_LOW
+#undef ONE_PAIR
+#undef ONE_CASE
+  return O355_EUNSUPPORTED;
+}
+
 int w4_gemv_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, bool pro, bool epi,
                      void* stream, int form = kFormChoose) {
+  if (a.M == 1 && form == kFormChoose && (!pro || a.ssq_in)) {  // one row: the kernel written for it
+    const int st1 = w4_one_dispatch(a, wt, st, zt, pro, epi, stream);
+    if (st1 != O355_EUNSUPPORTED) return st1;
+  }
   GemvPlan p = plan_gemv(a.M, a.N, a.K, true, pro, epi);
   const u32x4* w = (const u32x4*)wt;
   const int sgpa = a.M <= 4 ? 4 : (a.M <= 8 ? 2 : 1);
