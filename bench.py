@@ -26,9 +26,9 @@ W4_BYTES_PER_WEIGHT = 0.5 + 2.0 / 128 + 0.5 / 128  # nibble + fp16 scale and 4-b
 # HBM bytes per launch of the int4 small-M linear, averaged over the four 7B block shapes, from two
 # rocprofv3 --pmc runs of `bench.py --traffic-probe` (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each
 # scaled by what the same counter reads for a 256 MiB device copy (FETCH_SIZE reads half the bytes: factor
-# 2.0; WRITE_SIZE factor 1.0).  Per shape, read: 26.29 / 8.92 / 46.99 / 23.74 MB against 26.15 / 8.72 /
+# 2.0; WRITE_SIZE factor 1.0).  Per shape, read: 26.29 / 8.89 / 46.97 / 23.73 MB against 26.15 / 8.72 /
 # 46.85 / 23.43 MB of packed weights, scales and zeros; written: the output rows.
-GEMV_TRAFFIC_BYTES_7B = 26.51e6
+GEMV_TRAFFIC_BYTES_7B = 26.49e6
 
 
 def log(*a):
@@ -250,11 +250,11 @@ def main() -> int:
     avg_s = timed_graph(one_step_of_linears, reps) / n_launch
     bytes_per_launch = sum(n * k * W4_BYTES_PER_WEIGHT + 2 * k + 2 * n for n, k in shapes) * cfg.n_layers / n_launch
     achieved = bytes_per_launch / avg_s / 1e9
-    roofline = {"bound": "hbm", "kernel": "w4_gemv_small_kernel (M=1): the decode step's own 4 block-Linear launches x 32 layers "
+    roofline = {"bound": "hbm", "kernel": "w4_gemv_one_kernel (M=1): the decode step's own 4 block-Linear launches x 32 layers "
                                           "(chained-norm prologues, SwiGLU epilogue, per-tile sums of squares)",
                 "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                 "traffic": GEMV_TRAFFIC_BYTES_7B,
-                "traffic_source": "profiles/w4_gemv_small_kernel_7b_m1_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE "
+                "traffic_source": "profiles/w4_gemv_one_kernel_7b_m1_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE "
                                   "of `bench.py --traffic-probe`, scaled by a 256 MiB copy)",
                 "avg_launch_us": avg_s * 1e6, "bytes_per_launch": bytes_per_launch}
     log(f"[bench] int4 decode linears (the step's own launches): {avg_s * 1e6:.2f} us/launch avg, {achieved:.0f} GB/s = "
