@@ -983,25 +983,24 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_one_kernel(OneArgs a) {
   u32x4 w[NG][NT];
   uint16_t s16[QUADS][NT];
   uint8_t z8[QUADS][NT];
-  {
-    const __amdgpu_buffer_rsrc_t rw = make_rsrc32(a.wt, a.wt_bytes), rs = make_rsrc32(a.st, a.st_bytes),
-                                 rz = make_rsrc32(a.zt, a.zt_bytes);
-    const int svoff = (kq * 16 + col) * 2, zvoff = kq * 8 + (col >> 1);  // the lanes of slot kq: scale and zero of group kq of the quad
-    const int last_voff = full ? wvoff : (int)0x80000000u;             // past every buffer: zeros, no traffic
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc32(a.wt, a.wt_bytes), rs = make_rsrc32(a.st, a.st_bytes), rz = make_rsrc32(a.zt, a.zt_bytes);
+  const int svoff = (kq * 16 + col) * 2, zvoff = kq * 8 + (col >> 1);  // the lanes of slot kq: scale and zero of group kq of the quad
+  const int last_voff = full ? wvoff : (int)0x80000000u;             // past every buffer: zeros, no traffic
+  auto request = [&](int nt) {
 #pragma unroll
     for (int g = 0; g < NG; ++g)
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-        w[g][nt] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, g == NG - 1 ? last_voff : wvoff, (tg[nt] + g_begin + g) * 1024, 2));
+      w[g][nt] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, g == NG - 1 ? last_voff : wvoff, (tg[nt] + g_begin + g) * 1024, 2));
     // (groups past the wave's run: another group's finite numbers or the range check's zeros, times zero)
 #pragma unroll
-    for (int q = 0; q < QUADS; ++q)
+    for (int q = 0; q < QUADS; ++q) {
+      s16[q][nt] = __builtin_amdgcn_raw_buffer_load_b16(rs, svoff, (tg[nt] + g_begin + 4 * q) * 32, 0);
+      z8[q][nt] = __builtin_amdgcn_raw_buffer_load_b8(rz, zvoff, (tg[nt] + g_begin + 4 * q) * 8, 0);
+    }
+  };
+  // (all of them ahead of the prologue: holding some back until the row is in LDS, which helps at eight rows, measured
+  // level or slower here)
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
-        s16[q][nt] = __builtin_amdgcn_raw_buffer_load_b16(rs, svoff, (tg[nt] + g_begin + 4 * q) * 32, 0);
-        z8[q][nt] = __builtin_amdgcn_raw_buffer_load_b8(rz, zvoff, (tg[nt] + g_begin + 4 * q) * 8, 0);
-      }
-  }
+  for (int nt = 0; nt < NT; ++nt) request(nt);
   // the wave's run of the zero row
 #pragma unroll
   for (int q = 0; q < QUADS; ++q)
@@ -1466,6 +1465,221 @@ __global__ __launch_bounds__(WAVES * 64) void b16_gemv_kernel(GemvArgs args, con
   gemv_epilogue<MT, NT, WAVES, EPI>(acc, red, args, tile, ntiles);
 }
 
+// ---- int4, up to 8 rows, every request of a wave issued at once ------------------------------------------------------
+// w4_gemv_r8_kernel's arithmetic (operand fragments of a wave's run of K in registers, two groups per matrix
+// instruction, the same order of additions) in the shape that made the one-row kernel faster: the units of a workgroup
+// (tiles, or up/gate pairs) are fixed at compile time and all asked for before anything is waited for, and every wave
+// issues the same requests in the same order -- what a wave does not have (a group or a pair past its run, a unit past
+// the last) is asked for past the end of the buffer -- so the compiler's own waits let the products of the first
+// pieces start while the rest travels, where the requests inside branches of the kernel above made every wait a wait
+// for everything.  One barrier for the reduction over the waves (one more with the prologue, for the rows' norms).
+// PRO: 0, or the chained norm prologue with 1 or 2 requests per lane for a row's sums of squares (K <= 4096 / 8192).
+// NP: pairs of groups of the wave with the longest run.  PER units per workgroup: b, b + gridDim.x, ...
+template <int WAVES, int PRO, int EPI, int NP, int PER>
+__global__ __launch_bounds__(WAVES * 64) void w4_gemv_rows_kernel(GemvArgs args, const u32x4* __restrict__ wt,
+                                                                  const uint16_t* __restrict__ st,
+                                                                  const uint8_t* __restrict__ zt, int units) {
+  constexpr int NT = EPI ? 2 * PER : PER;  // tiles; EPI: nt = 2 unit + (0 up, 1 gate)
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* red = reinterpret_cast<float*>(smem);  // [WAVES][NT][8 rows][16 columns]
+  float* rstd_l = red + WAVES * NT * 128;       // [8]
+  const int M = args.M, K = args.K;
+  const int G = K >> 7, ntiles = args.N >> 4;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  unsigned char* xs = smem + (WAVES * NT * 128 + 8) * 4 + wave * kR8WaveBytes;  // this wave's own 16 blocks
+  const int col = lane & 15, kq = lane >> 4;
+  const int ul = kq >> 1;  // the group of a pair whose results this lane keeps
+  const int g_begin = (G * wave) / WAVES, g_end = (G * (wave + 1)) / WAVES;
+  constexpr int kNowhere = 0x40000000;  // past every buffer here: such a request returns zeros and moves nothing
+  const int wvoff = lane * 16;
+  const int half = lane >> 5, c32 = lane & 31, cu = c32 >> 4;  // request i of a pair: rows 2 i + half, group cu of the pair
+
+  // ---- 1. the rows (from L2: first), then every weight request ------------------------------------------------------
+  u32x4 xa[NP][4];  // first the rows as asked for (PRO: of the tensor to be normalised), then the operand fragments
+  u32x4 xr[PRO ? NP : 1][4], xw[PRO ? NP : 1];
+  f32x4 pv[PRO == 2 ? 2 : 1];
+  {
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc32(args.x, (uint32_t)(M * K * 2));
+    if constexpr (PRO != 0) {  // the sum of squares of row `wave` (waves past M: of the last row, unused)
+      const int n_ssq = K >> 4;
+      const __amdgpu_buffer_rsrc_t rp = make_rsrc32(args.ssq_in + min(wave, M - 1) * n_ssq, (uint32_t)(n_ssq * 4));
+      pv[0] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rp, wvoff, 0, 0));
+      if constexpr (PRO == 2) pv[1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rp, wvoff, 1024, 0));
+    }
+    // rows past M lie past the buffer and read as zeros; so must the second group of a pair that reaches past the run
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int g = g_begin + 2 * p;
+      const int xo = (g + cu < g_end) ? half * K * 2 + 256 * g + 16 * c32 : kNowhere;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        xa[p][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rx, xo + 2 * i * K * 2, 0, 0));
+    }
+    if constexpr (PRO != 0) {
+      const __amdgpu_buffer_rsrc_t rr = make_rsrc32(args.resid, (uint32_t)(M * K * 2)), rn = make_rsrc32(args.norm_w, (uint32_t)(K * 2));
+#pragma unroll
+      for (int p = 0; p < NP; ++p) {
+        const int g = g_begin + 2 * p;
+        const bool in = g + cu < g_end;
+        const int xo = in ? half * K * 2 + 256 * g + 16 * c32 : kNowhere;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          xr[p][i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rr, xo + 2 * i * K * 2, 0, 0));
+        xw[p] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rn, in ? 256 * g + 16 * c32 : kNowhere, 0, 0));
+      }
+    }
+  }
+  u32x4 w[NT][NP][2];
+  uint16_t s16[NT][NP];
+  uint8_t z8[NT][NP];
+  const uint32_t n_groups = (uint32_t)ntiles * (uint32_t)G;
+  const __amdgpu_buffer_rsrc_t rw = make_rsrc32(wt, n_groups * 1024u), rs = make_rsrc32(st, n_groups * 32u), rz = make_rsrc32(zt, n_groups * 8u);
+  auto request = [&](int nt) {
+    const int un = (int)blockIdx.x + (EPI ? nt >> 1 : nt) * (int)gridDim.x;
+    const bool have = un < units;  // uniform
+    const int tg = (EPI ? un + (nt & 1) * (ntiles >> 1) : un) * G;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int g = g_begin + 2 * p;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)  // a group past the run: nothing is moved, and its rows of x are zero
+        w[nt][p][u] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, have && g + u < g_end ? wvoff : kNowhere, (tg + g + u) * 1024, 2));
+      // the lanes that keep group g + ul hold its scale and zero
+      const bool real = have && g + ul < g_end;
+      s16[nt][p] = __builtin_amdgcn_raw_buffer_load_b16(rs, real ? (ul * 16 + col) * 2 : kNowhere, (tg + g) * 32, 0);
+      z8[nt][p] = __builtin_amdgcn_raw_buffer_load_b8(rz, real ? ul * 8 + (col >> 1) : kNowhere, (tg + g) * 8, 0);
+    }
+  };
+  // With the prologue only the first unit's weights are asked for ahead of it and the others after it (measured at
+  // eight rows, att_proj / ff_proj of the 7B model: 10.7 / 15.2 us; two units ahead 12.0 / 16.2, all three 12.4 /
+  // 17.6; the others asked for right after the norms' barrier, before the rows are normalised, 11.5 / 16.1): the
+  // prologue is what such a launch waits for, and a CU's whole share of the weights in flight holds it back.
+  constexpr int AHEAD = PRO != 0 ? (EPI ? 2 : 1) : NT;
+#pragma unroll
+  for (int nt = 0; nt < AHEAD; ++nt) request(nt);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- 2. the rows: normalised in place (ChainNorm's arithmetic), then turned into operand fragments -------------------
+  if constexpr (PRO != 0) {
+    float ss = (pv[0][0] + pv[0][1]) + (pv[0][2] + pv[0][3]);
+    if constexpr (PRO == 2) ss += (pv[1][0] + pv[1][1]) + (pv[1][2] + pv[1][3]);
+    ss = wave_sum_dpp(ss);
+    if (lane == 0 && wave < 8) rstd_l[wave] = 1.f / sqrtf(ss / (float)K + args.eps);
+    __syncthreads();
+    float rstd[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) rstd[i] = rstd_l[2 * i + half];  // rows past M: some finite number, dropped below
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int g = g_begin + 2 * p;
+      float wn[8];
+      unpack8(xw[p], wn);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (2 * i >= M) continue;  // both rows of the request lie past M: zeros came back, zeros stay (uniform)
+        const int row = 2 * i + half;
+        const bool mine = row < M && g + cu < g_end;
+        float f[8], r[8];
+        unpack8(xa[p][i], f);
+        unpack8(xr[p][i], r);
+        u32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float y0 = round_bf16(wn[2 * e] * round_bf16(f[2 * e] * rstd[i]));
+          const float y1 = round_bf16(wn[2 * e + 1] * round_bf16(f[2 * e + 1] * rstd[i]));
+          o[e] = pack_bf16x2(r[2 * e] + y0, r[2 * e + 1] + y1);
+        }
+        xa[p][i] = mine ? o : u32x4{0u, 0u, 0u, 0u};
+        if (blockIdx.x == 0 && mine)
+          *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(args.x_out) + row * K * 2 + 256 * g + 16 * c32) = o;
+      }
+    }
+  }
+  // rows as asked for -> operand fragments, a pair at a time through the wave's own blocks: block (row, group of the
+  // pair) holds that row's 128 columns; the fragment of k-step j is chunk 4 j + kq of block (col & 7, col >> 3)
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      *reinterpret_cast<u32x4*>(xs + (2 * (2 * i + half) + cu) * kR8BlockBytes + (c32 & 15) * 16) = xa[p][i];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      xa[p][j] = *reinterpret_cast<const u32x4*>(xs + (2 * (col & 7) + (col >> 3)) * kR8BlockBytes + (4 * j + kq) * 16);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int nt = AHEAD; nt < NT; ++nt) request(nt);
+  __builtin_amdgcn_sched_barrier(0);
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  const bf16x8 ones = ones_bf16x8();
+  const UnpackConsts uc;
+  f32x4 xsum[NP];  // the sums of the activations over each group do not depend on the tile
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    xsum[p] = zero4;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      xsum[p] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[p][j]), ones, xsum[p], 0, 0, 0);
+  }
+
+  // ---- 3. products, tile by tile in the order the pieces were asked for ------------------------------------------------
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    f32x4 acc = zero4;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      f32x4 t[2] = {zero4, zero4};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bf16x8 af = __builtin_bit_cast(bf16x8, xa[p][j]);
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+          t[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af, unpack_w4_bias128(w[nt][p][u][j], uc), t[u], 0, 0, 0);
+      }
+      // this lane's rows are 4 kq + r of the operand: group g for kq < 2, group g + 1 otherwise
+      const float sc = (float)__builtin_bit_cast(_Float16, s16[nt][p]);
+      const float nzc = -(float)(129 + (int)(((uint32_t)z8[nt][p] >> (4 * (col & 1))) & 15u));  // -(128 + (stored + 1))
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float tv = ul ? t[1][r] : t[0][r];
+        acc[r] = __builtin_fmaf(sc, __builtin_fmaf(nzc, xsum[p][r], tv), acc[r]);
+      }
+    }
+    // the two groups of a pair inside the wave; the waves through LDS below
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float v = combine_xor32(acc[r], AddOp{});
+      if (kq < 2) red[((wave * NT + nt) * 8 + 4 * kq + r) * 16 + col] = v;
+    }
+  }
+  __syncthreads();
+  auto total_of = [&](int nt, int mm, int c) {
+    float v = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv) v += red[((wv * NT + nt) * 8 + mm) * 16 + c];
+    return v;
+  };
+  for (int i = tid; i < PER * 128; i += WAVES * 64) {  // whole waves: 16 lanes = one (row, unit)
+    const int c = i & 15, mm = (i >> 4) & 7, iu = i >> 7;
+    const int un = (int)blockIdx.x + iu * (int)gridDim.x;
+    const bool live = un < units && mm < M;
+    if constexpr (EPI == 0) {
+      const float v = live ? round_bf16(total_of(iu, mm, c)) : 0.f;
+      if (live) args.y[mm * args.N + un * 16 + c] = f32_to_bf16_bits(v);
+      if (args.ssq_out) {  // sum of squares of the 16 outputs of (row, tile): one row of 16 lanes
+        const float q = row16_sum(v * v);
+        if (live && c == 0) args.ssq_out[mm * ntiles + un] = q;
+      }
+    } else if (live) {
+      const float up = round_bf16(total_of(2 * iu, mm, c));  // the Linear's bf16 output
+      const float gate = round_bf16(total_of(2 * iu + 1, mm, c));
+      const float sg = round_bf16(gate / (1.f + expf(-gate)));
+      args.y[mm * (args.N >> 1) + un * 16 + c] = f32_to_bf16_bits(sg * up);
+    }
+  }
+}
+
 // ---- launch plans -------------------------------------------------------------------------------
 struct GemvPlan {
   int mt, nt, waves;
@@ -1615,6 +1829,62 @@ constexpr bool r8_exists(int nt, int waves, int pmax, bool pro, bool epi, bool p
   return nt == 1 || pmax == 1;
 }
 
+// CUs of the device first used (a grid only has to be about as large as the machine); 0 if the query fails
+int cu_count() {
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0)
+      n_cu = cus;
+  }
+  return n_cu;
+}
+
+// Up to 8 rows through w4_gemv_rows_kernel when the units of the product can be dealt out over one workgroup per CU
+// (at most four tiles or three up/gate pairs each); O355_EUNSUPPORTED otherwise (the caller goes on to the kernel
+// that walks sets of tiles).
+int w4_rows_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, bool pro, bool epi,
+                     void* stream) {
+  const int G = a.K >> 7, ntiles = a.N >> 4, n_cu = std::max(cu_count(), 1);
+  const int units = epi ? ntiles >> 1 : ntiles;
+  // 16 waves from 32 groups on, unless the groups split much more evenly into pairs over 8 (K = 5120: 16 runs of 2 or
+  // 3 groups -- two pairs each, a third of them empty -- or 8 runs of 5), as measured for the set-walking kernel
+  auto pairs_of = [&](int wv) { return std::max(1, ((G + wv - 1) / wv + 1) >> 1); };
+  const double fill16 = (double)G / (2.0 * pairs_of(16) * 16), fill8 = (double)G / (2.0 * pairs_of(8) * 8);
+  const int waves = G >= 32 && !(fill8 > fill16 + 0.15) ? 16 : 8;
+  if (G < waves) return O355_EUNSUPPORTED;
+  const int np = pairs_of(waves);
+  const int prov = !pro ? 0 : (a.K <= 4096 ? 1 : (a.K <= 8192 ? 2 : -1));
+  const int per = (units + n_cu - 1) / n_cu;
+  if (prov < 0 || np > 3 || per > (epi ? 3 : 4)) return O355_EUNSUPPORTED;
+  const int nt = epi ? 2 * per : per;
+  // registers of the pieces in flight (weights, rows, and with the prologue the residual and the norm weight): past
+  // these counts the instantiations spill (128 registers per lane at 16 waves, 256 at 8)
+  if (nt * np * 8 + np * 16 + (pro ? np * 20 : 0) > (waves == 16 ? 90 : 208)) return O355_EUNSUPPORTED;
+  const size_t lds = (size_t)waves * nt * 128 * 4 + 32 + (size_t)waves * kR8WaveBytes;
+  if (lds > 160 * 1024) return O355_EUNSUPPORTED;
+  const unsigned blocks = (unsigned)(per == 1 ? units : n_cu);
+  const u32x4* w = (const u32x4*)wt;
+  hipStream_t s = as_stream(stream);
+#define ROWS_CASE(Wv, Pv, Ev, Nv, Uv)                                                                                  \
+  if (waves == Wv && prov == Pv && (int)epi == Ev && np == Nv && per == Uv) {                                          \
+    auto kern = w4_gemv_rows_kernel<Wv, Pv, Ev, Nv, Uv>;                                                               \
+    if (lds > 48 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                               (int)lds) != hipSuccess)                                                \
+      return O355_ELAUNCH;                                                                                             \
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(Wv * 64), lds, s, a, w, st, zt, units);                                \
+    O355_CHECK_LAUNCH();                                                                                               \
+  }
+#define ROWS_FORMS(Wv, Pv, Nv)                                                                                    \
+  ROWS_CASE(Wv, Pv, 0, Nv, 1) ROWS_CASE(Wv, Pv, 0, Nv, 2) ROWS_CASE(Wv, Pv, 0, Nv, 3) ROWS_CASE(Wv, Pv, 0, Nv, 4) \
+  ROWS_CASE(Wv, Pv, 1, Nv, 1) ROWS_CASE(Wv, Pv, 1, Nv, 2) ROWS_CASE(Wv, Pv, 1, Nv, 3)
+  ROWS_FORMS(16, 0, 1) ROWS_FORMS(16, 0, 2) ROWS_FORMS(16, 0, 3) ROWS_FORMS(16, 1, 1) ROWS_FORMS(16, 2, 2)
+  ROWS_FORMS(8, 0, 1) ROWS_FORMS(8, 0, 3) ROWS_FORMS(8, 1, 1) ROWS_FORMS(8, 2, 3)
+#undef ROWS_FORMS
+#undef ROWS_CASE
+  return O355_EUNSUPPORTED;
+}
+
 int w4_r8_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, const uint8_t* zt, bool pro, bool epi, int nt,
                    int waves, void* stream) {
   const int G = a.K >> 7, ntiles = a.N >> 4;
@@ -1622,6 +1892,10 @@ int w4_r8_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, co
   if ((int64_t)a.M * a.K * 2 >= 0x40000000 || (int64_t)ntiles * G * 1024 >= (1ll << 31)) return O355_EUNSUPPORTED;
   if (pro && (!a.ssq_in || !a.resid || !a.norm_w || !a.x_out || (a.K >> 4) > 1024)) return O355_EUNSUPPORTED;
   if (a.ssq_out && epi) return O355_EUNSUPPORTED;
+  if (nt == 0 && waves == 0) {  // no form asked for: the kernel that issues everything at once, where it covers the shape
+    const int st_rows = w4_rows_dispatch(a, wt, st, zt, pro, epi, stream);
+    if (st_rows != O355_EUNSUPPORTED) return st_rows;
+  }
   static int n_cu = 0;  // of the device first used: the grid only has to be about as large as the machine
   if (n_cu == 0) {
     int dev = 0, cus = 0;
@@ -1676,17 +1950,6 @@ int w4_r8_dispatch(const GemvArgs& a, const uint32_t* wt, const uint16_t* st, co
   R8_CASE(2, 8, 1, false, 0, true) R8_CASE(2, 8, 2, false, 0, true) R8_CASE(2, 8, 1, true, 0, true) R8_CASE(2, 8, 2, true, 0, true)
   R8_CASE(2, 8, 1, false, 1, true) R8_CASE(2, 8, 2, false, 1, true) R8_CASE(2, 8, 1, true, 1, true) R8_CASE(2, 8, 2, true, 1, true)
   return O355_EUNSUPPORTED;
-}
-
-// CUs of the device first used (a grid only has to be about as large as the machine); 0 if the query fails
-int cu_count() {
-  static int n_cu = 0;
-  if (n_cu == 0) {
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0)
-      n_cu = cus;
-  }
-  return n_cu;
 }
 
 // One row through w4_gemv_one_kernel; O355_EUNSUPPORTED for what it does not cover (the caller goes on to the
