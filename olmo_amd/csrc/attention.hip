@@ -755,6 +755,12 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   __shared__ __align__(16) u32x4 knew[HD / 8], vnew[HD / 8];
   __shared__ int s_last;
   __shared__ uint32_t s_flag;
+  // Every argument at once: fetched where each is first used they come in seven batches, each a round trip of the
+  // scalar cache to memory that the wave waits out.
+  if constexpr (!RELAY)
+    asm volatile("" ::"s"(qkv), "s"(qw), "s"(kw), "s"(sin_t), "s"(cos_t), "s"(kc), "s"(vc), "s"(key_bias), "s"(ws), "s"(H), "s"(Hkv),
+                 "s"(Lmax), "s"(n_pos), "s"(past_len), "s"(past_dev), "s"(nchunks_max), "s"(bias_stride), "s"(eps), "s"(qk_ssq),
+                 "s"(rope_now), "s"(out), "s"(tickets), "s"(ll));
   const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z, gsz = H / Hkv, hk = h / gsz;
   const int tid = threadIdx.x, lane = tid & 63;
   // ll (flags in the data): the workgroup of the head's last chunk merges.  Workgroups start in the order of their
@@ -782,7 +788,14 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   // may depend on it: the rotary rows of the current position are then taken from rope_now ([sin | cos],
   // refreshed once per decode step by olmo355_rope_advance) rather than looked up by position, and the
   // position itself is first needed for masking, long after it has arrived.
-  const int pos = past_dev ? *past_dev : past_len;
+  // It is asked for as a vector request (an offset the compiler cannot see to be uniform): as a scalar one it would
+  // hold up every later wait for a scalar, the scalar counter having no order.
+  int pos_v = past_len;
+  if (past_dev) {
+    int zero_v = 0;
+    asm volatile("" : "+v"(zero_v));
+    pos_v = __builtin_amdgcn_raw_buffer_load_b32(make_rsrc(past_dev, 4), zero_v, 0, 0);
+  }
 
   // ---- 1. this head's q / new-k pieces, norm weights, rotary rows, sums of squares; then the cache rows
   // of this wave.  Cache rows come through a buffer resource with a scalar offset per request and the
@@ -807,8 +820,9 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
       w1 = reinterpret_cast<const u32x4*>(wsrc + j)[0];
       w2 = reinterpret_cast<const u32x4*>(wsrc + j + HALF)[0];
     }
-    const float* sp = rope_now ? rope_now : sin_t + (int64_t)min(pos, n_pos - 1) * HD;
-    const float* cp = rope_now ? rope_now + HD : cos_t + (int64_t)min(pos, n_pos - 1) * HD;
+    const int pos_r = rope_now ? 0 : min(__builtin_amdgcn_readfirstlane(pos_v), n_pos - 1);  // (waits for it: the path without rope_now)
+    const float* sp = rope_now ? rope_now : sin_t + (int64_t)pos_r * HD;
+    const float* cp = rope_now ? rope_now + HD : cos_t + (int64_t)pos_r * HD;
 #pragma unroll
     for (int v4 = 0; v4 < 2; ++v4) {
       cs1[v4] = reinterpret_cast<const f32x4*>(cp + j)[v4], cs2[v4] = reinterpret_cast<const f32x4*>(cp + j + HALF)[v4];
@@ -857,7 +871,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   u32x4 t[4], pq[2], pk[2];
   // workgroups whose chunk lies past the current length (a captured launch covers the cache's capacity) leave below
   // without having waited for anything
-  const bool relay_work = RELAY && (chunk * kDecodeChunk < pos + 1 || (ll && chunk == nchunks_max - 1));
+  const bool relay_work = RELAY && (chunk * kDecodeChunk < __builtin_amdgcn_readfirstlane(pos_v) + 1 || (ll && chunk == nchunks_max - 1));
   // (every request goes past the L2 -- device-coherent -- so that no poll finds a line there that was fetched before
   // the projection's stores)
   auto relay_ask = [&]() {
@@ -895,10 +909,17 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
 #pragma unroll
   for (int it = 0; it < ITERS; ++it)
     kreg[it] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rk, lane * 16, min(kbase + it * KPI, rowcap) * HD * 2, 2));
-#pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
+  // The value rows are asked for further down, once the query is in LDS: a CU takes a wave's requests only as fast
+  // as earlier ones come back (24 of them occupy a wave for 2 to 3 us, measured with time stamps), and a wave that
+  // is issuing them cannot look at the token's pieces when they arrive.  With the key rows alone ahead of it the
+  // query is ready 1 us earlier and the scores of the first keys are formed while the value rows travel.
+  auto ask_v = [&](int it) {
     vreg[it] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rv, lane * 16, min(kbase + it * KPI, rowcap) * HD * 2, 2));
     bias[it] = key_bias ? key_bias[(int64_t)b * bias_stride + min(min(kbase + it * KPI + kslot, kmax), bias_stride - 1)] : 0.f;  // keys past the row's end are past L
+  };
+  if constexpr (RELAY) {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) ask_v(it);
   }
 
   if constexpr (RELAY) {
@@ -1032,6 +1053,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   }
   if (role_v) vnew[tid - 64] = vrow;
   // ---- the position is needed from here on ----------------------------------------------------------------
+  const int pos = __builtin_amdgcn_readfirstlane(pos_v);
   const int L = pos + 1;
   const bool bad_pos = pos >= Lmax || pos >= n_pos || pos > kmax;
   bool merger = false, active = chunk * kDecodeChunk < L;
@@ -1056,6 +1078,10 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(
   float qr[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) qr[i] = qs[sub * 8 + i];
+  if constexpr (!RELAY) {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) ask_v(it);
+  }
 
   // ---- 3. scores, softmax partial and P.V per key slot (the LPK lanes that share a key) ------------
   float s[ITERS];
