@@ -1619,11 +1619,22 @@ FusedPlan fused_plan(int B, int H, int n_keys_max, int merge) {
   // (measured at the 7B shapes, context 2048: the in-kernel merge wins while the launch is a single round of
   // workgroups -- 17.0 against 20.4 us at batch 1 -- and loses once workgroups queue up -- 69.7 against 61.6 us
   // at batch 8, where one workgroup per (batch, head) takes 66.9)
-  p.merge_in_kernel = merge == 0 || merge == 1 || (merge < 0 && (int64_t)B * H * p.nch <= 1536);
+  // (measured again with the value rows asked for behind the query, batch 8 and more, 32 heads: the flag form
+  // 51.7 / 93.2 / 92.3 / 176.2 us at 8 x 2049, 16 x 2049, 8 x 4097, 32 x 2049 keys against 52.8 / 95.3 / 95.1 / 181.9 for
+  // the separate kernel and 54.4 / 102.5 / 103.1 / 193.2 for tickets -- when the workgroups fill whole rounds of the
+  // CUs; at 8 x 40 heads, 11.25 rounds, the separate kernel stays ahead, 63.1 against 65.1)
+  static int n_cu = 0;
+  if (n_cu == 0) {
+    int dev = 0, cus = 0;
+    n_cu = hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0 ? cus : 256;
+  }
+  const int64_t wgs = (int64_t)B * H * p.nch;
+  const bool whole_rounds = wgs > 1536 && wgs % n_cu == 0;
+  p.merge_in_kernel = merge == 0 || merge == 1 || (merge < 0 && (wgs <= 1536 || whole_rounds));
   // (measured with 128-key chunks, batch 1: the flag form is level with the ticket form at 17 chunks per head -- 17.2
   // against 16.4 us, 7B at context 2048 -- and ahead from about two dozen -- 34.4 against 36.5 us, 13B at context 4090;
   // with that launch's 256-key chunks, 17 per head, the two forms are level again at 29.6 us)
-  p.ll = p.merge_in_kernel && (merge == 1 || (merge < 0 && p.nch >= kFlagMergeFromChunks)) ? 1 : 0;  // needs the counters
+  p.ll = p.merge_in_kernel && (merge == 1 || (merge < 0 && (p.nch >= kFlagMergeFromChunks || whole_rounds))) ? 1 : 0;  // needs the counters
   return p;
 }
 

@@ -1491,7 +1491,7 @@ __global__ __launch_bounds__(WAVES * 64) void w4_gemv_rows_kernel(GemvArgs args,
   const int col = lane & 15, kq = lane >> 4;
   const int ul = kq >> 1;  // the group of a pair whose results this lane keeps
   const int g_begin = (G * wave) / WAVES, g_end = (G * (wave + 1)) / WAVES;
-  constexpr int kNowhere = 0x40000000;  // past every buffer here: such a request returns zeros and moves nothing
+  constexpr int kNowhere = (int)0x80000000u;  // past every buffer: such a request returns zeros and moves nothing
   const int wvoff = lane * 16;
   const int half = lane >> 5, c32 = lane & 31, cu = c32 >> 4;  // request i of a pair: rows 2 i + half, group cu of the pair
 
