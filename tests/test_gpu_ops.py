@@ -1041,6 +1041,59 @@ def test_w4_gemv_chain(dev, M, N, K, epi):
         assert torch.allclose(ssq.cpu(), want, rtol=1e-5, atol=1e-6 * want.max().item())
 
 
+@pytest.mark.parametrize("M", [1, 8])
+@pytest.mark.parametrize("N,K,epi", [
+    (6144, 2048, False), (2048, 8192, False), (16384, 2048, True),       # the 1B shapes: one group per wave; K = 8192; 512 up/gate pairs
+    (5120, 5120, False), (5120, 13824, False), (27648, 5120, True),      # the 13B shapes: runs of 2 or 3, of 6 or 7 and of 5 groups
+    (4112, 4096, False), (24576, 4096, False), (50176, 4096, False),     # 257 tiles; 1536 tiles = 512 workgroups of three; many tiles
+    (1024, 1024, False), (2048, 640, False),                            # eight groups; five (fewer than waves: the general kernel)
+])
+def test_w4_one_row_and_rows_kernels_over_shapes(dev, M, N, K, epi):
+    """The kernels written for the decode step (one row; up to 8 rows with every request issued at once) over the
+    splits of K and N their templates distinguish -- runs of equal and unequal length per wave, one and several units
+    per workgroup, the slot or unit a wave or workgroup lacks asked for past the buffer -- against the oracle's norm +
+    linear (+ SwiGLU); shapes they do not cover take the general kernels through the same call."""
+    say("w4 one/rows shapes", M, N, K, epi)
+    ops = _ops()
+    gen = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    resid = torch.randn(M, K, generator=gen).to(torch.bfloat16)
+    nw = (1 + 0.1 * torch.randn(K, generator=gen)).to(torch.bfloat16)
+    qw, qz, sc = ow4.random_quantized(K, N, 128, seed=N + K)
+    Wf = ow4.dequantize(qw, qz, sc, 128).float()
+    w = ops.w4_repack(qw.to(dev), qz.to(dev), sc.to(dev), 128)
+    # plain product (and the sums of squares of its output)
+    y0 = ops.w4_linear(a.to(dev), w)
+    y0_ref = (a.float() @ Wf).to(torch.bfloat16)
+    assert (y0.cpu().float() - y0_ref.float()).abs().max().item() <= 2 ** -6 * y0_ref.float().abs().max().item()
+    if not epi:
+        r = ops.w4_linear_chain(a.to(dev), w, want_ssq=True)
+        if r is not None:
+            y1, _, ssq1 = r
+            assert (y1.cpu().float() - y0_ref.float()).abs().max().item() <= 2 ** -6 * y0_ref.float().abs().max().item()
+            want = (y1.float().cpu() ** 2).view(M, -1, 16).sum(-1)
+            assert torch.allclose(ssq1.cpu(), want, rtol=1e-5, atol=1e-6 * want.max().item())
+    # with the chained norm prologue (and the SwiGLU epilogue)
+    ssq_in = (a.float() ** 2).view(M, -1, 16).sum(-1)
+    r = ops.w4_linear_chain(a.to(dev), w, resid=resid.to(dev), norm_w=nw.to(dev), eps=1e-6, ssq_in=ssq_in.to(dev),
+                            swiglu_out=epi, want_ssq=not epi)
+    if r is None:
+        assert K > 4096 or K < 1024  # a consumer may decline long or very short rows; never the model shapes at one row
+        assert not (M == 1 and 1024 <= K <= 8192)
+        return
+    y, x_new, ssq = r
+    x_ref = resid + om.rms_norm(a, nw, 1e-6)
+    y_ref = (x_ref.float() @ Wf).to(torch.bfloat16)
+    if epi:
+        y_ref = om.swiglu(y_ref)
+    dx = (x_new.cpu().float() - x_ref.float()).abs()
+    assert (dx <= 2.0 ** (torch.floor(torch.log2(x_ref.float().abs().clamp_min(1e-30))) - 7)).all()
+    assert (y.cpu().float() - y_ref.float()).abs().max().item() <= 2 ** -6 * y_ref.float().abs().max().item()
+    if ssq is not None:
+        want = (y.float().cpu() ** 2).view(M, -1, 16).sum(-1)
+        assert torch.allclose(ssq.cpu(), want, rtol=1e-5, atol=1e-6 * want.max().item())
+
+
 @pytest.mark.parametrize("M", [3, 8])
 @pytest.mark.parametrize("N,K,epi,pro", [(12288, 4096, False, True), (4096, 4096, False, False), (22016, 4096, True, True),
                                          (4096, 11008, False, False), (2064, 640, False, True)])
