@@ -175,8 +175,11 @@ def main() -> int:
 
     def run_decode(B: int):
         ids = torch.randint(0, cfg.vocab_size, (B, ctx), generator=gen).to(dev)
-        # prefill (timed separately, second run = warm)
+        # prefill (timed separately, second run = warm; the first run's cache is given back before it, as a server
+        # that finished a request would have done, so that the allocator hands the same memory out again)
+        out = cache = first = kb = None
         for rep in range(2):
+            out = cache = first = kb = None
             torch.cuda.synchronize()
             tp = time.perf_counter()
             out, cache, first, kb = _prefill(model, ids, None)

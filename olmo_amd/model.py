@@ -51,8 +51,12 @@ class KVCache:
     """Contiguous per-layer key/value buffers ``[B, n_kv_heads, capacity, hd]`` (keys rotated)."""
 
     def __init__(self, n_layers: int, B: int, Hkv: int, capacity: int, hd: int, dtype, device):
-        self.k = [torch.empty(B, Hkv, capacity, hd, dtype=dtype, device=device) for _ in range(n_layers)]
-        self.v = [torch.empty(B, Hkv, capacity, hd, dtype=dtype, device=device) for _ in range(n_layers)]
+        # one allocation for all layers (a fresh cache is made per prompt: 2 * n_layers separate ones cost a 7B
+        # prefill 2.9 ms of allocator calls when none of them was cached); a layer's keys and values are the
+        # contiguous slices [B, Hkv, capacity, hd] of it
+        kv = torch.empty(2, n_layers, B, Hkv, capacity, hd, dtype=dtype, device=device)
+        self.k = list(kv[0].unbind(0))
+        self.v = list(kv[1].unbind(0))
         self.B, self.capacity, self.length = B, capacity, 0
         # device copy of the number of cached positions, for captured decode steps
         self.length_dev = torch.zeros(1, dtype=torch.int32, device=device)
