@@ -191,6 +191,12 @@ int olmo355_f32_linear(const float* x, const float* w_nk, float* y, int M, int N
  * residual add of olmo/model.py:786-794,814-821).  weight may be NULL.  rows x d. */
 int olmo355_rmsnorm(const void* x, const void* weight, const void* residual, void* out, int rows, int d, float eps,
                     int dtype, void* stream);
+/* The last block's post-norm update and the final norm of a decode step in one launch
+ * (olmo/model.py:814-821 followed by olmo/model.py:1421-1423): x1 = residual + rmsnorm(x; w1),
+ * out = rmsnorm(x1; w2), with every rounding of the two olmo355_rmsnorm calls it replaces (bit-identical to them).
+ * O355_EUNSUPPORTED when d is not a multiple of 8 (4 for fp32) or above 8192 (4096): issue the two calls then. */
+int olmo355_rmsnorm_pair(const void* x, const void* w1, const void* residual, const void* w2, void* out, int rows, int d,
+                         float eps, int dtype, void* stream);
 /* Non-parametric LayerNorm.forward (olmo/model.py:212-225): F.layer_norm without weight/bias. */
 int olmo355_layernorm_np(const void* x, void* out, int rows, int d, float eps, int dtype, void* stream);
 
@@ -318,6 +324,13 @@ int olmo355_add_bias_f16(const uint16_t* x, const uint16_t* bias_f16, uint16_t* 
 /* Greedy step (olmo/beam_search.py:102-113 with beam 1): first index of the row maximum,
  * written as int64 to out[r], and the same value appended at ids_next when non-NULL. */
 int olmo355_argmax(const void* logits, int64_t* out, int rows, int n, int dtype, void* stream);
+/* The end of a greedy decode step in one launch: olmo355_argmax per row into ids_out, the chosen token's row of the
+ * embedding table (olmo/model.py:1318) into x_next [rows, d] as the next step's input, and olmo355_rope_advance(pos, 1,
+ * ...) for the step that follows.  Ids at or past `vocab` (rows of the table) read its last row, as
+ * olmo355_embedding does. */
+int olmo355_greedy_next(const void* logits, int64_t* ids_out, const void* table, void* x_next, int rows, int n, int d,
+                        int vocab, int32_t* pos, const float* sin_tab, const float* cos_tab, float* rope_now, int hd,
+                        int n_pos, int dtype, void* stream);
 /* The two selections of a beam-search step (olmo/beam_search.py:813-1045 with the DeterministicSampler,
  * :102-113), one workgroup per row.
  * olmo355_log_softmax: F.log_softmax of the step function (olmo/model.py:1705) over rows of n logits in the

@@ -49,6 +49,7 @@ EXPORTS = {
     "olmo355_f16_gemm": (I, [P, P, P, I, I, I, P]),
     "olmo355_f32_linear": (I, [P, P, P, I, I, I, P]),
     "olmo355_rmsnorm": (I, [P, P, P, P, I, I, F, I, P]),
+    "olmo355_rmsnorm_pair": (I, [P, P, P, P, P, I, I, F, I, P]),
     "olmo355_layernorm_np": (I, [P, P, I, I, F, I, P]),
     "olmo355_qknorm_rope_kvwrite": (I, [P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P, F, I, P]),
     "olmo355_attn_prefill": (I, [P, P, P, P, P, I, I, I, I, I, I, I, I, I, P]),
@@ -84,6 +85,7 @@ EXPORTS = {
     "olmo355_add_bias_bf16": (I, [P, P, P, I, I, P]),
     "olmo355_add_bias_f16": (I, [P, P, P, I, I, P]),
     "olmo355_argmax": (I, [P, P, I, I, I, P]),
+    "olmo355_greedy_next": (I, [P, P, P, P, I, I, I, I, P, P, P, P, I, I, I, P]),
     "olmo355_incr_i32": (I, [P, P]),
 }
 

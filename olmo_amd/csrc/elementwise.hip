@@ -106,6 +106,60 @@ __global__ __launch_bounds__(256) void rmsnorm_vec_kernel(const void* __restrict
   }
 }
 
+// Two norms in one launch, for the end of a decode step: x1 = res + rmsnorm(x; w1), out = rmsnorm(x1; w2), every
+// rounding where the two separate launches have it (x1 is rounded to the activation type before its squares are summed).
+template <int DT, int VPT>
+__global__ __launch_bounds__(256) void rmsnorm_pair_kernel(const void* __restrict__ x, const void* __restrict__ w1,
+                                                           const void* __restrict__ res, const void* __restrict__ w2,
+                                                           void* __restrict__ out, int d, float eps) {
+  constexpr int N = Vec<DT>::N;
+  __shared__ float red[16];
+  const int nvec = d / N;
+  const int64_t vbase = (int64_t)blockIdx.x * nvec;
+  float v[VPT][N];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int idx = threadIdx.x + i * 256;
+    if (idx < nvec) {
+      Vec<DT>::ld(x, vbase + idx, v[i]);
+#pragma unroll
+      for (int e = 0; e < N; ++e) ss += v[i][e] * v[i][e];
+    }
+  }
+  ss = block_sum(ss, red);
+  const float rstd = 1.f / sqrtf(ss / (float)d + eps);
+  float ss2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int idx = threadIdx.x + i * 256;
+    if (idx < nvec) {
+      float wv[N], rv[N];
+      Vec<DT>::ld(w1, idx, wv);
+      Vec<DT>::ld(res, vbase + idx, rv);
+#pragma unroll
+      for (int e = 0; e < N; ++e) {
+        const float y = Act<DT>::rnd(wv[e] * Act<DT>::rnd(v[i][e] * rstd));
+        v[i][e] = Act<DT>::rnd(rv[e] + y);
+        ss2 += v[i][e] * v[i][e];
+      }
+    }
+  }
+  ss2 = block_sum(ss2, red);
+  const float rstd2 = 1.f / sqrtf(ss2 / (float)d + eps);
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const int idx = threadIdx.x + i * 256;
+    if (idx < nvec) {
+      float wv[N];
+      Vec<DT>::ld(w2, idx, wv);
+#pragma unroll
+      for (int e = 0; e < N; ++e) v[i][e] = Act<DT>::rnd(wv[e] * Act<DT>::rnd(v[i][e] * rstd2));
+      Vec<DT>::st(out, vbase + idx, v[i]);
+    }
+  }
+}
+
 // any d (element-wise fallback)
 template <int DT>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const void* __restrict__ x, const void* __restrict__ w,
@@ -450,6 +504,81 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const void* __restrict__ x
   }
 }
 
+// The end of a greedy decode step in one launch: argmax_kernel's choice per row, the chosen token's embedding row as
+// the next step's input, and (row 0's workgroup) the position advanced by one with its rotary rows, as
+// olmo355_rope_advance leaves them.
+template <int DT>
+__global__ __launch_bounds__(1024) void greedy_next_kernel(const void* __restrict__ x, int64_t* __restrict__ out, int n,
+                                                           const void* __restrict__ tab, void* __restrict__ x_next, int d,
+                                                           int vocab, int32_t* __restrict__ pos,
+                                                           const float* __restrict__ sin_t, const float* __restrict__ cos_t,
+                                                           float* __restrict__ rope_now, int hd, int n_pos) {
+  constexpr int N = Vec<DT>::N;
+  constexpr int VPT = 16;
+  __shared__ float sv[16];
+  __shared__ int si[16];
+  const int64_t base = (int64_t)blockIdx.x * n;
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  if (n % N == 0 && n / N <= VPT * 1024) {
+    const int nvec = n / N;
+    float v[VPT][N];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int idx = threadIdx.x + i * 1024;
+      if (idx < nvec) Vec<DT>::ld(x, (base / N) + idx, v[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int idx = threadIdx.x + i * 1024;
+      if (idx < nvec) {
+#pragma unroll
+        for (int e = 0; e < N; ++e)
+          if (v[i][e] > best) best = v[i][e], bi = idx * N + e;  // indices ascend per thread: first max kept
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+      const float v = Act<DT>::ld(x, base + i);
+      if (v > best || (v == best && i < bi)) best = v, bi = i;
+    }
+  }
+  wave_first_pair(best, bi, [](float ov, int oi, float v, int i) { return ov > v || (ov == v && oi < i); });
+  const int w = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) sv[w] = best, si[w] = bi;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int i = 1; i < (int)(blockDim.x >> 6); ++i)
+      if (sv[i] > best || (sv[i] == best && si[i] < bi)) best = sv[i], bi = si[i];
+    bi = bi == 0x7fffffff ? 0 : bi;
+    out[blockIdx.x] = bi;
+    si[0] = bi;
+  }
+  __syncthreads();
+  // the chosen token's row of the embedding table (clamped like embedding_kernel's)
+  int64_t id = si[0];
+  id = id >= vocab ? vocab - 1 : id;
+  typedef typename Act<DT>::T T;
+  const T* src = (const T*)tab + id * d;
+  T* dst = (T*)x_next + (int64_t)blockIdx.x * d;
+  if (((d * sizeof(T)) & 15) == 0) {
+    const int nv = (int)(d * sizeof(T) / 16);
+    for (int i = threadIdx.x; i < nv; i += blockDim.x) reinterpret_cast<u32x4*>(dst)[i] = reinterpret_cast<const u32x4*>(src)[i];
+  } else {
+    for (int i = threadIdx.x; i < d; i += blockDim.x) dst[i] = src[i];
+  }
+  if (blockIdx.x == 0) {
+    const int p = *pos + 1;
+    __syncthreads();  // every thread has read the old value
+    if (threadIdx.x == 0) *pos = p;
+    const int r = min(max(p, 0), n_pos - 1);
+    for (int i = threadIdx.x; i < hd; i += blockDim.x) {
+      rope_now[i] = sin_t[(int64_t)r * hd + i];
+      rope_now[hd + i] = cos_t[(int64_t)r * hd + i];
+    }
+  }
+}
+
 __global__ void incr_kernel(int32_t* p) { *p += 1; }
 
 }  // namespace
@@ -488,6 +617,23 @@ extern "C" int olmo355_rmsnorm(const void* x, const void* weight, const void* re
   } else {
     DT_SWITCH(dtype,
               hipLaunchKernelGGL(rmsnorm_kernel<DT>, dim3(rows), dim3(256), 0, s, x, weight, residual, out, d, eps));
+  }
+  O355_CHECK_LAUNCH();
+}
+
+extern "C" int olmo355_rmsnorm_pair(const void* x, const void* w1, const void* residual, const void* w2, void* out,
+                                    int rows, int d, float eps, int dtype, void* stream) {
+  if (!x || !w1 || !residual || !w2 || !out || rows <= 0 || d <= 0) return O355_EINVAL;
+  hipStream_t s = as_stream(stream);
+  const int vn = dtype == O355_F32 ? 4 : 8;
+  const int nvec = d / vn;
+  if (d % vn != 0 || nvec > 4 * 256) return O355_EUNSUPPORTED;  // the caller issues the two norms one after the other
+  if (nvec <= 256) {
+    DT_SWITCH(dtype, hipLaunchKernelGGL((rmsnorm_pair_kernel<DT, 1>), dim3(rows), dim3(256), 0, s, x, w1, residual, w2, out, d, eps));
+  } else if (nvec <= 512) {
+    DT_SWITCH(dtype, hipLaunchKernelGGL((rmsnorm_pair_kernel<DT, 2>), dim3(rows), dim3(256), 0, s, x, w1, residual, w2, out, d, eps));
+  } else {
+    DT_SWITCH(dtype, hipLaunchKernelGGL((rmsnorm_pair_kernel<DT, 4>), dim3(rows), dim3(256), 0, s, x, w1, residual, w2, out, d, eps));
   }
   O355_CHECK_LAUNCH();
 }
@@ -619,6 +765,16 @@ extern "C" int olmo355_argmax(const void* logits, int64_t* out, int rows, int n,
   if (!logits || !out || rows <= 0 || n <= 0) return O355_EINVAL;
   DT_SWITCH(dtype,
             hipLaunchKernelGGL(argmax_kernel<DT>, dim3(rows), dim3(1024), 0, as_stream(stream), logits, out, n));
+  O355_CHECK_LAUNCH();
+}
+
+extern "C" int olmo355_greedy_next(const void* logits, int64_t* ids_out, const void* table, void* x_next, int rows, int n,
+                                   int d, int vocab, int32_t* pos, const float* sin_tab, const float* cos_tab,
+                                   float* rope_now, int hd, int n_pos, int dtype, void* stream) {
+  if (!logits || !ids_out || !table || !x_next || !pos || !sin_tab || !cos_tab || !rope_now) return O355_EINVAL;
+  if (rows <= 0 || n <= 0 || d <= 0 || vocab <= 0 || hd <= 0 || n_pos <= 0) return O355_EINVAL;
+  DT_SWITCH(dtype, hipLaunchKernelGGL(greedy_next_kernel<DT>, dim3(rows), dim3(1024), 0, as_stream(stream), logits,
+                                      ids_out, n, table, x_next, d, vocab, pos, sin_tab, cos_tab, rope_now, hd, n_pos));
   O355_CHECK_LAUNCH();
 }
 

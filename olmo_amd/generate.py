@@ -42,12 +42,20 @@ class DecodeSession:
         sin, cos = model._rope
         cache.rope_now = torch.empty(2 * sin.shape[1], dtype=torch.float32, device=sin.device)
         ops.rope_advance(cache.length_dev, 0, sin, cos, cache.rope_now)
+        # greedy: the step's last launch picks the token, looks up its embedding row for the next step and advances
+        # the position (three launches otherwise, and the next step's first)
+        wte = model.transformer["wte"].weight.data
+        self.x_next = model.transformer["wte"](self.ids) if sampling is None and wte.is_contiguous() else None
 
     def _step_kernels(self) -> None:
         m = self.model
-        x = m.transformer["wte"](self.ids)
+        x = self.x_next if self.x_next is not None else m.transformer["wte"](self.ids)
         logits, _ = m._forward_tokens(x, self.cache, self.B, 1, 0, self.key_bias, self.cache.length_dev, False)
         self.logits = logits
+        if self.x_next is not None:
+            ops.greedy_next(logits.view(self.B, -1), self.ids.view(self.B), m.transformer["wte"].weight.data, self.x_next,
+                            self.cache.length_dev, *m._rope, self.cache.rope_now)
+            return
         if self.sampling is None:
             ops.argmax(logits.view(self.B, -1), out=self.ids.view(self.B))
         else:

@@ -771,11 +771,20 @@ class OLMo(nn.Module):
                 x, pend = self._block_decode_fused(blk, x, pend, kc, vc, B, past_len, key_bias, graph_pos, n_keys_max)
             else:
                 x = self._block(blk, x, kc, vc, B, T, past_len, key_bias, graph_pos, n_keys_max)
+        done = False
         if pend is not None:  # the last block's update has no following linear to ride on
-            x = ops.rmsnorm(pend[0], pend[1], self.config.layer_norm_eps, residual=x)
+            ln_f = self.transformer["ln_f"]
+            w2 = getattr(ln_f, "weight", None)
+            if not collect_hidden and isinstance(ln_f, RMSLayerNorm) and w2 is not None and ln_f.eps == self.config.layer_norm_eps:
+                y = ops.rmsnorm_pair(pend[0], pend[1], x, w2.data, ln_f.eps)  # with the final norm, in one launch
+                if y is not None:
+                    x, done = y, True
+            if not done:
+                x = ops.rmsnorm(pend[0], pend[1], self.config.layer_norm_eps, residual=x)
         if last_logits_only and T > 1:
             x = x[:, -1, :].unsqueeze(1).contiguous()
-        x = self.transformer["ln_f"](x)
+        if not done:
+            x = self.transformer["ln_f"](x)
         if collect_hidden:
             hidden.append(x)
         logits = self._head(x)

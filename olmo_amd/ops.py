@@ -586,6 +586,25 @@ def rmsnorm(x, weight: Optional[torch.Tensor], eps: float, residual: Optional[to
     return out
 
 
+def rmsnorm_pair(x, w1: torch.Tensor, residual: torch.Tensor, w2: torch.Tensor, eps: float) -> Optional[torch.Tensor]:
+    """``rmsnorm(residual + rmsnorm(x; w1); w2)`` in one launch, bit-identical to the two :func:`rmsnorm` calls
+    (the end of a decode step: the last block's update, then the final norm); ``None`` for widths the kernel
+    does not take."""
+    _dev(x, w1, residual, w2)
+    d = x.shape[-1]
+    if any(w.dtype != x.dtype or w.numel() != d for w in (w1, w2)) or residual.dtype != x.dtype or residual.shape != x.shape:
+        raise ValueError("weights and residual must match x")
+    out = torch.empty_like(x)
+    rows = x.numel() // d
+    if not rows:
+        return out
+    st = lib().olmo355_rmsnorm_pair(_p(x), _p(w1), _p(residual), _p(w2), _p(out), rows, d, float(eps), _dt(x), _stream())
+    if st == 2:
+        return None
+    check("olmo355_rmsnorm_pair", st)
+    return out
+
+
 def layernorm_np(x: torch.Tensor, eps: float) -> torch.Tensor:
     _dev(x)
     d = x.shape[-1]
@@ -676,6 +695,25 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Te
         out = torch.empty(logits.shape[:-1], dtype=torch.int64, device=logits.device)
     check("olmo355_argmax", lib().olmo355_argmax(_p(logits), _p(out), rows, n, _dt(logits), _stream()))
     return out
+
+
+def greedy_next(logits: torch.Tensor, ids_out: torch.Tensor, table: torch.Tensor, x_next: torch.Tensor,
+                pos_dev: torch.Tensor, sin_tab: torch.Tensor, cos_tab: torch.Tensor, rope_now: torch.Tensor) -> None:
+    """The end of a greedy decode step in one launch: :func:`argmax` of every row into ``ids_out`` (int64), the
+    chosen tokens' embedding rows into ``x_next [rows, d]``, and :func:`rope_advance` by one position."""
+    _dev(logits, ids_out, table, x_next, pos_dev, sin_tab, cos_tab, rope_now)
+    n = logits.shape[-1]
+    rows = logits.numel() // n
+    d, hd = table.shape[1], sin_tab.shape[1]
+    if ids_out.dtype != torch.int64 or ids_out.numel() != rows or x_next.numel() != rows * d:
+        raise ValueError("ids_out int64 [rows] and x_next [rows, d] expected")
+    if table.dtype != logits.dtype or x_next.dtype != logits.dtype or not table.is_contiguous() or not x_next.is_contiguous():
+        raise TypeError("table and x_next: contiguous, of the logits' dtype")
+    if pos_dev.dtype != torch.int32 or rope_now.dtype != torch.float32 or rope_now.numel() != 2 * hd:
+        raise TypeError("pos_dev int32, rope_now float32 [2 * hd] expected")
+    check("olmo355_greedy_next",
+          lib().olmo355_greedy_next(_p(logits), _p(ids_out), _p(table), _p(x_next), rows, n, d, table.shape[0], _p(pos_dev),
+                                    _p(sin_tab), _p(cos_tab), _p(rope_now), hd, sin_tab.shape[0], _dt(logits), _stream()))
 
 
 def log_softmax(logits: torch.Tensor) -> torch.Tensor:

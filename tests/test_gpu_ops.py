@@ -618,6 +618,59 @@ def test_rmsnorm(dev, dtype, rows, d):
         assert (out_r.float() - (r + ref).float()).abs().max().item() <= 2 * ulp.max().item()
 
 
+@pytest.mark.parametrize("dtype", _ACT_DTYPES)
+@pytest.mark.parametrize("rows,d", [(1, 4096), (8, 5120), (3, 256), (2, 8192)])
+def test_rmsnorm_pair_equals_the_two_norms(dev, dtype, rows, d):
+    """The one-launch form of a decode step's last two norms, bit for bit against the two launches it replaces (which
+    test_rmsnorm holds against the oracle); a width it does not take is declined."""
+    ops = _ops()
+    gen = torch.Generator().manual_seed(rows + d)
+    if dtype == torch.float32 and d > 4096:
+        d = 4096
+    x = (torch.randn(rows, d, generator=gen) * 3).to(dtype).to(dev)
+    r = torch.randn(rows, d, generator=gen).to(dtype).to(dev)
+    w1 = (1 + 0.1 * torch.randn(d, generator=gen)).to(dtype).to(dev)
+    w2 = (1 + 0.1 * torch.randn(d, generator=gen)).to(dtype).to(dev)
+    two = ops.rmsnorm(ops.rmsnorm(x, w1, 1e-6, residual=r), w2, 1e-6)
+    one = ops.rmsnorm_pair(x, w1, r, w2, 1e-6)
+    assert one is not None and torch.equal(one, two)
+    odd = torch.randn(2, 1002, generator=gen).to(dtype).to(dev)
+    wo = torch.ones(1002, dtype=dtype, device=dev)
+    assert ops.rmsnorm_pair(odd, wo, odd, wo, 1e-6) is None
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("rows,n", [(1, 100352), (8, 100352), (3, 1003)])
+def test_greedy_next_equals_argmax_embedding_and_rope_advance(dev, dtype, rows, n):
+    """The one-launch end of a greedy decode step against the three launches it replaces: tokens (ties: first index),
+    embedding rows of the chosen tokens, position and rotary rows; a table with fewer rows than the logits are wide
+    reads its last row for ids past it."""
+    ops = _ops()
+    gen = torch.Generator().manual_seed(rows + n)
+    lg = torch.randn(rows, n, generator=gen).to(dtype)
+    lg[0, 77] = lg[0, 900] = 9.0
+    if rows > 1:
+        lg[1, n - 1] = 11.0  # past a table of n - 5 rows
+    lg = lg.to(dev)
+    d, hd, n_pos = 520, 64, 40
+    tab = torch.randn(n - 5, d, generator=gen).to(dtype).to(dev)
+    sin, cos = ops.rope_tables(hd, 10000.0, n_pos, dev)
+    for start in (0, 17, n_pos - 1):  # the last: the position runs past the table, its last row stays
+        pos_a = torch.full((1,), start, dtype=torch.int32, device=dev)
+        pos_b = pos_a.clone()
+        now_a = torch.zeros(2 * hd, dtype=torch.float32, device=dev)
+        now_b = torch.zeros_like(now_a)
+        ids_a = ops.argmax(lg)
+        x_a = ops.embedding(ids_a, tab)
+        ops.rope_advance(pos_a, 1, sin, cos, now_a)
+        ids_b = torch.full((rows,), -1, dtype=torch.int64, device=dev)
+        x_b = torch.full((rows, d), float("nan"), dtype=dtype, device=dev)
+        ops.greedy_next(lg, ids_b, tab, x_b, pos_b, sin, cos, now_b)
+        assert torch.equal(ids_a, ids_b) and int(ids_b[0]) == 77
+        assert torch.equal(x_a.view(rows, d), x_b)
+        assert torch.equal(pos_a, pos_b) and int(pos_b) == start + 1 and torch.equal(now_a, now_b)
+
+
 @pytest.mark.parametrize("rows,d", [(2048, 256), (3, 1000)])
 def test_layernorm_np(dev, rows, d):
     ops = _ops()
