@@ -518,6 +518,7 @@ constexpr int kDecodeMinChunk = 128;  // the smallest chunk: what the workspace 
 //   16 heads x 2101 keys  13.6 / 11.6 / 11.9     32 heads x 1001 keys  11.7 / 11.0 / 11.5
 //   16 heads x 1001 keys   9.6 /  9.9 / 10.5     32 heads x  301 keys   9.0 / 10.1 / 11.3
 //   40 heads x 4091 keys  34.1 / 29.4 / 29.1     8 x 32 heads x 2049 keys  65.8 / 67.0 / 63.4
+// (the kernels as they are now, 32 heads x 2101 keys in a cache of 2192: 40 / 48 / 56 keys per wave 13.0 / 12.6 / 14.2)
 // So: the longest run of keys per workgroup that still leaves the launch with clearly more workgroups than CUs, and
 // short runs for short contexts, where a workgroup's serial walk over its keys is most of the launch.
 inline int decode_keys_per_wave(int B, int H, int n_keys_max) {
