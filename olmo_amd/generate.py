@@ -63,8 +63,16 @@ class DecodeSession:
                        logprob=self.logprob, **self.sampling)
         ops.rope_advance(self.cache.length_dev, 1, *m._rope, self.cache.rope_now)
 
+    def feed(self, ids: torch.Tensor) -> None:
+        """Replace the token that the next step reads (``self.ids`` is what the last step chose): writes it where
+        the step looks for it, the embedding row included when the greedy step keeps that ahead."""
+        self.ids.copy_(ids.view(self.B, 1))
+        if self.x_next is not None:
+            self.x_next.copy_(self.model.transformer["wte"](self.ids))
+
     def step(self) -> None:
-        """Advance by one token: afterwards ``self.ids`` holds the new token of every sequence."""
+        """Advance by one token: afterwards ``self.ids`` holds the new token of every sequence.  (A greedy step has
+        already looked up that token's embedding row for the step after it: to feed another token use :meth:`feed`.)"""
         if self.cache.length + 1 > self.cache.capacity:
             raise ValueError("KV cache capacity exceeded")
         if self.graph is not None:

@@ -828,6 +828,52 @@ def test_sampled_generation(dev):
         model.generate(ids, max_steps=2, sampler=TopKSampler(k=0))
 
 
+def test_decode_session_feed_and_step_tail(dev):
+    """A greedy step's last launch has already looked up the chosen token's embedding row: the session with that
+    launch gives, bit for bit, the tokens and logits of one that ends its steps with the separate arg-max, position
+    advance and lookup (eager and captured); a token fed in place of the chosen one goes through the next step like
+    the last token of a full forward over the sequence that ends with it."""
+    say("decode session: step tail, feed")
+    from olmo_amd.generate import DecodeSession, _prefill
+
+    cfg = small_cfg("olmo2")
+    model, _ = build_pair(cfg, torch.bfloat16, dev, seed=5)
+    ids = torch.randint(0, cfg.vocab_size, (3, 11), generator=torch.Generator().manual_seed(2)).to(dev)
+
+    def run(fused, graph):
+        _, cache, first, kb = _prefill(model, ids, None)
+        sess = DecodeSession(model, cache, first, kb)
+        if not fused:
+            sess.x_next = None
+        toks, logits = [], []
+        for i in range(6):
+            if graph and i == 2:
+                sess.capture()
+            sess.step()
+            toks.append(sess.ids.view(-1).clone())
+            logits.append(sess.logits.view(3, -1).clone())
+        return torch.stack(toks, 1), torch.stack(logits, 1)
+
+    t_ref, l_ref = run(False, False)
+    for fused, graph in ((True, False), (True, True), (False, True)):
+        t, l = run(fused, graph)
+        assert torch.equal(t, t_ref) and torch.equal(l, l_ref), (fused, graph)
+
+    _, cache, first, kb = _prefill(model, ids, None)
+    sess = DecodeSession(model, cache, first, kb)
+    assert sess.x_next is not None
+    sess.step()
+    other = (sess.ids.view(-1) + 7) % cfg.vocab_size
+    sess.feed(other)
+    sess.step()
+    full = torch.cat((ids, first.view(3, 1), other.view(3, 1)), dim=1)
+    ref = model(full, last_logits_only=True).logits.view(3, -1)
+    assert softmax_err(sess.logits.view(3, -1), ref) <= 2e-2
+    wrong = model(torch.cat((ids, first.view(3, 1), ((other + 1) % cfg.vocab_size).view(3, 1)), dim=1),
+                  last_logits_only=True).logits.view(3, -1)
+    assert softmax_err(sess.logits.view(3, -1), wrong) > softmax_err(sess.logits.view(3, -1), ref)
+
+
 # ------------------------------------------------------------------------------------------------
 # the 7B / 13B int4 configurations at their real widths
 # ------------------------------------------------------------------------------------------------
